@@ -1,0 +1,211 @@
+/*
+ * rpa.h -- C ABI of the MI355X (gfx950) ragged paged attention library.
+ *
+ * The reference project (sglang-jax) has no native FFI on this path: its
+ * operator boundary is a jitted Python callable.  Each entry point below names
+ * the reference callable it stands in for (paths relative to the reference
+ * checkout, python/sgl_jax/srt/...).  A jax.ffi custom call, a ctypes stub or
+ * any other host binds exactly these symbols.
+ *
+ * Conventions
+ *   - every pointer marked "device" is caller-owned device memory; the library
+ *     never allocates or frees device memory and never synchronises a stream;
+ *   - every launch is enqueued on the hipStream_t passed as `stream` (NULL is
+ *     the legacy default stream), so calls are graph-capturable;
+ *   - functions return RPA_OK (0) or a negative RpaStatus; rpa_last_error()
+ *     returns a thread-local, human readable description of the last failure;
+ *   - metadata (kv_lens, page_indices, cu_q_lens, cu_kv_lens) is read on the
+ *     device only.  Host copies can be checked with rpa_validate_host().
+ */
+#ifndef RPA_MI355_H_
+#define RPA_MI355_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RPA_VERSION 100 /* 0.1.0 */
+
+typedef enum RpaStatus {
+  RPA_OK = 0,
+  RPA_EINVAL_SHAPE = -1,
+  RPA_EINVAL_DTYPE = -2,
+  RPA_EINVAL_HEADS = -3,
+  RPA_EINVAL_PAGE_RANGE = -4,
+  RPA_EINVAL_QLEN_GT_KVLEN = -5,
+  RPA_EINVAL_WINDOW = -6,
+  RPA_EINVAL_SOFTCAP = -7,
+  RPA_EINVAL_WORKSPACE = -8,
+  RPA_EHIP = -9,
+  RPA_EINVAL_DISTRIBUTION = -10,
+  RPA_EUNSUPPORTED = -11,
+  RPA_EINVAL_NULL = -12
+} RpaStatus;
+
+typedef enum RpaKvDtype {
+  RPA_KV_BF16 = 0,
+  RPA_KV_FP8_E4M3 = 1 /* OCP e4m3fn, max 448 */
+} RpaKvDtype;
+
+typedef enum RpaLayout {
+  /* one buffer [pages, P, 2*Hkv, D], heads stored K0,V0,K1,V1,...
+   * (mem_cache/memory_pool.py:56-91, 580-588) */
+  RPA_LAYOUT_FUSED = 0,
+  /* two buffers k_pages, v_pages [pages, P, Hkv, D]
+   * (kernels/ragged_paged_attention/ragged_paged_attention_v3.py:96-97) */
+  RPA_LAYOUT_SPLIT = 1
+} RpaLayout;
+
+/*
+ * One ragged paged attention call.  Field meanings follow the arguments of
+ * ragged_paged_attention (ragged_paged_attention_v3.py:1667-1700) and of
+ * ref_ragged_paged_attention (same file, :94-114).
+ */
+typedef struct RpaParams {
+  /* ---- device buffers ---- */
+  const void* q;              /* bf16 [T, Hq, D] */
+  void* out;                  /* bf16 [T, Hq, D]; rows >= cu_q_lens[num_seqs] untouched */
+  const void* kv_cache;       /* FUSED: the cache; SPLIT: k_pages */
+  const void* v_pages;        /* SPLIT only, else NULL */
+  const int32_t* kv_lens;     /* i32[S]  (kv length INCLUDING the new q tokens) */
+  const int32_t* page_indices;/* i32 flat (cu_kv_lens != NULL) or [S, pages_per_seq] */
+  const int32_t* cu_q_lens;   /* i32[S+1] */
+  const int32_t* cu_kv_lens;  /* i32[S+1] cumulative page-aligned kv lens; NULL => padded 2-D table */
+  const float* k_scale;       /* f32[Hkv] dequantisation scale of K, or NULL (= 1) */
+  const float* v_scale;       /* f32[Hkv] or NULL */
+  void* workspace;            /* split-KV partials; >= rpa_workspace_bytes() */
+  size_t workspace_bytes;
+  /* ---- static shape ---- */
+  int32_t num_tokens;         /* T */
+  int32_t num_seqs;           /* S = distribution[2]: sequences to process */
+  int32_t num_q_heads;        /* Hq */
+  int32_t num_kv_heads;       /* Hkv, Hq % Hkv == 0 */
+  int32_t head_dim;           /* D (128 supported) */
+  int32_t page_size;          /* P */
+  int32_t total_pages;
+  int32_t pages_per_seq;      /* row stride of the padded table (cu_kv_lens == NULL) */
+  int32_t layout;             /* RpaLayout */
+  int32_t kv_dtype;           /* RpaKvDtype */
+  /* ---- batch composition: distribution = (decode_end, prefill_end, num_seqs)
+   *      (ragged_paged_attention_v3.py:82-91); sequences [0, decode_end) have
+   *      q_len == 1, the rest any q_len >= 1 ---- */
+  int32_t decode_end;
+  /* ---- host-side bounds used only to size grids (never to index memory) ---- */
+  int32_t max_kv_len;         /* upper bound of kv_lens[0:num_seqs]; 0 => pages_per_seq*P or total_pages*P */
+  int32_t max_q_len;          /* upper bound of q_len over [decode_end, num_seqs); 0 => T */
+  int32_t num_splits;         /* decode split-KV count per sequence; 0 => automatic */
+  /* ---- options ---- */
+  int32_t sliding_window;     /* 0 => off */
+  float sm_scale;
+  float soft_cap;             /* 0 => off */
+  float mask_value;           /* 0 => default -0.7 * FLT_MAX */
+} RpaParams;
+
+/*
+ * Absorbed-MLA decode (mla_ragged_paged_attention, kernels/mla/v2/kernel.py:1338-1370;
+ * oracle ref_mla_ragged_paged_attention, kernels/mla/v1/ref.py:108-248).
+ * One shared latent row per token: [kv_c (lkv_dim) | k_pe (rope_dim)], rows of
+ * `row_stride` elements (576 compact, 640 in the reference's 128-aligned layout
+ * with rope at element offset `rope_offset`).
+ */
+typedef struct RpaMlaParams {
+  const void* ql_nope;        /* bf16 [T, Hq, lkv_dim] */
+  const void* q_pe;           /* bf16 [T, Hq, rope_dim] */
+  void* out;                  /* bf16 [T, Hq, lkv_dim] */
+  const void* cache_kv;       /* bf16 [pages, P, row_stride] */
+  const int32_t* kv_lens;
+  const int32_t* page_indices;
+  const int32_t* cu_q_lens;
+  const int32_t* cu_kv_lens;  /* NULL => padded table with pages_per_seq stride */
+  void* workspace;
+  size_t workspace_bytes;
+  int32_t num_tokens;
+  int32_t num_seqs;           /* all must be decode rows (q_len == 1) */
+  int32_t num_q_heads;
+  int32_t lkv_dim;            /* 512 */
+  int32_t rope_dim;           /* 64 */
+  int32_t row_stride;         /* elements per cached token row */
+  int32_t rope_offset;        /* element offset of k_pe inside a row */
+  int32_t page_size;
+  int32_t total_pages;
+  int32_t pages_per_seq;
+  int32_t max_kv_len;
+  int32_t num_splits;         /* 0 => automatic */
+  int32_t sliding_window;     /* 0 => off */
+  float sm_scale;
+  float soft_cap;             /* 0 => off */
+  float mask_value;           /* 0 => default */
+} RpaMlaParams;
+
+/* Library version (RPA_VERSION of the build). */
+int rpa_version(void);
+
+/* Thread-local description of the last error returned on this thread. */
+const char* rpa_last_error(void);
+
+/*
+ * Static contract check: static_validate_inputs,
+ * ragged_paged_attention_v3.py:1314-1439 (3-D q, Hq % Hkv == 0,
+ * sliding_window > 0, soft_cap != 0, ...).  Called by every entry point.
+ */
+int rpa_validate(const RpaParams* p);
+
+/*
+ * Value check on HOST copies of the metadata: dynamic_validate_inputs,
+ * ragged_paged_attention_v3.py:1442-1487 (0 < q_len <= kv_len, page count and
+ * page index ranges, distribution ordering).  Pointers are host memory.
+ */
+int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t* page_indices,
+                      int64_t num_page_indices, const int32_t* cu_q_lens,
+                      const int32_t* cu_kv_lens, const int32_t* distribution);
+
+/* Bytes of split-KV workspace rpa_decode / rpa_attention need for `p`. */
+size_t rpa_workspace_bytes(const RpaParams* p);
+size_t rpa_mla_workspace_bytes(const RpaMlaParams* p);
+
+/*
+ * Page-table gather of one sequence (the indexing expression
+ * k_pages[page_indices[i]].reshape(-1, Hkv, D)[:kv_len] of
+ * ragged_paged_attention_v3.py:138-139).  Copies, bit for bit, the K rows and
+ * V rows of sequence `seq` into k_out / v_out [kv_len, Hkv, D] (kv dtype).
+ */
+int rpa_gather_pages(const RpaParams* p, int32_t seq, void* k_out, void* v_out,
+                     int32_t max_tokens, void* stream);
+
+/*
+ * Decode rows [0, decode_end): split-KV pass + combine pass.  Stands in for the
+ * DECODE pallas_call of ragged_paged_attention_v3.py:2065-2072.
+ */
+int rpa_decode(const RpaParams* p, void* stream);
+
+/*
+ * Prefill / mixed rows [decode_end, num_seqs): flash-style MFMA kernel.  Stands
+ * in for the PREFILL and MIXED pallas_calls, ragged_paged_attention_v3.py:2074-2090.
+ */
+int rpa_prefill(const RpaParams* p, void* stream);
+
+/*
+ * Whole call: dispatch by distribution exactly as
+ * ragged_paged_attention_v3.py:2060-2090 does (decode rows, then the rest).
+ */
+int rpa_attention(const RpaParams* p, void* stream);
+
+/*
+ * Scatter the new K/V rows of every sequence into the paged cache: the fused
+ * cache update of ragged_paged_attention_v3.py:670-719 / the standalone
+ * kv_cache_update of kernels/update_kv_cache/update_kv_cache.py:120.  Token j of
+ * sequence i goes to position kv_len_i - q_len_i + j.  keys/values are
+ * [T, Hkv, D] in the cache dtype.
+ */
+int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void* stream);
+
+/* Absorbed-MLA decode, see RpaMlaParams. */
+int rpa_mla_decode(const RpaMlaParams* p, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RPA_MI355_H_ */

@@ -1,0 +1,22 @@
+"""MI355X-native ragged paged attention behind sglang-jax's operator surface.
+
+The directory name carries a hyphen, so the package is registered under the
+importable name ``sglang_jax_amd`` by ``__graft_entry__.load_package()``.
+"""
+
+from . import _lib  # noqa: F401
+from .mla import mla_ragged_paged_attention  # noqa: F401
+from .ragged_paged_attention import (  # noqa: F401
+    DEFAULT_MASK_VALUE,
+    gather_pages,
+    ragged_paged_attention,
+    ragged_paged_attention_ref_surface,
+)
+
+__all__ = [
+    "DEFAULT_MASK_VALUE",
+    "gather_pages",
+    "mla_ragged_paged_attention",
+    "ragged_paged_attention",
+    "ragged_paged_attention_ref_surface",
+]

@@ -1,0 +1,66 @@
+"""Build recipe of the HIP library: ``python sglang-jax_amd/build.py``.
+
+Compiles every translation unit under ``csrc/`` for gfx950 with hipcc (it
+cross-compiles without a GPU) and links ``lib/librpa_mi355.so`` in-tree.
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OUT_DIR = os.path.join(HERE, "lib")
+LIB_PATH = os.path.join(OUT_DIR, "librpa_mi355.so")
+
+SOURCES = ["rpa_capi.hip", "rpa_decode.hip", "rpa_prefill.hip", "rpa_mla.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-fPIC",
+    "-std=c++17",
+    "-ffp-contract=fast",
+    # never let the compiler form packed-fp32 VALU ops
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+    noise = ("is not a recognized feature for this target",)
+    out = "\n".join(ln for ln in proc.stdout.splitlines() if not any(n in ln for n in noise))
+    return out
+
+
+def build(verbose: bool = False, extra_flags=()) -> str:
+    os.makedirs(OUT_DIR, exist_ok=True)
+    objs = []
+
+    def compile_one(src):
+        obj = os.path.join(OUT_DIR, src.replace(".hip", ".o"))
+        out = _run([HIPCC, *FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj])
+        if verbose and out.strip():
+            print(out)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    tmp = LIB_PATH + ".tmp"
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp])
+    os.replace(tmp, LIB_PATH)
+    for o in objs:
+        os.remove(o)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    path = build(verbose=True, extra_flags=sys.argv[1:])
+    print("built", path)

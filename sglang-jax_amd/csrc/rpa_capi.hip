@@ -1,0 +1,392 @@
+// C ABI of the library (declared in include/rpa.h): argument checking,
+// grid sizing from the host-side bounds, and dispatch to the kernel launchers.
+// No device allocation, no synchronisation, no host reads of device memory.
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "../../include/rpa.h"
+#include "rpa_kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  if (!v || !*v) return dflt;
+  return atoi(v);
+}
+
+constexpr float kDefaultMask = -0.7f * 3.4028234663852886e38f;
+
+int esize_of(int kv_dtype) { return kv_dtype == RPA_KV_FP8_E4M3 ? 1 : 2; }
+
+rpa::KvAddr kv_addr(const RpaParams* p) {
+  rpa::KvAddr kv;
+  const int es = esize_of(p->kv_dtype);
+  const int64_t D = p->head_dim, H = p->num_kv_heads, P = p->page_size;
+  kv.k_base = static_cast<const char*>(p->kv_cache);
+  if (p->layout == RPA_LAYOUT_FUSED) {
+    kv.v_base = kv.k_base + D * es;
+    kv.head_stride = (int32_t)(2 * D * es);
+    kv.tok_stride = (int32_t)(2 * H * D * es);
+  } else {
+    kv.v_base = static_cast<const char*>(p->v_pages);
+    kv.head_stride = (int32_t)(D * es);
+    kv.tok_stride = (int32_t)(H * D * es);
+  }
+  kv.page_stride = (int64_t)kv.tok_stride * P;
+  return kv;
+}
+
+rpa::PageTable page_table(const RpaParams* p) {
+  rpa::PageTable pt;
+  pt.kv_lens = p->kv_lens;
+  pt.page_indices = p->page_indices;
+  pt.cu_q_lens = p->cu_q_lens;
+  pt.cu_kv_lens = p->cu_kv_lens;
+  pt.pages_per_seq = p->pages_per_seq;
+  pt.page_size = p->page_size;
+  return pt;
+}
+
+rpa::SoftmaxOpts softmax_opts(float sm_scale, float soft_cap, float mask_value, int window) {
+  rpa::SoftmaxOpts s;
+  s.sm_scale = sm_scale;
+  s.soft_cap = soft_cap;
+  s.mask_value = (mask_value == 0.0f) ? kDefaultMask : mask_value;
+  s.window = window;
+  return s;
+}
+
+int64_t kv_len_bound(int max_kv_len, int pages_per_seq, int page_size, int total_pages, bool ragged) {
+  if (max_kv_len > 0) return max_kv_len;
+  if (!ragged && pages_per_seq > 0) return (int64_t)pages_per_seq * page_size;
+  return (int64_t)total_pages * page_size;
+}
+
+// Split-KV plan.  `units` = independent wave jobs per split (rows * kv heads).
+// Aim for a few thousand waves on the 256-CU part while keeping every split at
+// least `min_chunk` tokens long so the partial write stays negligible.
+struct SplitPlan {
+  int chunk;
+  int splits;
+};
+
+SplitPlan plan_splits(int64_t max_len, int window, int64_t units, int forced, int min_chunk, int target) {
+  int64_t eff = max_len;
+  if (window > 0 && eff > (int64_t)window + 31) eff = (int64_t)window + 31;
+  if (eff < 1) eff = 1;
+  int64_t splits;
+  if (forced > 0) {
+    splits = forced;
+  } else {
+    splits = (target + units - 1) / (units > 0 ? units : 1);
+    const int64_t cap = (eff + min_chunk - 1) / min_chunk;
+    if (splits > cap) splits = cap;
+    if (splits < 1) splits = 1;
+  }
+  int64_t chunk = (eff + splits - 1) / splits;
+  chunk = (chunk + 31) / 32 * 32;
+  if (chunk < 32) chunk = 32;
+  splits = (eff + chunk - 1) / chunk;
+  if (splits < 1) splits = 1;
+  SplitPlan sp;
+  sp.chunk = (int)chunk;
+  sp.splits = (int)splits;
+  return sp;
+}
+
+SplitPlan decode_plan(const RpaParams* p) {
+  const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
+                                     p->cu_kv_lens != nullptr);
+  const int64_t units = (int64_t)p->decode_end * p->num_kv_heads;
+  return plan_splits(bound, p->sliding_window, units, p->num_splits,
+                     env_int("RPA_DECODE_MIN_CHUNK", 128), env_int("RPA_DECODE_TARGET_WAVES", 4096));
+}
+
+int check_hip(hipError_t e, const char* what) {
+  if (e == hipSuccess) return RPA_OK;
+  return fail(RPA_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+}  // namespace
+
+extern "C" {
+
+int rpa_version(void) { return RPA_VERSION; }
+
+const char* rpa_last_error(void) { return g_err; }
+
+int rpa_validate(const RpaParams* p) {
+  if (!p) return fail(RPA_EINVAL_NULL, "params is NULL");
+  if (p->num_tokens < 0 || p->num_seqs < 0 || p->num_q_heads <= 0 || p->num_kv_heads <= 0 ||
+      p->head_dim <= 0 || p->page_size <= 0 || p->total_pages <= 0)
+    return fail(RPA_EINVAL_SHAPE, "expected positive shape: T=%d S=%d Hq=%d Hkv=%d D=%d P=%d pages=%d",
+                p->num_tokens, p->num_seqs, p->num_q_heads, p->num_kv_heads, p->head_dim,
+                p->page_size, p->total_pages);
+  if (p->num_q_heads % p->num_kv_heads != 0)
+    return fail(RPA_EINVAL_HEADS, "expected num_q_heads=%d to be divisible by num_kv_heads=%d",
+                p->num_q_heads, p->num_kv_heads);
+  if (p->head_dim != 128)
+    return fail(RPA_EUNSUPPORTED, "head_dim=%d: only 128 is built", p->head_dim);
+  if (p->kv_dtype != RPA_KV_BF16 && p->kv_dtype != RPA_KV_FP8_E4M3)
+    return fail(RPA_EINVAL_DTYPE, "kv_dtype=%d is not a floating point cache dtype", p->kv_dtype);
+  if (p->layout != RPA_LAYOUT_FUSED && p->layout != RPA_LAYOUT_SPLIT)
+    return fail(RPA_EINVAL_SHAPE, "layout=%d unknown", p->layout);
+  if (p->layout == RPA_LAYOUT_SPLIT && !p->v_pages)
+    return fail(RPA_EINVAL_NULL, "split layout needs v_pages");
+  if (p->sliding_window < 0) return fail(RPA_EINVAL_WINDOW, "sliding_window=%d must be positive", p->sliding_window);
+  if (std::isnan(p->soft_cap)) return fail(RPA_EINVAL_SOFTCAP, "soft_cap must not be NaN");
+  if (p->decode_end < 0 || p->decode_end > p->num_seqs)
+    return fail(RPA_EINVAL_DISTRIBUTION, "distribution must satisfy 0 <= decode_end=%d <= num_seqs=%d",
+                p->decode_end, p->num_seqs);
+  if (p->num_seqs > 0) {
+    if (!p->q || !p->out || !p->kv_cache || !p->kv_lens || !p->page_indices || !p->cu_q_lens)
+      return fail(RPA_EINVAL_NULL, "q/out/kv_cache/kv_lens/page_indices/cu_q_lens must be non-NULL");
+    if (!p->cu_kv_lens && p->pages_per_seq <= 0)
+      return fail(RPA_EINVAL_SHAPE, "padded page table needs pages_per_seq > 0");
+  }
+  if (p->mask_value > 0.0f) return fail(RPA_EINVAL_SHAPE, "mask_value=%g must be negative", p->mask_value);
+  return RPA_OK;
+}
+
+int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t* page_indices,
+                      int64_t num_page_indices, const int32_t* cu_q_lens, const int32_t* cu_kv_lens,
+                      const int32_t* distribution) {
+  int rc = rpa_validate(p);
+  if (rc != RPA_OK) return rc;
+  if (!kv_lens || !page_indices || !cu_q_lens) return fail(RPA_EINVAL_NULL, "host metadata is NULL");
+  int i = 0, j = 0, k = p->num_seqs;
+  if (distribution) {
+    i = distribution[0]; j = distribution[1]; k = distribution[2];
+    if (!(i <= j && j <= k)) return fail(RPA_EINVAL_DISTRIBUTION, "distribution must satisfy i <= j <= k, got %d, %d, %d", i, j, k);
+    if (k != p->num_seqs || i != p->decode_end)
+      return fail(RPA_EINVAL_DISTRIBUTION, "distribution (%d,%d,%d) disagrees with decode_end=%d num_seqs=%d", i, j, k, p->decode_end, p->num_seqs);
+  } else {
+    i = p->decode_end;
+  }
+  if (cu_q_lens[k] > p->num_tokens)
+    return fail(RPA_EINVAL_SHAPE, "cu_q_lens[%d]=%d exceeds max_num_tokens=%d", k, cu_q_lens[k], p->num_tokens);
+  const int P = p->page_size;
+  for (int s = 0; s < k; ++s) {
+    const int q_len = cu_q_lens[s + 1] - cu_q_lens[s];
+    const int kv_len = kv_lens[s];
+    if (q_len <= 0) return fail(RPA_EINVAL_QLEN_GT_KVLEN, "Sequence %d: q_len=%d must be > 0", s, q_len);
+    if (q_len > kv_len) return fail(RPA_EINVAL_QLEN_GT_KVLEN, "Sequence %d: q_len=%d > kv_len=%d", s, q_len, kv_len);
+    if (s < i && q_len != 1) return fail(RPA_EINVAL_DISTRIBUTION, "Sequence %d is in the decode range but q_len=%d", s, q_len);
+    const int page_cnt = (kv_len + P - 1) / P;
+    int64_t start;
+    if (cu_kv_lens) {
+      if (cu_kv_lens[s] % P != 0) return fail(RPA_EINVAL_SHAPE, "cu_kv_lens[%d]=%d is not page aligned", s, cu_kv_lens[s]);
+      if (cu_kv_lens[s + 1] - cu_kv_lens[s] < page_cnt * P)
+        return fail(RPA_EINVAL_PAGE_RANGE, "Sequence %d: page_cnt=%d does not fit cu_kv_lens", s, page_cnt);
+      start = cu_kv_lens[s] / P;
+    } else {
+      if (page_cnt > p->pages_per_seq)
+        return fail(RPA_EINVAL_PAGE_RANGE, "Sequence %d: page_cnt=%d > pages_per_seq=%d", s, page_cnt, p->pages_per_seq);
+      start = (int64_t)s * p->pages_per_seq;
+    }
+    if (start + page_cnt > num_page_indices)
+      return fail(RPA_EINVAL_PAGE_RANGE, "Sequence %d: page list [%lld, %lld) exceeds page_indices length %lld", s,
+                  (long long)start, (long long)(start + page_cnt), (long long)num_page_indices);
+    for (int pg = 0; pg < page_cnt; ++pg) {
+      const int idx = page_indices[start + pg];
+      if (idx < 0 || idx >= p->total_pages)
+        return fail(RPA_EINVAL_PAGE_RANGE, "Sequence %d, page %d: index=%d out of [0, %d)", s, pg, idx, p->total_pages);
+    }
+    if (p->max_kv_len > 0 && kv_len > p->max_kv_len)
+      return fail(RPA_EINVAL_SHAPE, "Sequence %d: kv_len=%d exceeds max_kv_len=%d", s, kv_len, p->max_kv_len);
+    if (s >= i && p->max_q_len > 0 && q_len > p->max_q_len)
+      return fail(RPA_EINVAL_SHAPE, "Sequence %d: q_len=%d exceeds max_q_len=%d", s, q_len, p->max_q_len);
+  }
+  return RPA_OK;
+}
+
+size_t rpa_workspace_bytes(const RpaParams* p) {
+  if (!p || p->decode_end <= 0) return 0;
+  const SplitPlan sp = decode_plan(p);
+  if (sp.splits <= 1) return 0;
+  return (size_t)p->decode_end * sp.splits * p->num_q_heads * (p->head_dim + 2) * sizeof(float);
+}
+
+int rpa_gather_pages(const RpaParams* p, int32_t seq, void* k_out, void* v_out, int32_t max_tokens,
+                     void* stream) {
+  int rc = rpa_validate(p);
+  if (rc != RPA_OK) return rc;
+  if (seq < 0 || seq >= p->num_seqs) return fail(RPA_EINVAL_SHAPE, "seq=%d out of [0, %d)", seq, p->num_seqs);
+  if (!k_out || !v_out) return fail(RPA_EINVAL_NULL, "k_out/v_out is NULL");
+  rpa::GatherArgs a;
+  a.kv = kv_addr(p);
+  a.pt = page_table(p);
+  a.seq = seq;
+  a.Hkv = p->num_kv_heads;
+  a.head_bytes = p->head_dim * esize_of(p->kv_dtype);
+  a.row_bytes = a.Hkv * a.head_bytes;
+  a.k_out = k_out;
+  a.v_out = v_out;
+  a.max_tokens = max_tokens;
+  return check_hip(rpa::launch_gather(a, static_cast<hipStream_t>(stream)), "rpa_gather_pages");
+}
+
+int rpa_decode(const RpaParams* p, void* stream) {
+  int rc = rpa_validate(p);
+  if (rc != RPA_OK) return rc;
+  if (p->decode_end <= 0) return RPA_OK;
+  const SplitPlan sp = decode_plan(p);
+  rpa::DecodeArgs a;
+  a.q = static_cast<const uint16_t*>(p->q);
+  a.out = static_cast<uint16_t*>(p->out);
+  a.kv = kv_addr(p);
+  a.pt = page_table(p);
+  a.sm = softmax_opts(p->sm_scale, p->soft_cap, p->mask_value, p->sliding_window);
+  a.k_scale = p->k_scale;
+  a.v_scale = p->v_scale;
+  a.num_rows = p->decode_end;
+  a.Hq = p->num_q_heads;
+  a.Hkv = p->num_kv_heads;
+  a.G = p->num_q_heads / p->num_kv_heads;
+  a.chunk = sp.chunk;
+  a.max_splits = sp.splits;
+  a.fp8 = p->kv_dtype == RPA_KV_FP8_E4M3;
+  a.ws_o = nullptr;
+  a.ws_ml = nullptr;
+  if (sp.splits > 1) {
+    const size_t need = rpa_workspace_bytes(p);
+    if (!p->workspace || p->workspace_bytes < need)
+      return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
+    a.ws_o = static_cast<float*>(p->workspace);
+    a.ws_ml = a.ws_o + (size_t)p->decode_end * sp.splits * p->num_q_heads * p->head_dim;
+  }
+  return check_hip(rpa::launch_decode(a, static_cast<hipStream_t>(stream)), "rpa_decode");
+}
+
+int rpa_prefill(const RpaParams* p, void* stream) {
+  int rc = rpa_validate(p);
+  if (rc != RPA_OK) return rc;
+  if (p->num_seqs <= p->decode_end) return RPA_OK;
+  rpa::PrefillArgs a;
+  a.q = static_cast<const uint16_t*>(p->q);
+  a.out = static_cast<uint16_t*>(p->out);
+  a.kv = kv_addr(p);
+  a.pt = page_table(p);
+  a.sm = softmax_opts(p->sm_scale, p->soft_cap, p->mask_value, p->sliding_window);
+  a.k_scale = p->k_scale;
+  a.v_scale = p->v_scale;
+  a.seq_begin = p->decode_end;
+  a.seq_end = p->num_seqs;
+  a.Hq = p->num_q_heads;
+  a.Hkv = p->num_kv_heads;
+  a.G = p->num_q_heads / p->num_kv_heads;
+  a.max_q_len = p->max_q_len > 0 ? p->max_q_len : p->num_tokens;
+  a.fp8 = p->kv_dtype == RPA_KV_FP8_E4M3;
+  return check_hip(rpa::launch_prefill(a, static_cast<hipStream_t>(stream)), "rpa_prefill");
+}
+
+int rpa_attention(const RpaParams* p, void* stream) {
+  int rc = rpa_decode(p, stream);
+  if (rc != RPA_OK) return rc;
+  return rpa_prefill(p, stream);
+}
+
+int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void* stream) {
+  int rc = rpa_validate(p);
+  if (rc != RPA_OK) return rc;
+  if (!keys || !values) return fail(RPA_EINVAL_NULL, "keys/values is NULL");
+  rpa::KvWriteArgs a;
+  a.kv = kv_addr(p);
+  a.pt = page_table(p);
+  a.keys = static_cast<const char*>(keys);
+  a.values = static_cast<const char*>(values);
+  a.num_seqs = p->num_seqs;
+  a.Hkv = p->num_kv_heads;
+  a.head_bytes = p->head_dim * esize_of(p->kv_dtype);
+  a.num_tokens = p->num_tokens;
+  return check_hip(rpa::launch_kv_write(a, static_cast<hipStream_t>(stream)), "rpa_kv_write");
+}
+
+// ---------------------------------------------------------------- MLA ----
+
+static SplitPlan mla_plan(const RpaMlaParams* p) {
+  const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
+                                     p->cu_kv_lens != nullptr);
+  return plan_splits(bound, p->sliding_window, p->num_seqs, p->num_splits,
+                     env_int("RPA_MLA_MIN_CHUNK", 256), env_int("RPA_MLA_TARGET_WGS", 512));
+}
+
+static int mla_validate(const RpaMlaParams* p) {
+  if (!p) return fail(RPA_EINVAL_NULL, "params is NULL");
+  if (p->num_seqs < 0 || p->num_q_heads <= 0 || p->page_size <= 0 || p->total_pages <= 0)
+    return fail(RPA_EINVAL_SHAPE, "expected positive shape");
+  if (p->lkv_dim != 512 || p->rope_dim != 64)
+    return fail(RPA_EUNSUPPORTED, "lkv_dim=%d rope_dim=%d: only 512+64 is built", p->lkv_dim, p->rope_dim);
+  if (p->row_stride < p->rope_offset + p->rope_dim || p->rope_offset < p->lkv_dim || (p->row_stride % 8) != 0 ||
+      (p->rope_offset % 8) != 0)
+    return fail(RPA_EINVAL_SHAPE, "row_stride=%d rope_offset=%d do not describe [kv_c | k_pe]", p->row_stride, p->rope_offset);
+  if (p->num_q_heads % 16 != 0) return fail(RPA_EUNSUPPORTED, "num_q_heads=%d must be a multiple of 16", p->num_q_heads);
+  if (p->sliding_window < 0) return fail(RPA_EINVAL_WINDOW, "sliding_window=%d must be positive", p->sliding_window);
+  if (p->num_seqs > p->num_tokens) return fail(RPA_EINVAL_SHAPE, "decode rows=%d exceed tokens=%d", p->num_seqs, p->num_tokens);
+  if (p->num_seqs > 0 && (!p->ql_nope || !p->q_pe || !p->out || !p->cache_kv || !p->kv_lens || !p->page_indices || !p->cu_q_lens))
+    return fail(RPA_EINVAL_NULL, "a required buffer is NULL");
+  if (!p->cu_kv_lens && p->pages_per_seq <= 0 && p->num_seqs > 0)
+    return fail(RPA_EINVAL_SHAPE, "padded page table needs pages_per_seq > 0");
+  return RPA_OK;
+}
+
+size_t rpa_mla_workspace_bytes(const RpaMlaParams* p) {
+  if (!p || p->num_seqs <= 0) return 0;
+  const SplitPlan sp = mla_plan(p);
+  if (sp.splits <= 1) return 0;
+  return (size_t)p->num_seqs * sp.splits * p->num_q_heads * (p->lkv_dim + 2) * sizeof(float);
+}
+
+int rpa_mla_decode(const RpaMlaParams* p, void* stream) {
+  int rc = mla_validate(p);
+  if (rc != RPA_OK) return rc;
+  if (p->num_seqs <= 0) return RPA_OK;
+  const SplitPlan sp = mla_plan(p);
+  rpa::MlaDecodeArgs a;
+  a.ql_nope = static_cast<const uint16_t*>(p->ql_nope);
+  a.q_pe = static_cast<const uint16_t*>(p->q_pe);
+  a.out = static_cast<uint16_t*>(p->out);
+  a.cache = static_cast<const char*>(p->cache_kv);
+  a.pt.kv_lens = p->kv_lens;
+  a.pt.page_indices = p->page_indices;
+  a.pt.cu_q_lens = p->cu_q_lens;
+  a.pt.cu_kv_lens = p->cu_kv_lens;
+  a.pt.pages_per_seq = p->pages_per_seq;
+  a.pt.page_size = p->page_size;
+  a.sm = softmax_opts(p->sm_scale, p->soft_cap, p->mask_value, p->sliding_window);
+  a.num_rows = p->num_seqs;
+  a.Hq = p->num_q_heads;
+  a.row_stride = p->row_stride;
+  a.rope_offset = p->rope_offset;
+  a.chunk = sp.chunk;
+  a.max_splits = sp.splits;
+  a.ws_o = nullptr;
+  a.ws_ml = nullptr;
+  if (sp.splits > 1) {
+    const size_t need = rpa_mla_workspace_bytes(p);
+    if (!p->workspace || p->workspace_bytes < need)
+      return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
+    a.ws_o = static_cast<float*>(p->workspace);
+    a.ws_ml = a.ws_o + (size_t)p->num_seqs * sp.splits * p->num_q_heads * p->lkv_dim;
+  }
+  return check_hip(rpa::launch_mla_decode(a, static_cast<hipStream_t>(stream)), "rpa_mla_decode");
+}
+
+}  // extern "C"

@@ -1,0 +1,75 @@
+// Shared device helpers for the gfx950 ragged paged attention kernels.
+//
+// Wavefront = 64 lanes.  Matrix work uses the CDNA4 bf16 MFMA instructions
+//   v_mfma_f32_16x16x32_bf16 : A[16x32] B[32x16] -> C[16x16] f32
+//   v_mfma_f32_32x32x16_bf16 : A[32x16] B[16x32] -> C[32x32] f32
+// with the operand layouts (lane l, c = l % 16, g = l / 16):
+//   16x16x32  A: row c, k = 8g..8g+7     B: col c, k = 8g..8g+7
+//             C: col c, rows 4g..4g+3 in the 4 result registers
+//   32x32x16  (c = l % 32, h = l / 32)
+//             A: row c, k = 8h..8h+7     B: col c, k = 8h..8h+7
+//             C: col c, rows 8*(v/4) + 4h + (v%4) in result register v = 0..15
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rpa {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kDefaultMaskValue = -0.7f * 3.4028234663852886e38f;
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2_t f = {lo, hi};
+  bf16x2_t h = __builtin_convertvector(f, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, h);
+}
+
+__device__ __forceinline__ float bf16_lo_to_f32(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi_to_f32(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+__device__ __forceinline__ f32x4_t mfma16(u32x4_t a, u32x4_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// cap * tanh(x / cap), written so that +-inf arguments give +-cap.
+__device__ __forceinline__ float soft_cap_f(float x, float cap, float inv_cap) {
+  float e = __expf(2.0f * x * inv_cap);
+  return cap * (1.0f - 2.0f / (e + 1.0f));
+}
+
+// 16-byte global loads / stores.
+__device__ __forceinline__ u32x4_t ld16(const void* p) { return *reinterpret_cast<const u32x4_t*>(p); }
+__device__ __forceinline__ u32x2_t ld8(const void* p) { return *reinterpret_cast<const u32x2_t*>(p); }
+__device__ __forceinline__ void st16(void* p, u32x4_t v) { *reinterpret_cast<u32x4_t*>(p) = v; }
+
+// Two fp8-e4m3 bytes (low or high half of `w`) -> two f32.
+__device__ __forceinline__ f32x2_t fp8x2_to_f32(uint32_t w, bool hi) {
+  return hi ? __builtin_amdgcn_cvt_pk_f32_fp8(w, true) : __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+}
+
+// Four fp8-e4m3 bytes -> four bf16 packed in two dwords (exact: e4m3 fits bf16).
+__device__ __forceinline__ u32x2_t fp8x4_to_bf16x4(uint32_t w) {
+  f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+  f32x2_t b = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+  u32x2_t r = {pack_bf16x2(a[0], a[1]), pack_bf16x2(b[0], b[1])};
+  return r;
+}
+
+}  // namespace rpa

@@ -1,0 +1,486 @@
+// Split-KV decode for ragged paged attention on gfx950, plus the combine pass,
+// the page-table gather and the new-token cache write.
+//
+// Decode is HBM-bound: every visible KV token is read exactly once.  One
+// wavefront owns one (sequence, kv head, kv split) and streams that head's K
+// and V rows (adjacent in the head-interleaved cache: K_h | V_h = 2*D elements)
+// through the page table with 16-byte loads straight into the MFMA operand
+// layout -- no LDS, no barriers, so every wave is independent and the grid is
+// just "enough waves to keep ~16 KiB per wave in flight on every SIMD".
+//
+// Per 32-token block (bf16):
+//   S^T[tok, qrow] = K[tok, :] . Q^T        2 x 4 MFMA 16x16x32 (A = K, B = Q^T)
+//   online softmax on the 8 scores each lane holds (row stats need one
+//   cross-lane max over the 4 lane groups)
+//   O^T[dim, qrow] += V^T[dim, tok] . P^T   8 MFMA 16x16x32 (A = V^T, B = P^T)
+// The S^T result layout (lane = q row, registers = tokens) is already the B
+// operand layout of the second product when the 32 tokens of a block are
+// enumerated as slot(g, i) = (i < 4 ? 4g + i : 16 + 4g + i - 4); V is loaded in
+// that token order and transposed in registers with v_perm_b32 (two bf16 of
+// neighbouring tokens -> one dword), 32 permutes per block.
+// GQA: the G query heads of a kv head are the (zero padded) 16 columns of Q^T.
+
+#include "rpa_common.h"
+#include "rpa_kernels.h"
+
+namespace rpa {
+
+namespace {
+
+constexpr int kBlk = 32;
+
+__device__ __forceinline__ int tok_slot(int g, int i) {
+  return (i < 4) ? (g * 4 + i) : (16 + g * 4 + (i - 4));
+}
+
+template <bool FP8>
+struct KvRegs;
+template <>
+struct KvRegs<false> {
+  u32x4_t k[2][4];  // [token half][k step]: 8 bf16 of dims 32*s + 8*g ..
+  u32x4_t v[8];     // [slot]: 8 bf16 of dims 8*c ..
+};
+template <>
+struct KvRegs<true> {
+  u32x4_t k[2][2];  // 32 fp8 of dims 32*g ..
+  u32x2_t v[8];     // 8 fp8 of dims 8*c ..
+};
+
+struct SeqView {
+  const int32_t* pages;  // this sequence's page ids
+  int32_t page_size;
+  int32_t page_shift;  // >= 0 when page_size is a power of two
+  int32_t last_tok;    // kv_len - 1
+};
+
+__device__ __forceinline__ int page_slot_of(const SeqView& s, int tok) {
+  return s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
+}
+
+// Issue the global loads of one 32-token block.  Token indices are clamped to
+// the last valid token so that nothing past kv_len (and nothing past the
+// sequence's page list) is ever dereferenced; clamped rows are masked later.
+template <bool FP8, bool UNIFORM_PAGE>
+__device__ __forceinline__ void load_block(KvRegs<FP8>& r, const SeqView& s, const KvAddr& kv,
+                                           const char* kh, const char* vh, int tb, int c, int g) {
+  constexpr int kLaneK = FP8 ? 32 : 16;  // byte offset step of lane group g inside a K row
+  constexpr int kLaneV = FP8 ? 8 : 16;   // byte offset step of lane c inside a V row
+  if constexpr (UNIFORM_PAGE) {
+    const int slot = page_slot_of(s, tb);
+    const int page = __builtin_amdgcn_readfirstlane(s.pages[slot]);
+    const char* kp = kh + (int64_t)page * kv.page_stride;
+    const char* vp = vh + (int64_t)page * kv.page_stride;
+    const int t0 = slot * s.page_size;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int tin = min(tb + b * 16 + c, s.last_tok) - t0;
+      const uint32_t off = (uint32_t)(tin * kv.tok_stride + g * kLaneK);
+      if constexpr (FP8) {
+        r.k[b][0] = ld16(kp + off);
+        r.k[b][1] = ld16(kp + off + 16);
+      } else {
+#pragma unroll
+        for (int st = 0; st < 4; ++st) r.k[b][st] = ld16(kp + off + st * 64);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int tin = min(tb + tok_slot(g, i), s.last_tok) - t0;
+      const uint32_t off = (uint32_t)(tin * kv.tok_stride + c * kLaneV);
+      if constexpr (FP8) r.v[i] = ld8(vp + off);
+      else r.v[i] = ld16(vp + off);
+    }
+  } else {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int tok = min(tb + b * 16 + c, s.last_tok);
+      const int slot = page_slot_of(s, tok);
+      const int page = s.pages[slot];
+      const char* kp = kh + (int64_t)page * kv.page_stride +
+                       (int64_t)((tok - slot * s.page_size) * kv.tok_stride + g * kLaneK);
+      if constexpr (FP8) {
+        r.k[b][0] = ld16(kp);
+        r.k[b][1] = ld16(kp + 16);
+      } else {
+#pragma unroll
+        for (int st = 0; st < 4; ++st) r.k[b][st] = ld16(kp + st * 64);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int tok = min(tb + tok_slot(g, i), s.last_tok);
+      const int slot = page_slot_of(s, tok);
+      const int page = s.pages[slot];
+      const char* vp = vh + (int64_t)page * kv.page_stride +
+                       (int64_t)((tok - slot * s.page_size) * kv.tok_stride + c * kLaneV);
+      if constexpr (FP8) r.v[i] = ld8(vp);
+      else r.v[i] = ld16(vp);
+    }
+  }
+}
+
+struct ScoreOpts {
+  float scale;      // sm_scale * k_scale            (soft-cap path)
+  float scale2;     // sm_scale * k_scale * log2(e)  (plain path)
+  float cap, inv_cap;
+  float mask2;      // mask value in log2 units (finite)
+  int t_lo;         // first visible token (sliding window), 0 otherwise
+  int kv_len;
+};
+
+template <int MT, bool FP8>
+__device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_t (&qB)[MT][4],
+                                              f32x4_t (&acc)[MT][8], float (&m)[MT], float (&l)[MT],
+                                              const ScoreOpts& so, int tb, int g) {
+  // ---- K operands (A of S^T = K Q^T) ----
+  u32x4_t kA[2][4];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    if constexpr (FP8) {
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const uint32_t w0 = r.k[b][st >> 1][(st & 1) * 2 + 0];
+        const uint32_t w1 = r.k[b][st >> 1][(st & 1) * 2 + 1];
+        const u32x2_t lo = fp8x4_to_bf16x4(w0);
+        const u32x2_t hi = fp8x4_to_bf16x4(w1);
+        kA[b][st] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+      }
+    } else {
+#pragma unroll
+      for (int st = 0; st < 4; ++st) kA[b][st] = r.k[b][st];
+    }
+  }
+  // ---- V^T operands (A of O^T = V^T P^T), one per output dim j of the lane's 8-dim chunk ----
+  u32x4_t vA[8];
+  if constexpr (FP8) {
+    float f[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const f32x2_t a0 = __builtin_amdgcn_cvt_pk_f32_fp8(r.v[i][0], false);
+      const f32x2_t a1 = __builtin_amdgcn_cvt_pk_f32_fp8(r.v[i][0], true);
+      const f32x2_t a2 = __builtin_amdgcn_cvt_pk_f32_fp8(r.v[i][1], false);
+      const f32x2_t a3 = __builtin_amdgcn_cvt_pk_f32_fp8(r.v[i][1], true);
+      f[i][0] = a0[0]; f[i][1] = a0[1]; f[i][2] = a1[0]; f[i][3] = a1[1];
+      f[i][4] = a2[0]; f[i][5] = a2[1]; f[i][6] = a3[0]; f[i][7] = a3[1];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      vA[j] = u32x4_t{pack_bf16x2(f[0][j], f[1][j]), pack_bf16x2(f[2][j], f[3][j]),
+                      pack_bf16x2(f[4][j], f[5][j]), pack_bf16x2(f[6][j], f[7][j])};
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+      const int jj = j >> 1;
+      vA[j] = u32x4_t{__builtin_amdgcn_perm(r.v[1][jj], r.v[0][jj], sel),
+                      __builtin_amdgcn_perm(r.v[3][jj], r.v[2][jj], sel),
+                      __builtin_amdgcn_perm(r.v[5][jj], r.v[4][jj], sel),
+                      __builtin_amdgcn_perm(r.v[7][jj], r.v[6][jj], sel)};
+    }
+  }
+  const bool need_mask = (tb + kBlk > so.kv_len) || (tb < so.t_lo);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    f32x4_t s[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      s[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int st = 0; st < 4; ++st) s[b] = mfma16(kA[b][st], qB[mt][st], s[b]);
+    }
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float v = s[i >> 2][i & 3];
+      if (so.cap != 0.f) v = soft_cap_f(v * so.scale, so.cap, so.inv_cap) * kLog2e;
+      else v = v * so.scale2;
+      x[i] = v;
+    }
+    if (need_mask) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int tok = tb + tok_slot(g, i);
+        if (tok >= so.kv_len || tok < so.t_lo) x[i] = so.mask2;
+      }
+    }
+    float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])),
+                     fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m[mt], mx);
+    const float alpha = fast_exp2(m[mt] - m_new);
+    float p[8];
+    float ps = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      p[i] = fast_exp2(x[i] - m_new);
+      ps += p[i];
+    }
+    l[mt] = l[mt] * alpha + ps;
+    m[mt] = m_new;
+    const u32x4_t pB = u32x4_t{pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]),
+                               pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7])};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      acc[mt][j] = acc[mt][j] * alpha;
+      acc[mt][j] = mfma16(vA[j], pB, acc[mt][j]);
+    }
+  }
+}
+
+__device__ __forceinline__ int first_block_token(int kv_len, int window) {
+  const int t_lo = (window > 0) ? max(0, kv_len - window) : 0;
+  return t_lo & ~(kBlk - 1);
+}
+
+// grid = (max_splits, decode rows, head groups * row groups); block = NW waves.
+template <int MT, bool FP8, bool UNIFORM_PAGE>
+__global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const DecodeArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int seq = blockIdx.y;
+  const int split = blockIdx.x;
+  const int head_groups = (a.Hkv + nw - 1) / nw;
+  const int hg = blockIdx.z % head_groups;
+  const int rg = blockIdx.z / head_groups;
+  const int hk = hg * nw + wave;
+  if (hk >= a.Hkv) return;
+
+  const int kv_len = a.pt.kv_lens[seq];
+  const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
+  const int t0 = t_lo & ~(kBlk - 1);
+  const int t_begin = t0 + split * a.chunk;
+  if (t_begin >= kv_len) return;
+  // the last split runs to kv_len even if the host's length bound was too small
+  const int t_end = (split == a.max_splits - 1) ? kv_len : min(kv_len, t_begin + a.chunk);
+  const int nblk = (t_end - t_begin + kBlk - 1) / kBlk;
+
+  SeqView sv;
+  sv.page_size = a.pt.page_size;
+  sv.page_shift = ((sv.page_size & (sv.page_size - 1)) == 0) ? (31 - __builtin_clz(sv.page_size)) : -1;
+  sv.last_tok = kv_len - 1;
+  sv.pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[seq] / a.pt.page_size)
+                                                  : (int64_t)seq * a.pt.pages_per_seq);
+
+  const char* kh = a.kv.k_base + (int64_t)hk * a.kv.head_stride;
+  const char* vh = a.kv.v_base + (int64_t)hk * a.kv.head_stride;
+
+  // ---- Q^T operands: column c = query head (row0 + 16*mt + c) of this kv head ----
+  const int tq = a.pt.cu_q_lens[seq];
+  const int row0 = rg * 16 * MT;
+  u32x4_t qB[MT][4];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int row = row0 + mt * 16 + c;
+    const uint16_t* qp = a.q + ((int64_t)tq * a.Hq + (int64_t)hk * a.G + row) * 128;
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      const int d0 = FP8 ? (g * 32 + st * 8) : (st * 32 + g * 8);
+      qB[mt][st] = (row < a.G) ? ld16(qp + d0) : u32x4_t{0u, 0u, 0u, 0u};
+    }
+  }
+
+  ScoreOpts so;
+  const float ks = a.k_scale ? a.k_scale[hk] : 1.0f;
+  so.scale = a.sm.sm_scale * ks;
+  so.scale2 = so.scale * kLog2e;
+  so.cap = a.sm.soft_cap;
+  so.inv_cap = (so.cap != 0.f) ? 1.0f / so.cap : 0.f;
+  so.mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
+  so.t_lo = t_lo;
+  so.kv_len = kv_len;
+
+  f32x4_t acc[MT][8];
+  float m[MT], l[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    m[mt] = -INFINITY;
+    l[mt] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[mt][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // ---- software pipeline: the loads of block i+1 are in flight while block i is consumed ----
+  KvRegs<FP8> ra, rb;
+  load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, t_begin, c, g);
+  int blk = 0;
+  while (true) {
+    if (blk + 1 < nblk) load_block<FP8, UNIFORM_PAGE>(rb, sv, a.kv, kh, vh, t_begin + (blk + 1) * kBlk, c, g);
+    compute_block<MT, FP8>(ra, qB, acc, m, l, so, t_begin + blk * kBlk, g);
+    if (++blk >= nblk) break;
+    if (blk + 1 < nblk) load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, t_begin + (blk + 1) * kBlk, c, g);
+    compute_block<MT, FP8>(rb, qB, acc, m, l, so, t_begin + blk * kBlk, g);
+    if (++blk >= nblk) break;
+  }
+
+  // ---- epilogue: lane (c, g) holds q row c, dims 32g + 8r + j in acc[mt][j][r] ----
+  const float vs = a.v_scale ? a.v_scale[hk] : 1.0f;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    float lt = l[mt];
+    lt += __shfl_xor(lt, 16);
+    lt += __shfl_xor(lt, 32);
+    const int row = row0 + mt * 16 + c;
+    if (row >= a.G) continue;
+    const int head = hk * a.G + row;
+    if (a.max_splits == 1) {
+      const float inv = vs / lt;
+      uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 128 + g * 32;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        u32x4_t w;
+#pragma unroll
+        for (int jp = 0; jp < 4; ++jp)
+          w[jp] = pack_bf16x2(acc[mt][2 * jp][r] * inv, acc[mt][2 * jp + 1][r] * inv);
+        st16(op + r * 8, w);
+      }
+    } else {
+      const int64_t slot = ((int64_t)seq * a.max_splits + split) * a.Hq + head;
+      float* wo = a.ws_o + slot * 128 + g * 32;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        f32x4_t w0 = {acc[mt][0][r] * vs, acc[mt][1][r] * vs, acc[mt][2][r] * vs, acc[mt][3][r] * vs};
+        f32x4_t w1 = {acc[mt][4][r] * vs, acc[mt][5][r] * vs, acc[mt][6][r] * vs, acc[mt][7][r] * vs};
+        *reinterpret_cast<f32x4_t*>(wo + r * 8) = w0;
+        *reinterpret_cast<f32x4_t*>(wo + r * 8 + 4) = w1;
+      }
+      if (g == 0) {
+        a.ws_ml[slot * 2 + 0] = m[mt];
+        a.ws_ml[slot * 2 + 1] = lt;
+      }
+    }
+  }
+}
+
+// Merge the split partials: out = sum_j o_j 2^(m_j - m*) / sum_j l_j 2^(m_j - m*).
+// grid = (Hq, decode rows); block = 64 threads, 2 dims each (D = 128).
+__global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a) {
+  const int head = blockIdx.x;
+  const int seq = blockIdx.y;
+  const int kv_len = a.pt.kv_lens[seq];
+  const int t0 = first_block_token(kv_len, a.sm.window);
+  const int n = min(a.max_splits, (kv_len - t0 + a.chunk - 1) / a.chunk);
+  if (n <= 0) return;
+  const int64_t base = ((int64_t)seq * a.max_splits) * a.Hq + head;
+  float mstar = -INFINITY;
+  for (int j = 0; j < n; ++j) mstar = fmaxf(mstar, a.ws_ml[(base + (int64_t)j * a.Hq) * 2]);
+  float den = 0.f, o0 = 0.f, o1 = 0.f;
+  const int d = threadIdx.x * 2;
+  for (int j = 0; j < n; ++j) {
+    const int64_t slot = base + (int64_t)j * a.Hq;
+    const float w = fast_exp2(a.ws_ml[slot * 2] - mstar);
+    den += a.ws_ml[slot * 2 + 1] * w;
+    const f32x2_t o = *reinterpret_cast<const f32x2_t*>(a.ws_o + slot * 128 + d);
+    o0 += o[0] * w;
+    o1 += o[1] * w;
+  }
+  const float inv = 1.0f / den;
+  const int tq = a.pt.cu_q_lens[seq];
+  uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * 128 + d);
+  *op = pack_bf16x2(o0 * inv, o1 * inv);
+}
+
+// One thread copies one 16-byte piece of one gathered row.
+__global__ __launch_bounds__(256) void rpa_gather_kernel(const GatherArgs a) {
+  const int kv_len = min(a.pt.kv_lens[a.seq], a.max_tokens);
+  const int pieces = a.row_bytes / 16;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = (int64_t)kv_len * pieces;
+  if (idx >= total) return;
+  const int tok = (int)(idx / pieces);
+  const int byte = (int)(idx % pieces) * 16;
+  const int head = byte / a.head_bytes;
+  const int inner = byte % a.head_bytes;
+  const int32_t* pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[a.seq] / a.pt.page_size)
+                                                              : (int64_t)a.seq * a.pt.pages_per_seq);
+  const int slot = tok / a.pt.page_size;
+  const int64_t off = (int64_t)pages[slot] * a.kv.page_stride +
+                      (int64_t)(tok - slot * a.pt.page_size) * a.kv.tok_stride +
+                      (int64_t)head * a.kv.head_stride + inner;
+  st16((char*)a.k_out + (int64_t)tok * a.row_bytes + byte, ld16(a.kv.k_base + off));
+  st16((char*)a.v_out + (int64_t)tok * a.row_bytes + byte, ld16(a.kv.v_base + off));
+}
+
+// New-token cache write: token j of sequence i lands at position kv_len-q_len+j.
+// grid.x covers (token, 16-byte piece); the sequence of a token is found by
+// binary search in cu_q_lens.
+__global__ __launch_bounds__(256) void rpa_kv_write_kernel(const KvWriteArgs a) {
+  const int pieces = a.Hkv * a.head_bytes / 16;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int total_tokens = min(a.num_tokens, a.pt.cu_q_lens[a.num_seqs]);
+  if (idx >= (int64_t)total_tokens * pieces) return;
+  const int t = (int)(idx / pieces);
+  const int byte = (int)(idx % pieces) * 16;
+  int lo = 0, hi = a.num_seqs;  // last i with cu_q_lens[i] <= t
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (a.pt.cu_q_lens[mid] <= t) lo = mid; else hi = mid;
+  }
+  const int seq = lo;
+  const int q0 = a.pt.cu_q_lens[seq], q1 = a.pt.cu_q_lens[seq + 1];
+  const int pos = a.pt.kv_lens[seq] - (q1 - q0) + (t - q0);
+  if (pos < 0) return;
+  const int32_t* pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[seq] / a.pt.page_size)
+                                                              : (int64_t)seq * a.pt.pages_per_seq);
+  const int slot = pos / a.pt.page_size;
+  const int head = byte / a.head_bytes;
+  const int inner = byte % a.head_bytes;
+  const int64_t off = (int64_t)pages[slot] * a.kv.page_stride +
+                      (int64_t)(pos - slot * a.pt.page_size) * a.kv.tok_stride +
+                      (int64_t)head * a.kv.head_stride + inner;
+  const int64_t src = (int64_t)t * a.Hkv * a.head_bytes + byte;
+  st16(const_cast<char*>(a.kv.k_base) + off, ld16(a.keys + src));
+  st16(const_cast<char*>(a.kv.v_base) + off, ld16(a.values + src));
+}
+
+template <int MT>
+hipError_t launch_decode_mt(const DecodeArgs& a, dim3 grid, dim3 block, bool uniform, hipStream_t st) {
+  if (a.fp8) {
+    if (uniform) hipLaunchKernelGGL((rpa_decode_splitkv_kernel<MT, true, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((rpa_decode_splitkv_kernel<MT, true, false>), grid, block, 0, st, a);
+  } else {
+    if (uniform) hipLaunchKernelGGL((rpa_decode_splitkv_kernel<MT, false, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((rpa_decode_splitkv_kernel<MT, false, false>), grid, block, 0, st, a);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream) {
+  if (a.num_rows <= 0) return hipSuccess;
+  const int nw = a.Hkv >= 4 ? 4 : a.Hkv;
+  const int head_groups = (a.Hkv + nw - 1) / nw;
+  // more than 16 query heads per kv head: further groups of 16 re-walk the KV (rare: MQA-like shapes)
+  const int row_groups = (a.G + 15) / 16;
+  const bool uniform = (a.pt.page_size % kBlk) == 0;
+  dim3 grid(a.max_splits, a.num_rows, head_groups * row_groups);
+  dim3 block(nw * 64);
+  hipError_t e = launch_decode_mt<1>(a, grid, block, uniform, stream);
+  if (e != hipSuccess) return e;
+  if (a.max_splits > 1) {
+    hipLaunchKernelGGL(rpa_combine_kernel, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
+    e = hipGetLastError();
+  }
+  return e;
+}
+
+hipError_t launch_gather(const GatherArgs& a, hipStream_t stream) {
+  if (a.max_tokens <= 0) return hipSuccess;
+  const int64_t total = (int64_t)a.max_tokens * (a.row_bytes / 16);
+  const int blocks = (int)((total + 255) / 256);
+  hipLaunchKernelGGL(rpa_gather_kernel, dim3(blocks), dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_kv_write(const KvWriteArgs& a, hipStream_t stream) {
+  if (a.num_tokens <= 0 || a.num_seqs <= 0) return hipSuccess;
+  const int64_t total = (int64_t)a.num_tokens * (a.Hkv * a.head_bytes / 16);
+  const int blocks = (int)((total + 255) / 256);
+  hipLaunchKernelGGL(rpa_kv_write_kernel, dim3(blocks), dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+}  // namespace rpa

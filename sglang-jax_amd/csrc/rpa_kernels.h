@@ -1,0 +1,114 @@
+// Host-visible launch interface between the C ABI (rpa_capi.hip) and the
+// kernel translation units.  Plain structs of device pointers and integers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rpa {
+
+// How K and V rows of one (page, token, kv head) are addressed, in bytes.
+//   fused  [pages, P, 2*Hkv, D]: v_base = k_base + D*esize, head_stride = 2*D*esize
+//   split  k_pages / v_pages [pages, P, Hkv, D]: head_stride = D*esize
+struct KvAddr {
+  const char* k_base;
+  const char* v_base;
+  int64_t page_stride;
+  int32_t tok_stride;
+  int32_t head_stride;
+};
+
+struct PageTable {
+  const int32_t* kv_lens;
+  const int32_t* page_indices;
+  const int32_t* cu_q_lens;
+  const int32_t* cu_kv_lens;  // nullptr => padded table, row stride pages_per_seq
+  int32_t pages_per_seq;
+  int32_t page_size;
+};
+
+struct SoftmaxOpts {
+  float sm_scale;
+  float soft_cap;    // 0 => off
+  float mask_value;  // finite, negative
+  int32_t window;    // 0 => off
+};
+
+struct DecodeArgs {
+  const uint16_t* q;  // bf16 [T, Hq, D]
+  uint16_t* out;      // bf16 [T, Hq, D]
+  KvAddr kv;
+  PageTable pt;
+  SoftmaxOpts sm;
+  const float* k_scale;  // f32[Hkv] or nullptr
+  const float* v_scale;
+  float* ws_o;   // [num_rows, max_splits, Hq, D] unnormalised partial outputs
+  float* ws_ml;  // [num_rows, max_splits, Hq, 2]  (running max in log2 units, sum)
+  int32_t num_rows;  // decode sequences
+  int32_t Hq, Hkv, G;
+  int32_t chunk;       // kv tokens per split (multiple of 32)
+  int32_t max_splits;  // grid.x
+  int32_t fp8;
+};
+
+struct PrefillArgs {
+  const uint16_t* q;
+  uint16_t* out;
+  KvAddr kv;
+  PageTable pt;
+  SoftmaxOpts sm;
+  const float* k_scale;
+  const float* v_scale;
+  int32_t seq_begin, seq_end;  // sequences [seq_begin, seq_end)
+  int32_t Hq, Hkv, G;
+  int32_t max_q_len;
+  int32_t fp8;
+};
+
+struct GatherArgs {
+  KvAddr kv;
+  PageTable pt;
+  int32_t seq;
+  int32_t row_bytes;  // Hkv * D * esize of one gathered K (or V) row
+  int32_t Hkv;
+  int32_t head_bytes;  // D * esize
+  void* k_out;
+  void* v_out;
+  int32_t max_tokens;
+};
+
+struct KvWriteArgs {
+  KvAddr kv;  // bases are written through
+  PageTable pt;
+  const char* keys;    // [T, Hkv, D] cache dtype
+  const char* values;
+  int32_t num_seqs;
+  int32_t Hkv;
+  int32_t head_bytes;
+  int32_t num_tokens;
+};
+
+struct MlaDecodeArgs {
+  const uint16_t* ql_nope;  // [T, Hq, lkv]
+  const uint16_t* q_pe;     // [T, Hq, rope]
+  uint16_t* out;            // [T, Hq, lkv]
+  const char* cache;        // [pages, P, row_stride] bf16
+  PageTable pt;
+  SoftmaxOpts sm;
+  float* ws_o;   // [T, max_splits, Hq, lkv]
+  float* ws_ml;  // [T, max_splits, Hq, 2]
+  int32_t num_rows;
+  int32_t Hq;
+  int32_t row_stride;   // elements
+  int32_t rope_offset;  // elements
+  int32_t chunk;
+  int32_t max_splits;
+};
+
+hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream);
+hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream);
+hipError_t launch_gather(const GatherArgs& a, hipStream_t stream);
+hipError_t launch_kv_write(const KvWriteArgs& a, hipStream_t stream);
+hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream);
+
+}  // namespace rpa

@@ -1,0 +1,407 @@
+"""Host-side mirror of the reference's ragged paged attention operator.
+
+Same names, argument meaning and error behaviour as
+``python/sgl_jax/srt/kernels/ragged_paged_attention/ragged_paged_attention_v3.py``
+of the reference (``rpa_v3`` below), but the arrays are torch tensors on a ROCm
+device and the computation is the HIP library behind the C ABI of
+``include/rpa.h``.  There is no CPU path here.
+
+Two call surfaces:
+
+* :func:`ragged_paged_attention` -- the production signature, rpa_v3:1667-1700:
+  new ``keys/values`` are written into the fused, head-interleaved cache and the
+  pair ``(output, updated_cache)`` is returned (the cache is updated in place and
+  returned, matching the donated-buffer aliasing of rpa_v3:1973-1976);
+* :func:`ragged_paged_attention_ref_surface` -- the argument list of
+  ``ref_ragged_paged_attention`` (rpa_v3:94-114): separate ``k_pages/v_pages``
+  that already hold every token, a zero-padded 2-D page table and ``num_seqs``.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import RpaParams
+
+# rpa_v3:47
+DEFAULT_MASK_VALUE = -0.7 * float(np.finfo(np.float32).max)
+
+_workspaces: dict = {}
+
+
+def _workspace(device, nbytes: int) -> torch.Tensor:
+    """Grow-only scratch for the split-KV partials, one per device and stream."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _kv_dtype_code(dtype) -> int:
+    if dtype == torch.bfloat16:
+        return _lib.RPA_KV_BF16
+    if dtype in (torch.float8_e4m3fn,):
+        return _lib.RPA_KV_FP8_E4M3
+    raise ValueError(f"Expected kv cache dtype bfloat16 or float8_e4m3fn, got {dtype}")
+
+
+def _per_head(scale, num_kv_heads, device):
+    if scale is None:
+        return None
+    t = torch.as_tensor(scale, dtype=torch.float32, device=device).reshape(-1)
+    if t.numel() == 1:
+        t = t.expand(num_kv_heads)
+    if t.numel() != num_kv_heads:
+        raise ValueError(f"Expected a scalar or {num_kv_heads} per-head scales, got {t.numel()}")
+    return t.contiguous()
+
+
+def _i32(t, device):
+    if isinstance(t, np.ndarray):
+        t = torch.from_numpy(t)
+    if t.dtype != torch.int32:
+        raise ValueError(f"Expected int32 dtype for metadata, got {t.dtype}")
+    return t.to(device).contiguous()
+
+
+def _host_max(t):
+    """Upper bound taken from a HOST copy only (never synchronises a device)."""
+    if isinstance(t, np.ndarray):
+        return int(t.max()) if t.size else 0
+    if isinstance(t, torch.Tensor) and t.device.type == "cpu":
+        return int(t.max()) if t.numel() else 0
+    return 0
+
+
+def static_validate_inputs(queries, keys, values, kv_cache_fused, kv_lens, page_indices, cu_q_lens,
+                           cu_kv_lens, distribution, *, causal=1, sliding_window=None, soft_cap=None,
+                           chunk_prefill_size=None, skip_kv_mask=False):
+    """Shape/dtype contract of rpa_v3:1314-1439 (same messages where they apply)."""
+    q, k, v = queries, keys, values
+    if k is not None:
+        if not (q.dim() == k.dim() == v.dim() == 3):
+            raise ValueError(f"Expected 3D array for q.shape={tuple(q.shape)}, k.shape={tuple(k.shape)}, v.shape={tuple(v.shape)}")
+        if k.shape != v.shape:
+            raise ValueError(f"Expected k.shape={tuple(k.shape)} to be equal to v.shape={tuple(v.shape)}")
+        if not (q.shape[0] == k.shape[0] == v.shape[0]):
+            raise ValueError(f"Expected q.shape[0]={q.shape[0]} to be equal to k.shape[0]={k.shape[0]} and v.shape[0]={v.shape[0]}")
+        if not (q.shape[2] == k.shape[2] == v.shape[2]):
+            raise ValueError(f"Expected q.shape[2]={q.shape[2]} to be equal to k.shape[2]={k.shape[2]} and v.shape[2]={v.shape[2]}")
+        num_kv_heads = k.shape[1]
+    else:
+        if q.dim() != 3:
+            raise ValueError(f"Expected 3D array for q.shape={tuple(q.shape)}")
+        num_kv_heads = kv_cache_fused.shape[2] // 2
+    if q.shape[1] % num_kv_heads != 0:
+        raise ValueError(f"Expected actual_num_q_heads={q.shape[1]} to be divisible by actual_num_kv_heads={num_kv_heads}.")
+    if not kv_cache_fused.dtype.is_floating_point:
+        raise ValueError(f"Expected kv_cache_fused.dtype={kv_cache_fused.dtype} to be a floating point.")
+    for name, t in (("kv_lens", kv_lens), ("page_indices", page_indices), ("cu_q_lens", cu_q_lens),
+                    ("cu_kv_lens", cu_kv_lens), ("distribution", distribution)):
+        if t.dtype != torch.int32:
+            raise ValueError(f"Expected int32 dtype for {name}.dtype={t.dtype}")
+    if not (kv_lens.dim() == page_indices.dim() == cu_q_lens.dim() == 1):
+        raise ValueError("Expected 1D array for kv_lens, page_indices, cu_q_lens")
+    max_num_seqs = kv_lens.shape[0]
+    if tuple(cu_q_lens.shape) != (max_num_seqs + 1,):
+        raise ValueError(f"Expected cu_q_lens.shape={tuple(cu_q_lens.shape)} to be ({max_num_seqs + 1},).")
+    if tuple(cu_kv_lens.shape) != (max_num_seqs + 1,):
+        raise ValueError(f"Expected cu_kv_lens.shape={tuple(cu_kv_lens.shape)} to be ({max_num_seqs + 1},).")
+    if tuple(distribution.shape) != (3,):
+        raise ValueError(f"Expected distribution.shape={tuple(distribution.shape)} to be (3,).")
+    if sliding_window is not None and sliding_window <= 0:
+        raise ValueError(f"sliding_window={sliding_window} must be positive.")
+    if soft_cap is not None and soft_cap == 0.0:
+        raise ValueError(f"soft_cap={soft_cap} must not be 0.0.")
+    if chunk_prefill_size is not None and chunk_prefill_size <= 0:
+        raise ValueError(f"chunk_prefill_size={chunk_prefill_size} must be positive.")
+    if skip_kv_mask and causal == 1:
+        raise ValueError("Cannot skip kv mask when using causal mask.")
+
+
+def dynamic_validate_inputs(params: RpaParams, kv_lens, page_indices, cu_q_lens, cu_kv_lens, distribution):
+    """Value checks of rpa_v3:1442-1487 on HOST copies of the metadata (numpy int32)."""
+    lib = _lib.load()
+    keep = [np.ascontiguousarray(a, dtype=np.int32) if a is not None else None
+            for a in (kv_lens, page_indices, cu_q_lens, cu_kv_lens, distribution)]
+    ptrs = [None if a is None else a.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)) for a in keep]
+    _lib.check(lib.rpa_validate_host(ctypes.byref(params), ptrs[0], ptrs[1], int(keep[1].size), ptrs[2], ptrs[3], ptrs[4]))
+
+
+def _fill_common(p: RpaParams, q, out, *, num_seqs, decode_end, page_size, total_pages, num_kv_heads,
+                 kv_dtype, sm_scale, sliding_window, soft_cap, mask_value, max_kv_len, max_q_len, num_splits):
+    p.q = q.data_ptr()
+    p.out = out.data_ptr()
+    p.num_tokens = q.shape[0]
+    p.num_seqs = int(num_seqs)
+    p.num_q_heads = q.shape[1]
+    p.num_kv_heads = int(num_kv_heads)
+    p.head_dim = q.shape[2]
+    p.page_size = int(page_size)
+    p.total_pages = int(total_pages)
+    p.kv_dtype = _kv_dtype_code(kv_dtype)
+    p.decode_end = int(decode_end)
+    p.max_kv_len = int(max_kv_len)
+    p.max_q_len = int(max_q_len)
+    p.num_splits = int(num_splits)
+    p.sliding_window = int(sliding_window) if sliding_window else 0
+    p.sm_scale = float(sm_scale)
+    p.soft_cap = float(soft_cap) if soft_cap else 0.0
+    p.mask_value = float(mask_value) if mask_value is not None else DEFAULT_MASK_VALUE
+
+
+def _launch(p: RpaParams, device, entry: str = "rpa_attention"):
+    lib = _lib.load()
+    need = lib.rpa_workspace_bytes(ctypes.byref(p))
+    ws = None
+    if need:
+        ws = _workspace(device, need)
+        p.workspace = ws.data_ptr()
+        p.workspace_bytes = ws.numel()
+    stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    _lib.check(getattr(lib, entry)(ctypes.byref(p), stream))
+    return ws
+
+
+def _require_gpu(t, name):
+    if not (isinstance(t, torch.Tensor) and t.is_cuda):
+        raise RuntimeError(f"{name} must be a tensor on a ROCm device: this operator has no CPU path")
+
+
+def ragged_paged_attention(
+    queries: torch.Tensor,  # [max_num_tokens, num_q_heads, head_dim]
+    keys: torch.Tensor | None,  # [max_num_tokens, num_kv_heads, head_dim] or None (cache already complete)
+    values: torch.Tensor | None,
+    kv_cache_fused: torch.Tensor,  # [total_num_pages, page_size, num_kv_heads * 2, head_dim]
+    kv_lens,  # i32[max_num_seqs]
+    page_indices,  # i32[flat]
+    cu_q_lens,  # i32[max_num_seqs + 1]
+    cu_kv_lens,  # i32[max_num_seqs + 1]
+    distribution,  # i32[3]  (host array or tensor)
+    custom_mask=None,
+    attention_sink=None,
+    *,
+    causal: int = 1,
+    sm_scale: float = 1.0,
+    sliding_window: int | None = None,
+    soft_cap: float | None = None,
+    mask_value: float | None = DEFAULT_MASK_VALUE,
+    q_scale: float | None = None,
+    k_scale=None,
+    v_scale=None,
+    xai_temperature_len: float | None = None,
+    softmax_dtype=None,
+    chunk_prefill_size: int | None = None,
+    d_block_sizes=None,
+    p_block_sizes=None,
+    m_block_sizes=None,
+    vmem_limit_bytes: int | None = None,
+    out_dtype=None,
+    skip_kv_mask: bool = False,
+    disable_semaphore_checks: bool = True,
+    debug_mode: bool = False,
+    mask_aligned_to_cu_kv: bool = False,
+    # ---- additions of this implementation (host-side bounds, never synchronise) ----
+    max_kv_len: int | None = None,
+    max_q_len: int | None = None,
+    num_splits: int = 0,
+    validate_values: bool = False,
+):
+    """Ragged paged attention with fused KV cache; returns (output, updated_kv_cache_fused).
+
+    Mirrors rpa_v3:1667-1733.  TPU tuning knobs (block sizes, vmem limit, semaphore
+    checks, debug mode) are accepted and ignored.  ``k_scale``/``v_scale`` may be a
+    float (reference) or one value per kv head.  ``distribution`` and the optional
+    ``max_kv_len``/``max_q_len`` are host values used only to size launch grids.
+    """
+    _require_gpu(queries, "queries")
+    _require_gpu(kv_cache_fused, "kv_cache_fused")
+    device = queries.device
+    if isinstance(distribution, torch.Tensor):
+        dist = distribution.cpu().numpy()
+    elif isinstance(distribution, np.ndarray):
+        dist = distribution
+    else:
+        dist = np.asarray(distribution, dtype=np.int32)
+    dist_t = torch.as_tensor(dist)
+    kv_lens_d, page_d, cu_q_d, cu_kv_d = (_i32(x, device) for x in (kv_lens, page_indices, cu_q_lens, cu_kv_lens))
+    static_validate_inputs(queries, keys, values, kv_cache_fused, kv_lens_d, page_d, cu_q_d, cu_kv_d, dist_t,
+                           causal=causal, sliding_window=sliding_window, soft_cap=soft_cap,
+                           chunk_prefill_size=chunk_prefill_size, skip_kv_mask=skip_kv_mask)
+    if causal != 1 or custom_mask is not None:
+        raise NotImplementedError("custom_mask / causal=0 (speculative tree verification) is not built")
+    for name, val in (("attention_sink", attention_sink), ("xai_temperature_len", xai_temperature_len),
+                      ("softmax_dtype", softmax_dtype), ("q_scale", q_scale)):
+        if val is not None:
+            raise NotImplementedError(f"{name} is not built")
+    if kv_cache_fused.dim() == 5:  # reference's packed view [pages, P, 2Hkv/pack, pack, D]
+        s = kv_cache_fused.shape
+        kv_cache_fused = kv_cache_fused.view(s[0], s[1], s[2] * s[3], s[4])
+    if not (queries.is_contiguous() and kv_cache_fused.is_contiguous()):
+        raise ValueError("queries and kv_cache_fused must be contiguous")
+    if queries.dtype != torch.bfloat16:
+        raise ValueError(f"Expected bfloat16 queries, got {queries.dtype}")
+    total_pages, page_size, h2, head_dim = kv_cache_fused.shape
+    num_kv_heads = h2 // 2
+    if head_dim != queries.shape[2]:
+        raise ValueError(f"Expected cache head_dim={head_dim} to equal q head_dim={queries.shape[2]}")
+    i, j, k = (int(x) for x in dist)
+    if not (i <= j <= k):
+        raise ValueError(f"distribution must satisfy i <= j <= k, got {i}, {j}, {k}")
+    if k > kv_lens_d.shape[0]:
+        raise ValueError(f"distribution[2]={k} exceeds max_num_seqs={kv_lens_d.shape[0]}")
+
+    out = torch.empty_like(queries) if out_dtype in (None, torch.bfloat16) else None
+    if out is None:
+        raise NotImplementedError("out_dtype other than bfloat16 is not built")
+    p = RpaParams()
+    _fill_common(p, queries, out, num_seqs=k, decode_end=i, page_size=page_size, total_pages=total_pages,
+                 num_kv_heads=num_kv_heads, kv_dtype=kv_cache_fused.dtype, sm_scale=sm_scale,
+                 sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
+                 max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
+                 max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits)
+    p.kv_cache = kv_cache_fused.data_ptr()
+    p.layout = _lib.RPA_LAYOUT_FUSED
+    p.kv_lens = kv_lens_d.data_ptr()
+    p.page_indices = page_d.data_ptr()
+    p.cu_q_lens = cu_q_d.data_ptr()
+    p.cu_kv_lens = cu_kv_d.data_ptr()
+    ks = _per_head(k_scale, num_kv_heads, device)
+    vs = _per_head(v_scale, num_kv_heads, device)
+    p.k_scale = ks.data_ptr() if ks is not None else None
+    p.v_scale = vs.data_ptr() if vs is not None else None
+    if validate_values:
+        dynamic_validate_inputs(p, kv_lens_d.cpu().numpy(), page_d.cpu().numpy(), cu_q_d.cpu().numpy(),
+                                cu_kv_d.cpu().numpy(), dist.astype(np.int32))
+    lib = _lib.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    if keys is not None:
+        _require_gpu(keys, "keys")
+        if keys.dtype != kv_cache_fused.dtype or values.dtype != kv_cache_fused.dtype:
+            raise ValueError(f"Expected keys/values dtype {kv_cache_fused.dtype}, got {keys.dtype}/{values.dtype}")
+        _lib.check(lib.rpa_kv_write(ctypes.byref(p), _ptr(keys.contiguous()), _ptr(values.contiguous()), stream))
+    keep = (_launch(p, device), ks, vs, kv_lens_d, page_d, cu_q_d, cu_kv_d)
+    del keep
+    return out, kv_cache_fused
+
+
+def ragged_paged_attention_ref_surface(
+    queries: torch.Tensor,  # [padded_num_tokens, num_q_heads, head_dim]
+    k_pages: torch.Tensor,  # [total_num_pages, page_size, num_kv_heads, head_dim]
+    v_pages: torch.Tensor,
+    kv_lens,  # i32[padded_batch_size]
+    page_indices,  # i32[padded_batch_size, max_pages_per_seq]
+    cu_q_lens,  # i32[padded_batch_size + 1]
+    num_seqs,  # i32[1] (host) or int
+    *,
+    causal: bool = True,
+    sm_scale: float = 1.0,
+    sliding_window: int | None = None,
+    soft_cap: float | None = None,
+    mask_value: float | None = DEFAULT_MASK_VALUE,
+    k_scale=None,
+    v_scale=None,
+    decode_end: int = 0,
+    max_kv_len: int | None = None,
+    max_q_len: int | None = None,
+    num_splits: int = 0,
+) -> torch.Tensor:
+    """The argument list of ref_ragged_paged_attention (rpa_v3:94-114) on the HIP
+    kernels.  Returns [padded_num_tokens, Hq, D]; only rows < cu_q_lens[num_seqs]
+    are defined (the reference returns exactly those rows).  ``decode_end`` tells
+    how many leading sequences are single-token rows (0 is always valid: the
+    flash kernel handles q_len == 1 too)."""
+    _require_gpu(queries, "queries")
+    if not causal:
+        raise NotImplementedError("causal=False is not built")
+    if sliding_window is not None and sliding_window <= 0:
+        raise ValueError(f"sliding_window={sliding_window} must be positive.")
+    if soft_cap is not None and soft_cap == 0.0:
+        raise ValueError(f"soft_cap={soft_cap} must not be 0.0.")
+    device = queries.device
+    n = int(num_seqs[0]) if not isinstance(num_seqs, int) else num_seqs
+    total_pages, page_size, num_kv_heads, head_dim = k_pages.shape
+    if queries.shape[1] % num_kv_heads != 0:
+        raise ValueError(f"Expected num_q_heads={queries.shape[1]} to be divisible by num_kv_heads={num_kv_heads}.")
+    if k_pages.shape != v_pages.shape:
+        raise ValueError(f"Expected k_pages.shape={tuple(k_pages.shape)} to be equal to v_pages.shape={tuple(v_pages.shape)}")
+    if not (k_pages.is_contiguous() and v_pages.is_contiguous() and queries.is_contiguous()):
+        raise ValueError("queries, k_pages and v_pages must be contiguous")
+    kv_lens_d, cu_q_d = _i32(kv_lens, device), _i32(cu_q_lens, device)
+    page_d = _i32(page_indices, device)
+    if page_d.dim() != 2:
+        raise ValueError(f"Expected 2D page_indices, got shape {tuple(page_d.shape)}")
+    out = torch.empty_like(queries)
+    p = RpaParams()
+    _fill_common(p, queries, out, num_seqs=n, decode_end=decode_end, page_size=page_size, total_pages=total_pages,
+                 num_kv_heads=num_kv_heads, kv_dtype=k_pages.dtype, sm_scale=sm_scale,
+                 sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
+                 max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
+                 max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits)
+    p.kv_cache = k_pages.data_ptr()
+    p.v_pages = v_pages.data_ptr()
+    p.layout = _lib.RPA_LAYOUT_SPLIT
+    p.kv_lens = kv_lens_d.data_ptr()
+    p.page_indices = page_d.data_ptr()
+    p.pages_per_seq = page_d.shape[1]
+    p.cu_q_lens = cu_q_d.data_ptr()
+    p.cu_kv_lens = None
+    ks = _per_head(k_scale, num_kv_heads, device)
+    vs = _per_head(v_scale, num_kv_heads, device)
+    p.k_scale = ks.data_ptr() if ks is not None else None
+    p.v_scale = vs.data_ptr() if vs is not None else None
+    keep = (_launch(p, device), ks, vs, kv_lens_d, page_d, cu_q_d)
+    del keep
+    return out
+
+
+def gather_pages(kv_cache_fused: torch.Tensor, kv_lens, page_indices, cu_kv_lens, seq: int, kv_len: int):
+    """K and V rows of sequence ``seq`` gathered through the page table, bit for
+    bit: the indexing expression of rpa_v3:138-139 on its own.  Returns
+    (k [kv_len, Hkv, D], v [kv_len, Hkv, D]) in the cache dtype."""
+    _require_gpu(kv_cache_fused, "kv_cache_fused")
+    device = kv_cache_fused.device
+    total_pages, page_size, h2, head_dim = kv_cache_fused.shape
+    num_kv_heads = h2 // 2
+    kv_lens_d, page_d, cu_kv_d = _i32(kv_lens, device), _i32(page_indices, device), _i32(cu_kv_lens, device)
+    k_out = torch.empty((kv_len, num_kv_heads, head_dim), dtype=kv_cache_fused.dtype, device=device)
+    v_out = torch.empty_like(k_out)
+    dummy = torch.zeros(2, dtype=torch.int32, device=device)
+    p = RpaParams()
+    p.q = dummy.data_ptr()
+    p.out = dummy.data_ptr()
+    p.kv_cache = kv_cache_fused.data_ptr()
+    p.layout = _lib.RPA_LAYOUT_FUSED
+    p.kv_lens = kv_lens_d.data_ptr()
+    p.page_indices = page_d.data_ptr()
+    p.cu_q_lens = dummy.data_ptr()
+    p.cu_kv_lens = cu_kv_d.data_ptr()
+    p.num_tokens = 0
+    p.num_seqs = kv_lens_d.shape[0]
+    p.num_q_heads = num_kv_heads
+    p.num_kv_heads = num_kv_heads
+    p.head_dim = head_dim
+    p.page_size = page_size
+    p.total_pages = total_pages
+    p.kv_dtype = _kv_dtype_code(kv_cache_fused.dtype)
+    p.sm_scale = 1.0
+    lib = _lib.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    _lib.check(lib.rpa_gather_pages(ctypes.byref(p), int(seq), _ptr(k_out), _ptr(v_out), int(kv_len), stream))
+    return k_out, v_out
+
+
+def default_sm_scale(head_dim: int) -> float:
+    """layers/attention/flashattention_backend.py:630-634: 1/sqrt(head_dim) unless the layer sets one."""
+    return 1.0 / math.sqrt(head_dim)

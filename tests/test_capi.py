@@ -1,0 +1,148 @@
+"""Host-side checks that need no GPU: the library loads, exports every symbol
+include/rpa.h declares, and its validation mirrors the reference's
+static/dynamic_validate_inputs
+(python/sgl_jax/srt/kernels/ragged_paged_attention/ragged_paged_attention_v3.py:1314-1487)."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "rpa.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rpa_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    lib = pkg._lib.load()
+    names = header_functions()
+    assert set(names) == set(pkg._lib.EXPORTED_SYMBOLS)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.rpa_version() == 100
+
+
+def test_struct_layout_matches_header(pkg):
+    # 11 pointers + size_t + 15 int32 + 3 float
+    assert ctypes.sizeof(pkg._lib.RpaParams) == 12 * 8 + 18 * 4
+    assert ctypes.sizeof(pkg._lib.RpaMlaParams) == 10 * 8 + 13 * 4 + 3 * 4
+
+
+def base_params(pkg):
+    p = pkg._lib.RpaParams()
+    for f in ("q", "out", "kv_cache", "kv_lens", "page_indices", "cu_q_lens", "cu_kv_lens"):
+        setattr(p, f, 0x1000)  # never dereferenced by the validators
+    p.num_tokens, p.num_seqs, p.num_q_heads, p.num_kv_heads = 8, 3, 8, 2
+    p.head_dim, p.page_size, p.total_pages = 128, 4, 16
+    p.decode_end = 1
+    p.sm_scale = 1.0
+    return p
+
+
+def status(pkg, code):
+    return pkg._lib.STATUS_NAMES[code]
+
+
+def test_static_validation_codes(pkg):
+    lib = pkg._lib.load()
+    p = base_params(pkg)
+    assert lib.rpa_validate(ctypes.byref(p)) == 0
+    p.num_q_heads = 7
+    assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EINVAL_HEADS"
+    assert b"divisible" in lib.rpa_last_error()
+    p = base_params(pkg); p.sliding_window = -1
+    assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EINVAL_WINDOW"
+    p = base_params(pkg); p.kv_dtype = 5
+    assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EINVAL_DTYPE"
+    p = base_params(pkg); p.decode_end = 4
+    assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EINVAL_DISTRIBUTION"
+    p = base_params(pkg); p.head_dim = 64
+    assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EUNSUPPORTED"
+    p = base_params(pkg); p.q = None
+    assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EINVAL_NULL"
+    p = base_params(pkg); p.layout = 1
+    assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EINVAL_NULL"  # split layout without v_pages
+    assert lib.rpa_validate(None) == -12
+
+
+def host_check(pkg, p, kv_lens, pages, cu_q, cu_kv, dist):
+    lib = pkg._lib.load()
+    arr = lambda a: None if a is None else np.ascontiguousarray(a, dtype=np.int32)
+    a = [arr(x) for x in (kv_lens, pages, cu_q, cu_kv, dist)]
+    ptr = lambda x: None if x is None else x.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
+    rc = lib.rpa_validate_host(ctypes.byref(p), ptr(a[0]), ptr(a[1]), len(a[1]), ptr(a[2]), ptr(a[3]), ptr(a[4]))
+    return pkg._lib.STATUS_NAMES[rc], lib.rpa_last_error().decode()
+
+
+def test_dynamic_validation_codes(pkg):
+    p = base_params(pkg)
+    kv, cu_q, cu_kv = [5, 8, 6], [0, 1, 4, 8], [0, 8, 16, 24]
+    pages = [1, 2, 3, 4, 5, 6]
+    ok = host_check(pkg, p, kv, pages, cu_q, cu_kv, [1, 1, 3])
+    assert ok[0] == "RPA_OK", ok
+    assert host_check(pkg, p, kv, pages, cu_q, cu_kv, [2, 1, 3])[0] == "RPA_EINVAL_DISTRIBUTION"
+    # q_len > kv_len (message of ragged_paged_attention_v3.py:1475-1476)
+    st, msg = host_check(pkg, p, [5, 2, 6], pages, cu_q, cu_kv, [1, 1, 3])
+    assert st == "RPA_EINVAL_QLEN_GT_KVLEN" and "q_len=3 > kv_len=2" in msg
+    # q_len == 0
+    assert host_check(pkg, p, kv, pages, [0, 1, 1, 8], cu_kv, [1, 1, 3])[0] == "RPA_EINVAL_QLEN_GT_KVLEN"
+    # page index out of range
+    st, msg = host_check(pkg, p, kv, [1, 2, 3, 16, 5, 6], cu_q, cu_kv, [1, 1, 3])
+    assert st == "RPA_EINVAL_PAGE_RANGE" and "out of [0, 16)" in msg
+    assert host_check(pkg, p, kv, [1, 2, -1, 4, 5, 6], cu_q, cu_kv, [1, 1, 3])[0] == "RPA_EINVAL_PAGE_RANGE"
+    # page list runs off the end of page_indices
+    assert host_check(pkg, p, kv, pages[:5], cu_q, cu_kv, [1, 1, 3])[0] == "RPA_EINVAL_PAGE_RANGE"
+    # tokens exceed T
+    assert host_check(pkg, p, [5, 8, 9], pages + [7], [0, 1, 4, 9], [0, 8, 16, 28], [1, 1, 3])[0] == "RPA_EINVAL_SHAPE"
+    # decode row with q_len 2
+    assert host_check(pkg, p, kv, pages, [0, 2, 4, 8], cu_kv, [1, 1, 3])[0] == "RPA_EINVAL_DISTRIBUTION"
+    # padded 2-D table: page_cnt > pages_per_seq
+    p2 = base_params(pkg); p2.cu_kv_lens = None; p2.pages_per_seq = 1
+    st, msg = host_check(pkg, p2, kv, [1, 2, 3], cu_q, None, [1, 1, 3])
+    assert st == "RPA_EINVAL_PAGE_RANGE" and "pages_per_seq=1" in msg
+
+
+def test_workspace_size_is_deterministic(pkg):
+    lib = pkg._lib.load()
+    p = base_params(pkg)
+    p.num_seqs = p.decode_end = 16
+    p.num_tokens = 16
+    p.num_q_heads, p.num_kv_heads, p.page_size, p.total_pages = 32, 8, 64, 8192
+    p.max_kv_len = 32768
+    a = lib.rpa_workspace_bytes(ctypes.byref(p))
+    assert a > 0 and a == lib.rpa_workspace_bytes(ctypes.byref(p))
+    assert a % (16 * 32 * 130 * 4) == 0
+    p.num_splits = 1
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+
+
+def test_python_wrapper_raises_like_the_reference(pkg):
+    import torch
+
+    q = torch.zeros(4, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        pkg.ragged_paged_attention(q, None, None, torch.zeros(2, 4, 4, 128, dtype=torch.bfloat16),
+                                   torch.zeros(2, dtype=torch.int32), torch.zeros(2, dtype=torch.int32),
+                                   torch.zeros(3, dtype=torch.int32), torch.zeros(3, dtype=torch.int32), [0, 0, 2], None)
+    m = __import__("sglang_jax_amd.ragged_paged_attention", fromlist=["x"])
+    i32 = lambda *s: torch.zeros(*s, dtype=torch.int32)
+    cache = torch.zeros(2, 4, 4, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="must be positive"):
+        m.static_validate_inputs(q, None, None, cache, i32(2), i32(2), i32(3), i32(3), i32(3), sliding_window=0)
+    with pytest.raises(ValueError, match="must not be 0.0"):
+        m.static_validate_inputs(q, None, None, cache, i32(2), i32(2), i32(3), i32(3), i32(3), soft_cap=0.0)
+    with pytest.raises(ValueError, match="divisible"):
+        m.static_validate_inputs(q, None, None, torch.zeros(2, 4, 6, 128, dtype=torch.bfloat16), i32(2), i32(2), i32(3),
+                                 i32(3), i32(3))
+    with pytest.raises(ValueError, match=r"cu_q_lens.shape"):
+        m.static_validate_inputs(q, None, None, cache, i32(2), i32(2), i32(4), i32(3), i32(3))
+    with pytest.raises(ValueError, match="int32"):
+        m.static_validate_inputs(q, None, None, cache, torch.zeros(2, dtype=torch.int64), i32(2), i32(3), i32(3), i32(3))
+    with pytest.raises(ValueError, match="Expected 3D"):
+        m.static_validate_inputs(q, torch.zeros(4, 2), torch.zeros(4, 2), cache, i32(2), i32(2), i32(3), i32(3), i32(3))
