@@ -1,0 +1,238 @@
+#!/usr/bin/env python3
+"""Benchmark of the ragged paged attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--all]
+
+A *step* is one pass of the hot path over one synthetic batch already resident
+in HBM: ``rpa_decode`` (split-KV kernel + combine) on the decode rows followed
+by ``rpa_prefill`` (flash kernel) on the prefill rows -- exactly what
+``rpa_attention`` issues.  The default workload is the mixed Llama-3-8B batch
+(BASELINE.json configs[1]).
+
+One JSON line is printed:
+  value       decode HBM GB/s of the workload's decode rows: algorithmic bytes /
+              measured time of the decode partition (split-KV + combine)
+  prefill_tflops, decode_frac_of_hbm_peak, prefill_frac_of_mfma_peak
+  roofline    the workload's dominant kernel (largest average launch time),
+              timed with events on the launch stream over the timed region
+  cpu_baseline  the CPU oracle timed on this box's host cores on a bounded sample
+  other_configs (with --all) decode GB/s of the remaining configurations
+"""
+
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def _events(n):
+    import torch
+
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def time_partitions(call, steps, warmup, has_decode, has_prefill):
+    """W warm-up steps, then exactly `steps` timed steps; returns wall ms per step and
+    the average event-timed duration of each partition inside the timed region."""
+    import torch
+
+    def one(ev=None):
+        if ev is not None:
+            ev[0].record()
+        if has_decode:
+            call.decode()
+        if ev is not None:
+            ev[1].record()
+        if has_prefill:
+            call.prefill()
+        if ev is not None:
+            ev[2].record()
+
+    for _ in range(warmup):
+        one()
+    evs = [_events(3) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        one(evs[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    dec = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    pre = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    return (t1 - t0) * 1e3 / steps, dec, pre
+
+
+def make_call(pkg, b):
+    import numpy as np
+
+    m = importlib.import_module("sglang_jax_amd.ragged_paged_attention")
+    n = int(b.distribution[2])
+    q_lens = b.q_lens()[:n]
+    dec_end = int(b.distribution[0])
+    return m.RpaCall(b.q, b.kv_cache, None, b.kv_lens, b.page_indices, b.cu_q_lens, b.cu_kv_lens, num_seqs=n,
+                     decode_end=dec_end, sm_scale=b.sm_scale, sliding_window=b.sliding_window, soft_cap=b.soft_cap,
+                     k_scale=b.k_scale, v_scale=b.v_scale, max_kv_len=int(max(b.meta["kv_lens"])),
+                     max_q_len=int(q_lens[dec_end:].max()) if n > dec_end else 0)
+
+
+def run_rpa_config(pkg, wl, b, steps, warmup):
+    dec_end, n = int(b.distribution[0]), int(b.distribution[2])
+    call = make_call(pkg, b)
+    ms, dec_ms, pre_ms = time_partitions(call, steps, warmup, dec_end > 0, n > dec_end)
+    res = {"workload": b.name, "ms_per_step": ms}
+    if dec_end > 0:
+        nbytes = wl.decode_bytes(b, 0, dec_end)
+        res.update(decode_ms=dec_ms, decode_bytes=nbytes, decode_gbps=nbytes / (dec_ms * 1e-3) / 1e9)
+    if n > dec_end:
+        flops = wl.prefill_flops(b, dec_end, n)
+        res.update(prefill_ms=pre_ms, prefill_flops=flops, prefill_tflops=flops / (pre_ms * 1e-3) / 1e12)
+    return res
+
+
+def run_mla_config(pkg, wl, b, steps, warmup):
+    import ctypes
+
+    import torch
+
+    n = int(b.distribution[2])
+    kw = dict(sm_scale=b.sm_scale, max_kv_len=int(max(b.meta["kv_lens"])))
+    dist = b.distribution.cpu().numpy()
+
+    def one():
+        pkg.mla_ragged_paged_attention(b.ql_nope, b.q_pe, None, None, b.cache_kv, b.kv_lens, b.page_indices,
+                                       b.cu_q_lens, b.cu_kv_lens, dist, **kw)
+
+    for _ in range(warmup):
+        one()
+    evs = [_events(2) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for e in evs:
+        e[0].record()
+        one()
+        e[1].record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    nbytes, flops = wl.mla_decode_bytes(b), wl.mla_decode_flops(b)
+    return {"workload": b.name, "ms_per_step": (t1 - t0) * 1e3 / steps, "decode_ms": ms, "decode_bytes": nbytes,
+            "decode_gbps": nbytes / (ms * 1e-3) / 1e9, "tflops": flops / (ms * 1e-3) / 1e12}
+
+
+def cpu_baseline(wl, budget_s=15.0):
+    """CPU oracle on a bounded sample of the default workload: its first decode rows
+    (same seeded lengths and layout, values drawn on the host)."""
+    import torch
+
+    from oracle.ref_rpa import ref_ragged_paged_attention_fused
+
+    import numpy as np
+
+    rng = np.random.Generator(np.random.PCG64(1002))
+    kv_d = rng.integers(512, 4096, size=56, endpoint=True)
+    rows = 8
+    b = wl.make_batch("c2_decode_rows_0_7", np.ones(rows, int), kv_d[:rows], num_q_heads=32, num_kv_heads=8,
+                      head_dim=128, page_size=64, seed=1002)
+    table = b.padded_page_table()
+    torch.set_num_threads(os.cpu_count() or 1)
+    f = lambda: ref_ragged_paged_attention_fused(b.q, b.kv_cache, b.kv_lens, table, b.cu_q_lens, [rows],
+                                                 sm_scale=b.sm_scale)
+    f()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        f()
+        reps += 1
+        if time.perf_counter() - t0 > budget_s or reps >= 1000:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    nbytes = wl.decode_bytes(b)
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"CPU oracle (torch f32) on decode rows 0..{rows - 1} of c2_llama3_8b_mixed "
+                      f"(kv_lens {kv_d[:rows].tolist()}), {reps} reps, {dt * 1e3:.1f} ms each"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5"])
+    ap.add_argument("--all", action="store_true", help="also time the other configurations")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no sharding, no collectives); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import __graft_entry__ as graft
+
+    graft.ensure_built()
+    pkg = graft.load_package()
+    wl = importlib.import_module("sglang_jax_amd.workloads")
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the operators have no CPU path", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+
+    def build(name):
+        return {"c1": lambda: wl.config_c1(dev), "c2": lambda: wl.config_c2(dev), "c3": lambda: wl.config_c3(dev),
+                "c4": lambda: wl.config_c4(dev), "c4swa": lambda: wl.config_c4(dev, window=True),
+                "c5": lambda: wl.config_c5(dev)}[name]()
+
+    def run(name):
+        b = build(name)
+        r = run_mla_config(pkg, wl, b, args.steps, args.warmup) if name == "c5" else \
+            run_rpa_config(pkg, wl, b, args.steps, args.warmup)
+        del b
+        torch.cuda.empty_cache()
+        return r
+
+    main_res = run(args.config)
+    dec_gbps = main_res.get("decode_gbps")
+    pre_tflops = main_res.get("prefill_tflops")
+    # dominant kernel of the workload
+    if pre_tflops is not None and main_res.get("prefill_ms", 0) >= main_res.get("decode_ms", 0):
+        roofline = {"kernel": "rpa_prefill_flash_kernel", "bound": "mfma", "achieved": pre_tflops,
+                    "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": pre_tflops / MFMA_BF16_PEAK_TFLOPS,
+                    "traffic": None, "avg_launch_ms": main_res["prefill_ms"], "flops_per_launch": main_res["prefill_flops"]}
+    else:
+        roofline = {"kernel": "rpa_mla_decode_kernel" if args.config == "c5" else "rpa_decode_splitkv_kernel",
+                    "bound": "hbm", "achieved": dec_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": dec_gbps / HBM_PEAK_GBPS, "traffic": None, "avg_launch_ms": main_res["decode_ms"],
+                    "bytes_per_launch": main_res["decode_bytes"]}
+    line = {
+        "metric": "ragged paged attn: decode HBM GB/s (% of peak), prefill TFLOP/s; 1 MI355X",
+        "value": dec_gbps if dec_gbps is not None else pre_tflops,
+        "unit": "GB/s" if dec_gbps is not None else "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.config not in ("c4", "c4swa") else "bf16 (fp8-e4m3 KV)", "data": "synthetic",
+        "config": {"workload": main_res["workload"], "value_is": "decode partition (split-KV + combine) algorithmic bytes / time"},
+        "decode_frac_of_hbm_peak": None if dec_gbps is None else dec_gbps / HBM_PEAK_GBPS,
+        "prefill_tflops": pre_tflops,
+        "prefill_frac_of_mfma_peak": None if pre_tflops is None else pre_tflops / MFMA_BF16_PEAK_TFLOPS,
+        "partitions": main_res,
+        "roofline": roofline,
+    }
+    if args.all:
+        line["other_configs"] = {n: run(n) for n in ("c1", "c2", "c3", "c4", "c4swa", "c5") if n != args.config}
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

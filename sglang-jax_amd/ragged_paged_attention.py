@@ -161,22 +161,71 @@ def _fill_common(p: RpaParams, q, out, *, num_seqs, decode_end, page_size, total
     p.mask_value = float(mask_value) if mask_value is not None else DEFAULT_MASK_VALUE
 
 
-def _launch(p: RpaParams, device, entry: str = "rpa_attention"):
-    lib = _lib.load()
-    need = lib.rpa_workspace_bytes(ctypes.byref(p))
-    ws = None
-    if need:
-        ws = _workspace(device, need)
-        p.workspace = ws.data_ptr()
-        p.workspace_bytes = ws.numel()
-    stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
-    _lib.check(getattr(lib, entry)(ctypes.byref(p), stream))
-    return ws
-
-
 def _require_gpu(t, name):
     if not (isinstance(t, torch.Tensor) and t.is_cuda):
         raise RuntimeError(f"{name} must be a tensor on a ROCm device: this operator has no CPU path")
+
+
+class RpaCall:
+    """One prepared call: the filled ``RpaParams`` plus every tensor it points at.
+
+    ``attention()`` = ``rpa_attention`` (decode rows, then prefill/mixed rows);
+    ``decode()`` / ``prefill()`` run the two partitions on their own, which is how
+    the benchmark times them separately.  Launches go to torch's current stream.
+    """
+
+    def __init__(self, queries, kv_cache, v_pages, kv_lens_d, page_d, cu_q_d, cu_kv_d, *, num_seqs, decode_end,
+                 sm_scale, sliding_window=None, soft_cap=None, mask_value=DEFAULT_MASK_VALUE, k_scale=None,
+                 v_scale=None, max_kv_len=0, max_q_len=0, num_splits=0, out=None):
+        self.lib = _lib.load()
+        self.device = queries.device
+        fused = v_pages is None
+        if fused:
+            total_pages, page_size, h2, _ = kv_cache.shape
+            num_kv_heads = h2 // 2
+        else:
+            total_pages, page_size, num_kv_heads, _ = kv_cache.shape
+        self.out = torch.empty_like(queries) if out is None else out
+        self.ks = _per_head(k_scale, num_kv_heads, self.device)
+        self.vs = _per_head(v_scale, num_kv_heads, self.device)
+        self.tensors = (queries, kv_cache, v_pages, kv_lens_d, page_d, cu_q_d, cu_kv_d)
+        p = RpaParams()
+        _fill_common(p, queries, self.out, num_seqs=num_seqs, decode_end=decode_end, page_size=page_size,
+                     total_pages=total_pages, num_kv_heads=num_kv_heads, kv_dtype=kv_cache.dtype, sm_scale=sm_scale,
+                     sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value, max_kv_len=max_kv_len,
+                     max_q_len=max_q_len, num_splits=num_splits)
+        p.kv_cache = kv_cache.data_ptr()
+        p.v_pages = None if fused else v_pages.data_ptr()
+        p.layout = _lib.RPA_LAYOUT_FUSED if fused else _lib.RPA_LAYOUT_SPLIT
+        p.kv_lens = kv_lens_d.data_ptr()
+        p.page_indices = page_d.data_ptr()
+        p.cu_q_lens = cu_q_d.data_ptr()
+        p.cu_kv_lens = None if cu_kv_d is None else cu_kv_d.data_ptr()
+        p.pages_per_seq = page_d.shape[1] if page_d.dim() == 2 else 0
+        p.k_scale = self.ks.data_ptr() if self.ks is not None else None
+        p.v_scale = self.vs.data_ptr() if self.vs is not None else None
+        need = self.lib.rpa_workspace_bytes(ctypes.byref(p))
+        self.workspace = None
+        if need:
+            self.workspace = _workspace(self.device, need)
+            p.workspace = self.workspace.data_ptr()
+            p.workspace_bytes = self.workspace.numel()
+        self.params = p
+
+    def _stream(self):
+        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def attention(self):
+        _lib.check(self.lib.rpa_attention(ctypes.byref(self.params), self._stream()))
+
+    def decode(self):
+        _lib.check(self.lib.rpa_decode(ctypes.byref(self.params), self._stream()))
+
+    def prefill(self):
+        _lib.check(self.lib.rpa_prefill(ctypes.byref(self.params), self._stream()))
+
+    def kv_write(self, keys, values):
+        _lib.check(self.lib.rpa_kv_write(ctypes.byref(self.params), _ptr(keys), _ptr(values), self._stream()))
 
 
 def ragged_paged_attention(
@@ -262,38 +311,23 @@ def ragged_paged_attention(
     if k > kv_lens_d.shape[0]:
         raise ValueError(f"distribution[2]={k} exceeds max_num_seqs={kv_lens_d.shape[0]}")
 
-    out = torch.empty_like(queries) if out_dtype in (None, torch.bfloat16) else None
-    if out is None:
+    if out_dtype not in (None, torch.bfloat16):
         raise NotImplementedError("out_dtype other than bfloat16 is not built")
-    p = RpaParams()
-    _fill_common(p, queries, out, num_seqs=k, decode_end=i, page_size=page_size, total_pages=total_pages,
-                 num_kv_heads=num_kv_heads, kv_dtype=kv_cache_fused.dtype, sm_scale=sm_scale,
-                 sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
-                 max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
-                 max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits)
-    p.kv_cache = kv_cache_fused.data_ptr()
-    p.layout = _lib.RPA_LAYOUT_FUSED
-    p.kv_lens = kv_lens_d.data_ptr()
-    p.page_indices = page_d.data_ptr()
-    p.cu_q_lens = cu_q_d.data_ptr()
-    p.cu_kv_lens = cu_kv_d.data_ptr()
-    ks = _per_head(k_scale, num_kv_heads, device)
-    vs = _per_head(v_scale, num_kv_heads, device)
-    p.k_scale = ks.data_ptr() if ks is not None else None
-    p.v_scale = vs.data_ptr() if vs is not None else None
+    call = RpaCall(queries, kv_cache_fused, None, kv_lens_d, page_d, cu_q_d, cu_kv_d, num_seqs=k, decode_end=i,
+                   sm_scale=sm_scale, sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
+                   k_scale=k_scale, v_scale=v_scale,
+                   max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
+                   max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits)
     if validate_values:
-        dynamic_validate_inputs(p, kv_lens_d.cpu().numpy(), page_d.cpu().numpy(), cu_q_d.cpu().numpy(),
+        dynamic_validate_inputs(call.params, kv_lens_d.cpu().numpy(), page_d.cpu().numpy(), cu_q_d.cpu().numpy(),
                                 cu_kv_d.cpu().numpy(), dist.astype(np.int32))
-    lib = _lib.load()
-    stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     if keys is not None:
         _require_gpu(keys, "keys")
         if keys.dtype != kv_cache_fused.dtype or values.dtype != kv_cache_fused.dtype:
             raise ValueError(f"Expected keys/values dtype {kv_cache_fused.dtype}, got {keys.dtype}/{values.dtype}")
-        _lib.check(lib.rpa_kv_write(ctypes.byref(p), _ptr(keys.contiguous()), _ptr(values.contiguous()), stream))
-    keep = (_launch(p, device), ks, vs, kv_lens_d, page_d, cu_q_d, cu_kv_d)
-    del keep
-    return out, kv_cache_fused
+        call.kv_write(keys.contiguous(), values.contiguous())
+    call.attention()
+    return call.out, kv_cache_fused
 
 
 def ragged_paged_attention_ref_surface(
@@ -342,28 +376,13 @@ def ragged_paged_attention_ref_surface(
     page_d = _i32(page_indices, device)
     if page_d.dim() != 2:
         raise ValueError(f"Expected 2D page_indices, got shape {tuple(page_d.shape)}")
-    out = torch.empty_like(queries)
-    p = RpaParams()
-    _fill_common(p, queries, out, num_seqs=n, decode_end=decode_end, page_size=page_size, total_pages=total_pages,
-                 num_kv_heads=num_kv_heads, kv_dtype=k_pages.dtype, sm_scale=sm_scale,
-                 sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
-                 max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
-                 max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits)
-    p.kv_cache = k_pages.data_ptr()
-    p.v_pages = v_pages.data_ptr()
-    p.layout = _lib.RPA_LAYOUT_SPLIT
-    p.kv_lens = kv_lens_d.data_ptr()
-    p.page_indices = page_d.data_ptr()
-    p.pages_per_seq = page_d.shape[1]
-    p.cu_q_lens = cu_q_d.data_ptr()
-    p.cu_kv_lens = None
-    ks = _per_head(k_scale, num_kv_heads, device)
-    vs = _per_head(v_scale, num_kv_heads, device)
-    p.k_scale = ks.data_ptr() if ks is not None else None
-    p.v_scale = vs.data_ptr() if vs is not None else None
-    keep = (_launch(p, device), ks, vs, kv_lens_d, page_d, cu_q_d)
-    del keep
-    return out
+    call = RpaCall(queries, k_pages, v_pages, kv_lens_d, page_d, cu_q_d, None, num_seqs=n, decode_end=decode_end,
+                   sm_scale=sm_scale, sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
+                   k_scale=k_scale, v_scale=v_scale,
+                   max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
+                   max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits)
+    call.attention()
+    return call.out
 
 
 def gather_pages(kv_cache_fused: torch.Tensor, kv_lens, page_indices, cu_kv_lens, seq: int, kv_len: int):
