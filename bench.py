@@ -83,7 +83,8 @@ def make_call(pkg, b):
     return m.RpaCall(b.q, b.kv_cache, None, b.kv_lens, b.page_indices, b.cu_q_lens, b.cu_kv_lens, num_seqs=n,
                      decode_end=dec_end, sm_scale=b.sm_scale, sliding_window=b.sliding_window, soft_cap=b.soft_cap,
                      k_scale=b.k_scale, v_scale=b.v_scale, max_kv_len=int(max(b.meta["kv_lens"])),
-                     max_q_len=int(q_lens[dec_end:].max()) if n > dec_end else 0)
+                     max_q_len=int(q_lens[dec_end:].max()) if n > dec_end else 0,
+                     sum_decode_kv_len=int(sum(b.meta["kv_lens"][:dec_end])))
 
 
 def run_rpa_config(pkg, wl, b, steps, warmup):

@@ -102,6 +102,8 @@ typedef struct RpaParams {
   float sm_scale;
   float soft_cap;             /* 0 => off */
   float mask_value;           /* 0 => default -0.7 * FLT_MAX */
+  /* sum of kv_lens over the decode rows (host-side, balances the split plan); 0 => unknown */
+  int64_t sum_decode_kv_len;
 } RpaParams;
 
 /*

@@ -82,6 +82,7 @@ class RpaParams(ctypes.Structure):
         ("sm_scale", ctypes.c_float),
         ("soft_cap", ctypes.c_float),
         ("mask_value", ctypes.c_float),
+        ("sum_decode_kv_len", ctypes.c_int64),
     ]
 
 

@@ -20,6 +20,8 @@
 // neighbouring tokens -> one dword), 32 permutes per block.
 // GQA: the G query heads of a kv head are the (zero padded) 16 columns of Q^T.
 
+#include <cstdlib>
+
 #include "rpa_common.h"
 #include "rpa_kernels.h"
 
@@ -62,12 +64,12 @@ __device__ __forceinline__ int page_slot_of(const SeqView& s, int tok) {
 // sequence's page list) is ever dereferenced; clamped rows are masked later.
 template <bool FP8, bool UNIFORM_PAGE>
 __device__ __forceinline__ void load_block(KvRegs<FP8>& r, const SeqView& s, const KvAddr& kv,
-                                           const char* kh, const char* vh, int tb, int c, int g) {
+                                           const char* kh, const char* vh, int tb, int page, int c, int g) {
   constexpr int kLaneK = FP8 ? 32 : 16;  // byte offset step of lane group g inside a K row
   constexpr int kLaneV = FP8 ? 8 : 16;   // byte offset step of lane c inside a V row
   if constexpr (UNIFORM_PAGE) {
+    // the whole block lies in one page whose id the caller fetched a block ahead
     const int slot = page_slot_of(s, tb);
-    const int page = __builtin_amdgcn_readfirstlane(s.pages[slot]);
     const char* kp = kh + (int64_t)page * kv.page_stride;
     const char* vp = vh + (int64_t)page * kv.page_stride;
     const int t0 = slot * s.page_size;
@@ -128,7 +130,7 @@ struct ScoreOpts {
   int kv_len;
 };
 
-template <int MT, bool FP8>
+template <int MT, bool FP8, bool CAP>
 __device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_t (&qB)[MT][4],
                                               f32x4_t (&acc)[MT][8], float (&m)[MT], float (&l)[MT],
                                               const ScoreOpts& so, int tb, int g) {
@@ -192,7 +194,7 @@ __device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       float v = s[i >> 2][i & 3];
-      if (so.cap != 0.f) v = soft_cap_f(v * so.scale, so.cap, so.inv_cap) * kLog2e;
+      if constexpr (CAP) v = soft_cap_f(v * so.scale, so.cap, so.inv_cap) * kLog2e;
       else v = v * so.scale2;
       x[i] = v;
     }
@@ -220,10 +222,21 @@ __device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_
     m[mt] = m_new;
     const u32x4_t pB = u32x4_t{pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]),
                                pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7])};
+    if constexpr (FP8) {
+      // fp8 blocks are VALU-bound (dequantisation): skip the accumulator rescale unless the
+      // running max moved in some lane, which is rare after the first blocks
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      acc[mt][j] = acc[mt][j] * alpha;
-      acc[mt][j] = mfma16(vA[j], pB, acc[mt][j]);
+        for (int j = 0; j < 8; ++j) acc[mt][j] = acc[mt][j] * alpha;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[mt][j] = mfma16(vA[j], pB, acc[mt][j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        acc[mt][j] = acc[mt][j] * alpha;
+        acc[mt][j] = mfma16(vA[j], pB, acc[mt][j]);
+      }
     }
   }
 }
@@ -234,7 +247,7 @@ __device__ __forceinline__ int first_block_token(int kv_len, int window) {
 }
 
 // grid = (max_splits, decode rows, head groups * row groups); block = NW waves.
-template <int MT, bool FP8, bool UNIFORM_PAGE>
+template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
 __global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const DecodeArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -302,17 +315,27 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const Decode
     for (int j = 0; j < 8; ++j) acc[mt][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- software pipeline: the loads of block i+1 are in flight while block i is consumed ----
+  // ---- software pipeline: the loads of block i+1 are in flight while block i is consumed.
+  // The prefetch is unconditional (past the end it re-reads the last block) so that the
+  // number of outstanding loads is the same on every path and the waits stay partial; the
+  // page id of block i+2 is fetched while block i is consumed.
+  const int t_last = t_begin + (nblk - 1) * kBlk;
+  auto block_tok = [&](int b) { return min(t_begin + b * kBlk, t_last); };
+  auto page_of = [&](int tb) -> int {
+    if constexpr (UNIFORM_PAGE) return __builtin_amdgcn_readfirstlane(sv.pages[page_slot_of(sv, tb)]);
+    else return 0;
+  };
   KvRegs<FP8> ra, rb;
-  load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, t_begin, c, g);
-  int blk = 0;
-  while (true) {
-    if (blk + 1 < nblk) load_block<FP8, UNIFORM_PAGE>(rb, sv, a.kv, kh, vh, t_begin + (blk + 1) * kBlk, c, g);
-    compute_block<MT, FP8>(ra, qB, acc, m, l, so, t_begin + blk * kBlk, g);
-    if (++blk >= nblk) break;
-    if (blk + 1 < nblk) load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, t_begin + (blk + 1) * kBlk, c, g);
-    compute_block<MT, FP8>(rb, qB, acc, m, l, so, t_begin + blk * kBlk, g);
-    if (++blk >= nblk) break;
+  int pg_next = page_of(block_tok(1));
+  load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, t_begin, page_of(t_begin), c, g);
+  for (int blk = 0; blk < nblk; blk += 2) {
+    load_block<FP8, UNIFORM_PAGE>(rb, sv, a.kv, kh, vh, block_tok(blk + 1), pg_next, c, g);
+    pg_next = page_of(block_tok(blk + 2));
+    compute_block<MT, FP8, CAP>(ra, qB, acc, m, l, so, t_begin + blk * kBlk, g);
+    if (blk + 1 >= nblk) break;
+    load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, block_tok(blk + 2), pg_next, c, g);
+    pg_next = page_of(block_tok(blk + 3));
+    compute_block<MT, FP8, CAP>(rb, qB, acc, m, l, so, t_begin + (blk + 1) * kBlk, g);
   }
 
   // ---- epilogue: lane (c, g) holds q row c, dims 32g + 8r + j in acc[mt][j][r] ----
@@ -355,26 +378,56 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const Decode
 }
 
 // Merge the split partials: out = sum_j o_j 2^(m_j - m*) / sum_j l_j 2^(m_j - m*).
-// grid = (Hq, decode rows); block = 64 threads, 2 dims each (D = 128).
+// grid = (Hq, decode rows); block = one wave, 2 dims per lane (D = 128).  Lane j
+// first fetches (m_j, l_j) of split j, the wave reduces m* and the denominator
+// with shuffles, then the weights are broadcast lane by lane while the partial
+// rows stream in with independent loads.
 __global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a) {
   const int head = blockIdx.x;
   const int seq = blockIdx.y;
+  const int lane = threadIdx.x;
   const int kv_len = a.pt.kv_lens[seq];
   const int t0 = first_block_token(kv_len, a.sm.window);
   const int n = min(a.max_splits, (kv_len - t0 + a.chunk - 1) / a.chunk);
   if (n <= 0) return;
   const int64_t base = ((int64_t)seq * a.max_splits) * a.Hq + head;
+  const int d = lane * 2;
   float mstar = -INFINITY;
-  for (int j = 0; j < n; ++j) mstar = fmaxf(mstar, a.ws_ml[(base + (int64_t)j * a.Hq) * 2]);
+  for (int j0 = 0; j0 < n; j0 += 64) {
+    const int j = j0 + lane;
+    float mj = (j < n) ? a.ws_ml[(base + (int64_t)j * a.Hq) * 2] : -INFINITY;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mj = fmaxf(mj, __shfl_xor(mj, off));
+    mstar = fmaxf(mstar, mj);
+  }
   float den = 0.f, o0 = 0.f, o1 = 0.f;
-  const int d = threadIdx.x * 2;
-  for (int j = 0; j < n; ++j) {
-    const int64_t slot = base + (int64_t)j * a.Hq;
-    const float w = fast_exp2(a.ws_ml[slot * 2] - mstar);
-    den += a.ws_ml[slot * 2 + 1] * w;
-    const f32x2_t o = *reinterpret_cast<const f32x2_t*>(a.ws_o + slot * 128 + d);
-    o0 += o[0] * w;
-    o1 += o[1] * w;
+  for (int j0 = 0; j0 < n; j0 += 64) {
+    const int j = j0 + lane;
+    float wj = 0.f, lj = 0.f;
+    if (j < n) {
+      const int64_t slot = base + (int64_t)j * a.Hq;
+      wj = fast_exp2(a.ws_ml[slot * 2] - mstar);
+      lj = a.ws_ml[slot * 2 + 1] * wj;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) lj += __shfl_xor(lj, off);
+    den += lj;
+    const int cnt = min(64, n - j0);
+    for (int jj = 0; jj < cnt; jj += 8) {
+      f32x2_t o[8];
+      float w[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int js = min(jj + u, cnt - 1);
+        w[u] = (jj + u < cnt) ? __shfl(wj, js) : 0.f;
+        o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + (base + (int64_t)(j0 + js) * a.Hq) * 128 + d);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        o0 += o[u][0] * w[u];
+        o1 += o[u][1] * w[u];
+      }
+    }
   }
   const float inv = 1.0f / den;
   const int tq = a.pt.cu_q_lens[seq];
@@ -435,14 +488,23 @@ __global__ __launch_bounds__(256) void rpa_kv_write_kernel(const KvWriteArgs a) 
   st16(const_cast<char*>(a.kv.v_base) + off, ld16(a.values + src));
 }
 
-template <int MT>
+template <bool FP8, bool UNIFORM, bool CAP>
+void launch_decode_variant(const DecodeArgs& a, dim3 grid, dim3 block, hipStream_t st) {
+  hipLaunchKernelGGL((rpa_decode_splitkv_kernel<1, FP8, UNIFORM, CAP>), grid, block, 0, st, a);
+}
+
 hipError_t launch_decode_mt(const DecodeArgs& a, dim3 grid, dim3 block, bool uniform, hipStream_t st) {
-  if (a.fp8) {
-    if (uniform) hipLaunchKernelGGL((rpa_decode_splitkv_kernel<MT, true, true>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((rpa_decode_splitkv_kernel<MT, true, false>), grid, block, 0, st, a);
-  } else {
-    if (uniform) hipLaunchKernelGGL((rpa_decode_splitkv_kernel<MT, false, true>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((rpa_decode_splitkv_kernel<MT, false, false>), grid, block, 0, st, a);
+  const bool cap = a.sm.soft_cap != 0.f;
+  const int key = (a.fp8 ? 4 : 0) | (uniform ? 2 : 0) | (cap ? 1 : 0);
+  switch (key) {
+    case 0: launch_decode_variant<false, false, false>(a, grid, block, st); break;
+    case 1: launch_decode_variant<false, false, true>(a, grid, block, st); break;
+    case 2: launch_decode_variant<false, true, false>(a, grid, block, st); break;
+    case 3: launch_decode_variant<false, true, true>(a, grid, block, st); break;
+    case 4: launch_decode_variant<true, false, false>(a, grid, block, st); break;
+    case 5: launch_decode_variant<true, false, true>(a, grid, block, st); break;
+    case 6: launch_decode_variant<true, true, false>(a, grid, block, st); break;
+    default: launch_decode_variant<true, true, true>(a, grid, block, st); break;
   }
   return hipGetLastError();
 }
@@ -451,14 +513,16 @@ hipError_t launch_decode_mt(const DecodeArgs& a, dim3 grid, dim3 block, bool uni
 
 hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream) {
   if (a.num_rows <= 0) return hipSuccess;
-  const int nw = a.Hkv >= 4 ? 4 : a.Hkv;
+  static const int nw_env = [] { const char* v = getenv("RPA_DECODE_WAVES_PER_WG"); return v ? atoi(v) : 0; }();
+  int nw = (nw_env >= 1 && nw_env <= 4) ? nw_env : 2;
+  if (nw > a.Hkv) nw = a.Hkv;
   const int head_groups = (a.Hkv + nw - 1) / nw;
   // more than 16 query heads per kv head: further groups of 16 re-walk the KV (rare: MQA-like shapes)
   const int row_groups = (a.G + 15) / 16;
   const bool uniform = (a.pt.page_size % kBlk) == 0;
   dim3 grid(a.max_splits, a.num_rows, head_groups * row_groups);
   dim3 block(nw * 64);
-  hipError_t e = launch_decode_mt<1>(a, grid, block, uniform, stream);
+  hipError_t e = launch_decode_mt(a, grid, block, uniform, stream);
   if (e != hipSuccess) return e;
   if (a.max_splits > 1) {
     hipLaunchKernelGGL(rpa_combine_kernel, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);

@@ -140,7 +140,8 @@ def dynamic_validate_inputs(params: RpaParams, kv_lens, page_indices, cu_q_lens,
 
 
 def _fill_common(p: RpaParams, q, out, *, num_seqs, decode_end, page_size, total_pages, num_kv_heads,
-                 kv_dtype, sm_scale, sliding_window, soft_cap, mask_value, max_kv_len, max_q_len, num_splits):
+                 kv_dtype, sm_scale, sliding_window, soft_cap, mask_value, max_kv_len, max_q_len, num_splits,
+                 sum_decode_kv_len=0):
     p.q = q.data_ptr()
     p.out = out.data_ptr()
     p.num_tokens = q.shape[0]
@@ -159,6 +160,16 @@ def _fill_common(p: RpaParams, q, out, *, num_seqs, decode_end, page_size, total
     p.sm_scale = float(sm_scale)
     p.soft_cap = float(soft_cap) if soft_cap else 0.0
     p.mask_value = float(mask_value) if mask_value is not None else DEFAULT_MASK_VALUE
+    p.sum_decode_kv_len = int(sum_decode_kv_len)
+
+
+def _host_decode_sum(kv_lens, decode_end):
+    """Sum of the decode rows' kv lengths, from a HOST copy only (0 when there is none)."""
+    if isinstance(kv_lens, torch.Tensor) and kv_lens.device.type == "cpu":
+        return int(kv_lens[:decode_end].sum()) if decode_end else 0
+    if isinstance(kv_lens, np.ndarray):
+        return int(kv_lens[:decode_end].sum()) if decode_end else 0
+    return 0
 
 
 def _require_gpu(t, name):
@@ -176,7 +187,7 @@ class RpaCall:
 
     def __init__(self, queries, kv_cache, v_pages, kv_lens_d, page_d, cu_q_d, cu_kv_d, *, num_seqs, decode_end,
                  sm_scale, sliding_window=None, soft_cap=None, mask_value=DEFAULT_MASK_VALUE, k_scale=None,
-                 v_scale=None, max_kv_len=0, max_q_len=0, num_splits=0, out=None):
+                 v_scale=None, max_kv_len=0, max_q_len=0, num_splits=0, out=None, sum_decode_kv_len=0):
         self.lib = _lib.load()
         self.device = queries.device
         fused = v_pages is None
@@ -193,7 +204,7 @@ class RpaCall:
         _fill_common(p, queries, self.out, num_seqs=num_seqs, decode_end=decode_end, page_size=page_size,
                      total_pages=total_pages, num_kv_heads=num_kv_heads, kv_dtype=kv_cache.dtype, sm_scale=sm_scale,
                      sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value, max_kv_len=max_kv_len,
-                     max_q_len=max_q_len, num_splits=num_splits)
+                     max_q_len=max_q_len, num_splits=num_splits, sum_decode_kv_len=sum_decode_kv_len)
         p.kv_cache = kv_cache.data_ptr()
         p.v_pages = None if fused else v_pages.data_ptr()
         p.layout = _lib.RPA_LAYOUT_FUSED if fused else _lib.RPA_LAYOUT_SPLIT
@@ -317,7 +328,8 @@ def ragged_paged_attention(
                    sm_scale=sm_scale, sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
                    k_scale=k_scale, v_scale=v_scale,
                    max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
-                   max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits)
+                   max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits,
+                   sum_decode_kv_len=_host_decode_sum(kv_lens, i))
     if validate_values:
         dynamic_validate_inputs(call.params, kv_lens_d.cpu().numpy(), page_d.cpu().numpy(), cu_q_d.cpu().numpy(),
                                 cu_kv_d.cpu().numpy(), dist.astype(np.int32))
@@ -380,7 +392,8 @@ def ragged_paged_attention_ref_surface(
                    sm_scale=sm_scale, sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
                    k_scale=k_scale, v_scale=v_scale,
                    max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
-                   max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits)
+                   max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits,
+                   sum_decode_kv_len=_host_decode_sum(kv_lens, decode_end))
     call.attention()
     return call.out
 
