@@ -16,9 +16,9 @@
 // that order (register transpose with v_perm_b32 while staging), so no data
 // crosses lanes between the two products.
 //
-// Workgroup ids are remapped so that consecutive logical tiles (all query
-// tiles and the G heads that share one kv head) run on the same XCD and hit
-// the same L2: hardware deals workgroup n to XCD n % 8.
+// Workgroup ids are remapped so that everything that reads one kv head of one
+// sequence runs on the same XCD (same L2) while the ragged sequences are spread
+// evenly over the 8 XCDs: hardware deals workgroup n to XCD n % 8.
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
@@ -35,6 +35,11 @@ constexpr int kVPitch = 144;  // bytes per V^T row in LDS (128 + 16 pad)
 __device__ __forceinline__ u32x4_t lds_ld16(const char* p) { return *reinterpret_cast<const u32x4_t*>(p); }
 __device__ __forceinline__ void lds_st16(char* p, u32x4_t v) { *reinterpret_cast<u32x4_t*>(p) = v; }
 
+// token (inside a 64-token tile) that lands at LDS position 8*tg + i of a V^T row
+__device__ __forceinline__ int vt_token(int tg, int i) {
+  return (tg >> 1) * 16 + (i >> 2) * 8 + (tg & 1) * 4 + (i & 3);
+}
+
 struct TileSrc {
   const int32_t* pages;
   int32_t page_size;
@@ -42,30 +47,51 @@ struct TileSrc {
   int32_t last_tok;
 };
 
-__device__ __forceinline__ int64_t row_offset(const TileSrc& s, const KvAddr& kv, int tok) {
-  tok = min(tok, s.last_tok);
-  const int slot = s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
-  const int page = s.pages[slot];
-  return (int64_t)page * kv.page_stride + (int64_t)(tok - slot * s.page_size) * kv.tok_stride;
+__device__ __forceinline__ int page_slot(const TileSrc& s, int tok) {
+  return s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
 }
 
-// token (inside a 64-token tile) that lands at LDS position 8*tg + i of a V^T row
-__device__ __forceinline__ int vt_token(int tg, int i) {
-  return (tg >> 1) * 16 + (i >> 2) * 8 + (tg & 1) * 4 + (i & 3);
-}
+// Page ids a thread needs for one tile, fetched one tile ahead of the rows themselves so
+// that the dependent chain "page id -> row address -> row" is never exposed.
+//   UNIFORM (page_size % 64 == 0): the whole tile lies in one page, one id.
+//   otherwise: the K loader needs 1 id, a V loader thread up to 8 (one per token it stages).
+template <bool UNIFORM>
+struct PageIds {
+  int32_t id[UNIFORM ? 1 : 8];
+};
 
 template <bool FP8>
 struct Stage {
   u32x4_t r[FP8 ? 4 : 8];
 };
 
+template <bool UNIFORM>
+__device__ __forceinline__ void fetch_page_ids(PageIds<UNIFORM>& pg, const TileSrc& s, int tb, int tid) {
+  if constexpr (UNIFORM) {
+    pg.id[0] = __builtin_amdgcn_readfirstlane(s.pages[page_slot(s, min(tb, s.last_tok))]);
+  } else {
+    if (tid < 128) {
+      pg.id[0] = s.pages[page_slot(s, min(tb + (tid >> 1), s.last_tok))];
+    } else {
+      const int tg = (tid - 128) & 7;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) pg.id[i] = s.pages[page_slot(s, min(tb + vt_token(tg, i), s.last_tok))];
+    }
+  }
+}
+
+__device__ __forceinline__ int64_t row_offset(const TileSrc& s, const KvAddr& kv, int tok, int page) {
+  tok = min(tok, s.last_tok);
+  return (int64_t)page * kv.page_stride + (int64_t)(tok - page_slot(s, tok) * s.page_size) * kv.tok_stride;
+}
+
 // Threads 0..127 stage K (one half row each), threads 128..255 stage V (8 tokens x 8 dims each).
-template <bool FP8>
-__device__ __forceinline__ void tile_gload(Stage<FP8>& st, const TileSrc& s, const KvAddr& kv,
-                                           const char* kh, const char* vh, int tb, int tid) {
+template <bool FP8, bool UNIFORM>
+__device__ __forceinline__ void tile_gload(Stage<FP8>& st, const TileSrc& s, const KvAddr& kv, const char* kh,
+                                           const char* vh, int tb, int tid, const PageIds<UNIFORM>& pg) {
   if (tid < 128) {
     const int tl = tid >> 1, half = tid & 1;
-    const char* p = kh + row_offset(s, kv, tb + tl) + half * (FP8 ? 64 : 128);
+    const char* p = kh + row_offset(s, kv, tb + tl, pg.id[0]) + half * (FP8 ? 64 : 128);
 #pragma unroll
     for (int i = 0; i < (FP8 ? 4 : 8); ++i) st.r[i] = ld16(p + i * 16);
   } else {
@@ -74,13 +100,14 @@ __device__ __forceinline__ void tile_gload(Stage<FP8>& st, const TileSrc& s, con
     if constexpr (FP8) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const u32x2_t w = ld8(vh + row_offset(s, kv, tb + vt_token(tg, i)) + dc * 8);
+        const u32x2_t w = ld8(vh + row_offset(s, kv, tb + vt_token(tg, i), pg.id[UNIFORM ? 0 : i]) + dc * 8);
         st.r[i >> 1][(i & 1) * 2 + 0] = w[0];
         st.r[i >> 1][(i & 1) * 2 + 1] = w[1];
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) st.r[i] = ld16(vh + row_offset(s, kv, tb + vt_token(tg, i)) + dc * 16);
+      for (int i = 0; i < 8; ++i)
+        st.r[i] = ld16(vh + row_offset(s, kv, tb + vt_token(tg, i), pg.id[UNIFORM ? 0 : i]) + dc * 16);
     }
   }
 }
@@ -140,19 +167,40 @@ __device__ __forceinline__ void tile_lstore(const Stage<FP8>& st, char* lds_k, c
   }
 }
 
-template <bool FP8>
+template <bool FP8, bool UNIFORM, bool CAP>
 __global__ __launch_bounds__(256, 2) void rpa_prefill_flash_kernel(const PrefillArgs a, int tiles, int nseq) {
-  __shared__ __attribute__((aligned(16))) char lds_k[kBN * kKPitch];
-  __shared__ __attribute__((aligned(16))) char lds_v[128 * kVPitch];
+  // two tile buffers: tile t+1 is written while tile t is read, one barrier per tile
+  __shared__ __attribute__((aligned(16))) char lds_k_buf[2][kBN * kKPitch];
+  __shared__ __attribute__((aligned(16))) char lds_v_buf[2][128 * kVPitch];
 
-  // ---- logical work id: XCD-chunked, query tile fastest, then head, then sequence ----
-  const int per_xcd = gridDim.x >> 3;
-  const int W = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  const int qt = tiles - 1 - (W % tiles);  // heavy (late) tiles first
-  const int rest = W / tiles;
-  const int head = rest % a.Hq;
-  const int si = rest / a.Hq;
-  if (si >= nseq) return;
+  // ---- work decomposition ----
+  // A unit is one (sequence, kv head): its G query heads and all their query tiles read the
+  // same K/V, so a unit stays on one XCD (one L2).  Hardware deals workgroup n to XCD n % 8;
+  // XCD x owns units x, x+8, ...: units of one sequence cost the same, so the XCDs stay
+  // balanced whatever the ragged lengths are.  Inside an XCD, late (long, causal) query
+  // tiles of every unit are issued first and the G heads of a unit sit next to each other.
+  const int units = nseq * a.Hkv;
+  int tile_rev, u, gi;
+  if (units >= 8) {
+    const int xcd = blockIdx.x & 7, r = blockIdx.x >> 3;
+    const int units_per_xcd = (units + 7) >> 3;
+    const int per_tile = units_per_xcd * a.G;
+    tile_rev = r / per_tile;
+    const int rest = r - tile_rev * per_tile;
+    u = xcd + 8 * (rest / a.G);
+    gi = rest % a.G;
+  } else {
+    const int per_tile = units * a.G;
+    tile_rev = blockIdx.x / per_tile;
+    const int rest = blockIdx.x - tile_rev * per_tile;
+    u = rest / a.G;
+    gi = rest % a.G;
+  }
+  if (u >= units || tile_rev >= tiles) return;
+  const int qt = tiles - 1 - tile_rev;
+  const int si = u / a.Hkv;
+  const int hk = u - si * a.Hkv;
+  const int head = hk * a.G + gi;
   const int seq = a.seq_begin + si;
   const int qg0 = a.pt.cu_q_lens[seq];
   const int q_len = a.pt.cu_q_lens[seq + 1] - qg0;
@@ -160,7 +208,6 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_flash_kernel(const Prefill
   if (q_start >= q_len) return;
   const int kv_len = a.pt.kv_lens[seq];
   const int prefix = kv_len - q_len;
-  const int hk = head / a.G;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -211,18 +258,32 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_flash_kernel(const Prefill
   int t_lo = 0;
   if (W_ > 0) t_lo = max(0, prefix + q_start - W_ + 1) & ~(kBN - 1);
 
+  // ---- pipeline: page ids run two tiles ahead, rows one tile ahead (in registers), LDS one
+  // tile ahead of the MFMAs.  Loads past the last tile re-read the last valid token.
   Stage<FP8> stg;
-  tile_gload<FP8>(stg, src, a.kv, kh, vh, t_lo, tid);
-  for (int tb = t_lo; tb < t_hi; tb += kBN) {
-    __syncthreads();
-    tile_lstore<FP8>(stg, lds_k, lds_v, tid);
-    __syncthreads();
-    if (tb + kBN < t_hi) tile_gload<FP8>(stg, src, a.kv, kh, vh, tb + kBN, tid);
+  PageIds<UNIFORM> pg;
+  fetch_page_ids<UNIFORM>(pg, src, t_lo, tid);
+  tile_gload<FP8, UNIFORM>(stg, src, a.kv, kh, vh, t_lo, tid, pg);
+  fetch_page_ids<UNIFORM>(pg, src, t_lo + kBN, tid);
+  tile_lstore<FP8>(stg, lds_k_buf[0], lds_v_buf[0], tid);
+  tile_gload<FP8, UNIFORM>(stg, src, a.kv, kh, vh, t_lo + kBN, tid, pg);
+  fetch_page_ids<UNIFORM>(pg, src, t_lo + 2 * kBN, tid);
+  __syncthreads();
+  int buf = 0;
+  for (int tb = t_lo; tb < t_hi; tb += kBN, buf ^= 1) {
+    const char* lds_k = lds_k_buf[buf];
+    const char* lds_v = lds_v_buf[buf];
+    if (tb + kBN < t_hi) {
+      // the other buffer was last read before the barrier that ended the previous tile
+      tile_lstore<FP8>(stg, lds_k_buf[buf ^ 1], lds_v_buf[buf ^ 1], tid);
+      tile_gload<FP8, UNIFORM>(stg, src, a.kv, kh, vh, tb + 2 * kBN, tid, pg);
+      fetch_page_ids<UNIFORM>(pg, src, tb + 3 * kBN, tid);
+    }
 
     // visible to this wave?  causal: some token <= last row's position; window: some token
     // newer than the first row's horizon
     const bool vis = wave_active && (tb <= prefix + r_hi) && (W_ <= 0 || tb + kBN - 1 > prefix + r_lo - W_);
-    if (!vis) continue;
+    if (vis) {
     const bool need_mask = (tb + kBN - 1 > prefix + r_lo) || (W_ > 0 && tb <= prefix + r_hi - W_);
 
     f32x16_t S[2];
@@ -235,7 +296,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_flash_kernel(const Prefill
       for (int ks = 0; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ks * 32), qB[ks], S[mt]);
     }
     // scores -> log2 units
-    if (cap != 0.f) {
+    if constexpr (CAP) {
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -280,10 +341,13 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_flash_kernel(const Prefill
       }
     l = l * alpha + ps;
     m = m_new;
+    // the running max rarely moves once a few tiles are in: rescale only if some lane needs it
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-    for (int d = 0; d < 4; ++d)
+      for (int d = 0; d < 4; ++d)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) O[d][v] *= alpha;
+        for (int v = 0; v < 16; ++v) O[d][v] *= alpha;
+    }
     u32x4_t pB[2][2];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -302,6 +366,8 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_flash_kernel(const Prefill
         for (int kk = 0; kk < 2; ++kk)
           O[d] = mfma32(lds_ld16(vp + (mt * 32 + kk * 16) * 2), pB[mt][kk], O[d]);
     }
+    }  // vis
+    __syncthreads();
   }
 
   // ---- epilogue: lane (c, h) holds query row c, dims 32d + 8*(v/4) + 4h + v%4 ----
@@ -326,13 +392,25 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const int nseq = a.seq_end - a.seq_begin;
   if (nseq <= 0 || a.max_q_len <= 0) return hipSuccess;
   const int tiles = (a.max_q_len + kBM - 1) / kBM;
-  const int64_t work = (int64_t)tiles * a.Hq * nseq;
-  const int64_t grid = (work + 7) / 8 * 8;
+  const int64_t units = (int64_t)nseq * a.Hkv;
+  const int64_t grid = (units >= 8 ? ((units + 7) / 8) * 8 : units) * a.G * tiles;
   if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
-  if (a.fp8)
-    hipLaunchKernelGGL(rpa_prefill_flash_kernel<true>, dim3((unsigned)grid), dim3(256), 0, stream, a, tiles, nseq);
-  else
-    hipLaunchKernelGGL(rpa_prefill_flash_kernel<false>, dim3((unsigned)grid), dim3(256), 0, stream, a, tiles, nseq);
+  const bool uniform = (a.pt.page_size % kBN) == 0;
+  const bool cap = a.sm.soft_cap != 0.f;
+  const dim3 g((unsigned)grid), blk(256);
+#define RPA_PREFILL_LAUNCH(F, U, C) \
+  hipLaunchKernelGGL((rpa_prefill_flash_kernel<F, U, C>), g, blk, 0, stream, a, tiles, nseq)
+  switch ((a.fp8 ? 4 : 0) | (uniform ? 2 : 0) | (cap ? 1 : 0)) {
+    case 0: RPA_PREFILL_LAUNCH(false, false, false); break;
+    case 1: RPA_PREFILL_LAUNCH(false, false, true); break;
+    case 2: RPA_PREFILL_LAUNCH(false, true, false); break;
+    case 3: RPA_PREFILL_LAUNCH(false, true, true); break;
+    case 4: RPA_PREFILL_LAUNCH(true, false, false); break;
+    case 5: RPA_PREFILL_LAUNCH(true, false, true); break;
+    case 6: RPA_PREFILL_LAUNCH(true, true, false); break;
+    default: RPA_PREFILL_LAUNCH(true, true, true); break;
+  }
+#undef RPA_PREFILL_LAUNCH
   return hipGetLastError();
 }
 
