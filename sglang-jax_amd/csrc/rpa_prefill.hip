@@ -2,23 +2,30 @@
 //
 // One workgroup (4 waves) owns a tile of 128 query positions of one query head
 // of one sequence; wave w owns 32 of them.  KV is walked in tiles of 64 tokens
-// gathered through the page table:
-//   global -> registers -> LDS   K tile  [64 tok][128 dims]  (row pitch 272 B)
-//                                V tile  transposed [128 dims][64 tok] (pitch 144 B)
+// gathered through the page table into a two-deep LDS ring (tile t+1 arrives
+// while tile t is consumed, one barrier per tile):
 //   S^T[tok, q]  = K . Q^T        v_mfma_f32_32x32x16_bf16, A = K rows from LDS,
 //                                 B = Q^T held in registers for the whole loop
 //   online softmax per query column (in-lane over tokens + one lane swap)
-//   O^T[dim, q] += V^T . P^T      A = V^T rows from LDS, B = P^T straight from
-//                                 the S^T result registers
+//   O^T[dim, q] += V^T . P^T      A = V^T from LDS, B = P^T straight from the
+//                                 S^T result registers
 // The S^T result layout (lane = query, registers = tokens) is the B operand
-// layout of the second product provided the 16 tokens of a k-step are ordered
-// 16kk + 8*(i/4) + 4h + i%4; the V loader writes its transposed rows in exactly
-// that order (register transpose with v_perm_b32 while staging), so no data
-// crosses lanes between the two products.
+// layout of the second product when the 16 tokens of a k-step are ordered
+// 16kk + 8*(i/4) + 4h + i%4 -- no data crosses lanes between the two products.
+//
+// Two data paths feed the LDS ring:
+//   * bf16 cache ("async"): global_load_lds_dwordx4 copies 16-byte chunks straight
+//     into LDS, rows kept row-major with XOR-swizzled chunk positions (no padding,
+//     no staging registers).  K operands are ds_read_b128; V^T operands come from
+//     the row-major V rows through the transposing LDS read ds_read_b64_tr_b16.
+//   * fp8 cache ("staged"): rows pass through registers, are dequantised to bf16
+//     once, and V is transposed in registers (v_perm_b32) before it is written.
 //
 // Workgroup ids are remapped so that everything that reads one kv head of one
 // sequence runs on the same XCD (same L2) while the ragged sequences are spread
 // evenly over the 8 XCDs: hardware deals workgroup n to XCD n % 8.
+
+#include <cstdlib>
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
@@ -27,15 +34,26 @@ namespace rpa {
 
 namespace {
 
-constexpr int kBM = 128;      // query rows per workgroup
-constexpr int kBN = 64;       // kv tokens per tile
-constexpr int kKPitch = 272;  // bytes per K row in LDS (256 + 16 pad: conflict-free b128 reads)
-constexpr int kVPitch = 144;  // bytes per V^T row in LDS (128 + 16 pad)
+constexpr int kBM = 128;  // query rows per workgroup
+constexpr int kBN = 64;   // kv tokens per tile
 
 __device__ __forceinline__ u32x4_t lds_ld16(const char* p) { return *reinterpret_cast<const u32x4_t*>(p); }
 __device__ __forceinline__ void lds_st16(char* p, u32x4_t v) { *reinterpret_cast<u32x4_t*>(p) = v; }
 
-// token (inside a 64-token tile) that lands at LDS position 8*tg + i of a V^T row
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+// ds_read_b64_tr_b16: inside every block of 16 lanes, lane i receives
+//   out[e] = M[(i >> 2) + 4e][i & 3],  e = 0..3,
+// where M[r][0..3] are the four 16-bit elements at the address supplied by lane r of
+// the block.  With lane r pointing at (token r >> 2, dims 4*(r & 3) ..) of a row-major
+// tile, lane i ends up with dim i of four tokens: the k-contiguous MFMA operand.
+__device__ __forceinline__ u32x2_t lds_tr16(const char* p) {
+  typedef __attribute__((address_space(3))) s16x4_t* lds_ptr_t;
+  const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p));
+  return __builtin_bit_cast(u32x2_t, v);
+}
+
+// token (inside a 64-token tile) that lands at LDS position 8*tg + i of a staged V^T row
 __device__ __forceinline__ int vt_token(int tg, int i) {
   return (tg >> 1) * 16 + (i >> 2) * 8 + (tg & 1) * 4 + (i & 3);
 }
@@ -51,10 +69,336 @@ __device__ __forceinline__ int page_slot(const TileSrc& s, int tok) {
   return s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
 }
 
-// Page ids a thread needs for one tile, fetched one tile ahead of the rows themselves so
-// that the dependent chain "page id -> row address -> row" is never exposed.
-//   UNIFORM (page_size % 64 == 0): the whole tile lies in one page, one id.
-//   otherwise: the K loader needs 1 id, a V loader thread up to 8 (one per token it stages).
+// Byte offset of token `tok` of the tile starting at `tb`.  UNIFORM (page_size % 64 == 0):
+// the tile lies inside the page `page`.
+template <bool UNIFORM>
+__device__ __forceinline__ int64_t row_offset(const TileSrc& s, const KvAddr& kv, int tb, int tok, int page) {
+  tok = min(tok, s.last_tok);
+  if constexpr (UNIFORM) {
+    const int page_tok0 = page_slot(s, tb) * s.page_size;  // wave-uniform
+    return (int64_t)page * kv.page_stride + (int64_t)((tok - page_tok0) * kv.tok_stride);
+  } else {
+    return (int64_t)page * kv.page_stride + (int64_t)(tok - page_slot(s, tok) * s.page_size) * kv.tok_stride;
+  }
+}
+
+// ------------------------------------------------------------------ work decomposition
+// A unit is one (sequence, kv head): its G query heads and all their query tiles read the
+// same K/V, so a unit stays on one XCD (one L2).  Hardware deals workgroup n to XCD n % 8;
+// XCD x owns units x, x+8, ...: units of one sequence cost the same, so the XCDs stay
+// balanced whatever the ragged lengths are.  Inside an XCD, late (long, causal) query
+// tiles of every unit are issued first and the G heads of a unit sit next to each other.
+struct Work {
+  int seq, hk, head, q_start, qg0, q_len, kv_len, prefix;
+  bool valid;
+};
+
+__device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int nseq) {
+  Work w;
+  w.valid = false;
+  const int units = nseq * a.Hkv;
+  int tile_rev, u, gi;
+  if (units >= 8) {
+    const int xcd = blockIdx.x & 7, r = blockIdx.x >> 3;
+    const int units_per_xcd = (units + 7) >> 3;
+    const int per_tile = units_per_xcd * a.G;
+    tile_rev = r / per_tile;
+    const int rest = r - tile_rev * per_tile;
+    u = xcd + 8 * (rest / a.G);
+    gi = rest % a.G;
+  } else {
+    const int per_tile = units * a.G;
+    tile_rev = blockIdx.x / per_tile;
+    const int rest = blockIdx.x - tile_rev * per_tile;
+    u = rest / a.G;
+    gi = rest % a.G;
+  }
+  if (u >= units || tile_rev >= tiles) return w;
+  const int si = u / a.Hkv;
+  w.hk = u - si * a.Hkv;
+  w.head = w.hk * a.G + gi;
+  w.seq = a.seq_begin + si;
+  w.qg0 = a.pt.cu_q_lens[w.seq];
+  w.q_len = a.pt.cu_q_lens[w.seq + 1] - w.qg0;
+  w.q_start = (tiles - 1 - tile_rev) * kBM;
+  if (w.q_start >= w.q_len) return w;
+  w.kv_len = a.pt.kv_lens[w.seq];
+  w.prefix = w.kv_len - w.q_len;
+  w.valid = true;
+  return w;
+}
+
+__device__ __forceinline__ TileSrc make_src(const PrefillArgs& a, const Work& w) {
+  TileSrc src;
+  src.page_size = a.pt.page_size;
+  src.page_shift = ((src.page_size & (src.page_size - 1)) == 0) ? (31 - __builtin_clz(src.page_size)) : -1;
+  src.last_tok = w.kv_len - 1;
+  src.pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[w.seq] / a.pt.page_size)
+                                                  : (int64_t)w.seq * a.pt.pages_per_seq);
+  return src;
+}
+
+// ------------------------------------------------------------------ per-wave state and softmax
+struct WaveRows {
+  int r_lo, r_hi, row, qpos;
+  bool active;
+};
+
+template <bool CAP>
+struct Softmax {
+  float scale, cap, inv_cap, sc2;
+};
+
+// Online-softmax update of one 64-token tile.  On entry S holds raw scores (MFMA units); on
+// exit it holds the probabilities.  Scores stay in MFMA units; sc2 turns them into log2 units
+// inside the exponent: p = 2^(s*sc2 - m*sc2) is one fused multiply-add per score (soft-capped
+// scores are already in log2 units, sc2 = 1).  The running max starts at a finite floor far
+// above the mask value, so a row whose tokens are all masked in this tile gets p = 0, not 2^0.
+constexpr float kMaxFloor = -1.0e30f;
+constexpr float kMaskRaw = -3.0e38f;
+
+template <bool CAP>
+__device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4], float& m, float& l,
+                                             const Softmax<CAP>& sm, bool need_mask, int tb, int h, int qpos,
+                                             int window) {
+  if constexpr (CAP) {
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) S[mt][v] = soft_cap_f(S[mt][v] * sm.scale, sm.cap, sm.inv_cap) * kLog2e;
+  }
+  if (need_mask) {
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int tok = tb + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        const bool masked = (tok > qpos) || (window > 0 && tok <= qpos - window);
+        S[mt][v] = masked ? kMaskRaw : S[mt][v];
+      }
+  }
+  float mx = fmaxf(S[0][0], S[1][0]);
+#pragma unroll
+  for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(S[0][v], S[1][v]));
+  mx = fmaxf(mx, __shfl_xor(mx, 32));
+  const float m_new = fmaxf(m, mx);
+  const float alpha = fast_exp2((m - m_new) * sm.sc2);
+  const float neg_m = -m_new * sm.sc2;
+  float ps = 0.f;
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float p = fast_exp2(__builtin_fmaf(S[mt][v], sm.sc2, neg_m));
+      S[mt][v] = p;
+      ps += p;
+    }
+  l = l * alpha + ps;
+  m = m_new;
+  // the running max rarely moves once a few tiles are in: rescale only if some lane needs it
+  if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) O[d][v] *= alpha;
+  }
+}
+
+__device__ __forceinline__ void pack_probs(const f32x16_t (&S)[2], u32x4_t (&pB)[2][2]) {
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+      pB[mt][kk] = u32x4_t{pack_bf16x2(S[mt][8 * kk + 0], S[mt][8 * kk + 1]),
+                           pack_bf16x2(S[mt][8 * kk + 2], S[mt][8 * kk + 3]),
+                           pack_bf16x2(S[mt][8 * kk + 4], S[mt][8 * kk + 5]),
+                           pack_bf16x2(S[mt][8 * kk + 6], S[mt][8 * kk + 7])};
+}
+
+// lane (c, h) holds query row c, dims 32d + 8*(v/4) + 4h + v%4 in O[d][v]
+__device__ __forceinline__ void write_rows(const PrefillArgs& a, const Work& w, const WaveRows& wr,
+                                           const f32x16_t (&O)[4], float l, int h) {
+  l += __shfl_xor(l, 32);
+  if (!wr.active || wr.row >= w.q_len) return;
+  const float vs = a.v_scale ? a.v_scale[w.hk] : 1.0f;
+  const float inv = vs / l;
+  uint16_t* op = a.out + ((int64_t)(w.qg0 + wr.row) * a.Hq + w.head) * 128 + 4 * h;
+#pragma unroll
+  for (int d = 0; d < 4; ++d)
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq) {
+      u32x2_t o = {pack_bf16x2(O[d][4 * vq + 0] * inv, O[d][4 * vq + 1] * inv),
+                   pack_bf16x2(O[d][4 * vq + 2] * inv, O[d][4 * vq + 3] * inv)};
+      *reinterpret_cast<u32x2_t*>(op + d * 32 + vq * 8) = o;
+    }
+}
+
+// ==================================================================== async path (bf16 cache)
+constexpr int kRowB = 256;             // one K or V row of a head: 128 bf16, unpadded
+constexpr int kTileB = kBN * kRowB;    // 16 KiB
+
+// 16-byte chunk j of row t sits at chunk position j ^ swizzle(t):
+//   K: swizzle = t & 15      (ds_read_b128: 16 consecutive tokens -> 16 distinct chunk columns)
+//   V: swizzle = 4 * (t & 3) (transposing read: 4 consecutive tokens -> 4 distinct 64-byte windows)
+template <bool UNIFORM>
+struct AsyncPages {
+  int32_t id[UNIFORM ? 1 : 4];
+};
+
+template <bool UNIFORM>
+__device__ __forceinline__ void async_fetch_pages(AsyncPages<UNIFORM>& pg, const TileSrc& s, int tb, int wave,
+                                                  int lane) {
+  tb = min(tb, s.last_tok & ~(kBN - 1));
+  if constexpr (UNIFORM) {
+    pg.id[0] = __builtin_amdgcn_readfirstlane(s.pages[page_slot(s, tb)]);
+  } else {
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const int t = (wave * 4 + n) * 4 + (lane >> 4);
+      pg.id[n] = s.pages[page_slot(s, min(tb + t, s.last_tok))];
+    }
+  }
+}
+
+// Every wave copies 4 x 64 chunks of K and of V: chunk position p = 64*(4*wave + n) + lane of
+// the tile, i.e. row p / 16, chunk column p % 16.
+template <bool UNIFORM>
+__device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const TileSrc& s, const KvAddr& kv,
+                                                const char* kh, const char* vh, int tb, int wave, int lane,
+                                                const AsyncPages<UNIFORM>& pg) {
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  tb = min(tb, s.last_tok & ~(kBN - 1));  // past the end: re-copy the last tile
+  const int cp = lane & 15;
+#pragma unroll
+  for (int n = 0; n < 4; ++n) {
+    const int blk = wave * 4 + n;
+    const int t = blk * 4 + (lane >> 4);
+    const int64_t ro = row_offset<UNIFORM>(s, kv, tb, tb + t, pg.id[UNIFORM ? 0 : n]);
+    const int jk = cp ^ (t & 15);
+    const int jv = cp ^ ((t & 3) << 2);
+    __builtin_amdgcn_global_load_lds((gptr_t)(kh + ro + jk * 16), (lptr_t)(lds_k + blk * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gptr_t)(vh + ro + jv * 16), (lptr_t)(lds_v + blk * 1024), 16, 0, 0);
+  }
+}
+
+template <bool UNIFORM, bool CAP>
+__global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const PrefillArgs a, int tiles, int nseq) {
+  __shared__ __attribute__((aligned(1024))) char lds_k_buf[2][kTileB];
+  __shared__ __attribute__((aligned(1024))) char lds_v_buf[2][kTileB];
+
+  const Work w = decompose(a, tiles, nseq);
+  if (!w.valid) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 31, h = lane >> 5;
+  const TileSrc src = make_src(a, w);
+  const char* kh = a.kv.k_base + (int64_t)w.hk * a.kv.head_stride;
+  const char* vh = a.kv.v_base + (int64_t)w.hk * a.kv.head_stride;
+
+  WaveRows wr;
+  wr.r_lo = w.q_start + wave * 32;
+  wr.r_hi = min(wr.r_lo + 31, w.q_len - 1);
+  wr.active = wr.r_lo < w.q_len;
+  wr.row = wr.r_lo + c;
+  wr.qpos = w.prefix + wr.row;
+  const int W_ = a.sm.window;
+
+  u32x4_t qB[8];
+  {
+    const int rr = min(wr.row, w.q_len - 1);
+    const uint16_t* qp = a.q + ((int64_t)(w.qg0 + rr) * a.Hq + w.head) * 128 + h * 8;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qB[ks] = ld16(qp + ks * 16);
+  }
+  Softmax<CAP> sm;
+  sm.scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f);
+  sm.cap = a.sm.soft_cap;
+  sm.inv_cap = (sm.cap != 0.f) ? 1.0f / sm.cap : 0.f;
+  sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e;
+
+  f32x16_t O[4];
+#pragma unroll
+  for (int d = 0; d < 4; ++d)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) O[d][v] = 0.f;
+  float m = kMaxFloor, l = 0.f;
+
+  const int wg_r_hi = min(w.q_start + kBM, w.q_len) - 1;
+  const int t_hi = min(w.kv_len, w.prefix + wg_r_hi + 1);  // exclusive
+  int t_lo = 0;
+  if (W_ > 0) t_lo = max(0, w.prefix + w.q_start - W_ + 1) & ~(kBN - 1);
+
+  // ---- operand addresses inside a tile (bytes) ----
+  // K operand of (m-tile mt, k-step ks): row 32mt + c, chunk (2ks + h) ^ (c & 15)
+  const int k_row = c * kRowB;
+  const int k_swz = (h ^ (c & 15)) << 4;  // chunk = (2ks) ^ (h ^ (c & 15)), in bytes: (32ks) ^ k_swz
+  // V^T operand of (dim tile d, m-tile mt, k-step kk), first / second half of the k-step:
+  //   source lane r = lane & 15 of its 16-lane block points at token 32mt + 16kk + 4h + (r >> 2) (+ 8),
+  //   dims 32d + 16*(block & 1) + 4*(r & 3); chunk = (4d + 2*(block & 1) + ((r & 3) >> 1)) ^ (4*(r >> 2))
+  const int r16 = lane & 15, b16 = lane >> 4;
+  const int v_row = (4 * h + (r16 >> 2)) * kRowB;
+  const int v_in = ((b16 & 1) << 5) + (((r16 & 3) >> 1) << 4) + ((r16 & 1) << 3);
+  const int v_swz = (r16 >> 2) << 6;  // byte offset of the 64-byte window: (64d) ^ v_swz
+
+  // ---- pipeline: page ids two tiles ahead, the asynchronous copy one tile ahead ----
+  AsyncPages<UNIFORM> pg;
+  async_fetch_pages<UNIFORM>(pg, src, t_lo, wave, lane);
+  async_copy_tile<UNIFORM>(lds_k_buf[0], lds_v_buf[0], src, a.kv, kh, vh, t_lo, wave, lane, pg);
+  async_fetch_pages<UNIFORM>(pg, src, t_lo + kBN, wave, lane);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the copies have landed in LDS
+  __syncthreads();
+  int buf = 0;
+  for (int tb = t_lo; tb < t_hi; tb += kBN, buf ^= 1) {
+    const char* lds_k = lds_k_buf[buf];
+    const char* lds_v = lds_v_buf[buf];
+    if (tb + kBN < t_hi) {
+      // the other buffer was last read before the barrier that ended the previous tile
+      async_copy_tile<UNIFORM>(lds_k_buf[buf ^ 1], lds_v_buf[buf ^ 1], src, a.kv, kh, vh, tb + kBN, wave, lane, pg);
+      async_fetch_pages<UNIFORM>(pg, src, tb + 2 * kBN, wave, lane);
+    }
+    // visible to this wave?  causal: some token <= last row's position; window: some token
+    // newer than the first row's horizon
+    const bool vis = wr.active && (tb <= w.prefix + wr.r_hi) && (W_ <= 0 || tb + kBN - 1 > w.prefix + wr.r_lo - W_);
+    if (vis) {
+      const bool need_mask = (tb + kBN - 1 > w.prefix + wr.r_lo) || (W_ > 0 && tb <= w.prefix + wr.r_hi - W_);
+      f32x16_t S[2];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) S[mt][v] = 0.f;
+        const char* kp = lds_k + mt * 32 * kRowB + k_row;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ((ks * 32) ^ k_swz)), qB[ks], S[mt]);
+      }
+      softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_);
+      u32x4_t pB[2][2];
+      pack_probs(S, pB);
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const char* vp = lds_v + v_row + v_in + ((d * 64) ^ v_swz);
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk) {
+            const char* vt = vp + (mt * 32 + kk * 16) * kRowB;
+            const u32x2_t lo = lds_tr16(vt);
+            const u32x2_t hi = lds_tr16(vt + 8 * kRowB);
+            O[d] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, pB[mt][kk], O[d]);
+          }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // the next tile has landed
+    __syncthreads();
+  }
+  write_rows(a, w, wr, O, l, h);
+}
+
+// ==================================================================== staged path (fp8 cache)
+constexpr int kKPitch = 272;  // bytes per K row in LDS (256 + 16 pad: conflict-free b128 reads)
+constexpr int kVPitch = 144;  // bytes per V^T row in LDS (128 + 16 pad)
+
 template <bool UNIFORM>
 struct PageIds {
   int32_t id[UNIFORM ? 1 : 8];
@@ -67,8 +411,9 @@ struct Stage {
 
 template <bool UNIFORM>
 __device__ __forceinline__ void fetch_page_ids(PageIds<UNIFORM>& pg, const TileSrc& s, int tb, int tid) {
+  tb = min(tb, s.last_tok & ~(kBN - 1));
   if constexpr (UNIFORM) {
-    pg.id[0] = __builtin_amdgcn_readfirstlane(s.pages[page_slot(s, min(tb, s.last_tok))]);
+    pg.id[0] = __builtin_amdgcn_readfirstlane(s.pages[page_slot(s, tb)]);
   } else {
     if (tid < 128) {
       pg.id[0] = s.pages[page_slot(s, min(tb + (tid >> 1), s.last_tok))];
@@ -80,18 +425,14 @@ __device__ __forceinline__ void fetch_page_ids(PageIds<UNIFORM>& pg, const TileS
   }
 }
 
-__device__ __forceinline__ int64_t row_offset(const TileSrc& s, const KvAddr& kv, int tok, int page) {
-  tok = min(tok, s.last_tok);
-  return (int64_t)page * kv.page_stride + (int64_t)(tok - page_slot(s, tok) * s.page_size) * kv.tok_stride;
-}
-
 // Threads 0..127 stage K (one half row each), threads 128..255 stage V (8 tokens x 8 dims each).
 template <bool FP8, bool UNIFORM>
 __device__ __forceinline__ void tile_gload(Stage<FP8>& st, const TileSrc& s, const KvAddr& kv, const char* kh,
                                            const char* vh, int tb, int tid, const PageIds<UNIFORM>& pg) {
+  tb = min(tb, s.last_tok & ~(kBN - 1));  // past the end: re-read the last tile
   if (tid < 128) {
     const int tl = tid >> 1, half = tid & 1;
-    const char* p = kh + row_offset(s, kv, tb + tl, pg.id[0]) + half * (FP8 ? 64 : 128);
+    const char* p = kh + row_offset<UNIFORM>(s, kv, tb, tb + tl, pg.id[0]) + half * (FP8 ? 64 : 128);
 #pragma unroll
     for (int i = 0; i < (FP8 ? 4 : 8); ++i) st.r[i] = ld16(p + i * 16);
   } else {
@@ -100,14 +441,15 @@ __device__ __forceinline__ void tile_gload(Stage<FP8>& st, const TileSrc& s, con
     if constexpr (FP8) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const u32x2_t w = ld8(vh + row_offset(s, kv, tb + vt_token(tg, i), pg.id[UNIFORM ? 0 : i]) + dc * 8);
-        st.r[i >> 1][(i & 1) * 2 + 0] = w[0];
-        st.r[i >> 1][(i & 1) * 2 + 1] = w[1];
+        const u32x2_t x =
+            ld8(vh + row_offset<UNIFORM>(s, kv, tb, tb + vt_token(tg, i), pg.id[UNIFORM ? 0 : i]) + dc * 8);
+        st.r[i >> 1][(i & 1) * 2 + 0] = x[0];
+        st.r[i >> 1][(i & 1) * 2 + 1] = x[1];
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        st.r[i] = ld16(vh + row_offset(s, kv, tb + vt_token(tg, i), pg.id[UNIFORM ? 0 : i]) + dc * 16);
+        st.r[i] = ld16(vh + row_offset<UNIFORM>(s, kv, tb, tb + vt_token(tg, i), pg.id[UNIFORM ? 0 : i]) + dc * 16);
     }
   }
 }
@@ -168,98 +510,54 @@ __device__ __forceinline__ void tile_lstore(const Stage<FP8>& st, char* lds_k, c
 }
 
 template <bool FP8, bool UNIFORM, bool CAP>
-__global__ __launch_bounds__(256, 2) void rpa_prefill_flash_kernel(const PrefillArgs a, int tiles, int nseq) {
-  // two tile buffers: tile t+1 is written while tile t is read, one barrier per tile
+__global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const PrefillArgs a, int tiles, int nseq) {
   __shared__ __attribute__((aligned(16))) char lds_k_buf[2][kBN * kKPitch];
   __shared__ __attribute__((aligned(16))) char lds_v_buf[2][128 * kVPitch];
 
-  // ---- work decomposition ----
-  // A unit is one (sequence, kv head): its G query heads and all their query tiles read the
-  // same K/V, so a unit stays on one XCD (one L2).  Hardware deals workgroup n to XCD n % 8;
-  // XCD x owns units x, x+8, ...: units of one sequence cost the same, so the XCDs stay
-  // balanced whatever the ragged lengths are.  Inside an XCD, late (long, causal) query
-  // tiles of every unit are issued first and the G heads of a unit sit next to each other.
-  const int units = nseq * a.Hkv;
-  int tile_rev, u, gi;
-  if (units >= 8) {
-    const int xcd = blockIdx.x & 7, r = blockIdx.x >> 3;
-    const int units_per_xcd = (units + 7) >> 3;
-    const int per_tile = units_per_xcd * a.G;
-    tile_rev = r / per_tile;
-    const int rest = r - tile_rev * per_tile;
-    u = xcd + 8 * (rest / a.G);
-    gi = rest % a.G;
-  } else {
-    const int per_tile = units * a.G;
-    tile_rev = blockIdx.x / per_tile;
-    const int rest = blockIdx.x - tile_rev * per_tile;
-    u = rest / a.G;
-    gi = rest % a.G;
-  }
-  if (u >= units || tile_rev >= tiles) return;
-  const int qt = tiles - 1 - tile_rev;
-  const int si = u / a.Hkv;
-  const int hk = u - si * a.Hkv;
-  const int head = hk * a.G + gi;
-  const int seq = a.seq_begin + si;
-  const int qg0 = a.pt.cu_q_lens[seq];
-  const int q_len = a.pt.cu_q_lens[seq + 1] - qg0;
-  const int q_start = qt * kBM;
-  if (q_start >= q_len) return;
-  const int kv_len = a.pt.kv_lens[seq];
-  const int prefix = kv_len - q_len;
-
+  const Work w = decompose(a, tiles, nseq);
+  if (!w.valid) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int c = lane & 31, h = lane >> 5;
+  const TileSrc src = make_src(a, w);
+  const char* kh = a.kv.k_base + (int64_t)w.hk * a.kv.head_stride;
+  const char* vh = a.kv.v_base + (int64_t)w.hk * a.kv.head_stride;
 
-  TileSrc src;
-  src.page_size = a.pt.page_size;
-  src.page_shift = ((src.page_size & (src.page_size - 1)) == 0) ? (31 - __builtin_clz(src.page_size)) : -1;
-  src.last_tok = kv_len - 1;
-  src.pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[seq] / a.pt.page_size)
-                                                  : (int64_t)seq * a.pt.pages_per_seq);
-  const char* kh = a.kv.k_base + (int64_t)hk * a.kv.head_stride;
-  const char* vh = a.kv.v_base + (int64_t)hk * a.kv.head_stride;
-
-  // ---- this wave's query rows ----
-  const int r_lo = q_start + wave * 32;
-  const int r_hi = min(r_lo + 31, q_len - 1);
-  const bool wave_active = r_lo < q_len;
-  const int row = r_lo + c;
-  const int qpos = prefix + row;  // position of this lane's query inside the sequence
+  WaveRows wr;
+  wr.r_lo = w.q_start + wave * 32;
+  wr.r_hi = min(wr.r_lo + 31, w.q_len - 1);
+  wr.active = wr.r_lo < w.q_len;
+  wr.row = wr.r_lo + c;
+  wr.qpos = w.prefix + wr.row;
   const int W_ = a.sm.window;
 
   u32x4_t qB[8];
   {
-    const int rr = min(row, q_len - 1);
-    const uint16_t* qp = a.q + ((int64_t)(qg0 + rr) * a.Hq + head) * 128 + h * 8;
+    const int rr = min(wr.row, w.q_len - 1);
+    const uint16_t* qp = a.q + ((int64_t)(w.qg0 + rr) * a.Hq + w.head) * 128 + h * 8;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qB[ks] = ld16(qp + ks * 16);
   }
-
-  const float ksc = a.k_scale ? a.k_scale[hk] : 1.0f;
-  const float scale = a.sm.sm_scale * ksc;
-  const float scale2 = scale * kLog2e;
-  const float cap = a.sm.soft_cap;
-  const float inv_cap = (cap != 0.f) ? 1.0f / cap : 0.f;
-  const float mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
+  Softmax<CAP> sm;
+  sm.scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f);
+  sm.cap = a.sm.soft_cap;
+  sm.inv_cap = (sm.cap != 0.f) ? 1.0f / sm.cap : 0.f;
+  sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e;
 
   f32x16_t O[4];
 #pragma unroll
   for (int d = 0; d < 4; ++d)
 #pragma unroll
     for (int v = 0; v < 16; ++v) O[d][v] = 0.f;
-  float m = -INFINITY, l = 0.f;
+  float m = kMaxFloor, l = 0.f;
 
-  // ---- kv tile range of the workgroup ----
-  const int wg_r_hi = min(q_start + kBM, q_len) - 1;
-  const int t_hi = min(kv_len, prefix + wg_r_hi + 1);  // exclusive
+  const int wg_r_hi = min(w.q_start + kBM, w.q_len) - 1;
+  const int t_hi = min(w.kv_len, w.prefix + wg_r_hi + 1);  // exclusive
   int t_lo = 0;
-  if (W_ > 0) t_lo = max(0, prefix + q_start - W_ + 1) & ~(kBN - 1);
+  if (W_ > 0) t_lo = max(0, w.prefix + w.q_start - W_ + 1) & ~(kBN - 1);
 
   // ---- pipeline: page ids run two tiles ahead, rows one tile ahead (in registers), LDS one
-  // tile ahead of the MFMAs.  Loads past the last tile re-read the last valid token.
+  // tile ahead of the MFMAs.  Loads past the last tile re-read the last tile.
   Stage<FP8> stg;
   PageIds<UNIFORM> pg;
   fetch_page_ids<UNIFORM>(pg, src, t_lo, tid);
@@ -279,111 +577,34 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_flash_kernel(const Prefill
       tile_gload<FP8, UNIFORM>(stg, src, a.kv, kh, vh, tb + 2 * kBN, tid, pg);
       fetch_page_ids<UNIFORM>(pg, src, tb + 3 * kBN, tid);
     }
-
-    // visible to this wave?  causal: some token <= last row's position; window: some token
-    // newer than the first row's horizon
-    const bool vis = wave_active && (tb <= prefix + r_hi) && (W_ <= 0 || tb + kBN - 1 > prefix + r_lo - W_);
+    const bool vis = wr.active && (tb <= w.prefix + wr.r_hi) && (W_ <= 0 || tb + kBN - 1 > w.prefix + wr.r_lo - W_);
     if (vis) {
-    const bool need_mask = (tb + kBN - 1 > prefix + r_lo) || (W_ > 0 && tb <= prefix + r_hi - W_);
-
-    f32x16_t S[2];
+      const bool need_mask = (tb + kBN - 1 > w.prefix + wr.r_lo) || (W_ > 0 && tb <= w.prefix + wr.r_hi - W_);
+      f32x16_t S[2];
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+      for (int mt = 0; mt < 2; ++mt) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) S[mt][v] = 0.f;
-      const char* kp = lds_k + (mt * 32 + c) * kKPitch + h * 16;
+        for (int v = 0; v < 16; ++v) S[mt][v] = 0.f;
+        const char* kp = lds_k + (mt * 32 + c) * kKPitch + h * 16;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ks * 32), qB[ks], S[mt]);
-    }
-    // scores -> log2 units
-    if constexpr (CAP) {
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) S[mt][v] = soft_cap_f(S[mt][v] * scale, cap, inv_cap) * kLog2e;
-    } else {
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) S[mt][v] *= scale2;
-    }
-    uint32_t mbits = 0;  // bit (mt*16+v) set => masked
-    if (need_mask) {
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int tok = tb + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-          const bool masked = (tok > qpos) || (W_ > 0 && tok <= qpos - W_);
-          if (masked) {
-            S[mt][v] = mask2;
-            mbits |= 1u << (mt * 16 + v);
-          }
-        }
-    }
-    float mx = S[0][0];
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[mt][v]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = fast_exp2(m - m_new);
-    float ps = 0.f;
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float p = fast_exp2(S[mt][v] - m_new);
-        if (need_mask && ((mbits >> (mt * 16 + v)) & 1u)) p = 0.f;
-        S[mt][v] = p;
-        ps += p;
+        for (int ks = 0; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ks * 32), qB[ks], S[mt]);
       }
-    l = l * alpha + ps;
-    m = m_new;
-    // the running max rarely moves once a few tiles are in: rescale only if some lane needs it
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+      softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_);
+      u32x4_t pB[2][2];
+      pack_probs(S, pB);
 #pragma unroll
-      for (int d = 0; d < 4; ++d)
+      for (int d = 0; d < 4; ++d) {
+        const char* vp = lds_v + (d * 32 + c) * kVPitch + h * 16;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) O[d][v] *= alpha;
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk)
+            O[d] = mfma32(lds_ld16(vp + (mt * 32 + kk * 16) * 2), pB[mt][kk], O[d]);
+      }
     }
-    u32x4_t pB[2][2];
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
-        pB[mt][kk] = u32x4_t{pack_bf16x2(S[mt][8 * kk + 0], S[mt][8 * kk + 1]),
-                             pack_bf16x2(S[mt][8 * kk + 2], S[mt][8 * kk + 3]),
-                             pack_bf16x2(S[mt][8 * kk + 4], S[mt][8 * kk + 5]),
-                             pack_bf16x2(S[mt][8 * kk + 6], S[mt][8 * kk + 7])};
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const char* vp = lds_v + (d * 32 + c) * kVPitch + h * 16;
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
-          O[d] = mfma32(lds_ld16(vp + (mt * 32 + kk * 16) * 2), pB[mt][kk], O[d]);
-    }
-    }  // vis
     __syncthreads();
   }
-
-  // ---- epilogue: lane (c, h) holds query row c, dims 32d + 8*(v/4) + 4h + v%4 ----
-  l += __shfl_xor(l, 32);
-  if (!wave_active || row >= q_len) return;
-  const float vs = a.v_scale ? a.v_scale[hk] : 1.0f;
-  const float inv = vs / l;
-  uint16_t* op = a.out + ((int64_t)(qg0 + row) * a.Hq + head) * 128 + 4 * h;
-#pragma unroll
-  for (int d = 0; d < 4; ++d)
-#pragma unroll
-    for (int vq = 0; vq < 4; ++vq) {
-      u32x2_t w = {pack_bf16x2(O[d][4 * vq + 0] * inv, O[d][4 * vq + 1] * inv),
-                   pack_bf16x2(O[d][4 * vq + 2] * inv, O[d][4 * vq + 3] * inv)};
-      *reinterpret_cast<u32x2_t*>(op + d * 32 + vq * 8) = w;
-    }
+  write_rows(a, w, wr, O, l, h);
 }
 
 }  // namespace
@@ -397,20 +618,36 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
   const bool uniform = (a.pt.page_size % kBN) == 0;
   const bool cap = a.sm.soft_cap != 0.f;
+  static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
+  const bool staged = a.fp8 || force_staged;
   const dim3 g((unsigned)grid), blk(256);
-#define RPA_PREFILL_LAUNCH(F, U, C) \
-  hipLaunchKernelGGL((rpa_prefill_flash_kernel<F, U, C>), g, blk, 0, stream, a, tiles, nseq)
-  switch ((a.fp8 ? 4 : 0) | (uniform ? 2 : 0) | (cap ? 1 : 0)) {
-    case 0: RPA_PREFILL_LAUNCH(false, false, false); break;
-    case 1: RPA_PREFILL_LAUNCH(false, false, true); break;
-    case 2: RPA_PREFILL_LAUNCH(false, true, false); break;
-    case 3: RPA_PREFILL_LAUNCH(false, true, true); break;
-    case 4: RPA_PREFILL_LAUNCH(true, false, false); break;
-    case 5: RPA_PREFILL_LAUNCH(true, false, true); break;
-    case 6: RPA_PREFILL_LAUNCH(true, true, false); break;
-    default: RPA_PREFILL_LAUNCH(true, true, true); break;
+#define RPA_STAGED(F, U, C) hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C>), g, blk, 0, stream, a, tiles, nseq)
+#define RPA_ASYNC(U, C) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C>), g, blk, 0, stream, a, tiles, nseq)
+  const int key = (uniform ? 2 : 0) | (cap ? 1 : 0);
+  if (!staged) {
+    switch (key) {
+      case 0: RPA_ASYNC(false, false); break;
+      case 1: RPA_ASYNC(false, true); break;
+      case 2: RPA_ASYNC(true, false); break;
+      default: RPA_ASYNC(true, true); break;
+    }
+  } else if (a.fp8) {
+    switch (key) {
+      case 0: RPA_STAGED(true, false, false); break;
+      case 1: RPA_STAGED(true, false, true); break;
+      case 2: RPA_STAGED(true, true, false); break;
+      default: RPA_STAGED(true, true, true); break;
+    }
+  } else {
+    switch (key) {
+      case 0: RPA_STAGED(false, false, false); break;
+      case 1: RPA_STAGED(false, false, true); break;
+      case 2: RPA_STAGED(false, true, false); break;
+      default: RPA_STAGED(false, true, true); break;
+    }
   }
-#undef RPA_PREFILL_LAUNCH
+#undef RPA_STAGED
+#undef RPA_ASYNC
   return hipGetLastError();
 }
 
