@@ -54,6 +54,17 @@ __device__ __forceinline__ float soft_cap_f(float x, float cap, float inv_cap) {
   return cap * (1.0f - 2.0f / (e + 1.0f));
 }
 
+// Load a 32-bit word through the scalar data cache.  `p` must be wave-uniform and point at
+// memory nobody writes during the kernel (page tables, lengths).  A scalar load is counted by
+// lgkmcnt, not vmcnt, so waiting for it never drains the vector-memory queue.
+__device__ __forceinline__ int32_t scalar_load_i32(const int32_t* p) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(a));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(a >> 32));
+  typedef const __attribute__((address_space(4))) int32_t* const_ptr_t;
+  return *reinterpret_cast<const_ptr_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 // 16-byte global loads / stores.
 __device__ __forceinline__ u32x4_t ld16(const void* p) { return *reinterpret_cast<const u32x4_t*>(p); }
 __device__ __forceinline__ u32x2_t ld8(const void* p) { return *reinterpret_cast<const u32x2_t*>(p); }

@@ -154,8 +154,29 @@ struct Softmax {
 // inside the exponent: p = 2^(s*sc2 - m*sc2) is one fused multiply-add per score (soft-capped
 // scores are already in log2 units, sc2 = 1).  The running max starts at a finite floor far
 // above the mask value, so a row whose tokens are all masked in this tile gets p = 0, not 2^0.
+constexpr f32x16_t kZero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 constexpr float kMaxFloor = -1.0e30f;
 constexpr float kMaskRaw = -3.0e38f;
+
+// The running max is allowed to go stale: it is raised (and the accumulators rescaled) only
+// when some row's new maximum exceeds it by more than 2^kMaxSlack, so probabilities stay
+// below 2^kMaxSlack -- harmless in f32 sums and bf16 operands -- and the 64-register rescale
+// of O happens a handful of times per row instead of once per tile.
+constexpr float kMaxSlack = 8.0f;
+
+template <int ND>
+__device__ __forceinline__ void update_running_max(float mx, float& m, float& l, f32x16_t (&O)[ND], float sc2) {
+  if (__builtin_amdgcn_ballot_w64((mx - m) * sc2 > kMaxSlack) != 0) {
+    const float m_new = fmaxf(m, mx);
+    const float alpha = fast_exp2((m - m_new) * sc2);
+    m = m_new;
+    l *= alpha;
+#pragma unroll
+    for (int d = 0; d < ND; ++d)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) O[d][v] *= alpha;
+  }
+}
 
 template <bool CAP>
 __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4], float& m, float& l,
@@ -177,13 +198,16 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4],
         S[mt][v] = masked ? kMaskRaw : S[mt][v];
       }
   }
-  float mx = fmaxf(S[0][0], S[1][0]);
+  // 32 scores -> 1 with three-operand maxima: 16 instructions instead of 31
+  float mx = __builtin_fmaxf(__builtin_fmaxf(S[0][0], S[0][1]), S[1][0]);
 #pragma unroll
-  for (int v = 1; v < 16; ++v) mx = fmaxf(mx, fmaxf(S[0][v], S[1][v]));
+  for (int v = 1; v < 16; ++v) {
+    if (v < 15) mx = __builtin_fmaxf(__builtin_fmaxf(mx, S[0][v + 1]), S[1][v]);
+    else mx = __builtin_fmaxf(mx, S[1][v]);
+  }
   mx = fmaxf(mx, __shfl_xor(mx, 32));
-  const float m_new = fmaxf(m, mx);
-  const float alpha = fast_exp2((m - m_new) * sm.sc2);
-  const float neg_m = -m_new * sm.sc2;
+  update_running_max<4>(mx, m, l, O, sm.sc2);
+  const float neg_m = -m * sm.sc2;
   float ps = 0.f;
 #pragma unroll
   for (int mt = 0; mt < 2; ++mt)
@@ -193,15 +217,7 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4],
       S[mt][v] = p;
       ps += p;
     }
-  l = l * alpha + ps;
-  m = m_new;
-  // the running max rarely moves once a few tiles are in: rescale only if some lane needs it
-  if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-    for (int d = 0; d < 4; ++d)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) O[d][v] *= alpha;
-  }
+  l += ps;
 }
 
 __device__ __forceinline__ void pack_probs(const f32x16_t (&S)[2], u32x4_t (&pB)[2][2]) {
@@ -250,7 +266,7 @@ __device__ __forceinline__ void async_fetch_pages(AsyncPages<UNIFORM>& pg, const
                                                   int lane) {
   tb = min(tb, s.last_tok & ~(kBN - 1));
   if constexpr (UNIFORM) {
-    pg.id[0] = __builtin_amdgcn_readfirstlane(s.pages[page_slot(s, tb)]);
+    pg.id[0] = scalar_load_i32(s.pages + __builtin_amdgcn_readfirstlane(page_slot(s, tb)));
   } else {
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
@@ -261,14 +277,48 @@ __device__ __forceinline__ void async_fetch_pages(AsyncPages<UNIFORM>& pg, const
 }
 
 // Every wave copies 4 x 64 chunks of K and of V: chunk position p = 64*(4*wave + n) + lane of
-// the tile, i.e. row p / 16, chunk column p % 16.
+// the tile, i.e. row p / 16, chunk column p % 16.  For a full tile inside one page the byte
+// offset of a lane's chunk from the tile's first row never changes: it is computed once
+// (AsyncOffsets) and a copy costs no vector ALU work, only a scalar tile base.
+struct AsyncOffsets {
+  uint32_t k[4], v[4];
+};
+
+__device__ __forceinline__ AsyncOffsets make_async_offsets(const KvAddr& kv, int wave, int lane) {
+  AsyncOffsets o;
+  const int cp = lane & 15;
+#pragma unroll
+  for (int n = 0; n < 4; ++n) {
+    const int t = (wave * 4 + n) * 4 + (lane >> 4);
+    o.k[n] = (uint32_t)(t * kv.tok_stride + ((cp ^ (t & 15)) << 4));
+    o.v[n] = (uint32_t)(t * kv.tok_stride + ((cp ^ ((t & 3) << 2)) << 4));
+  }
+  return o;
+}
+
 template <bool UNIFORM>
 __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const TileSrc& s, const KvAddr& kv,
                                                 const char* kh, const char* vh, int tb, int wave, int lane,
-                                                const AsyncPages<UNIFORM>& pg) {
+                                                const AsyncPages<UNIFORM>& pg, const AsyncOffsets& ofs) {
   typedef const __attribute__((address_space(1))) void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
   tb = min(tb, s.last_tok & ~(kBN - 1));  // past the end: re-copy the last tile
+  if constexpr (UNIFORM) {
+    if (tb + kBN - 1 <= s.last_tok) {
+      const int64_t base = (int64_t)pg.id[0] * kv.page_stride +
+                           (int64_t)(tb - page_slot(s, tb) * s.page_size) * kv.tok_stride;  // scalar
+      const char* kb = kh + base;
+      const char* vb = vh + base;
+#pragma unroll
+      for (int n = 0; n < 4; ++n) {
+        const int blk = wave * 4 + n;
+        __builtin_amdgcn_global_load_lds((gptr_t)(kb + ofs.k[n]), (lptr_t)(lds_k + blk * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(vb + ofs.v[n]), (lptr_t)(lds_v + blk * 1024), 16, 0, 0);
+      }
+      return;
+    }
+  }
+  // last, partial tile (rows clamped to the last valid token) or pages smaller than a tile
   const int cp = lane & 15;
 #pragma unroll
   for (int n = 0; n < 4; ++n) {
@@ -284,8 +334,13 @@ __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const 
 
 template <bool UNIFORM, bool CAP>
 __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const PrefillArgs a, int tiles, int nseq) {
-  __shared__ __attribute__((aligned(1024))) char lds_k_buf[2][kTileB];
-  __shared__ __attribute__((aligned(1024))) char lds_v_buf[2][kTileB];
+  // Four separate arrays (not one indexed array): the compiler can then prove that the
+  // asynchronous copy into one ring slot does not alias the LDS reads of the other slot and
+  // does not drain the vector-memory queue in the middle of a tile.
+  __shared__ __attribute__((aligned(1024))) char lds_k0[kTileB];
+  __shared__ __attribute__((aligned(1024))) char lds_k1[kTileB];
+  __shared__ __attribute__((aligned(1024))) char lds_v0[kTileB];
+  __shared__ __attribute__((aligned(1024))) char lds_v1[kTileB];
 
   const Work w = decompose(a, tiles, nseq);
   if (!w.valid) return;
@@ -343,19 +398,19 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
   const int v_swz = (r16 >> 2) << 6;  // byte offset of the 64-byte window: (64d) ^ v_swz
 
   // ---- pipeline: page ids two tiles ahead, the asynchronous copy one tile ahead ----
+  const AsyncOffsets ofs = make_async_offsets(a.kv, wave, lane);
   AsyncPages<UNIFORM> pg;
   async_fetch_pages<UNIFORM>(pg, src, t_lo, wave, lane);
-  async_copy_tile<UNIFORM>(lds_k_buf[0], lds_v_buf[0], src, a.kv, kh, vh, t_lo, wave, lane, pg);
+  async_copy_tile<UNIFORM>(lds_k0, lds_v0, src, a.kv, kh, vh, t_lo, wave, lane, pg, ofs);
   async_fetch_pages<UNIFORM>(pg, src, t_lo + kBN, wave, lane);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the copies have landed in LDS
   __syncthreads();
-  int buf = 0;
-  for (int tb = t_lo; tb < t_hi; tb += kBN, buf ^= 1) {
-    const char* lds_k = lds_k_buf[buf];
-    const char* lds_v = lds_v_buf[buf];
+
+  // one tile: consume (lds_k, lds_v), fill (nxt_k, nxt_v) with the tile after it
+  auto tile_step = [&](const char* lds_k, const char* lds_v, char* nxt_k, char* nxt_v, int tb) {
     if (tb + kBN < t_hi) {
-      // the other buffer was last read before the barrier that ended the previous tile
-      async_copy_tile<UNIFORM>(lds_k_buf[buf ^ 1], lds_v_buf[buf ^ 1], src, a.kv, kh, vh, tb + kBN, wave, lane, pg);
+      // the other slot was last read before the barrier that ended the previous tile
+      async_copy_tile<UNIFORM>(nxt_k, nxt_v, src, a.kv, kh, vh, tb + kBN, wave, lane, pg, ofs);
       async_fetch_pages<UNIFORM>(pg, src, tb + 2 * kBN, wave, lane);
     }
     // visible to this wave?  causal: some token <= last row's position; window: some token
@@ -363,34 +418,43 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
     const bool vis = wr.active && (tb <= w.prefix + wr.r_hi) && (W_ <= 0 || tb + kBN - 1 > w.prefix + wr.r_lo - W_);
     if (vis) {
       const bool need_mask = (tb + kBN - 1 > w.prefix + wr.r_lo) || (W_ > 0 && tb <= w.prefix + wr.r_hi - W_);
-      f32x16_t S[2];
+      const char* kp0 = lds_k + k_row;
+      const char* kp1 = kp0 + 32 * kRowB;
+      const char* vbase = lds_v + v_row + v_in;
+      {
+        f32x16_t S[2];
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
+        for (int mt = 0; mt < 2; ++mt) {
+          const char* kp = mt ? kp1 : kp0;
+          S[mt] = mfma32(lds_ld16(kp + k_swz), qB[0], kZero16);  // zero accumulator as an inline constant
 #pragma unroll
-        for (int v = 0; v < 16; ++v) S[mt][v] = 0.f;
-        const char* kp = lds_k + mt * 32 * kRowB + k_row;
+          for (int ks = 1; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ((ks * 32) ^ k_swz)), qB[ks], S[mt]);
+        }
+        softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_);
+        u32x4_t pB[2][2];
+        pack_probs(S, pB);
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ((ks * 32) ^ k_swz)), qB[ks], S[mt]);
-      }
-      softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_);
-      u32x4_t pB[2][2];
-      pack_probs(S, pB);
+        for (int d = 0; d < 4; ++d) {
+          const char* vp = vbase + ((d * 64) ^ v_swz);
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        const char* vp = lds_v + v_row + v_in + ((d * 64) ^ v_swz);
+          for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-          for (int kk = 0; kk < 2; ++kk) {
-            const char* vt = vp + (mt * 32 + kk * 16) * kRowB;
-            const u32x2_t lo = lds_tr16(vt);
-            const u32x2_t hi = lds_tr16(vt + 8 * kRowB);
-            O[d] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, pB[mt][kk], O[d]);
-          }
+            for (int kk = 0; kk < 2; ++kk) {
+              const char* vt = vp + (mt * 32 + kk * 16) * kRowB;
+              const u32x2_t lo = lds_tr16(vt);
+              const u32x2_t hi = lds_tr16(vt + 8 * kRowB);
+              O[d] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, pB[mt][kk], O[d]);
+            }
+        }
       }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // the next tile has landed
     __syncthreads();
+  };
+  for (int tb = t_lo; tb < t_hi; tb += 2 * kBN) {
+    tile_step(lds_k0, lds_v0, lds_k1, lds_v1, tb);
+    if (tb + kBN >= t_hi) break;
+    tile_step(lds_k1, lds_v1, lds_k0, lds_v0, tb + kBN);
   }
   write_rows(a, w, wr, O, l, h);
 }
@@ -413,7 +477,7 @@ template <bool UNIFORM>
 __device__ __forceinline__ void fetch_page_ids(PageIds<UNIFORM>& pg, const TileSrc& s, int tb, int tid) {
   tb = min(tb, s.last_tok & ~(kBN - 1));
   if constexpr (UNIFORM) {
-    pg.id[0] = __builtin_amdgcn_readfirstlane(s.pages[page_slot(s, tb)]);
+    pg.id[0] = scalar_load_i32(s.pages + __builtin_amdgcn_readfirstlane(page_slot(s, tb)));
   } else {
     if (tid < 128) {
       pg.id[0] = s.pages[page_slot(s, min(tb + (tid >> 1), s.last_tok))];
@@ -583,11 +647,10 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
       f32x16_t S[2];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) S[mt][v] = 0.f;
         const char* kp = lds_k + (mt * 32 + c) * kKPitch + h * 16;
+        S[mt] = mfma32(lds_ld16(kp), qB[0], kZero16);
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ks * 32), qB[ks], S[mt]);
+        for (int ks = 1; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ks * 32), qB[ks], S[mt]);
       }
       softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_);
       u32x4_t pB[2][2];
