@@ -422,30 +422,30 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
       const char* kp1 = kp0 + 32 * kRowB;
       const char* vbase = lds_v + v_row + v_in;
       {
+        // the two 32-token halves form two independent accumulator chains, issued alternately
         f32x16_t S[2];
+        S[0] = mfma32(lds_ld16(kp0 + k_swz), qB[0], kZero16);  // zero accumulator as an inline constant
+        S[1] = mfma32(lds_ld16(kp1 + k_swz), qB[0], kZero16);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-          const char* kp = mt ? kp1 : kp0;
-          S[mt] = mfma32(lds_ld16(kp + k_swz), qB[0], kZero16);  // zero accumulator as an inline constant
-#pragma unroll
-          for (int ks = 1; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ((ks * 32) ^ k_swz)), qB[ks], S[mt]);
+        for (int ks = 1; ks < 8; ++ks) {
+          S[0] = mfma32(lds_ld16(kp0 + ((ks * 32) ^ k_swz)), qB[ks], S[0]);
+          S[1] = mfma32(lds_ld16(kp1 + ((ks * 32) ^ k_swz)), qB[ks], S[1]);
         }
         softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_);
         u32x4_t pB[2][2];
         pack_probs(S, pB);
+        // four independent accumulator chains (dim tiles), issued round-robin
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          const char* vp = vbase + ((d * 64) ^ v_swz);
+        for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-          for (int mt = 0; mt < 2; ++mt)
+          for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-              const char* vt = vp + (mt * 32 + kk * 16) * kRowB;
+            for (int d = 0; d < 4; ++d) {
+              const char* vt = vbase + ((d * 64) ^ v_swz) + (mt * 32 + kk * 16) * kRowB;
               const u32x2_t lo = lds_tr16(vt);
               const u32x2_t hi = lds_tr16(vt + 8 * kRowB);
               O[d] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, pB[mt][kk], O[d]);
             }
-        }
       }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // the next tile has landed
