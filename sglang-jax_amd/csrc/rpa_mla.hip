@@ -2,16 +2,26 @@
 //
 // Every token has ONE shared latent row [kv_c (512) | k_pe (64)]; all query
 // heads attend to it (scores over 576 dims, values = the first 512 dims).  A
-// workgroup of 8 waves owns one (sequence, kv split) and ALL heads in groups of
-// 128 (wave w owns 16 heads), so the latent rows are fetched from HBM once:
-//   global -> registers -> LDS      K tile [32 tok][576]        (pitch 1168 B)
-//   LDS -> registers -> LDS         V^T tile [512 dims][32 tok] (pitch 80 B),
-//                                   register transpose with v_perm_b32
-//   S^T[tok, head] = K . Q^T        36 MFMA 16x16x32 per wave and tile
+// workgroup of 8 waves owns one (sequence, kv split) and 128 heads (wave w owns
+// heads 16w..16w+15), so each latent row is fetched from HBM exactly once:
+//   global -> LDS   global_load_lds_dwordx4 copies 32-token tiles (rows of 72
+//                   16-byte chunks, row-major, XOR-swizzled) into a 3-slot ring,
+//                   two tiles ahead of the MFMAs; no staging registers
+//   S^T[tok, head] = K . Q^T       36 MFMA 16x16x32 per wave and tile, A = rows
+//                                  read with ds_read_b128, B = Q^T in registers
 //   online softmax, P rounded to bf16 (as the reference rounds it)
-//   O^T[dim, head] += V^T . P^T     32 MFMA 16x16x32 per wave and tile
+//   O^T[dim, head] += V^T . P^T    32 MFMA 16x16x32; A = V^T read from the SAME
+//                                  row-major rows with ds_read_b64_tr_b16
 // Partials (unnormalised O, running max, sum) go to the workspace and are merged
 // by rpa_mla_combine_kernel; with a single split the output is written directly.
+//
+// LDS layout of a tile: row r (token) at r * 1152 bytes; 16-byte chunk j of the row
+// at chunk position j ^ key(r), key(r) = ((r >> 1 & 3) << 1) | (r >> 3 & 1)  (j and
+// j ^ key stay inside the same aligned group of 8 chunks; 72 = 9 groups).  The 16 MFMA
+// rows of a score tile map to tokens row(m) = 16b + 8(m >> 3) + 2(m & 3) + (m >> 2 & 1):
+// with that pairing both the b128 reads of K (16 lanes, one chunk column each, two bank
+// halves) and the transposing reads of V (4 tokens x 32 bytes per 16-lane block) are
+// free of bank conflicts without padding.
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
@@ -20,17 +30,26 @@ namespace rpa {
 
 namespace {
 
-constexpr int kTok = 32;         // tokens per tile
-constexpr int kRowB = 1152;      // compact latent row bytes (576 bf16)
-constexpr int kKPitch = 1168;    // LDS pitch of a K row
-constexpr int kVPitch = 80;      // LDS pitch of a V^T row (32 tok * 2 B + 16)
-constexpr int kPieces = kTok * 72;  // 16-byte pieces per tile
+constexpr int kTok = 32;                 // tokens per tile
+constexpr int kRowB = 1152;              // compact latent row in LDS (576 bf16)
+constexpr int kChunks = 72;              // 16-byte chunks per row
+constexpr int kSlotB = 40 * 1024;        // one ring slot: 40 copy blocks of 64 chunks (36 used + 4 dummy)
+constexpr int kCopiesPerWave = 5;        // every wave issues 5 copy instructions per tile
 
 __device__ __forceinline__ u32x4_t lds_ld16(const char* p) { return *reinterpret_cast<const u32x4_t*>(p); }
-__device__ __forceinline__ void lds_st16(char* p, u32x4_t v) { *reinterpret_cast<u32x4_t*>(p) = v; }
 
-__device__ __forceinline__ int tok_slot(int g, int i) {
-  return (i < 4) ? (g * 4 + i) : (16 + g * 4 + (i - 4));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2_t lds_tr16(const char* p) {
+  typedef __attribute__((address_space(3))) s16x4_t* lds_ptr_t;
+  const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(p));
+  return __builtin_bit_cast(u32x2_t, v);
+}
+
+__device__ __forceinline__ int row_key(int r) { return (((r >> 1) & 3) << 1) | ((r >> 3) & 1); }
+
+// token (inside a tile) behind slot i = 4b + r of lane group g in the S^T result registers
+__device__ __forceinline__ int tok_of(int g, int i) {
+  return 16 * (i >> 2) + 8 * (g >> 1) + 2 * (i & 3) + (g & 1);
 }
 
 struct Src {
@@ -41,22 +60,70 @@ struct Src {
   int32_t rope_byte;    // byte offset of k_pe inside a cached row
 };
 
-__device__ __forceinline__ u32x4_t load_piece(const Src& s, const char* cache, int tb, int idx) {
-  const int tl = idx / 72, piece = idx - tl * 72;
-  const int tok = min(tb + tl, s.last_tok);
-  const int slot = s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
-  const int page = s.pages[slot];
-  const int inner = piece < 64 ? piece * 16 : s.rope_byte + (piece - 64) * 16;
-  return ld16(cache + (int64_t)page * s.page_stride + (int64_t)(tok - slot * s.page_size) * s.row_bytes + inner);
+__device__ __forceinline__ int page_slot(const Src& s, int tok) {
+  return s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
+}
+
+// A lane's 5 chunks of a tile: position p = 64*(5*wave + n) + lane; row p / 72, chunk
+// column p % 72.  Positions >= 32*72 are padding copies of the tile's first chunk.
+__device__ __forceinline__ void chunk_of(const Src& s, int wave, int lane, int n, int& row, int& inner) {
+  int p = (wave * kCopiesPerWave + n) * 64 + lane;
+  if (p >= kTok * kChunks) p = 0;
+  row = p / kChunks;
+  const int j = (p - row * kChunks) ^ row_key(row);
+  inner = j < 64 ? j * 16 : s.rope_byte + (j - 64) * 16;
+}
+
+template <bool UNIFORM>
+__device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* cache, int tb, int wave, int lane,
+                                          int page) {
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  tb = min(tb, s.last_tok & ~(kTok - 1));  // past the end: re-copy the last tile
+  if constexpr (UNIFORM) {
+    if (tb + kTok - 1 <= s.last_tok) {
+      const char* base = cache + (int64_t)page * s.page_stride +
+                         (int64_t)(tb - page_slot(s, tb) * s.page_size) * s.row_bytes;  // scalar
+      // chunk offsets are recomputed per tile (a dozen integer ops) rather than kept in
+      // registers: the accumulators and Q^T leave no room, and a spill reload would be a
+      // vector-memory load that drains the copy queue
+      int ln = lane;
+      asm volatile("" : "+v"(ln));  // opaque: keeps the offset arithmetic inside the loop
+#pragma unroll
+      for (int n = 0; n < kCopiesPerWave; ++n) {
+        int row, inner;
+        chunk_of(s, wave, ln, n, row, inner);
+        __builtin_amdgcn_global_load_lds((gptr_t)(base + (uint32_t)(row * s.row_bytes + inner)),
+                                         (lptr_t)(slot + (wave * kCopiesPerWave + n) * 1024), 16, 0, 0);
+      }
+      return;
+    }
+  }
+  // last, partial tile (rows clamped to the last valid token) or pages smaller than a tile
+#pragma unroll
+  for (int n = 0; n < kCopiesPerWave; ++n) {
+    int row, inner;
+    chunk_of(s, wave, lane, n, row, inner);
+    const int tok = min(tb + row, s.last_tok);
+    const int ps = page_slot(s, tok);
+    const int pg = UNIFORM ? page : s.pages[ps];
+    const char* src = cache + (int64_t)pg * s.page_stride + (int64_t)(tok - ps * s.page_size) * s.row_bytes + inner;
+    __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(slot + (wave * kCopiesPerWave + n) * 1024), 16, 0, 0);
+  }
 }
 
 // grid = (max_splits, rows, head groups of 128); block = 512 threads.
+template <bool UNIFORM, bool CAP>
 __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeArgs a) {
-  __shared__ __attribute__((aligned(16))) char lds_k[kTok * kKPitch];
-  __shared__ __attribute__((aligned(16))) char lds_v[512 * kVPitch];
+  // three separate arrays: lets the compiler see that a copy into one slot does not alias the
+  // reads of another, so it does not drain the vector-memory queue before LDS reads
+  __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, g = lane >> 4;
   const int seq = blockIdx.y, split = blockIdx.x;
   const int head0 = blockIdx.z * 128 + wave * 16;
@@ -78,6 +145,14 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   src.row_bytes = a.row_stride * 2;
   src.page_stride = (int64_t)src.row_bytes * a.pt.page_size;
   src.rope_byte = a.rope_offset * 2;
+  auto page_of = [&](int tb) -> int {
+    if constexpr (UNIFORM) {
+      tb = min(tb, src.last_tok & ~(kTok - 1));
+      return scalar_load_i32(src.pages + __builtin_amdgcn_readfirstlane(page_slot(src, tb)));
+    } else {
+      return 0;
+    }
+  };
 
   // ---- Q^T operands of this wave: column c = head head0 + c, k-step ks covers dims 32ks + 8g .. ----
   const int tq = a.pt.cu_q_lens[seq];
@@ -98,102 +173,104 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   const float inv_cap = (cap != 0.f) ? 1.0f / cap : 0.f;
   const float mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
 
+  // ---- LDS operand addresses (bytes inside a slot) ----
+  // K operand of score tile b (tokens 16b..), k-step ks: row 16b + 8(c>>3) + 2(c&3) + (c>>2 & 1)
+  const int k_row = (8 * (c >> 3) + 2 * (c & 3) + ((c >> 2) & 1));
+  const int k_off = k_row * kRowB;
+  const int k_swz = (g ^ row_key(k_row)) << 4;  // chunk (4ks + g) ^ key = (4ks) ^ (g ^ key)
+  // V^T operand of dim chunk j: source lane r = c points at token 8(g>>1) + 2(r>>2) + (g&1) (+16),
+  // dims 16j + 4(r&3); chunk (2j + (r&3 >> 1)) ^ key, key = ((r>>2) << 1) | (g >> 1)
+  const int v_row = 8 * (g >> 1) + 2 * (c >> 2) + (g & 1);
+  const int v_off = v_row * kRowB + ((c & 1) << 3);
+  const int v_swz = ((((c & 3) >> 1)) ^ row_key(v_row)) << 4;
+
   f32x4_t acc[32];
 #pragma unroll
   for (int j = 0; j < 32; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  u32x4_t stg[5];
-#pragma unroll
-  for (int r = 0; r < 5; ++r) {
-    const int idx = tid + r * 512;
-    if (idx < kPieces) stg[r] = load_piece(src, a.cache, t_begin, idx);
-  }
+  // ---- pipeline: copies run two tiles ahead of the MFMAs (3-slot ring) ----
+  int pg_next = page_of(t_begin + 2 * kTok);
+  copy_tile<UNIFORM>(slot0, src, a.cache, t_begin, wave, lane, page_of(t_begin));
+  copy_tile<UNIFORM>(slot1, src, a.cache, t_begin + kTok, wave, lane, page_of(t_begin + kTok));
+  // wait for the Q loads and the first tile (all but the 5 newest copies), then meet
+  __builtin_amdgcn_s_waitcnt(0x0F70 | kCopiesPerWave);
+  __syncthreads();
 
-  for (int tb = t_begin; tb < t_end; tb += kTok) {
-    __syncthreads();  // previous tile fully consumed
+  auto tile_step = [&](const char* cur, char* fill, int tb) {
+    // `fill` held tile tb - 32, which every wave finished before the last barrier
+    copy_tile<UNIFORM>(fill, src, a.cache, tb + 2 * kTok, wave, lane, pg_next);
+    pg_next = page_of(tb + 3 * kTok);
+    if (wave_on) {
+      f32x4_t s[2];
 #pragma unroll
-    for (int r = 0; r < 5; ++r) {
-      const int idx = tid + r * 512;
-      if (idx < kPieces) {
-        const int tl = idx / 72, piece = idx - tl * 72;
-        lds_st16(lds_k + tl * kKPitch + piece * 16, stg[r]);
-      }
-    }
-    __syncthreads();
-    if (tb + kTok < t_end) {
+      for (int b = 0; b < 2; ++b) {
+        s[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        const char* kp = cur + k_off + b * 16 * kRowB;
 #pragma unroll
-      for (int r = 0; r < 5; ++r) {
-        const int idx = tid + r * 512;
-        if (idx < kPieces) stg[r] = load_piece(src, a.cache, tb + kTok, idx);
-      }
-    }
-    // ---- transpose the value part: thread (tg, dc) turns 8 tokens x 8 dims into 8 dims x 8 tokens ----
-    if (tid < 256) {
-      const int tg = tid & 3, dc = tid >> 2;
-      // two passes of 4 tokens keep only 16 staging registers live
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        u32x4_t v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = lds_ld16(lds_k + tok_slot(tg, half * 4 + i) * kKPitch + dc * 16);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-          const int jj = j >> 1;
-          const u32x2_t w = {__builtin_amdgcn_perm(v[1][jj], v[0][jj], sel), __builtin_amdgcn_perm(v[3][jj], v[2][jj], sel)};
-          *reinterpret_cast<u32x2_t*>(lds_v + (dc * 8 + j) * kVPitch + tg * 16 + half * 8) = w;
+        for (int ks = 0; ks < 18; ++ks) {
+          s[b] = mfma16(lds_ld16(kp + ((ks * 64) ^ k_swz)), qB[ks], s[b]);
+          // fence the scheduler every few MFMAs: it would otherwise hoist all LDS reads of the
+          // tile, run out of registers and spill (a spill reload drains the copy queue)
+          if (ks % 3 == 2) __builtin_amdgcn_sched_barrier(0);
         }
       }
-    }
-    __syncthreads();
-    if (!wave_on) continue;
-
-    f32x4_t s[2];
-#pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      s[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      const char* kp = lds_k + (b * 16 + c) * kKPitch + g * 16;
-#pragma unroll
-      for (int ks = 0; ks < 18; ++ks) s[b] = mfma16(lds_ld16(kp + ks * 64), qB[ks], s[b]);
-    }
-    float x[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float v = s[i >> 2][i & 3];
-      if (cap != 0.f) v = soft_cap_f(v * scale, cap, inv_cap) * kLog2e;
-      else v = v * scale2;
-      x[i] = v;
-    }
-    if ((tb + kTok > kv_len) || (tb < t_lo)) {
+      float x[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const int tok = tb + tok_slot(g, i);
-        if (tok >= kv_len || tok < t_lo) x[i] = mask2;
+        float v = s[i >> 2][i & 3];
+        if constexpr (CAP) v = soft_cap_f(v * scale, cap, inv_cap) * kLog2e;
+        else v = v * scale2;
+        x[i] = v;
+      }
+      if ((tb + kTok > kv_len) || (tb < t_lo)) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int tok = tb + tok_of(g, i);
+          if (tok >= kv_len || tok < t_lo) x[i] = mask2;
+        }
+      }
+      float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m, mx);
+      const float alpha = fast_exp2(m - m_new);
+      float p[8], ps = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        p[i] = fast_exp2(x[i] - m_new);
+        ps += p[i];
+      }
+      l = l * alpha + ps;
+      m = m_new;
+      const u32x4_t pB = u32x4_t{pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
+                                 pack_bf16x2(p[6], p[7])};
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int j = 0; j < 32; ++j) acc[j] = acc[j] * alpha;
+      }
+      const char* vp = cur + v_off;
+#pragma unroll
+      for (int j = 0; j < 32; ++j) {
+        const char* vt = vp + ((j * 32) ^ v_swz);
+        const u32x2_t lo = lds_tr16(vt);
+        const u32x2_t hi = lds_tr16(vt + 16 * kRowB);
+        acc[j] = mfma16(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, pB, acc[j]);
+        if (j % 2 == 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
-    float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = fast_exp2(m - m_new);
-    float p[8], ps = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      p[i] = fast_exp2(x[i] - m_new);
-      ps += p[i];
-    }
-    l = l * alpha + ps;
-    m = m_new;
-    const u32x4_t pB = u32x4_t{pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
-                               pack_bf16x2(p[6], p[7])};
-    const char* vp = lds_v + c * kVPitch + g * 16;
-#pragma unroll
-    for (int j = 0; j < 32; ++j) {
-      acc[j] = acc[j] * alpha;
-      acc[j] = mfma16(lds_ld16(vp + j * 16 * kVPitch), pB, acc[j]);
-    }
+    // tile tb + 32 has landed once at most the 5 copies of tile tb + 64 are outstanding
+    __builtin_amdgcn_s_waitcnt(0x0F70 | kCopiesPerWave);
+    __syncthreads();
+  };
+  for (int tb = t_begin; tb < t_end; tb += 3 * kTok) {
+    tile_step(slot0, slot2, tb);
+    if (tb + kTok >= t_end) break;
+    tile_step(slot1, slot0, tb + kTok);
+    if (tb + 2 * kTok >= t_end) break;
+    tile_step(slot2, slot1, tb + 2 * kTok);
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the copies issued past the end
 
   // ---- epilogue: lane (c, g) holds head head0+c, dims 16j + 4g + r in acc[j][r] ----
   l += __shfl_xor(l, 16);
@@ -251,7 +328,16 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_kernel(const MlaDecodeArg
 hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   if (a.num_rows <= 0) return hipSuccess;
   const int head_groups = (a.Hq + 127) / 128;
-  hipLaunchKernelGGL(rpa_mla_decode_kernel, dim3(a.max_splits, a.num_rows, head_groups), dim3(512), 0, stream, a);
+  const dim3 grid(a.max_splits, a.num_rows, head_groups), block(512);
+  const bool uniform = (a.pt.page_size % kTok) == 0;
+  const bool cap = a.sm.soft_cap != 0.f;
+  if (uniform) {
+    if (cap) hipLaunchKernelGGL((rpa_mla_decode_kernel<true, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((rpa_mla_decode_kernel<true, false>), grid, block, 0, stream, a);
+  } else {
+    if (cap) hipLaunchKernelGGL((rpa_mla_decode_kernel<false, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((rpa_mla_decode_kernel<false, false>), grid, block, 0, stream, a);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (a.max_splits > 1) {
