@@ -107,7 +107,7 @@ def run_mla_config(pkg, wl, b, steps, warmup):
     import torch
 
     n = int(b.distribution[2])
-    kw = dict(sm_scale=b.sm_scale, max_kv_len=int(max(b.meta["kv_lens"])))
+    kw = dict(sm_scale=b.sm_scale, max_kv_len=int(max(b.meta["kv_lens"])), sum_kv_len=int(sum(b.meta["kv_lens"])))
     dist = b.distribution.cpu().numpy()
 
     def one():

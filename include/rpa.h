@@ -140,6 +140,7 @@ typedef struct RpaMlaParams {
   float sm_scale;
   float soft_cap;             /* 0 => off */
   float mask_value;           /* 0 => default */
+  int64_t sum_kv_len;         /* sum of kv_lens (host-side, balances the split plan); 0 => unknown */
 } RpaMlaParams;
 
 /* Library version (RPA_VERSION of the build). */

@@ -114,6 +114,7 @@ class RpaMlaParams(ctypes.Structure):
         ("sm_scale", ctypes.c_float),
         ("soft_cap", ctypes.c_float),
         ("mask_value", ctypes.c_float),
+        ("sum_kv_len", ctypes.c_int64),
     ]
 
 

@@ -28,6 +28,7 @@ FLAGS = [
     # never let the compiler form packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",  # async_copy16 names m0, which the compiler reports as reserved
 ]
 
 

@@ -351,7 +351,13 @@ int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void*
 static SplitPlan mla_plan(const RpaMlaParams* p) {
   const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                      p->cu_kv_lens != nullptr);
-  return plan_splits(bound, p->sliding_window, p->num_seqs, 0, p->num_splits,
+  // one 8-wave workgroup per (row, split, 128 heads) and per CU; every split costs a 256 KiB
+  // partial write per 128 heads, so splits are kept as few as fill the CUs once
+  const int64_t groups = (p->num_q_heads + 127) / 128;
+  const int64_t units = (int64_t)p->num_seqs * groups;
+  int64_t work = p->sum_kv_len > 0 ? p->sum_kv_len * groups : 0;
+  if (p->sliding_window > 0) work = 0;
+  return plan_splits(bound, p->sliding_window, units, work, p->num_splits,
                      env_int("RPA_MLA_MIN_CHUNK", 256), env_int("RPA_MLA_WG_CAPACITY", wave_capacity() / 8));
 }
 

@@ -65,6 +65,17 @@ __device__ __forceinline__ int32_t scalar_load_i32(const int32_t* p) {
   return *reinterpret_cast<const_ptr_t>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
+// Asynchronous 16-byte copy global -> LDS (global_load_lds_dwordx4): lane l's 16 bytes land at
+// lds_base + 16*l; the data never touches a VGPR and completion is counted by vmcnt.  Issued as
+// inline assembly so that the compiler does not model it as an LDS store: it would otherwise
+// wait for ALL outstanding copies (vmcnt(0)) in front of every LDS read it cannot disambiguate,
+// which destroys a multi-tile prefetch.  The caller waits with s_waitcnt vmcnt(n) itself.
+__device__ __forceinline__ void async_copy16(const void* gsrc, const void* lds_base_uniform) {
+  typedef const __attribute__((address_space(3))) char* lds_ptr_t;
+  const uint32_t m0v = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds_base_uniform));
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(gsrc) : "memory", "m0");
+}
+
 // 16-byte global loads / stores.
 __device__ __forceinline__ u32x4_t ld16(const void* p) { return *reinterpret_cast<const u32x4_t*>(p); }
 __device__ __forceinline__ u32x2_t ld8(const void* p) { return *reinterpret_cast<const u32x2_t*>(p); }

@@ -15,13 +15,12 @@
 // Partials (unnormalised O, running max, sum) go to the workspace and are merged
 // by rpa_mla_combine_kernel; with a single split the output is written directly.
 //
-// LDS layout of a tile: row r (token) at r * 1152 bytes; 16-byte chunk j of the row
-// at chunk position j ^ key(r), key(r) = ((r >> 1 & 3) << 1) | (r >> 3 & 1)  (j and
-// j ^ key stay inside the same aligned group of 8 chunks; 72 = 9 groups).  The 16 MFMA
-// rows of a score tile map to tokens row(m) = 16b + 8(m >> 3) + 2(m & 3) + (m >> 2 & 1):
-// with that pairing both the b128 reads of K (16 lanes, one chunk column each, two bank
-// halves) and the transposing reads of V (4 tokens x 32 bytes per 16-lane block) are
-// free of bank conflicts without padding.
+// LDS layout of a tile: row r (token) at r * 1168 bytes = 73 chunks of 16 bytes, the last one
+// padding.  1168 bytes = 292 dwords = 36 (mod 64 banks): the 16 rows of a b128 operand read
+// start at 16 distinct multiples of 4 banks, and the 8 even (or 8 odd) rows of a transposing
+// read at 8 distinct 8-bank windows -- no bank conflicts and no address swizzle, so every LDS
+// address is a per-lane base plus a compile-time offset.  MFMA row m of a score tile is token
+// 16b + 2(m & 7) + (m >> 3), which puts even tokens in lane groups 0-1 and odd ones in 2-3.
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
@@ -31,9 +30,9 @@ namespace rpa {
 namespace {
 
 constexpr int kTok = 32;                 // tokens per tile
-constexpr int kRowB = 1152;              // compact latent row in LDS (576 bf16)
-constexpr int kChunks = 72;              // 16-byte chunks per row
-constexpr int kSlotB = 40 * 1024;        // one ring slot: 40 copy blocks of 64 chunks (36 used + 4 dummy)
+constexpr int kRowB = 1168;              // latent row in LDS: 576 bf16 + 16 bytes of padding
+constexpr int kChunks = 73;              // 16-byte chunks per row (72 data + 1 pad)
+constexpr int kSlotB = 40 * 1024;        // one ring slot: 40 copy blocks of 64 chunks (36.5 used)
 constexpr int kCopiesPerWave = 5;        // every wave issues 5 copy instructions per tile
 
 __device__ __forceinline__ u32x4_t lds_ld16(const char* p) { return *reinterpret_cast<const u32x4_t*>(p); }
@@ -45,11 +44,9 @@ __device__ __forceinline__ u32x2_t lds_tr16(const char* p) {
   return __builtin_bit_cast(u32x2_t, v);
 }
 
-__device__ __forceinline__ int row_key(int r) { return (((r >> 1) & 3) << 1) | ((r >> 3) & 1); }
-
 // token (inside a tile) behind slot i = 4b + r of lane group g in the S^T result registers
 __device__ __forceinline__ int tok_of(int g, int i) {
-  return 16 * (i >> 2) + 8 * (g >> 1) + 2 * (i & 3) + (g & 1);
+  return 16 * (i >> 2) + 8 * (g & 1) + 2 * (i & 3) + (g >> 1);
 }
 
 struct Src {
@@ -64,21 +61,20 @@ __device__ __forceinline__ int page_slot(const Src& s, int tok) {
   return s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
 }
 
-// A lane's 5 chunks of a tile: position p = 64*(5*wave + n) + lane; row p / 72, chunk
-// column p % 72.  Positions >= 32*72 are padding copies of the tile's first chunk.
+// A lane's 5 chunks of a tile: position p = 64*(5*wave + n) + lane; row p / 73, chunk
+// column p % 73.  The pad column and positions >= 32*73 copy the tile's first chunk.
 __device__ __forceinline__ void chunk_of(const Src& s, int wave, int lane, int n, int& row, int& inner) {
   int p = (wave * kCopiesPerWave + n) * 64 + lane;
   if (p >= kTok * kChunks) p = 0;
   row = p / kChunks;
-  const int j = (p - row * kChunks) ^ row_key(row);
+  int j = p - row * kChunks;
+  if (j == kChunks - 1) { row = 0; j = 0; }
   inner = j < 64 ? j * 16 : s.rope_byte + (j - 64) * 16;
 }
 
 template <bool UNIFORM>
 __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* cache, int tb, int wave, int lane,
                                           int page) {
-  typedef const __attribute__((address_space(1))) void* gptr_t;
-  typedef __attribute__((address_space(3))) void* lptr_t;
   tb = min(tb, s.last_tok & ~(kTok - 1));  // past the end: re-copy the last tile
   if constexpr (UNIFORM) {
     if (tb + kTok - 1 <= s.last_tok) {
@@ -93,8 +89,7 @@ __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* 
       for (int n = 0; n < kCopiesPerWave; ++n) {
         int row, inner;
         chunk_of(s, wave, ln, n, row, inner);
-        __builtin_amdgcn_global_load_lds((gptr_t)(base + (uint32_t)(row * s.row_bytes + inner)),
-                                         (lptr_t)(slot + (wave * kCopiesPerWave + n) * 1024), 16, 0, 0);
+        async_copy16(base + (uint32_t)(row * s.row_bytes + inner), slot + (wave * kCopiesPerWave + n) * 1024);
       }
       return;
     }
@@ -108,7 +103,7 @@ __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* 
     const int ps = page_slot(s, tok);
     const int pg = UNIFORM ? page : s.pages[ps];
     const char* src = cache + (int64_t)pg * s.page_stride + (int64_t)(tok - ps * s.page_size) * s.row_bytes + inner;
-    __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(slot + (wave * kCopiesPerWave + n) * 1024), 16, 0, 0);
+    async_copy16(src, slot + (wave * kCopiesPerWave + n) * 1024);
   }
 }
 
@@ -174,15 +169,11 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   const float mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
 
   // ---- LDS operand addresses (bytes inside a slot) ----
-  // K operand of score tile b (tokens 16b..), k-step ks: row 16b + 8(c>>3) + 2(c&3) + (c>>2 & 1)
-  const int k_row = (8 * (c >> 3) + 2 * (c & 3) + ((c >> 2) & 1));
-  const int k_off = k_row * kRowB;
-  const int k_swz = (g ^ row_key(k_row)) << 4;  // chunk (4ks + g) ^ key = (4ks) ^ (g ^ key)
-  // V^T operand of dim chunk j: source lane r = c points at token 8(g>>1) + 2(r>>2) + (g&1) (+16),
-  // dims 16j + 4(r&3); chunk (2j + (r&3 >> 1)) ^ key, key = ((r>>2) << 1) | (g >> 1)
-  const int v_row = 8 * (g >> 1) + 2 * (c >> 2) + (g & 1);
-  const int v_off = v_row * kRowB + ((c & 1) << 3);
-  const int v_swz = ((((c & 3) >> 1)) ^ row_key(v_row)) << 4;
+  // K operand of score tile b, k-step ks: row 16b + 2(c & 7) + (c >> 3), bytes 64ks + 16g
+  const int k_off = (2 * (c & 7) + (c >> 3)) * kRowB + g * 16;
+  // V^T operand of dim chunk j: source lane r = c points at token 8(g & 1) + 2(r >> 2) + (g >> 1)
+  // (+16 for the second half of the k-step), dims 16j + 4(r & 3)
+  const int v_off = (8 * (g & 1) + 2 * (c >> 2) + (g >> 1)) * kRowB + (c & 3) * 8;
 
   f32x4_t acc[32];
 #pragma unroll
@@ -193,7 +184,12 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   int pg_next = page_of(t_begin + 2 * kTok);
   copy_tile<UNIFORM>(slot0, src, a.cache, t_begin, wave, lane, page_of(t_begin));
   copy_tile<UNIFORM>(slot1, src, a.cache, t_begin + kTok, wave, lane, page_of(t_begin + kTok));
-  // wait for the Q loads and the first tile (all but the 5 newest copies), then meet
+  // Touch every Q^T register here: the compiler then waits for the Q loads now, instead of
+  // re-checking them with s_waitcnt vmcnt(0..4) inside the loop, where such a wait would also
+  // drain the copy queue.
+#pragma unroll
+  for (int ks = 0; ks < 18; ++ks) asm volatile("" ::"v"(qB[ks]));
+  // wait for the first tile (all but the 5 newest copies), then meet
   __builtin_amdgcn_s_waitcnt(0x0F70 | kCopiesPerWave);
   __syncthreads();
 
@@ -202,18 +198,18 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
     copy_tile<UNIFORM>(fill, src, a.cache, tb + 2 * kTok, wave, lane, pg_next);
     pg_next = page_of(tb + 3 * kTok);
     if (wave_on) {
+      // two independent accumulator chains (token halves), issued alternately
       f32x4_t s[2];
+      s[0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      s[1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const char* kp = cur + k_off;
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        s[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        const char* kp = cur + k_off + b * 16 * kRowB;
-#pragma unroll
-        for (int ks = 0; ks < 18; ++ks) {
-          s[b] = mfma16(lds_ld16(kp + ((ks * 64) ^ k_swz)), qB[ks], s[b]);
-          // fence the scheduler every few MFMAs: it would otherwise hoist all LDS reads of the
-          // tile, run out of registers and spill (a spill reload drains the copy queue)
-          if (ks % 3 == 2) __builtin_amdgcn_sched_barrier(0);
-        }
+      for (int ks = 0; ks < 18; ++ks) {
+        s[0] = mfma16(lds_ld16(kp + ks * 64), qB[ks], s[0]);
+        s[1] = mfma16(lds_ld16(kp + 16 * kRowB + ks * 64), qB[ks], s[1]);
+        // fence the scheduler every few MFMAs: it would otherwise hoist all LDS reads of the
+        // tile, run out of registers and spill (a spill reload drains the copy queue)
+        if (ks % 3 == 2) __builtin_amdgcn_sched_barrier(0);
       }
       float x[8];
 #pragma unroll
@@ -252,16 +248,22 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
       const char* vp = cur + v_off;
 #pragma unroll
       for (int j = 0; j < 32; ++j) {
-        const char* vt = vp + ((j * 32) ^ v_swz);
+        const char* vt = vp + j * 32;
         const u32x2_t lo = lds_tr16(vt);
         const u32x2_t hi = lds_tr16(vt + 16 * kRowB);
         acc[j] = mfma16(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, pB, acc[j]);
         if (j % 2 == 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // tile tb + 32 has landed once at most the 5 copies of tile tb + 64 are outstanding
+    // Tile tb + 32 has landed once at most the 5 copies of tile tb + 64 are outstanding.  A bare
+    // s_barrier is used instead of __syncthreads(): the fence in the latter makes the compiler
+    // wait for ALL outstanding copies, which would shorten the prefetch distance to one tile.
+    // Every LDS read of this tile has returned (its MFMA consumed it) before the barrier, and
+    // each wave has waited for its own share of the next tile, so no fence is needed.
     __builtin_amdgcn_s_waitcnt(0x0F70 | kCopiesPerWave);
-    __syncthreads();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
   };
   for (int tb = t_begin; tb < t_end; tb += 3 * kTok) {
     tile_step(slot0, slot2, tb);

@@ -16,7 +16,7 @@ import torch
 
 from . import _lib
 from ._lib import RpaMlaParams
-from .ragged_paged_attention import DEFAULT_MASK_VALUE, _host_max, _i32, _require_gpu, _workspace
+from .ragged_paged_attention import DEFAULT_MASK_VALUE, _host_decode_sum, _host_max, _i32, _require_gpu, _workspace
 
 
 def mla_ragged_paged_attention(
@@ -46,6 +46,7 @@ def mla_ragged_paged_attention(
     debug_mode: bool = False,
     max_kv_len: int | None = None,
     num_splits: int = 0,
+    sum_kv_len: int | None = None,
 ):
     """Returns (output [max_num_tokens, num_q_heads, lkv_dim], cache_kv).
 
@@ -113,6 +114,7 @@ def mla_ragged_paged_attention(
     p.pages_per_seq = (page_d.numel() // max(kv_lens_d.shape[0], 1)) if cu_kv_d is None else 0
     p.max_kv_len = int(max_kv_len) if max_kv_len is not None else _host_max(kv_lens)
     p.num_splits = int(num_splits)
+    p.sum_kv_len = int(sum_kv_len) if sum_kv_len is not None else _host_decode_sum(kv_lens, k)
     p.sliding_window = int(sliding_window) if sliding_window else 0
     p.sm_scale = float(sm_scale)
     p.soft_cap = float(soft_cap) if soft_cap else 0.0
