@@ -35,6 +35,16 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
+# HBM bytes per launch (read + write) of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE scaled by a 1 GiB device copy (profiles/hbm_traffic_pmc.txt).  Counter runs cannot be
+# taken inside this process, so these are the figures of the committed profile, not live ones.
+MEASURED_TRAFFIC_BYTES = {
+    ("c2", "rpa_prefill_async_kernel"): 359.6e6 + 77.3e6,
+    ("c2", "rpa_decode_splitkv_kernel"): 501.5e6 + 3.5e6,
+    ("c3", "rpa_decode_splitkv_kernel"): 2149.9e6 + 4.3e6,
+    ("c5", "rpa_mla_decode_kernel"): 787.1e6 + 57.4e6,
+}
+
 
 def _events(n):
     import torch
@@ -171,6 +181,9 @@ def main():
     ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5"])
     ap.add_argument("--all", action="store_true", help="also time the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 1 GiB device-to-device copy (10 launches): the known-size kernel "
+                         "against which rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no sharding, no collectives); run with --gpus 1", file=sys.stderr)
@@ -187,6 +200,14 @@ def main():
         print("bench.py: no GPU visible; the operators have no CPU path", file=sys.stderr)
         sys.exit(3)
     dev = torch.device("cuda:0")
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "launches": 10}))
+        return
 
     def build(name):
         return {"c1": lambda: wl.config_c1(dev), "c2": lambda: wl.config_c2(dev), "c3": lambda: wl.config_c3(dev),
@@ -204,16 +225,21 @@ def main():
     main_res = run(args.config)
     dec_gbps = main_res.get("decode_gbps")
     pre_tflops = main_res.get("prefill_tflops")
-    # dominant kernel of the workload
+    # dominant kernel of the workload (largest average launch time inside the timed region)
+    dec_kernel = "rpa_mla_decode_kernel" if args.config == "c5" else "rpa_decode_splitkv_kernel"
+    roofline_decode = None
+    if dec_gbps is not None:
+        roofline_decode = {"kernel": dec_kernel + (" + combine" if args.config != "c1" else ""), "bound": "hbm",
+                           "achieved": dec_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": dec_gbps / HBM_PEAK_GBPS,
+                           "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dec_kernel)),
+                           "avg_launch_ms": main_res["decode_ms"], "bytes_per_launch": main_res["decode_bytes"]}
     if pre_tflops is not None and main_res.get("prefill_ms", 0) >= main_res.get("decode_ms", 0):
-        roofline = {"kernel": "rpa_prefill_flash_kernel", "bound": "mfma", "achieved": pre_tflops,
+        roofline = {"kernel": "rpa_prefill_async_kernel", "bound": "mfma", "achieved": pre_tflops,
                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": pre_tflops / MFMA_BF16_PEAK_TFLOPS,
-                    "traffic": None, "avg_launch_ms": main_res["prefill_ms"], "flops_per_launch": main_res["prefill_flops"]}
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, "rpa_prefill_async_kernel")),
+                    "avg_launch_ms": main_res["prefill_ms"], "flops_per_launch": main_res["prefill_flops"]}
     else:
-        roofline = {"kernel": "rpa_mla_decode_kernel" if args.config == "c5" else "rpa_decode_splitkv_kernel",
-                    "bound": "hbm", "achieved": dec_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                    "frac": dec_gbps / HBM_PEAK_GBPS, "traffic": None, "avg_launch_ms": main_res["decode_ms"],
-                    "bytes_per_launch": main_res["decode_bytes"]}
+        roofline = roofline_decode
     line = {
         "metric": "ragged paged attn: decode HBM GB/s (% of peak), prefill TFLOP/s; 1 MI355X",
         "value": dec_gbps if dec_gbps is not None else pre_tflops,
@@ -227,6 +253,7 @@ def main():
         "prefill_frac_of_mfma_peak": None if pre_tflops is None else pre_tflops / MFMA_BF16_PEAK_TFLOPS,
         "partitions": main_res,
         "roofline": roofline,
+        "roofline_decode": roofline_decode,
     }
     if args.all:
         line["other_configs"] = {n: run(n) for n in ("c1", "c2", "c3", "c4", "c4swa", "c5") if n != args.config}
