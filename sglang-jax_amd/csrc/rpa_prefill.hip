@@ -178,10 +178,16 @@ __device__ __forceinline__ void update_running_max(float mx, float& m, float& l,
   }
 }
 
+// xor-32 lane exchange of a maximum through v_permlane32_swap (no LDS round trip)
+__device__ __forceinline__ float swap_max(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 template <bool CAP>
 __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4], float& m, float& l,
                                              const Softmax<CAP>& sm, bool need_mask, int tb, int h, int qpos,
-                                             int window) {
+                                             int window, u32x4_t (&pB)[2][2]) {
   if constexpr (CAP) {
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -205,30 +211,29 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4],
     if (v < 15) mx = __builtin_fmaxf(__builtin_fmaxf(mx, S[0][v + 1]), S[1][v]);
     else mx = __builtin_fmaxf(mx, S[1][v]);
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 32));
+  mx = swap_max(mx);
   update_running_max<4>(mx, m, l, O, sm.sc2);
   const float neg_m = -m * sm.sc2;
-  float ps = 0.f;
+  // probabilities go straight into bf16 pairs (the B operands of the second product); the row
+  // sum is taken over the rounded pairs, one dot instruction per pair
+  const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+  float ps0 = 0.f, ps1 = 0.f;
 #pragma unroll
   for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const float p = fast_exp2(__builtin_fmaf(S[mt][v], sm.sc2, neg_m));
-      S[mt][v] = p;
-      ps += p;
+    for (int kk = 0; kk < 2; ++kk) {
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float p0 = fast_exp2(__builtin_fmaf(S[mt][8 * kk + 2 * j], sm.sc2, neg_m));
+        const float p1 = fast_exp2(__builtin_fmaf(S[mt][8 * kk + 2 * j + 1], sm.sc2, neg_m));
+        w[j] = pack_bf16x2(p0, p1);
+        if (j & 1) ps1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[j]), ones, ps1, false);
+        else ps0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[j]), ones, ps0, false);
+      }
+      pB[mt][kk] = u32x4_t{w[0], w[1], w[2], w[3]};
     }
-  l += ps;
-}
-
-__device__ __forceinline__ void pack_probs(const f32x16_t (&S)[2], u32x4_t (&pB)[2][2]) {
-#pragma unroll
-  for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
-      pB[mt][kk] = u32x4_t{pack_bf16x2(S[mt][8 * kk + 0], S[mt][8 * kk + 1]),
-                           pack_bf16x2(S[mt][8 * kk + 2], S[mt][8 * kk + 3]),
-                           pack_bf16x2(S[mt][8 * kk + 4], S[mt][8 * kk + 5]),
-                           pack_bf16x2(S[mt][8 * kk + 6], S[mt][8 * kk + 7])};
+  l += ps0 + ps1;
 }
 
 // lane (c, h) holds query row c, dims 32d + 8*(v/4) + 4h + v%4 in O[d][v]
@@ -396,6 +401,20 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
   const int v_row = (4 * h + (r16 >> 2)) * kRowB;
   const int v_in = ((b16 & 1) << 5) + (((r16 & 3) >> 1) << 4) + ((r16 & 1) << 3);
   const int v_swz = (r16 >> 2) << 6;  // byte offset of the 64-byte window: (64d) ^ v_swz
+  // The swizzled offsets are kept in registers for the whole loop (12 of them) instead of being
+  // recomputed in front of each of the 48 LDS reads of a tile; slot bases and row steps fold
+  // into the instructions' immediate offsets.
+  int koff[8], voff[4];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    koff[ks] = k_row + ((ks * 32) ^ k_swz);
+    asm volatile("" : "+v"(koff[ks]));
+  }
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    voff[d] = v_row + v_in + ((d * 64) ^ v_swz);
+    asm volatile("" : "+v"(voff[d]));
+  }
 
   // ---- pipeline: page ids two tiles ahead, the asynchronous copy one tile ahead ----
   const AsyncOffsets ofs = make_async_offsets(a.kv, wave, lane);
@@ -418,22 +437,18 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
     const bool vis = wr.active && (tb <= w.prefix + wr.r_hi) && (W_ <= 0 || tb + kBN - 1 > w.prefix + wr.r_lo - W_);
     if (vis) {
       const bool need_mask = (tb + kBN - 1 > w.prefix + wr.r_lo) || (W_ > 0 && tb <= w.prefix + wr.r_hi - W_);
-      const char* kp0 = lds_k + k_row;
-      const char* kp1 = kp0 + 32 * kRowB;
-      const char* vbase = lds_v + v_row + v_in;
       {
         // the two 32-token halves form two independent accumulator chains, issued alternately
         f32x16_t S[2];
-        S[0] = mfma32(lds_ld16(kp0 + k_swz), qB[0], kZero16);  // zero accumulator as an inline constant
-        S[1] = mfma32(lds_ld16(kp1 + k_swz), qB[0], kZero16);
+        S[0] = mfma32(lds_ld16(lds_k + koff[0]), qB[0], kZero16);  // zero accumulator as an inline constant
+        S[1] = mfma32(lds_ld16(lds_k + koff[0] + 32 * kRowB), qB[0], kZero16);
 #pragma unroll
         for (int ks = 1; ks < 8; ++ks) {
-          S[0] = mfma32(lds_ld16(kp0 + ((ks * 32) ^ k_swz)), qB[ks], S[0]);
-          S[1] = mfma32(lds_ld16(kp1 + ((ks * 32) ^ k_swz)), qB[ks], S[1]);
+          S[0] = mfma32(lds_ld16(lds_k + koff[ks]), qB[ks], S[0]);
+          S[1] = mfma32(lds_ld16(lds_k + koff[ks] + 32 * kRowB), qB[ks], S[1]);
         }
-        softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_);
         u32x4_t pB[2][2];
-        pack_probs(S, pB);
+        softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB);
         // four independent accumulator chains (dim tiles), issued round-robin
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -441,7 +456,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
           for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-              const char* vt = vbase + ((d * 64) ^ v_swz) + (mt * 32 + kk * 16) * kRowB;
+              const char* vt = lds_v + voff[d] + (mt * 32 + kk * 16) * kRowB;
               const u32x2_t lo = lds_tr16(vt);
               const u32x2_t hi = lds_tr16(vt + 8 * kRowB);
               O[d] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, pB[mt][kk], O[d]);
@@ -652,9 +667,8 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
 #pragma unroll
         for (int ks = 1; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ks * 32), qB[ks], S[mt]);
       }
-      softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_);
       u32x4_t pB[2][2];
-      pack_probs(S, pB);
+      softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB);
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
         const char* vp = lds_v + (d * 32 + c) * kVPitch + h * 16;
