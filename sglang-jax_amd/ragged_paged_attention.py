@@ -277,13 +277,16 @@ def ragged_paged_attention(
     max_q_len: int | None = None,
     num_splits: int = 0,
     validate_values: bool = False,
+    host_kv_lens=None,
 ):
     """Ragged paged attention with fused KV cache; returns (output, updated_kv_cache_fused).
 
     Mirrors rpa_v3:1667-1733.  TPU tuning knobs (block sizes, vmem limit, semaphore
     checks, debug mode) are accepted and ignored.  ``k_scale``/``v_scale`` may be a
     float (reference) or one value per kv head.  ``distribution`` and the optional
-    ``max_kv_len``/``max_q_len`` are host values used only to size launch grids.
+    ``max_kv_len``/``max_q_len`` are host values used only to size launch grids;
+    ``host_kv_lens`` is an optional host copy of ``kv_lens`` (the split plan balances on its
+    sum) for callers that pass ``kv_lens`` as a device tensor.
     """
     _require_gpu(queries, "queries")
     _require_gpu(kv_cache_fused, "kv_cache_fused")
@@ -327,9 +330,10 @@ def ragged_paged_attention(
     call = RpaCall(queries, kv_cache_fused, None, kv_lens_d, page_d, cu_q_d, cu_kv_d, num_seqs=k, decode_end=i,
                    sm_scale=sm_scale, sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
                    k_scale=k_scale, v_scale=v_scale,
-                   max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
+                   max_kv_len=max_kv_len if max_kv_len is not None else _host_max(
+                       host_kv_lens if host_kv_lens is not None else kv_lens),
                    max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits,
-                   sum_decode_kv_len=_host_decode_sum(kv_lens, i))
+                   sum_decode_kv_len=_host_decode_sum(host_kv_lens if host_kv_lens is not None else kv_lens, i))
     if validate_values:
         dynamic_validate_inputs(call.params, kv_lens_d.cpu().numpy(), page_d.cpu().numpy(), cu_q_d.cpu().numpy(),
                                 cu_kv_d.cpu().numpy(), dist.astype(np.int32))
