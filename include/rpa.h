@@ -50,6 +50,12 @@ typedef enum RpaKvDtype {
   RPA_KV_FP8_E4M3 = 1 /* OCP e4m3fn, max 448 */
 } RpaKvDtype;
 
+typedef enum RpaMaskMode {
+  RPA_MASK_CAUSAL = 0, /* query j of a sequence sees tokens <= kv_len - q_len + j */
+  RPA_MASK_CUSTOM = 1, /* causal = 0 with custom_mask (speculative tree verification) */
+  RPA_MASK_NONE = 2    /* causal = 0 without a mask: every query sees all kv_len tokens */
+} RpaMaskMode;
+
 typedef enum RpaLayout {
   /* one buffer [pages, P, 2*Hkv, D], heads stored K0,V0,K1,V1,...
    * (mem_cache/memory_pool.py:56-91, 580-588) */
@@ -104,6 +110,18 @@ typedef struct RpaParams {
   float mask_value;           /* 0 => default -0.7 * FLT_MAX */
   /* sum of kv_lens over the decode rows (host-side, balances the split plan); 0 => unknown */
   int64_t sum_decode_kv_len;
+  /* ---- further options of ref_ragged_paged_attention (ragged_paged_attention_v3.py:103-113) ---- */
+  const float* attention_sink;  /* device f32[Hq]: one extra logit per query head that enters only the
+                                   softmax denominator (:185-196), or NULL */
+  const int32_t* custom_mask;   /* device i32, flat: sequence i, query row j, token t at
+                                   cu_mask_lens[i] + j * row_width_i + t; >= 1 keeps, < 1 masks (:154-163).
+                                   Read only when mask_mode == RPA_MASK_CUSTOM */
+  const int32_t* cu_mask_lens;  /* device i32[S+1]: cumulative q_len_i * row_width_i (:123-129, 1801-1806) */
+  float xai_temperature_len;    /* > 0: logits of a query at position p > len are multiplied by
+                                   log2(p) / log2(len) (:171-177); 0 => off */
+  int32_t mask_mode;            /* RpaMaskMode */
+  int32_t mask_rows_page_aligned; /* custom mask row_width_i: 0 => kv_len_i, 1 => kv_len_i rounded up to
+                                   pages (cu_kv_lens delta; mask_aligned_to_cu_kv, :1791-1806) */
 } RpaParams;
 
 /*

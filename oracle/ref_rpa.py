@@ -102,7 +102,7 @@ def _attend_one_sequence(
     add_mask = torch.where(mask, torch.tensor(mask_value, dtype=torch.float32), torch.tensor(0.0))
 
     temp = None
-    if xai_temperature_len is not None:  # rpa_v3:171-177  (parity unpinned)
+    if xai_temperature_len is not None:  # rpa_v3:171-177
         qidx = torch.arange(kv_len - q_len, kv_len)
         scale = 1.0 / math.log2(float(xai_temperature_len))
         qtemp = torch.log2(qidx.to(torch.float32)) * scale

@@ -83,7 +83,16 @@ class RpaParams(ctypes.Structure):
         ("soft_cap", ctypes.c_float),
         ("mask_value", ctypes.c_float),
         ("sum_decode_kv_len", ctypes.c_int64),
+        ("attention_sink", ctypes.c_void_p),
+        ("custom_mask", ctypes.c_void_p),
+        ("cu_mask_lens", ctypes.c_void_p),
+        ("xai_temperature_len", ctypes.c_float),
+        ("mask_mode", ctypes.c_int32),
+        ("mask_rows_page_aligned", ctypes.c_int32),
     ]
+
+
+MASK_CAUSAL, MASK_CUSTOM, MASK_NONE = 0, 1, 2
 
 
 class RpaMlaParams(ctypes.Structure):

@@ -70,6 +70,23 @@ rpa::SoftmaxOpts softmax_opts(float sm_scale, float soft_cap, float mask_value, 
   s.soft_cap = soft_cap;
   s.mask_value = (mask_value == 0.0f) ? kDefaultMask : mask_value;
   s.window = window;
+  s.sink = nullptr;
+  s.xai_len = 0.f;
+  s.mask_mode = RPA_MASK_CAUSAL;
+  s.mask_rows_page_aligned = 0;
+  s.custom_mask = nullptr;
+  s.cu_mask_lens = nullptr;
+  return s;
+}
+
+rpa::SoftmaxOpts softmax_opts(const RpaParams* p) {
+  rpa::SoftmaxOpts s = softmax_opts(p->sm_scale, p->soft_cap, p->mask_value, p->sliding_window);
+  s.sink = p->attention_sink;
+  s.xai_len = p->xai_temperature_len;
+  s.mask_mode = p->mask_mode;
+  s.mask_rows_page_aligned = p->mask_rows_page_aligned;
+  s.custom_mask = p->custom_mask;
+  s.cu_mask_lens = p->cu_mask_lens;
   return s;
 }
 
@@ -189,6 +206,14 @@ int rpa_validate(const RpaParams* p) {
       return fail(RPA_EINVAL_SHAPE, "padded page table needs pages_per_seq > 0");
   }
   if (p->mask_value > 0.0f) return fail(RPA_EINVAL_SHAPE, "mask_value=%g must be negative", p->mask_value);
+  if (p->mask_mode < RPA_MASK_CAUSAL || p->mask_mode > RPA_MASK_NONE)
+    return fail(RPA_EINVAL_SHAPE, "mask_mode=%d is not an RpaMaskMode", p->mask_mode);
+  if (p->mask_mode == RPA_MASK_CUSTOM && (!p->custom_mask || !p->cu_mask_lens))
+    return fail(RPA_EINVAL_NULL, "RPA_MASK_CUSTOM needs custom_mask and cu_mask_lens");
+  if (p->mask_mode == RPA_MASK_CUSTOM && p->mask_rows_page_aligned && !p->cu_kv_lens)
+    return fail(RPA_EINVAL_NULL, "page-aligned mask rows need cu_kv_lens");
+  if (p->xai_temperature_len < 0.0f || std::isnan(p->xai_temperature_len))
+    return fail(RPA_EINVAL_SHAPE, "xai_temperature_len=%g must be positive", p->xai_temperature_len);
   return RPA_OK;
 }
 
@@ -274,13 +299,14 @@ int rpa_decode(const RpaParams* p, void* stream) {
   int rc = rpa_validate(p);
   if (rc != RPA_OK) return rc;
   if (p->decode_end <= 0) return RPA_OK;
+  if (p->mask_mode == RPA_MASK_CUSTOM) return RPA_OK;  // masked rows all go through the prefill kernel
   const SplitPlan sp = decode_plan(p);
   rpa::DecodeArgs a;
   a.q = static_cast<const uint16_t*>(p->q);
   a.out = static_cast<uint16_t*>(p->out);
   a.kv = kv_addr(p);
   a.pt = page_table(p);
-  a.sm = softmax_opts(p->sm_scale, p->soft_cap, p->mask_value, p->sliding_window);
+  a.sm = softmax_opts(p);
   a.k_scale = p->k_scale;
   a.v_scale = p->v_scale;
   a.num_rows = p->decode_end;
@@ -305,16 +331,16 @@ int rpa_decode(const RpaParams* p, void* stream) {
 int rpa_prefill(const RpaParams* p, void* stream) {
   int rc = rpa_validate(p);
   if (rc != RPA_OK) return rc;
-  if (p->num_seqs <= p->decode_end) return RPA_OK;
+  if (p->num_seqs <= p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) return RPA_OK;
   rpa::PrefillArgs a;
   a.q = static_cast<const uint16_t*>(p->q);
   a.out = static_cast<uint16_t*>(p->out);
   a.kv = kv_addr(p);
   a.pt = page_table(p);
-  a.sm = softmax_opts(p->sm_scale, p->soft_cap, p->mask_value, p->sliding_window);
+  a.sm = softmax_opts(p);
   a.k_scale = p->k_scale;
   a.v_scale = p->v_scale;
-  a.seq_begin = p->decode_end;
+  a.seq_begin = (p->mask_mode == RPA_MASK_CUSTOM) ? 0 : p->decode_end;
   a.seq_end = p->num_seqs;
   a.Hq = p->num_q_heads;
   a.Hkv = p->num_kv_heads;

@@ -54,6 +54,24 @@ __device__ __forceinline__ float soft_cap_f(float x, float cap, float inv_cap) {
   return cap * (1.0f - 2.0f / (e + 1.0f));
 }
 
+// Temperature factor of a query at position qpos (ragged_paged_attention_v3.py:171-177):
+// log2(qpos) / log2(T) beyond position T, 1 before.
+__device__ __forceinline__ float xai_factor(int qpos, float xai_len) {
+  if (!(xai_len > 0.f)) return 1.0f;
+  return ((float)qpos > xai_len) ? __log2f((float)qpos) / __log2f(xai_len) : 1.0f;
+}
+
+// Softmax denominator with an attention sink: given the running maximum m2 (log2 units), the
+// sum l of 2^(x - m2) and a sink logit (natural units), returns the factor that turns the
+// unnormalised output into out = sum p v / (sum p + e^sink)
+// (ragged_paged_attention_v3.py:185-196: the sink is a logit column dropped after softmax).
+__device__ __forceinline__ float sink_inverse(float m2, float l, float sink) {
+  const float s2 = sink * kLog2e;
+  const float mm = fmaxf(m2, s2);
+  const float w = __builtin_amdgcn_exp2f(m2 - mm);
+  return w / (l * w + __builtin_amdgcn_exp2f(s2 - mm));
+}
+
 // Load a 32-bit word through the scalar data cache.  `p` must be wave-uniform and point at
 // memory nobody writes during the kernel (page tables, lengths).  A scalar load is counted by
 // lgkmcnt, not vmcnt, so waiting for it never drains the vector-memory queue.

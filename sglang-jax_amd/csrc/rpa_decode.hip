@@ -125,6 +125,7 @@ struct ScoreOpts {
   float scale;      // sm_scale * k_scale            (soft-cap path)
   float scale2;     // sm_scale * k_scale * log2(e)  (plain path)
   float cap, inv_cap;
+  float post;       // log2(e) * temperature factor, applied after the soft cap
   float mask2;      // mask value in log2 units (finite)
   int t_lo;         // first visible token (sliding window), 0 otherwise
   int kv_len;
@@ -194,7 +195,7 @@ __device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       float v = s[i >> 2][i & 3];
-      if constexpr (CAP) v = soft_cap_f(v * so.scale, so.cap, so.inv_cap) * kLog2e;
+      if constexpr (CAP) v = soft_cap_f(v * so.scale, so.cap, so.inv_cap) * so.post;
       else v = v * so.scale2;
       x[i] = v;
     }
@@ -297,8 +298,11 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const Decode
 
   ScoreOpts so;
   const float ks = a.k_scale ? a.k_scale[hk] : 1.0f;
+  // the one query of a decode row sits at position kv_len - 1
+  const float temp = xai_factor(kv_len - 1, a.sm.xai_len);
   so.scale = a.sm.sm_scale * ks;
-  so.scale2 = so.scale * kLog2e;
+  so.scale2 = so.scale * kLog2e * temp;
+  so.post = kLog2e * temp;
   so.cap = a.sm.soft_cap;
   so.inv_cap = (so.cap != 0.f) ? 1.0f / so.cap : 0.f;
   so.mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
@@ -349,7 +353,7 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const Decode
     if (row >= a.G) continue;
     const int head = hk * a.G + row;
     if (a.max_splits == 1) {
-      const float inv = vs / lt;
+      const float inv = a.sm.sink ? vs * sink_inverse(m[mt], lt, a.sm.sink[head]) : vs / lt;
       uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 128 + g * 32;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -429,7 +433,7 @@ __global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a) {
       }
     }
   }
-  const float inv = 1.0f / den;
+  const float inv = a.sm.sink ? sink_inverse(mstar, den, a.sm.sink[head]) : 1.0f / den;
   const int tq = a.pt.cu_q_lens[seq];
   uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * 128 + d);
   *op = pack_bf16x2(o0 * inv, o1 * inv);

@@ -32,6 +32,13 @@ struct SoftmaxOpts {
   float soft_cap;    // 0 => off
   float mask_value;  // finite, negative
   int32_t window;    // 0 => off
+  const float* sink;  // f32[Hq] extra logit per query head that only enters the denominator, or nullptr
+  float xai_len;      // > 0: logits of a query at position p > xai_len are multiplied by log2(p)/log2(xai_len)
+  // prefill kernels only: 0 causal, 1 custom mask, 2 no mask
+  int32_t mask_mode;
+  int32_t mask_rows_page_aligned;
+  const int32_t* custom_mask;
+  const int32_t* cu_mask_lens;
 };
 
 struct DecodeArgs {

@@ -146,7 +146,9 @@ struct WaveRows {
 
 template <bool CAP>
 struct Softmax {
-  float scale, cap, inv_cap, sc2;
+  float scale, cap, inv_cap;
+  float sc2;   // raw score -> log2 units inside the exponent (per row: carries the temperature factor)
+  float post;  // soft-cap path: log2(e) * temperature factor
 };
 
 // Online-softmax update of one 64-token tile.  On entry S holds raw scores (MFMA units); on
@@ -184,15 +186,36 @@ __device__ __forceinline__ float swap_max(float x) {
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
-template <bool CAP>
+// Which tokens a query row may see.  mode 0: causal (token <= row position); mode 1: the
+// caller's mask row (>= 1 keeps), mode 2: everything; modes 1 and 2 still hide the tokens of a
+// partial last tile beyond kv_len.  The sliding window applies on top in every mode.
+struct MaskCtx {
+  int mode;
+  int kv_len;
+  const int32_t* row;  // mode 1: this lane's mask row (token t at row[t])
+};
+
+__device__ __forceinline__ MaskCtx make_mask_ctx(const PrefillArgs& a, const Work& w, int row) {
+  MaskCtx mc;
+  mc.mode = a.sm.mask_mode;
+  mc.kv_len = w.kv_len;
+  mc.row = nullptr;
+  if (mc.mode == 1) {
+    const int width = a.sm.mask_rows_page_aligned ? (a.pt.cu_kv_lens[w.seq + 1] - a.pt.cu_kv_lens[w.seq]) : w.kv_len;
+    mc.row = a.sm.custom_mask + a.sm.cu_mask_lens[w.seq] + (int64_t)min(row, w.q_len - 1) * width;
+  }
+  return mc;
+}
+
+template <bool CAP, bool EXT>
 __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4], float& m, float& l,
                                              const Softmax<CAP>& sm, bool need_mask, int tb, int h, int qpos,
-                                             int window, u32x4_t (&pB)[2][2]) {
+                                             int window, u32x4_t (&pB)[2][2], const MaskCtx& mc) {
   if constexpr (CAP) {
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) S[mt][v] = soft_cap_f(S[mt][v] * sm.scale, sm.cap, sm.inv_cap) * kLog2e;
+      for (int v = 0; v < 16; ++v) S[mt][v] = soft_cap_f(S[mt][v] * sm.scale, sm.cap, sm.inv_cap) * sm.post;
   }
   if (need_mask) {
 #pragma unroll
@@ -200,7 +223,10 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4],
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int tok = tb + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-        const bool masked = (tok > qpos) || (window > 0 && tok <= qpos - window);
+        bool masked;
+        if (!EXT || mc.mode == 0) masked = tok > qpos;
+        else masked = (tok >= mc.kv_len) || (mc.mode == 1 && mc.row[tok] < 1);
+        masked = masked || (window > 0 && tok <= qpos - window);
         S[mt][v] = masked ? kMaskRaw : S[mt][v];
       }
   }
@@ -238,11 +264,11 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4],
 
 // lane (c, h) holds query row c, dims 32d + 8*(v/4) + 4h + v%4 in O[d][v]
 __device__ __forceinline__ void write_rows(const PrefillArgs& a, const Work& w, const WaveRows& wr,
-                                           const f32x16_t (&O)[4], float l, int h) {
+                                           const f32x16_t (&O)[4], float l, int h, float m2) {
   l += __shfl_xor(l, 32);
   if (!wr.active || wr.row >= w.q_len) return;
   const float vs = a.v_scale ? a.v_scale[w.hk] : 1.0f;
-  const float inv = vs / l;
+  const float inv = a.sm.sink ? vs * sink_inverse(m2, l, a.sm.sink[w.head]) : vs / l;
   uint16_t* op = a.out + ((int64_t)(w.qg0 + wr.row) * a.Hq + w.head) * 128 + 4 * h;
 #pragma unroll
   for (int d = 0; d < 4; ++d)
@@ -337,7 +363,9 @@ __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const 
   }
 }
 
-template <bool UNIFORM, bool CAP>
+// EXT compiles in the rarely used options (temperature factor, custom mask / no mask); the
+// plain causal instantiation keeps its scale in a scalar register and its mask test to one compare.
+template <bool UNIFORM, bool CAP, bool EXT>
 __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const PrefillArgs a, int tiles, int nseq) {
   // Four separate arrays (not one indexed array): the compiler can then prove that the
   // asynchronous copy into one ring slot does not alias the LDS reads of the other slot and
@@ -376,7 +404,11 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
   sm.scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f);
   sm.cap = a.sm.soft_cap;
   sm.inv_cap = (sm.cap != 0.f) ? 1.0f / sm.cap : 0.f;
-  sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e;
+  {
+    const float temp = EXT ? xai_factor(wr.qpos, a.sm.xai_len) : 1.0f;  // per query row
+    sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e * temp;
+    sm.post = kLog2e * temp;
+  }
 
   f32x16_t O[4];
 #pragma unroll
@@ -386,7 +418,11 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
   float m = kMaxFloor, l = 0.f;
 
   const int wg_r_hi = min(w.q_start + kBM, w.q_len) - 1;
-  const int t_hi = min(w.kv_len, w.prefix + wg_r_hi + 1);  // exclusive
+  const bool causal = !EXT || a.sm.mask_mode == 0;
+  MaskCtx mc;
+  mc.mode = 0;
+  if constexpr (EXT) mc = make_mask_ctx(a, w, wr.row);
+  const int t_hi = causal ? min(w.kv_len, w.prefix + wg_r_hi + 1) : w.kv_len;  // exclusive
   int t_lo = 0;
   if (W_ > 0) t_lo = max(0, w.prefix + w.q_start - W_ + 1) & ~(kBN - 1);
 
@@ -434,9 +470,11 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
     }
     // visible to this wave?  causal: some token <= last row's position; window: some token
     // newer than the first row's horizon
-    const bool vis = wr.active && (tb <= w.prefix + wr.r_hi) && (W_ <= 0 || tb + kBN - 1 > w.prefix + wr.r_lo - W_);
+    const bool vis = wr.active && (!causal || tb <= w.prefix + wr.r_hi) &&
+                     (W_ <= 0 || tb + kBN - 1 > w.prefix + wr.r_lo - W_);
     if (vis) {
-      const bool need_mask = (tb + kBN - 1 > w.prefix + wr.r_lo) || (W_ > 0 && tb <= w.prefix + wr.r_hi - W_);
+      const bool need_mask = (causal ? (tb + kBN - 1 > w.prefix + wr.r_lo) : (mc.mode == 1 || tb + kBN > w.kv_len)) ||
+                             (W_ > 0 && tb <= w.prefix + wr.r_hi - W_);
       {
         // the two 32-token halves form two independent accumulator chains, issued alternately
         f32x16_t S[2];
@@ -448,7 +486,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
           S[1] = mfma32(lds_ld16(lds_k + koff[ks] + 32 * kRowB), qB[ks], S[1]);
         }
         u32x4_t pB[2][2];
-        softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB);
+        softmax_tile<CAP, EXT>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc);
         // four independent accumulator chains (dim tiles), issued round-robin
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -471,7 +509,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
     if (tb + kBN >= t_hi) break;
     tile_step(lds_k1, lds_v1, lds_k0, lds_v0, tb + kBN);
   }
-  write_rows(a, w, wr, O, l, h);
+  write_rows(a, w, wr, O, l, h, m * sm.sc2);
 }
 
 // ==================================================================== staged path (fp8 cache)
@@ -588,7 +626,7 @@ __device__ __forceinline__ void tile_lstore(const Stage<FP8>& st, char* lds_k, c
   }
 }
 
-template <bool FP8, bool UNIFORM, bool CAP>
+template <bool FP8, bool UNIFORM, bool CAP, bool EXT>
 __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const PrefillArgs a, int tiles, int nseq) {
   __shared__ __attribute__((aligned(16))) char lds_k_buf[2][kBN * kKPitch];
   __shared__ __attribute__((aligned(16))) char lds_v_buf[2][128 * kVPitch];
@@ -621,7 +659,11 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
   sm.scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f);
   sm.cap = a.sm.soft_cap;
   sm.inv_cap = (sm.cap != 0.f) ? 1.0f / sm.cap : 0.f;
-  sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e;
+  {
+    const float temp = EXT ? xai_factor(wr.qpos, a.sm.xai_len) : 1.0f;  // per query row
+    sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e * temp;
+    sm.post = kLog2e * temp;
+  }
 
   f32x16_t O[4];
 #pragma unroll
@@ -631,7 +673,11 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
   float m = kMaxFloor, l = 0.f;
 
   const int wg_r_hi = min(w.q_start + kBM, w.q_len) - 1;
-  const int t_hi = min(w.kv_len, w.prefix + wg_r_hi + 1);  // exclusive
+  const bool causal = !EXT || a.sm.mask_mode == 0;
+  MaskCtx mc;
+  mc.mode = 0;
+  if constexpr (EXT) mc = make_mask_ctx(a, w, wr.row);
+  const int t_hi = causal ? min(w.kv_len, w.prefix + wg_r_hi + 1) : w.kv_len;  // exclusive
   int t_lo = 0;
   if (W_ > 0) t_lo = max(0, w.prefix + w.q_start - W_ + 1) & ~(kBN - 1);
 
@@ -656,9 +702,11 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
       tile_gload<FP8, UNIFORM>(stg, src, a.kv, kh, vh, tb + 2 * kBN, tid, pg);
       fetch_page_ids<UNIFORM>(pg, src, tb + 3 * kBN, tid);
     }
-    const bool vis = wr.active && (tb <= w.prefix + wr.r_hi) && (W_ <= 0 || tb + kBN - 1 > w.prefix + wr.r_lo - W_);
+    const bool vis = wr.active && (!causal || tb <= w.prefix + wr.r_hi) &&
+                     (W_ <= 0 || tb + kBN - 1 > w.prefix + wr.r_lo - W_);
     if (vis) {
-      const bool need_mask = (tb + kBN - 1 > w.prefix + wr.r_lo) || (W_ > 0 && tb <= w.prefix + wr.r_hi - W_);
+      const bool need_mask = (causal ? (tb + kBN - 1 > w.prefix + wr.r_lo) : (mc.mode == 1 || tb + kBN > w.kv_len)) ||
+                             (W_ > 0 && tb <= w.prefix + wr.r_hi - W_);
       f32x16_t S[2];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
@@ -668,7 +716,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
         for (int ks = 1; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ks * 32), qB[ks], S[mt]);
       }
       u32x4_t pB[2][2];
-      softmax_tile<CAP>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB);
+      softmax_tile<CAP, EXT>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc);
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
         const char* vp = lds_v + (d * 32 + c) * kVPitch + h * 16;
@@ -681,7 +729,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
     }
     __syncthreads();
   }
-  write_rows(a, w, wr, O, l, h);
+  write_rows(a, w, wr, O, l, h, m * sm.sc2);
 }
 
 }  // namespace
@@ -698,31 +746,33 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
   const bool staged = a.fp8 || force_staged;
   const dim3 g((unsigned)grid), blk(256);
-#define RPA_STAGED(F, U, C) hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C>), g, blk, 0, stream, a, tiles, nseq)
-#define RPA_ASYNC(U, C) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C>), g, blk, 0, stream, a, tiles, nseq)
-  const int key = (uniform ? 2 : 0) | (cap ? 1 : 0);
-  if (!staged) {
-    switch (key) {
-      case 0: RPA_ASYNC(false, false); break;
-      case 1: RPA_ASYNC(false, true); break;
-      case 2: RPA_ASYNC(true, false); break;
-      default: RPA_ASYNC(true, true); break;
-    }
-  } else if (a.fp8) {
-    switch (key) {
-      case 0: RPA_STAGED(true, false, false); break;
-      case 1: RPA_STAGED(true, false, true); break;
-      case 2: RPA_STAGED(true, true, false); break;
-      default: RPA_STAGED(true, true, true); break;
-    }
-  } else {
-    switch (key) {
-      case 0: RPA_STAGED(false, false, false); break;
-      case 1: RPA_STAGED(false, false, true); break;
-      case 2: RPA_STAGED(false, true, false); break;
-      default: RPA_STAGED(false, true, true); break;
-    }
+  const bool ext = a.sm.xai_len > 0.f || a.sm.mask_mode != 0;
+#define RPA_STAGED(F, U, C, E) \
+  hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C, E>), g, blk, 0, stream, a, tiles, nseq)
+#define RPA_ASYNC(U, C, E) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E>), g, blk, 0, stream, a, tiles, nseq)
+#define RPA_PICK(M, ...)                                            \
+  switch ((uniform ? 4 : 0) | (cap ? 2 : 0) | (ext ? 1 : 0)) {        \
+    case 0: M(__VA_ARGS__ false, false, false); break;              \
+    case 1: M(__VA_ARGS__ false, false, true); break;               \
+    case 2: M(__VA_ARGS__ false, true, false); break;               \
+    case 3: M(__VA_ARGS__ false, true, true); break;                \
+    case 4: M(__VA_ARGS__ true, false, false); break;               \
+    case 5: M(__VA_ARGS__ true, false, true); break;                \
+    case 6: M(__VA_ARGS__ true, true, false); break;                \
+    default: M(__VA_ARGS__ true, true, true); break;                \
   }
+#define RPA_STAGED_FP8(U, C, E) RPA_STAGED(true, U, C, E)
+#define RPA_STAGED_BF16(U, C, E) RPA_STAGED(false, U, C, E)
+  if (!staged) {
+    RPA_PICK(RPA_ASYNC, )
+  } else if (a.fp8) {
+    RPA_PICK(RPA_STAGED_FP8, )
+  } else {
+    RPA_PICK(RPA_STAGED_BF16, )
+  }
+#undef RPA_STAGED_FP8
+#undef RPA_STAGED_BF16
+#undef RPA_PICK
 #undef RPA_STAGED
 #undef RPA_ASYNC
   return hipGetLastError();

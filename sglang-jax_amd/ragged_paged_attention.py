@@ -187,7 +187,9 @@ class RpaCall:
 
     def __init__(self, queries, kv_cache, v_pages, kv_lens_d, page_d, cu_q_d, cu_kv_d, *, num_seqs, decode_end,
                  sm_scale, sliding_window=None, soft_cap=None, mask_value=DEFAULT_MASK_VALUE, k_scale=None,
-                 v_scale=None, max_kv_len=0, max_q_len=0, num_splits=0, out=None, sum_decode_kv_len=0):
+                 v_scale=None, max_kv_len=0, max_q_len=0, num_splits=0, out=None, sum_decode_kv_len=0,
+                 attention_sink=None, xai_temperature_len=None, causal=True, custom_mask=None,
+                 mask_aligned_to_cu_kv=False):
         self.lib = _lib.load()
         self.device = queries.device
         fused = v_pages is None
@@ -215,6 +217,48 @@ class RpaCall:
         p.pages_per_seq = page_d.shape[1] if page_d.dim() == 2 else 0
         p.k_scale = self.ks.data_ptr() if self.ks is not None else None
         p.v_scale = self.vs.data_ptr() if self.vs is not None else None
+        # ---- attention sink: scalar or one logit per query head (rpa_v3:185-193)
+        self.sink = None
+        if attention_sink is not None:
+            sink = torch.as_tensor(attention_sink, dtype=torch.float32).reshape(-1)
+            if sink.numel() == 1:
+                sink = sink.expand(queries.shape[1])
+            if sink.numel() != queries.shape[1]:
+                raise ValueError(f"Expected attention_sink with {queries.shape[1]} entries, got {sink.numel()}")
+            self.sink = sink.to(self.device).contiguous()
+            p.attention_sink = self.sink.data_ptr()
+        if xai_temperature_len is not None:
+            if not xai_temperature_len > 0:
+                raise ValueError(f"xai_temperature_len={xai_temperature_len} must be positive.")
+            p.xai_temperature_len = float(xai_temperature_len)
+        # ---- mask mode (rpa_v3:152-165): causal, the caller's flat mask, or none
+        self.mask = self.cu_mask = None
+        if causal:
+            p.mask_mode = _lib.MASK_CAUSAL
+        elif custom_mask is None:
+            p.mask_mode = _lib.MASK_NONE
+        else:
+            mask = custom_mask
+            if mask.dtype == torch.bool:
+                mask = mask.to(torch.int32)
+            if mask.dtype != torch.int32:
+                raise ValueError(f"Expected int32 (or bool) custom_mask, got {mask.dtype}")
+            self.mask = mask.to(self.device).contiguous().reshape(-1)
+            # cu_seq_mask_lens = [0, cumsum(q_len * row width)] on the device (rpa_v3:1801-1806)
+            q_lens = (cu_q_d[1:] - cu_q_d[:-1]).to(torch.int64)
+            if mask_aligned_to_cu_kv:
+                if cu_kv_d is None:
+                    raise ValueError("mask_aligned_to_cu_kv needs cu_kv_lens")
+                widths = (cu_kv_d[1:] - cu_kv_d[:-1]).to(torch.int64)
+            else:
+                widths = kv_lens_d[: q_lens.shape[0]].to(torch.int64)
+            cu = torch.zeros(q_lens.shape[0] + 1, dtype=torch.int64, device=self.device)
+            cu[1:] = torch.cumsum(q_lens * widths[: q_lens.shape[0]], dim=0)
+            self.cu_mask = cu.to(torch.int32)
+            p.mask_mode = _lib.MASK_CUSTOM
+            p.custom_mask = self.mask.data_ptr()
+            p.cu_mask_lens = self.cu_mask.data_ptr()
+            p.mask_rows_page_aligned = 1 if mask_aligned_to_cu_kv else 0
         need = self.lib.rpa_workspace_bytes(ctypes.byref(p))
         self.workspace = None
         if need:
@@ -302,10 +346,7 @@ def ragged_paged_attention(
     static_validate_inputs(queries, keys, values, kv_cache_fused, kv_lens_d, page_d, cu_q_d, cu_kv_d, dist_t,
                            causal=causal, sliding_window=sliding_window, soft_cap=soft_cap,
                            chunk_prefill_size=chunk_prefill_size, skip_kv_mask=skip_kv_mask)
-    if causal != 1 or custom_mask is not None:
-        raise NotImplementedError("custom_mask / causal=0 (speculative tree verification) is not built")
-    for name, val in (("attention_sink", attention_sink), ("xai_temperature_len", xai_temperature_len),
-                      ("softmax_dtype", softmax_dtype), ("q_scale", q_scale)):
+    for name, val in (("softmax_dtype", softmax_dtype), ("q_scale", q_scale)):
         if val is not None:
             raise NotImplementedError(f"{name} is not built")
     if kv_cache_fused.dim() == 5:  # reference's packed view [pages, P, 2Hkv/pack, pack, D]
@@ -333,7 +374,9 @@ def ragged_paged_attention(
                    max_kv_len=max_kv_len if max_kv_len is not None else _host_max(
                        host_kv_lens if host_kv_lens is not None else kv_lens),
                    max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits,
-                   sum_decode_kv_len=_host_decode_sum(host_kv_lens if host_kv_lens is not None else kv_lens, i))
+                   sum_decode_kv_len=_host_decode_sum(host_kv_lens if host_kv_lens is not None else kv_lens, i),
+                   attention_sink=attention_sink, xai_temperature_len=xai_temperature_len, causal=bool(causal),
+                   custom_mask=custom_mask, mask_aligned_to_cu_kv=mask_aligned_to_cu_kv)
     if validate_values:
         dynamic_validate_inputs(call.params, kv_lens_d.cpu().numpy(), page_d.cpu().numpy(), cu_q_d.cpu().numpy(),
                                 cu_kv_d.cpu().numpy(), dist.astype(np.int32))
@@ -362,6 +405,10 @@ def ragged_paged_attention_ref_surface(
     mask_value: float | None = DEFAULT_MASK_VALUE,
     k_scale=None,
     v_scale=None,
+    custom_mask=None,
+    xai_temperature_len: float | None = None,
+    attention_sink=None,
+    softmax_dtype=None,
     decode_end: int = 0,
     max_kv_len: int | None = None,
     max_q_len: int | None = None,
@@ -373,8 +420,8 @@ def ragged_paged_attention_ref_surface(
     how many leading sequences are single-token rows (0 is always valid: the
     flash kernel handles q_len == 1 too)."""
     _require_gpu(queries, "queries")
-    if not causal:
-        raise NotImplementedError("causal=False is not built")
+    if softmax_dtype is not None:
+        raise NotImplementedError("softmax_dtype is not built")
     if sliding_window is not None and sliding_window <= 0:
         raise ValueError(f"sliding_window={sliding_window} must be positive.")
     if soft_cap is not None and soft_cap == 0.0:
@@ -397,7 +444,8 @@ def ragged_paged_attention_ref_surface(
                    k_scale=k_scale, v_scale=v_scale,
                    max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
                    max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits,
-                   sum_decode_kv_len=_host_decode_sum(kv_lens, decode_end))
+                   sum_decode_kv_len=_host_decode_sum(kv_lens, decode_end), attention_sink=attention_sink,
+                   xai_temperature_len=xai_temperature_len, causal=bool(causal), custom_mask=custom_mask)
     call.attention()
     return call.out
 

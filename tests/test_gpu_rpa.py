@@ -42,8 +42,8 @@ def gpu_out(pkg, b, dev, **kw):
     dist = b.distribution.cpu().numpy()
     n = int(dist[2])
     out, _ = pkg.ragged_paged_attention(
-        g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens, dist, None,
-        sm_scale=b.sm_scale, sliding_window=b.sliding_window, soft_cap=b.soft_cap, k_scale=g.k_scale,
+        g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens, dist,
+        kw.pop("custom_mask", None), sm_scale=b.sm_scale, sliding_window=b.sliding_window, soft_cap=b.soft_cap, k_scale=g.k_scale,
         v_scale=g.v_scale, max_kv_len=int(max(b.meta["kv_lens"])), max_q_len=int(q_lens[:n].max()), **kw)
     torch.cuda.synchronize()
     T = int(b.cu_q_lens[n])
@@ -336,3 +336,83 @@ def test_full_size_page_permutation_invariance(pkg, wl, gpu, name):
     assert torch.equal(a.view(torch.int16), run(c).view(torch.int16))
     one = run(b, num_splits=1)
     torch.testing.assert_close(a.float(), one.float(), rtol=1e-2, atol=4e-3)
+
+
+# ------------------------------------------------------------------ further options of the oracle
+def options_batch(wl, name, seed, P=64):
+    # decode rows (short, long, at a page edge), then chunks with and without a prefix
+    q_lens = [1, 1, 1, 7, 130, 64]
+    kv_lens = [5, 700, 2 * P, 7, 300, 1000]
+    return q_lens, kv_lens, wl.make_batch(name, q_lens, kv_lens, num_q_heads=16, num_kv_heads=4, head_dim=128,
+                                          page_size=P, seed=seed)
+
+
+@pytest.mark.parametrize("window,cap", [(None, None), (100, 20.0)])
+def test_attention_sink(pkg, wl, gpu, window, cap):
+    """One extra logit per query head in the softmax denominator (ragged_paged_attention_v3.py:185-196);
+    sink vectors drawn as the reference's tests draw them (test_flashattention_mha.py:171)."""
+    q_lens, kv_lens, b = options_batch(wl, "sink", 71)
+    b.sliding_window, b.soft_cap = window, cap
+    sink = torch.from_numpy(np.random.RandomState(123).randn(16).astype(np.float32)) * 3.0
+    say(f"case sink window={window} cap={cap}")
+    want = oracle_out(b, attention_sink=sink)
+    got = gpu_out(pkg, b, gpu, attention_sink=sink)
+    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    # a sink far below every logit changes nothing; one far above takes all the weight
+    none = gpu_out(pkg, b, gpu)
+    low = gpu_out(pkg, b, gpu, attention_sink=torch.full((16,), -1.0e4))
+    torch.testing.assert_close(low.float(), none.float(), rtol=8e-3, atol=1e-3)  # one bf16 ulp
+    high = gpu_out(pkg, b, gpu, attention_sink=1.0e4)
+    assert float(high.float().abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("cap", [None, 20.0])
+def test_xai_temperature(pkg, wl, gpu, cap):
+    """Logits of queries beyond position T are multiplied by log2(pos)/log2(T)
+    (ragged_paged_attention_v3.py:171-177)."""
+    q_lens, kv_lens, b = options_batch(wl, "xai", 72)
+    b.soft_cap = cap
+    say(f"case xai cap={cap}")
+    for T in (64.0, 8192.0):  # rows on both sides of T / no row beyond T
+        want = oracle_out(b, xai_temperature_len=T)
+        got = gpu_out(pkg, b, gpu, xai_temperature_len=T)
+        torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    assert torch.equal(gpu_out(pkg, b, gpu, xai_temperature_len=8192.0), gpu_out(pkg, b, gpu))
+
+
+def flat_mask(masks):
+    return torch.from_numpy(np.concatenate([m.reshape(-1) for m in masks]).astype(np.int32))
+
+
+@pytest.mark.parametrize("P", [16, 64])
+def test_custom_mask_and_no_mask(pkg, wl, gpu, P):
+    """causal = 0: tree-verification masks (ragged_paged_attention_v3.py:152-165) and full attention."""
+    q_lens, kv_lens = [4, 1, 33, 8], [70, 130, 33, 300]
+    b = wl.make_batch("cmask", q_lens, kv_lens, num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=P, seed=73)
+    rng = np.random.default_rng(9)
+    masks = []
+    for ql, kv in zip(q_lens, kv_lens):
+        m = (rng.random((ql, kv)) < 0.6).astype(np.int32)
+        m[:, 0] = 1  # every row keeps a token
+        masks.append(m)
+    cm = flat_mask(masks)
+    say(f"case custom mask P={P}")
+    want = oracle_out(b, causal=False, custom_mask=cm)
+    got = gpu_out(pkg, b, gpu, causal=0, custom_mask=cm.to(gpu))
+    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    # rows padded to whole pages (mask_aligned_to_cu_kv, ragged_paged_attention_v3.py:1791-1806)
+    padded = []
+    for m in masks:
+        w = -(-m.shape[1] // P) * P
+        mp = np.zeros((m.shape[0], w), dtype=np.int32)
+        mp[:, : m.shape[1]] = m
+        padded.append(mp)
+    got2 = gpu_out(pkg, b, gpu, causal=0, custom_mask=flat_mask(padded).to(gpu), mask_aligned_to_cu_kv=True)
+    assert torch.equal(got2, got)
+    # the causal pattern spelled out as a mask equals the causal kernel path
+    causal = [(np.arange(kv)[None, :] <= (kv - ql) + np.arange(ql)[:, None]).astype(np.int32)
+              for ql, kv in zip(q_lens, kv_lens)]
+    got3 = gpu_out(pkg, b, gpu, causal=0, custom_mask=flat_mask(causal).to(gpu))
+    torch.testing.assert_close(got3.float(), oracle_out(b).float(), **BF16_TOL)
+    say("case no mask")
+    torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=0).float(), oracle_out(b, causal=False).float(), **BF16_TOL)

@@ -7,7 +7,7 @@ and jnp oracle on fresh random inputs), so the oracle is pinned by
   * a float64 scalar-loop brute force (tests/bruteforce.py),
   * closed forms and invariants of masked softmax attention,
   * the committed fixtures under tests/golden/ (brute-force outputs).
-xai_temperature_len and softmax_dtype have no such pin: parity unpinned.
+softmax_dtype has no such pin: parity unpinned.
 """
 
 import math
@@ -318,3 +318,87 @@ def test_forward_metadata_closed_forms():
     assert dist.tolist() == [0, 3, 3]
     table = ragged_to_padded_page_table(pi, cu_kv, P, 3)
     assert table.tolist() == [[7, 2], [3, 9], [5, 0]]
+
+
+# ---------------------------------------------------------------- temperature (rpa_v3:171-177)
+def test_temperature_reduces_to_a_per_row_scale():
+    """With T = 4 a query at position 16 has factor log2(16)/log2(4) = 2 exactly and a query at
+    position 64 has 3: each such row equals the plain oracle with sm_scale doubled / tripled;
+    rows at positions <= T are unchanged."""
+    D = 16
+    # decode rows at chosen positions (position = kv_len - 1) and one chunk crossing T
+    q_lens, kv_lens = [1, 1, 1, 1, 3], [17, 65, 5, 3, 6]
+    c = make_case(q_lens, kv_lens, 4, 2, D, 4, seed=31, dtype=torch.float32)
+    out = run(c, sm_scale=0.25, xai_temperature_len=4.0)
+    plain = run(c, sm_scale=0.25)
+    x2 = run(c, sm_scale=0.5)
+    x3 = run(c, sm_scale=0.75)
+    torch.testing.assert_close(out[0], x2[0], rtol=1e-5, atol=1e-6)      # position 16
+    torch.testing.assert_close(out[1], x3[1], rtol=1e-5, atol=1e-6)      # position 64
+    torch.testing.assert_close(out[2], plain[2], rtol=0, atol=0)         # position 4 == T: not beyond
+    torch.testing.assert_close(out[3], plain[3], rtol=0, atol=0)         # position 2
+    # chunk rows at positions 3, 4, 5: only the last is beyond T (factor log2(5)/2)
+    torch.testing.assert_close(out[4:6], plain[4:6], rtol=0, atol=0)
+    f = math.log2(5.0) / 2.0
+    scaled = run(c, sm_scale=0.25 * f)
+    torch.testing.assert_close(out[6], scaled[6], rtol=1e-5, atol=1e-6)
+
+
+def test_temperature_applies_after_the_soft_cap():
+    """cap*tanh(s/cap) is bounded by cap; with factor 2 the logits reach 2*cap, which a factor
+    applied before the cap could never produce: compare with the float64 brute force fed the
+    doubled cap-ed scores through its own scale/cap arguments."""
+    q_lens, kv_lens = [1], [17]
+    c = make_case(q_lens, kv_lens, 2, 1, 8, 4, seed=32, dtype=torch.float32)
+    cap, sm = 1.5, 0.9
+    out = run(c, sm_scale=sm, soft_cap=cap, xai_temperature_len=4.0).double().numpy()
+    k, v = gathered(c, 0)
+    q = c["q"].double().numpy()
+    kk, vv = k.double().numpy(), v.double().numpy()
+    want = np.zeros_like(out)
+    for h in range(2):
+        sc = np.array([2.0 * cap * math.tanh(sm * float(q[0, h] @ kk[t, 0]) / cap) for t in range(17)])
+        w = np.exp(sc - sc.max())
+        want[0, h] = (w / w.sum()) @ vv[:, 0]
+    np.testing.assert_allclose(out, want, rtol=2e-5, atol=2e-6)
+
+
+# ---------------------------------------------------------------- custom mask (rpa_v3:152-165)
+def _flat_mask(masks):
+    return torch.from_numpy(np.concatenate([m.reshape(-1) for m in masks]).astype(np.int32))
+
+
+def test_custom_mask_special_cases_and_brute_force():
+    q_lens, kv_lens = [3, 1, 5], [9, 6, 5]
+    Hq, Hkv, D, P = 4, 2, 8, 4
+    c = make_case(q_lens, kv_lens, Hq, Hkv, D, P, seed=33, dtype=torch.float32)
+    sm = 0.4
+    # (1) a mask that spells out the causal pattern reproduces causal attention
+    causal = [(np.arange(kv)[None, :] <= (kv - ql) + np.arange(ql)[:, None]) for ql, kv in zip(q_lens, kv_lens)]
+    out = run(c, sm_scale=sm, causal=False, custom_mask=_flat_mask(causal))
+    torch.testing.assert_close(out, run(c, sm_scale=sm), rtol=1e-6, atol=1e-6)
+    # (2) an all-ones mask equals causal=False without a mask
+    ones = [np.ones((ql, kv)) for ql, kv in zip(q_lens, kv_lens)]
+    torch.testing.assert_close(run(c, sm_scale=sm, causal=False, custom_mask=_flat_mask(ones)),
+                               run(c, sm_scale=sm, causal=False), rtol=0, atol=0)
+    # (3) a random tree-like mask (every row keeps at least one token) against a float64 loop
+    rng = np.random.default_rng(5)
+    masks = []
+    for ql, kv in zip(q_lens, kv_lens):
+        mk = rng.integers(0, 2, size=(ql, kv))
+        mk[:, 0] = 1
+        masks.append(mk)
+    out = run(c, sm_scale=sm, causal=False, custom_mask=_flat_mask(masks)).double().numpy()
+    o = 0
+    for i, (ql, kv) in enumerate(zip(q_lens, kv_lens)):
+        k, v = gathered(c, i)
+        q = c["q"][o:o + ql].double().numpy()
+        kk, vv = k.double().numpy(), v.double().numpy()
+        for j in range(ql):
+            for h in range(Hq):
+                keep = [t for t in range(kv) if masks[i][j, t] >= 1]
+                sc = np.array([sm * float(q[j, h] @ kk[t, h // 2]) for t in keep])
+                w = np.exp(sc - sc.max())
+                want = (w / w.sum()) @ vv[keep, h // 2]
+                np.testing.assert_allclose(out[o + j, h], want, rtol=2e-5, atol=2e-6)
+        o += ql
