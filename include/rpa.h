@@ -143,7 +143,7 @@ typedef struct RpaMlaParams {
   void* workspace;
   size_t workspace_bytes;
   int32_t num_tokens;
-  int32_t num_seqs;           /* all must be decode rows (q_len == 1) */
+  int32_t num_seqs;           /* rpa_mla_decode: all must be decode rows (q_len == 1) */
   int32_t num_q_heads;
   int32_t lkv_dim;            /* 512 */
   int32_t rope_dim;           /* 64 */
@@ -223,8 +223,25 @@ int rpa_attention(const RpaParams* p, void* stream);
  */
 int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void* stream);
 
-/* Absorbed-MLA decode, see RpaMlaParams. */
+/* Absorbed-MLA decode, see RpaMlaParams: every sequence contributes exactly one query token. */
 int rpa_mla_decode(const RpaMlaParams* p, void* stream);
+
+/*
+ * Absorbed-MLA attention for any batch composition (decode, prefill chunks, mixed): the three
+ * launches of mla_ragged_paged_attention (kernels/mla/v2/kernel.py:1338-1744) in one.  Query
+ * token j of a sequence with q_len new tokens attends to the cache tokens 0 .. kv_len - q_len + j.
+ * Workspace: rpa_mla_attention_workspace_bytes(); max_kv_len / sum_kv_len bound, resp. sum, the
+ * per-token visible lengths.
+ */
+size_t rpa_mla_attention_workspace_bytes(const RpaMlaParams* p);
+int rpa_mla_attention(const RpaMlaParams* p, void* stream);
+
+/*
+ * Write the new latent rows into the paged cache: update_kv_cache of kernels/mla/v1/ref.py:56-105
+ * (the fused cache update of kernels/mla/v2/kernel.py).  new_kv_c bf16 [T, lkv_dim], new_k_pe bf16
+ * [T, rope_dim]; token j of sequence i goes to position kv_len_i - q_len_i + j.
+ */
+int rpa_mla_kv_write(const RpaMlaParams* p, const void* new_kv_c, const void* new_k_pe, void* stream);
 
 #ifdef __cplusplus
 }

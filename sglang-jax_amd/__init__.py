@@ -5,7 +5,13 @@ importable name ``sglang_jax_amd`` by ``__graft_entry__.load_package()``.
 """
 
 from . import _lib  # noqa: F401
-from .backend import FlashAttention, FlashAttentionMetadata, ForwardMode, build_forward_metadata  # noqa: F401
+from .backend import (  # noqa: F401
+    FlashAttention,
+    FlashAttentionMetadata,
+    ForwardMode,
+    MLAAttentionBackend,
+    build_forward_metadata,
+)
 from .mla import mla_ragged_paged_attention  # noqa: F401
 from .ragged_paged_attention import (  # noqa: F401
     DEFAULT_MASK_VALUE,
@@ -18,6 +24,7 @@ __all__ = [
     "FlashAttention",
     "FlashAttentionMetadata",
     "ForwardMode",
+    "MLAAttentionBackend",
     "build_forward_metadata",
     "DEFAULT_MASK_VALUE",
     "gather_pages",

@@ -47,6 +47,9 @@ EXPORTED_SYMBOLS = (
     "rpa_attention",
     "rpa_kv_write",
     "rpa_mla_decode",
+    "rpa_mla_attention_workspace_bytes",
+    "rpa_mla_attention",
+    "rpa_mla_kv_write",
 )
 
 
@@ -170,6 +173,12 @@ def load() -> ctypes.CDLL:
     lib.rpa_kv_write.argtypes = [P(RpaParams), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     lib.rpa_mla_decode.restype = ctypes.c_int
     lib.rpa_mla_decode.argtypes = [P(RpaMlaParams), ctypes.c_void_p]
+    lib.rpa_mla_attention_workspace_bytes.restype = ctypes.c_size_t
+    lib.rpa_mla_attention_workspace_bytes.argtypes = [P(RpaMlaParams)]
+    lib.rpa_mla_attention.restype = ctypes.c_int
+    lib.rpa_mla_attention.argtypes = [P(RpaMlaParams), ctypes.c_void_p]
+    lib.rpa_mla_kv_write.restype = ctypes.c_int
+    lib.rpa_mla_kv_write.argtypes = [P(RpaMlaParams), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     _lib = lib
     return lib
 

@@ -27,6 +27,7 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 
+from .mla import mla_ragged_paged_attention
 from .ragged_paged_attention import ragged_paged_attention
 
 
@@ -56,6 +57,7 @@ def build_forward_metadata(
     dp_size: int = 1,
     per_dp_bs_size: int | None = None,
     swa_index_mapping=None,
+    extend_distribution_is_mixed: bool = False,
 ) -> dict:
     """Host arithmetic of ``FlashAttention.get_forward_metadata``
     (flashattention_backend.py:146-237), as numpy int32 arrays:
@@ -64,7 +66,9 @@ def build_forward_metadata(
     cumulative extend lengths, each section starting at 0; ``cu_kv_lens`` = cumulative
     page-aligned sequence lengths; ``distribution`` = (n, n, n) for decode and (0, n, n) for
     extend with n = number of sequences of non-zero length; the sliding-window pool's page
-    ids through ``swa_index_mapping`` when one is given.
+    ids through ``swa_index_mapping`` when one is given.  The MLA backend builds the same
+    arrays but declares an extend batch as (0, 0, n) (mla_backend.py:192-199):
+    ``extend_distribution_is_mixed``.
     """
     seq_lens = np.asarray(seq_lens, dtype=np.int32)
     cache_loc = np.asarray(cache_loc, dtype=np.int32)
@@ -118,7 +122,8 @@ def build_forward_metadata(
     if mode == "DECODE":
         distribution = np.repeat(n, 3).astype(np.int32)
     else:
-        distribution = np.column_stack([np.zeros_like(n), n, n]).ravel().astype(np.int32)
+        mid = np.zeros_like(n) if extend_distribution_is_mixed else n
+        distribution = np.column_stack([np.zeros_like(n), mid, n]).ravel().astype(np.int32)
 
     return {
         "cu_q_lens": cu_q_lens,
@@ -145,6 +150,7 @@ class FlashAttentionMetadata:
     host_distribution: np.ndarray | None = None
     max_kv_len: int = 0
     max_q_len: int = 0
+    sum_visible: int = 0
     host_seq_lens: np.ndarray | None = field(default=None, repr=False)
 
 
@@ -248,3 +254,79 @@ class FlashAttention:
             f"max running requests: {res} must larger than 0, please increase page size or decrease max context length"
         )
         return res
+
+
+class MLAAttentionBackend:
+    """One-GPU counterpart of the reference's absorbed-MLA backend
+    (python/sgl_jax/srt/layers/attention/mla_backend.py:83-389): same metadata as the MHA
+    backend except that an extend batch is declared (0, 0, n), and a layer call that takes
+    the absorbed latent query, the new latent row and the two rope parts."""
+
+    def __init__(self, num_attn_heads: int, kv_lora_rank: int, qk_nope_head_dim: int, qk_rope_head_dim: int,
+                 v_head_dim: int, page_size: int = 1, device=None):
+        assert page_size > 1, "MLA attention backend does not support page_size=1."
+        self.num_heads = num_attn_heads
+        self.kv_lora_rank = kv_lora_rank
+        self.qk_nope_head_dim = qk_nope_head_dim
+        self.qk_rope_head_dim = qk_rope_head_dim
+        self.v_head_dim = v_head_dim
+        self.page_size = page_size
+        self.device = torch.device(device) if device is not None else torch.device("cuda:0")
+        self.forward_metadata = FlashAttentionMetadata()
+
+    def get_forward_metadata(self, batch) -> FlashAttentionMetadata:
+        if getattr(batch, "dp_size", 1) != 1:
+            raise NotImplementedError("one GPU: data-parallel sections (dp_size > 1) are not built")
+        host = build_forward_metadata(
+            forward_mode=batch.forward_mode,
+            seq_lens=batch.seq_lens,
+            cache_loc=batch.cache_loc,
+            extend_seq_lens=getattr(batch, "extend_seq_lens", None),
+            page_size=self.page_size,
+            dp_size=1,
+            per_dp_bs_size=getattr(batch, "per_dp_bs_size", None) or len(batch.seq_lens),
+            extend_distribution_is_mixed=True,
+        )
+        md = FlashAttentionMetadata()
+        for name in ("cu_q_lens", "cu_kv_lens", "page_indices", "seq_lens", "distribution"):
+            setattr(md, name, torch.from_numpy(np.ascontiguousarray(host[name])).to(self.device, non_blocking=True))
+        md.host_distribution = host["distribution"]
+        md.host_seq_lens = host["seq_lens"]
+        md.max_kv_len = int(host["seq_lens"].max()) if len(host["seq_lens"]) else 0
+        q_lens = np.diff(host["cu_q_lens"])
+        md.max_q_len = int(q_lens.max()) if len(q_lens) else 0
+        # work of one row per query token: token j of a chunk sees kv_len - q_len + j + 1 tokens
+        n = int(host["distribution"][2])
+        kv, ql = host["seq_lens"][:n].astype(np.int64), q_lens[:n].astype(np.int64)
+        md.sum_visible = int((ql * kv - ql * (ql - 1) // 2).sum())
+        return md
+
+    def __call__(self, q, k, v, layer, forward_batch, token_to_kv_pool, **kwargs):
+        """q: ``[T, n_h, kv_lora_rank]`` (absorbed latent query), k: ``[T, 1, kv_lora_rank]`` or
+        ``[T, kv_lora_rank]`` (new latent row; v is the same tensor), ``q_rope`` / ``k_rope``
+        keyword arguments: the rope parts.  Returns ``(o_latent [T, n_h, kv_lora_rank], cache)``."""
+        del v
+        q_rope, k_rope = kwargs.get("q_rope"), kwargs.get("k_rope")
+        if q_rope is None or k_rope is None:
+            raise ValueError(
+                "MLAAttentionBackend requires q_rope/k_rope kwargs (q_pe/k_pe) "
+                "alongside the non-rope q/k tensors."
+            )
+        md = self.forward_metadata
+        if md.page_indices is None:
+            raise ValueError("forward_metadata is not set: call get_forward_metadata(batch) first")
+        new_kv_c = k if k.dim() == 2 else k.squeeze(1)
+        new_k_pe = k_rope if k_rope.dim() == 2 else k_rope.squeeze(1)
+        cache = token_to_kv_pool.get_fused_kv_buffer(layer.layer_id)
+        scaling = getattr(layer, "scaling", None)
+        sm_scale = float(scaling) if scaling is not None else 1.0 / float(
+            np.sqrt(self.qk_nope_head_dim + self.qk_rope_head_dim))
+        return mla_ragged_paged_attention(
+            q, q_rope, new_kv_c, new_k_pe, cache, md.seq_lens, md.page_indices, md.cu_q_lens, md.cu_kv_lens,
+            md.host_distribution,
+            sm_scale=sm_scale,
+            sliding_window=getattr(layer, "sliding_window_size", None) or None,
+            soft_cap=getattr(layer, "logit_cap", None) or None,
+            max_kv_len=md.max_kv_len,
+            sum_kv_len=getattr(md, "sum_visible", 0),
+        )

@@ -374,13 +374,13 @@ int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void*
 
 // ---------------------------------------------------------------- MLA ----
 
-static SplitPlan mla_plan(const RpaMlaParams* p) {
+static SplitPlan mla_plan(const RpaMlaParams* p, int64_t rows) {
   const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                      p->cu_kv_lens != nullptr);
   // one 8-wave workgroup per (row, split, 128 heads) and per CU; every split costs a 256 KiB
   // partial write per 128 heads, so splits are kept as few as fill the CUs once
   const int64_t groups = (p->num_q_heads + 127) / 128;
-  const int64_t units = (int64_t)p->num_seqs * groups;
+  const int64_t units = rows * groups;
   int64_t work = p->sum_kv_len > 0 ? p->sum_kv_len * groups : 0;
   if (p->sliding_window > 0) work = 0;
   return plan_splits(bound, p->sliding_window, units, work, p->num_splits,
@@ -398,7 +398,6 @@ static int mla_validate(const RpaMlaParams* p) {
     return fail(RPA_EINVAL_SHAPE, "row_stride=%d rope_offset=%d do not describe [kv_c | k_pe]", p->row_stride, p->rope_offset);
   if (p->num_q_heads % 16 != 0) return fail(RPA_EUNSUPPORTED, "num_q_heads=%d must be a multiple of 16", p->num_q_heads);
   if (p->sliding_window < 0) return fail(RPA_EINVAL_WINDOW, "sliding_window=%d must be positive", p->sliding_window);
-  if (p->num_seqs > p->num_tokens) return fail(RPA_EINVAL_SHAPE, "decode rows=%d exceed tokens=%d", p->num_seqs, p->num_tokens);
   if (p->num_seqs > 0 && (!p->ql_nope || !p->q_pe || !p->out || !p->cache_kv || !p->kv_lens || !p->page_indices || !p->cu_q_lens))
     return fail(RPA_EINVAL_NULL, "a required buffer is NULL");
   if (!p->cu_kv_lens && p->pages_per_seq <= 0 && p->num_seqs > 0)
@@ -406,18 +405,26 @@ static int mla_validate(const RpaMlaParams* p) {
   return RPA_OK;
 }
 
-size_t rpa_mla_workspace_bytes(const RpaMlaParams* p) {
-  if (!p || p->num_seqs <= 0) return 0;
-  const SplitPlan sp = mla_plan(p);
+static size_t mla_workspace(const RpaMlaParams* p, int64_t rows) {
+  if (!p || p->num_seqs <= 0 || rows <= 0) return 0;
+  const SplitPlan sp = mla_plan(p, rows);
   if (sp.splits <= 1) return 0;
-  return (size_t)p->num_seqs * sp.splits * p->num_q_heads * (p->lkv_dim + 2) * sizeof(float);
+  return (size_t)rows * sp.splits * p->num_q_heads * (p->lkv_dim + 2) * sizeof(float);
 }
 
-int rpa_mla_decode(const RpaMlaParams* p, void* stream) {
+size_t rpa_mla_workspace_bytes(const RpaMlaParams* p) { return mla_workspace(p, p ? p->num_seqs : 0); }
+
+size_t rpa_mla_attention_workspace_bytes(const RpaMlaParams* p) { return mla_workspace(p, p ? p->num_tokens : 0); }
+
+static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   int rc = mla_validate(p);
   if (rc != RPA_OK) return rc;
   if (p->num_seqs <= 0) return RPA_OK;
-  const SplitPlan sp = mla_plan(p);
+  if (!token_rows && p->num_seqs > p->num_tokens)
+    return fail(RPA_EINVAL_SHAPE, "decode rows=%d exceed tokens=%d", p->num_seqs, p->num_tokens);
+  const int64_t rows = token_rows ? p->num_tokens : p->num_seqs;
+  if (rows <= 0) return RPA_OK;
+  const SplitPlan sp = mla_plan(p, rows);
   rpa::MlaDecodeArgs a;
   a.ql_nope = static_cast<const uint16_t*>(p->ql_nope);
   a.q_pe = static_cast<const uint16_t*>(p->q_pe);
@@ -430,7 +437,9 @@ int rpa_mla_decode(const RpaMlaParams* p, void* stream) {
   a.pt.pages_per_seq = p->pages_per_seq;
   a.pt.page_size = p->page_size;
   a.sm = softmax_opts(p->sm_scale, p->soft_cap, p->mask_value, p->sliding_window);
-  a.num_rows = p->num_seqs;
+  a.num_rows = (int32_t)rows;
+  a.num_seqs = p->num_seqs;
+  a.rows_are_tokens = token_rows ? 1 : 0;
   a.Hq = p->num_q_heads;
   a.row_stride = p->row_stride;
   a.rope_offset = p->rope_offset;
@@ -439,13 +448,40 @@ int rpa_mla_decode(const RpaMlaParams* p, void* stream) {
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
   if (sp.splits > 1) {
-    const size_t need = rpa_mla_workspace_bytes(p);
+    const size_t need = mla_workspace(p, rows);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
     a.ws_o = static_cast<float*>(p->workspace);
-    a.ws_ml = a.ws_o + (size_t)p->num_seqs * sp.splits * p->num_q_heads * p->lkv_dim;
+    a.ws_ml = a.ws_o + (size_t)rows * sp.splits * p->num_q_heads * p->lkv_dim;
   }
-  return check_hip(rpa::launch_mla_decode(a, static_cast<hipStream_t>(stream)), "rpa_mla_decode");
+  return check_hip(rpa::launch_mla_decode(a, static_cast<hipStream_t>(stream)),
+                   token_rows ? "rpa_mla_attention" : "rpa_mla_decode");
+}
+
+int rpa_mla_decode(const RpaMlaParams* p, void* stream) { return mla_run(p, stream, false); }
+
+int rpa_mla_attention(const RpaMlaParams* p, void* stream) { return mla_run(p, stream, true); }
+
+int rpa_mla_kv_write(const RpaMlaParams* p, const void* new_kv_c, const void* new_k_pe, void* stream) {
+  int rc = mla_validate(p);
+  if (rc != RPA_OK) return rc;
+  if (!new_kv_c || !new_k_pe) return fail(RPA_EINVAL_NULL, "new_kv_c/new_k_pe is NULL");
+  if (p->num_seqs <= 0 || p->num_tokens <= 0) return RPA_OK;
+  rpa::MlaWriteArgs a;
+  a.cache = static_cast<char*>(const_cast<void*>(p->cache_kv));
+  a.pt.kv_lens = p->kv_lens;
+  a.pt.page_indices = p->page_indices;
+  a.pt.cu_q_lens = p->cu_q_lens;
+  a.pt.cu_kv_lens = p->cu_kv_lens;
+  a.pt.pages_per_seq = p->pages_per_seq;
+  a.pt.page_size = p->page_size;
+  a.new_kv_c = static_cast<const uint16_t*>(new_kv_c);
+  a.new_k_pe = static_cast<const uint16_t*>(new_k_pe);
+  a.num_tokens = p->num_tokens;
+  a.num_seqs = p->num_seqs;
+  a.row_stride = p->row_stride;
+  a.rope_offset = p->rope_offset;
+  return check_hip(rpa::launch_mla_kv_write(a, static_cast<hipStream_t>(stream)), "rpa_mla_kv_write");
 }
 
 }  // extern "C"

@@ -104,7 +104,9 @@ struct MlaDecodeArgs {
   SoftmaxOpts sm;
   float* ws_o;   // [T, max_splits, Hq, lkv]
   float* ws_ml;  // [T, max_splits, Hq, 2]
-  int32_t num_rows;
+  int32_t num_rows;     // grid rows: sequences (rows_are_tokens == 0) or query tokens
+  int32_t num_seqs;
+  int32_t rows_are_tokens;  // 1: row r is query token r of whatever sequence owns it (any q_len)
   int32_t Hq;
   int32_t row_stride;   // elements
   int32_t rope_offset;  // elements
@@ -112,10 +114,22 @@ struct MlaDecodeArgs {
   int32_t max_splits;
 };
 
+struct MlaWriteArgs {
+  char* cache;              // [pages, P, row_stride] bf16
+  PageTable pt;
+  const uint16_t* new_kv_c;  // [T, 512]
+  const uint16_t* new_k_pe;  // [T, 64]
+  int32_t num_tokens;
+  int32_t num_seqs;
+  int32_t row_stride;
+  int32_t rope_offset;
+};
+
 hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream);
 hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream);
 hipError_t launch_gather(const GatherArgs& a, hipStream_t stream);
 hipError_t launch_kv_write(const KvWriteArgs& a, hipStream_t stream);
 hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream);
+hipError_t launch_mla_kv_write(const MlaWriteArgs& a, hipStream_t stream);
 
 }  // namespace rpa

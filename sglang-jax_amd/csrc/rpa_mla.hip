@@ -107,6 +107,49 @@ __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* 
   }
 }
 
+// Sequence that owns query token `row`: the last one whose first token is <= row
+// (zero-length sequences are skipped).  cu_q_lens[0 .. num_seqs] is non-decreasing.
+__device__ __forceinline__ int owner_of_token(const int32_t* cu_q_lens, int num_seqs, int row) {
+  int lo = 0, hi = num_seqs;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (scalar_load_i32(cu_q_lens + mid) <= row) lo = mid;
+    else hi = mid;
+  }
+  return lo;
+}
+
+// What a grid row attends to.  Sequence rows (decode batches): the one query of sequence `row`
+// sees all kv_len tokens.  Token rows: query token `row` of a sequence with q_len new tokens
+// sits at position kv_len - q_len + j and sees the tokens up to itself -- an absorbed-MLA
+// prefill row is a decode row over a shorter prefix (mla/v1/ref.py:229-233).
+struct MlaRow {
+  int seq, kv_len, tq;
+  bool valid;
+};
+
+__device__ __forceinline__ MlaRow mla_row(const MlaDecodeArgs& a, int row) {
+  MlaRow r;
+  r.valid = true;
+  if (a.rows_are_tokens) {
+    if (row >= scalar_load_i32(a.pt.cu_q_lens + a.num_seqs)) {
+      r.valid = false;
+      r.seq = r.kv_len = r.tq = 0;
+      return r;
+    }
+    r.seq = owner_of_token(a.pt.cu_q_lens, a.num_seqs, row);
+    const int q0 = scalar_load_i32(a.pt.cu_q_lens + r.seq);
+    const int q_len = scalar_load_i32(a.pt.cu_q_lens + r.seq + 1) - q0;
+    r.kv_len = scalar_load_i32(a.pt.kv_lens + r.seq) - q_len + (row - q0) + 1;
+    r.tq = row;
+  } else {
+    r.seq = row;
+    r.kv_len = a.pt.kv_lens[row];
+    r.tq = a.pt.cu_q_lens[row];
+  }
+  return r;
+}
+
 // grid = (max_splits, rows, head groups of 128); block = 512 threads.
 template <bool UNIFORM, bool CAP>
 __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeArgs a) {
@@ -120,11 +163,15 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, g = lane >> 4;
-  const int seq = blockIdx.y, split = blockIdx.x;
+  const int row_id = blockIdx.y, split = blockIdx.x;
   const int head0 = blockIdx.z * 128 + wave * 16;
   const bool wave_on = head0 < a.Hq;
 
-  const int kv_len = a.pt.kv_lens[seq];
+  const MlaRow mr = mla_row(a, row_id);
+  if (!mr.valid) return;
+  const int seq = mr.seq;
+  const int kv_len = mr.kv_len;
+  if (kv_len <= 0) return;
   const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
   const int t0 = t_lo & ~(kTok - 1);
   const int t_begin = t0 + split * a.chunk;
@@ -150,7 +197,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   };
 
   // ---- Q^T operands of this wave: column c = head head0 + c, k-step ks covers dims 32ks + 8g .. ----
-  const int tq = a.pt.cu_q_lens[seq];
+  const int tq = mr.tq;
   u32x4_t qB[18];
   {
     const int head = min(head0 + c, a.Hq - 1);
@@ -288,7 +335,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
       *reinterpret_cast<u32x2_t*>(op + j * 16) = w;
     }
   } else {
-    const int64_t slot = ((int64_t)seq * a.max_splits + split) * a.Hq + head;
+    const int64_t slot = ((int64_t)row_id * a.max_splits + split) * a.Hq + head;
     float* wo = a.ws_o + slot * 512 + g * 4;
 #pragma unroll
     for (int j = 0; j < 32; ++j) *reinterpret_cast<f32x4_t*>(wo + j * 16) = acc[j];
@@ -301,13 +348,15 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
 
 // grid = (Hq, rows); block = 128 threads, 4 dims each.
 __global__ __launch_bounds__(128) void rpa_mla_combine_kernel(const MlaDecodeArgs a) {
-  const int head = blockIdx.x, seq = blockIdx.y;
-  const int kv_len = a.pt.kv_lens[seq];
+  const int head = blockIdx.x, row_id = blockIdx.y;
+  const MlaRow mr = mla_row(a, row_id);
+  if (!mr.valid || mr.kv_len <= 0) return;
+  const int kv_len = mr.kv_len;
   const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
   const int t0 = t_lo & ~(kTok - 1);
   const int n = min(a.max_splits, (kv_len - t0 + a.chunk - 1) / a.chunk);
   if (n <= 0) return;
-  const int64_t base = ((int64_t)seq * a.max_splits) * a.Hq + head;
+  const int64_t base = ((int64_t)row_id * a.max_splits) * a.Hq + head;
   float mstar = -INFINITY;
   for (int j = 0; j < n; ++j) mstar = fmaxf(mstar, a.ws_ml[(base + (int64_t)j * a.Hq) * 2]);
   float den = 0.f;
@@ -320,12 +369,39 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_kernel(const MlaDecodeArg
     o += *reinterpret_cast<const f32x4_t*>(a.ws_o + slot * 512 + d) * w;
   }
   const float inv = 1.0f / den;
-  const int tq = a.pt.cu_q_lens[seq];
+  const int tq = mr.tq;
   u32x2_t w = {pack_bf16x2(o[0] * inv, o[1] * inv), pack_bf16x2(o[2] * inv, o[3] * inv)};
   *reinterpret_cast<u32x2_t*>(a.out + ((int64_t)tq * a.Hq + head) * 512 + d) = w;
 }
 
+// New latent rows into the paged cache (mla/v1/ref.py:56-105): token j of sequence i goes to
+// position kv_len_i - q_len_i + j; kv_c to elements [0, 512), k_pe to [rope_offset, +64).
+// grid = tokens; block = 128 threads of which 72 move 16 bytes each.
+__global__ __launch_bounds__(128) void rpa_mla_kv_write_kernel(const MlaWriteArgs a) {
+  const int tok = blockIdx.x;
+  if (tok >= scalar_load_i32(a.pt.cu_q_lens + a.num_seqs)) return;
+  const int seq = owner_of_token(a.pt.cu_q_lens, a.num_seqs, tok);
+  const int q0 = scalar_load_i32(a.pt.cu_q_lens + seq);
+  const int q_len = scalar_load_i32(a.pt.cu_q_lens + seq + 1) - q0;
+  const int pos = scalar_load_i32(a.pt.kv_lens + seq) - q_len + (tok - q0);
+  if (pos < 0) return;
+  const int P = a.pt.page_size;
+  const int32_t* pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[seq] / P)
+                                                              : (int64_t)seq * a.pt.pages_per_seq);
+  const int page = pages[pos / P];
+  char* row = a.cache + ((int64_t)page * P + (pos % P)) * a.row_stride * 2;
+  const int t = threadIdx.x;
+  if (t < 64) st16(row + t * 16, ld16(a.new_kv_c + (int64_t)tok * 512 + t * 8));
+  else if (t < 72) st16(row + a.rope_offset * 2 + (t - 64) * 16, ld16(a.new_k_pe + (int64_t)tok * 64 + (t - 64) * 8));
+}
+
 }  // namespace
+
+hipError_t launch_mla_kv_write(const MlaWriteArgs& a, hipStream_t stream) {
+  if (a.num_tokens <= 0 || a.num_seqs <= 0) return hipSuccess;
+  hipLaunchKernelGGL(rpa_mla_kv_write_kernel, dim3(a.num_tokens), dim3(128), 0, stream, a);
+  return hipGetLastError();
+}
 
 hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   if (a.num_rows <= 0) return hipSuccess;

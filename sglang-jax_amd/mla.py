@@ -1,6 +1,8 @@
 """Host-side mirror of the reference's absorbed-MLA ragged paged attention
 (``mla_ragged_paged_attention``, python/sgl_jax/srt/kernels/mla/v2/kernel.py:1338-1370)
-for decode rows, on the HIP kernels behind ``rpa_mla_decode`` (include/rpa.h).
+on the HIP kernels behind ``rpa_mla_kv_write`` / ``rpa_mla_decode`` / ``rpa_mla_attention``
+(include/rpa.h): new latent rows are written into the cache, then every query token attends to
+the cache up to its own position.
 
 The latent cache may be the compact ``[pages, P, lkv+rope]`` (576-wide rows) or
 the reference's 128-aligned ``[pages, P, 512+128]`` (kernel.py:74-86; also its
@@ -48,11 +50,11 @@ def mla_ragged_paged_attention(
     num_splits: int = 0,
     sum_kv_len: int | None = None,
 ):
-    """Returns (output [max_num_tokens, num_q_heads, lkv_dim], cache_kv).
+    """Returns (output [max_num_tokens, num_q_heads, lkv_dim], cache_kv updated in place).
 
-    Only decode batches are built (every sequence contributes one query token,
-    ``distribution = (n, n, n)``); the fused write of ``new_kv_c/new_k_pe`` is not
-    built either, so the cache must already hold all ``kv_len`` tokens."""
+    ``new_kv_c`` / ``new_k_pe`` may be None when the cache already holds all ``kv_len``
+    tokens.  A decode batch (``distribution = (n, n, n)``) takes the one-row-per-sequence
+    entry point; anything else (prefill chunks, mixed) runs one row per query token."""
     _require_gpu(ql_nope, "ql_nope")
     _require_gpu(cache_kv, "cache_kv")
     if ql_nope.dim() != 3:
@@ -65,14 +67,15 @@ def mla_ragged_paged_attention(
         raise ValueError(f"sliding_window={sliding_window} must be positive.")
     if soft_cap is not None and soft_cap == 0.0:
         raise ValueError(f"soft_cap={soft_cap} must not be 0.0.")
-    if new_kv_c is not None or new_k_pe is not None:
-        raise NotImplementedError("fused latent cache write is not built: pass new_kv_c=None with a complete cache")
+    if (new_kv_c is None) != (new_k_pe is None):
+        raise ValueError("new_kv_c and new_k_pe must be given together")
     if q_scale is not None or k_scale is not None or v_scale is not None:
         raise NotImplementedError("q_scale/k_scale/v_scale are not built for MLA")
     dist = np.asarray(distribution.cpu() if isinstance(distribution, torch.Tensor) else distribution)
     i, j, k = (int(x) for x in dist)
-    if not (i == j == k):
-        raise NotImplementedError(f"only decode batches are built, got distribution=({i}, {j}, {k})")
+    if not (0 <= i <= j <= k):
+        raise ValueError(f"distribution must satisfy 0 <= i <= j <= k, got ({i}, {j}, {k})")
+    decode_only = i == j == k
     device = ql_nope.device
     if cache_kv.dim() == 4:
         s = cache_kv.shape
@@ -120,11 +123,20 @@ def mla_ragged_paged_attention(
     p.soft_cap = float(soft_cap) if soft_cap else 0.0
     p.mask_value = float(mask_value) if mask_value is not None else DEFAULT_MASK_VALUE
     lib = _lib.load()
-    need = lib.rpa_mla_workspace_bytes(ctypes.byref(p))
+    stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    if new_kv_c is not None:
+        _require_gpu(new_kv_c, "new_kv_c")
+        if new_kv_c.shape != (T, lkv) or new_k_pe.shape != (T, rope):
+            raise ValueError(f"Expected new_kv_c {(T, lkv)} and new_k_pe {(T, rope)}, got "
+                             f"{tuple(new_kv_c.shape)} and {tuple(new_k_pe.shape)}")
+        if not (new_kv_c.dtype == new_k_pe.dtype == cache_kv.dtype):
+            raise ValueError("new_kv_c / new_k_pe must have the cache dtype")
+        nk, nr = new_kv_c.contiguous(), new_k_pe.contiguous()
+        _lib.check(lib.rpa_mla_kv_write(ctypes.byref(p), nk.data_ptr(), nr.data_ptr(), stream))
+    need = (lib.rpa_mla_workspace_bytes if decode_only else lib.rpa_mla_attention_workspace_bytes)(ctypes.byref(p))
     if need:
         ws = _workspace(device, need)
         p.workspace = ws.data_ptr()
         p.workspace_bytes = ws.numel()
-    stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
-    _lib.check(lib.rpa_mla_decode(ctypes.byref(p), stream))
+    _lib.check((lib.rpa_mla_decode if decode_only else lib.rpa_mla_attention)(ctypes.byref(p), stream))
     return out, cache_kv

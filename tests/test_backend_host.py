@@ -105,3 +105,15 @@ def test_max_running_requests(pkg):
     assert pkg.FlashAttention.get_max_running_reqests(4096, 64) == 1024 * 1024 // 2 // 64 // 4
     with pytest.raises(AssertionError):
         pkg.FlashAttention.get_max_running_reqests(1 << 30, 1)
+
+
+def test_mla_extend_distribution(pkg):
+    """mla_backend.py:192-199: an extend batch is declared (0, 0, n)."""
+    md = pkg.build_forward_metadata(forward_mode="EXTEND", seq_lens=np.array([5, 8, 0], dtype=np.int32),
+                                    cache_loc=np.arange(16, dtype=np.int32), extend_seq_lens=np.array([2, 8, 0]),
+                                    page_size=4, extend_distribution_is_mixed=True)
+    assert md["distribution"].tolist() == [0, 0, 2]
+    md = pkg.build_forward_metadata(forward_mode="DECODE", seq_lens=np.array([5, 8, 0], dtype=np.int32),
+                                    cache_loc=np.arange(16, dtype=np.int32), page_size=4,
+                                    extend_distribution_is_mixed=True)
+    assert md["distribution"].tolist() == [2, 2, 2]

@@ -116,3 +116,59 @@ def test_extend_then_decode_steps(pkg, gpu, P, window, cap):
         assert backend.forward_metadata.host_distribution.tolist() == [3, 3, 3]
     say("chunked extend on top of the existing prefix")
     run_step(pkg.ForwardMode.EXTEND, [9, 4, 33, 0])
+
+
+def test_mla_backend_extend_then_decode(pkg, gpu):
+    """MLAAttentionBackend (mla_backend.py:83-389): prompt, then decode steps, on the
+    reference's 640-wide latent rows; output and cache against the CPU oracle."""
+    from oracle.ref_mla import ref_mla_ragged_paged_attention
+
+    Hq, P, pool_pages, W = 16, 16, 48, 640
+    rng = np.random.default_rng(17)
+    gen = torch.Generator().manual_seed(19)
+    host_cache = torch.zeros(pool_pages, P, W, dtype=torch.bfloat16)
+    pool = SimpleNamespace(buf=host_cache.to(gpu))
+    pool.get_fused_kv_buffer = lambda layer_id: pool.buf
+    backend = pkg.MLAAttentionBackend(Hq, 512, 128, 64, 128, page_size=P, device=gpu)
+    layer = SimpleNamespace(layer_id=0, scaling=None, sliding_window_size=None, logit_cap=None)
+    free = list(rng.permutation(pool_pages))
+    bs = 3
+    pages = [[] for _ in range(bs)]
+    seq_lens = np.zeros(bs, dtype=np.int32)
+
+    def step(mode, new_lens):
+        nonlocal seq_lens, host_cache
+        new_lens = np.asarray(new_lens, dtype=np.int32)
+        seq_lens = seq_lens + new_lens
+        for i in range(bs):
+            while len(pages[i]) * P < seq_lens[i]:
+                pages[i].append(int(free.pop()))
+        cache_loc = np.concatenate([np.arange(p * P, p * P + P) for ps in pages for p in ps]).astype(np.int32)
+        batch = SimpleNamespace(forward_mode=mode, seq_lens=seq_lens.copy(), cache_loc=cache_loc,
+                                extend_seq_lens=new_lens, dp_size=1, per_dp_bs_size=bs)
+        backend.forward_metadata = backend.get_forward_metadata(batch)
+        T = int(new_lens.sum())
+        q = (torch.randn(T, Hq, 512, generator=gen) * 0.5).to(torch.bfloat16)
+        qr = (torch.randn(T, Hq, 64, generator=gen) * 0.5).to(torch.bfloat16)
+        kc = (torch.randn(T, 1, 512, generator=gen) * 0.5).to(torch.bfloat16)
+        kr = (torch.randn(T, 1, 64, generator=gen) * 0.5).to(torch.bfloat16)
+        out, cache = backend(q.to(gpu), kc.to(gpu), kc.to(gpu), layer, batch, pool, q_rope=qr.to(gpu), k_rope=kr.to(gpu))
+        torch.cuda.synchronize()
+        width = max(len(p) for p in pages)
+        table = np.zeros((bs, width), dtype=np.int32)
+        for i, ps in enumerate(pages):
+            table[i, :len(ps)] = ps
+        cu_q = np.concatenate([[0], np.cumsum(new_lens)]).astype(np.int32)
+        want, host_cache = ref_mla_ragged_paged_attention(
+            q, qr, kc[:, 0], kr[:, 0], host_cache, torch.from_numpy(seq_lens.copy()),
+            torch.from_numpy(table.reshape(-1)), torch.from_numpy(cu_q), [0, 0, bs],
+            sm_scale=1.0 / np.sqrt(192.0), layout="padded")
+        assert torch.equal(cache.cpu().view(torch.int16), host_cache.view(torch.int16))
+        torch.testing.assert_close(out.cpu().float(), want.float(), **TOL)
+
+    say("mla extend")
+    step(pkg.ForwardMode.EXTEND, [37, 70, 5])
+    assert backend.forward_metadata.host_distribution.tolist() == [0, 0, 3]
+    for s_ in range(2):
+        say(f"mla decode {s_}")
+        step(pkg.ForwardMode.DECODE, [1, 1, 1])

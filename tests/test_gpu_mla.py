@@ -106,3 +106,77 @@ def test_c5_scaled_against_oracle(pkg, wl, gpu):
     b = wl.config_c5(scale=0.06)
     got = run_gpu(pkg, b, gpu)
     torch.testing.assert_close(got.float(), oracle(b).float(), **TOL)
+
+
+# ------------------------------------------------------------------ prefill / mixed rows, fused latent write
+@pytest.mark.parametrize("P,window,cap", [(16, None, None), (64, None, None), (64, 128, 30.0)])
+def test_mla_prefill_and_mixed_rows(pkg, wl, gpu, P, window, cap):
+    """Decode rows, chunks with a prefix and whole prompts in one batch
+    (kernels/mla/v2/kernel.py:1338-1744 runs them as three launches)."""
+    q_lens = [1, 1, 5, 64, 33, 130]
+    kv_lens = [77, 1, 5, 300, 33, 131]
+    say(f"mla mixed P={P} window={window} cap={cap} q={q_lens} kv={kv_lens}")
+    b = wl.make_mla_batch("mla_mixed", q_lens, kv_lens, num_q_heads=16, lkv_dim=512, rope_dim=64, page_size=P,
+                          seed=81, sliding_window=window, soft_cap=cap)
+    want = oracle(b)
+    got = run_gpu(pkg, b, gpu)
+    T = sum(q_lens)
+    assert torch.isfinite(got[:T].float()).all()
+    torch.testing.assert_close(got[:T].float(), want.float(), **TOL)
+    # any split count gives the same rows
+    got4 = run_gpu(pkg, b, gpu, num_splits=3)
+    torch.testing.assert_close(got4[:T].float(), got[:T].float(), rtol=1e-2, atol=1e-2)
+
+
+def test_mla_token_rows_equal_sequence_rows_on_a_decode_batch(pkg, wl, gpu):
+    kv_lens = [40, 1000, 257, 64]
+    b = wl.make_mla_batch("mla_dec", [1] * 4, kv_lens, num_q_heads=32, lkv_dim=512, rope_dim=64, page_size=64, seed=82)
+    seq_rows = run_gpu(pkg, b, gpu)
+    # the same batch declared as "mixed" takes the one-row-per-token entry point
+    g = b.to(gpu)
+    out, _ = pkg.mla_ragged_paged_attention(
+        g.ql_nope, g.q_pe, None, None, g.cache_kv, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+        [0, 0, 4], sm_scale=b.sm_scale, max_kv_len=1000)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), seq_rows)
+
+
+@pytest.mark.parametrize("padded", [False, True])
+def test_mla_new_rows_are_written_into_the_cache(pkg, wl, gpu, padded):
+    """The cache holds kv_len - q_len rows, new_kv_c / new_k_pe bring the rest
+    (kernels/mla/v1/ref.py:56-105): cache bit for bit, output within tolerance."""
+    q_lens, kv_lens, P = [1, 1, 20, 65], [64, 200, 20, 300], 16
+    b = wl.make_mla_batch("mla_write", q_lens, kv_lens, num_q_heads=16, lkv_dim=512, rope_dim=64, page_size=P, seed=83)
+    say(f"mla write padded={padded}")
+    cache = b.cache_kv
+    if padded:  # the reference's 128-aligned rows: [kv_c 512 | k_pe 64 | 64 unused]
+        wide = torch.zeros(cache.shape[0], P, 640, dtype=cache.dtype)
+        wide[..., :576] = cache
+        cache = wide
+    table = b.padded_page_indices().view(len(q_lens), -1)
+    T = sum(q_lens)
+    new_c = torch.empty(T, 512, dtype=torch.bfloat16)
+    new_r = torch.empty(T, 64, dtype=torch.bfloat16)
+    holed = cache.clone()
+    t = 0
+    for i, (ql, kv) in enumerate(zip(q_lens, kv_lens)):
+        for j in range(ql):
+            pos = kv - ql + j
+            page, row = int(table[i, pos // P]), pos % P
+            new_c[t], new_r[t] = cache[page, row, :512], cache[page, row, 512:576]
+            holed[page, row] = float("nan")
+            if padded:
+                holed[page, row, 576:] = 0
+            t += 1
+    n = len(q_lens)
+    want, want_cache = ref_mla_ragged_paged_attention(
+        b.ql_nope, b.q_pe, new_c, new_r, holed, b.kv_lens, b.padded_page_indices(), b.cu_q_lens, [0, 0, n],
+        sm_scale=b.sm_scale, layout="padded" if padded else "compact")
+    assert torch.equal(want_cache.view(torch.int16), cache.view(torch.int16))
+    g = b.to(gpu)
+    out, got_cache = pkg.mla_ragged_paged_attention(
+        g.ql_nope, g.q_pe, new_c.to(gpu), new_r.to(gpu), holed.to(gpu), g.kv_lens, g.page_indices, g.cu_q_lens,
+        g.cu_kv_lens, b.distribution.numpy(), sm_scale=b.sm_scale, max_kv_len=300)
+    torch.cuda.synchronize()
+    assert torch.equal(got_cache.cpu().view(torch.int16), cache.view(torch.int16))
+    torch.testing.assert_close(out.cpu()[:T].float(), want.float(), **TOL)
