@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -163,6 +164,44 @@ SplitPlan decode_plan(const RpaParams* p) {
                      env_int("RPA_DECODE_MIN_CHUNK", 128), env_int("RPA_DECODE_WAVE_CAPACITY", wave_capacity()));
 }
 
+// Balanced decode plan: a fixed number of waves (every wave slot of the GPU once) share the
+// 32-token blocks of the batch evenly; the device works the partition out from kv_lens.
+bool decode_balanced() {
+  static const bool on = env_int("RPA_DECODE_BALANCED", 1) != 0;
+  return on;
+}
+
+// The balanced plan pays for itself on ragged batches that need splitting.  Rows of one known
+// length (the host's sum equals rows x bound) split evenly under the fixed plan already, and
+// batches the fixed plan does not split at all finish in one launch with no partial rows.
+int decode_waves_per_wg(int num_kv_heads);
+int decode_wgs(int num_kv_heads);
+
+bool use_balanced(const RpaParams* p, const SplitPlan& fixed) {
+  if (!decode_balanced() || fixed.splits <= 1) return false;
+  if (p->num_splits > 0) return true;
+  // too little work to hand every workgroup its minimum piece: latency-bound, keep the launch count low
+  const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
+                                     p->cu_kv_lens != nullptr);
+  const int nw = decode_waves_per_wg(p->num_kv_heads);
+  const int64_t units = (int64_t)((p->num_kv_heads + nw - 1) / nw) * ((p->num_q_heads / p->num_kv_heads + 15) / 16);
+  const int64_t min_blocks = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 128) / 32);
+  if ((int64_t)p->decode_end * ((bound + 31) / 32) * units <= (int64_t)decode_wgs(p->num_kv_heads) * min_blocks)
+    return false;
+  const bool equal_lengths = p->sum_decode_kv_len > 0 && p->max_kv_len > 0 &&
+                             p->sum_decode_kv_len == (int64_t)p->decode_end * p->max_kv_len;
+  return !equal_lengths;
+}
+
+int decode_waves_per_wg(int num_kv_heads) {
+  const int nw = env_int("RPA_DECODE_WAVES_PER_WG", 2);
+  return std::max(1, std::min(std::min(nw, 4), num_kv_heads));
+}
+
+int decode_wgs(int num_kv_heads) {
+  return std::max(1, env_int("RPA_DECODE_WAVE_CAPACITY", wave_capacity()) / decode_waves_per_wg(num_kv_heads));
+}
+
 int check_hip(hipError_t e, const char* what) {
   if (e == hipSuccess) return RPA_OK;
   return fail(RPA_EHIP, "%s: %s", what, hipGetErrorString(e));
@@ -272,6 +311,10 @@ int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t*
 size_t rpa_workspace_bytes(const RpaParams* p) {
   if (!p || p->decode_end <= 0) return 0;
   const SplitPlan sp = decode_plan(p);
+  if (use_balanced(p, sp))
+    return (size_t)decode_wgs(p->num_kv_heads) * decode_waves_per_wg(p->num_kv_heads) * 2 * 16 * (p->head_dim + 2) *
+               sizeof(float) +
+           ((size_t)p->decode_end + 1) * sizeof(int32_t);
   if (sp.splits <= 1) return 0;
   return (size_t)p->decode_end * sp.splits * p->num_q_heads * (p->head_dim + 2) * sizeof(float);
 }
@@ -318,7 +361,25 @@ int rpa_decode(const RpaParams* p, void* stream) {
   a.fp8 = p->kv_dtype == RPA_KV_FP8_E4M3;
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
-  if (sp.splits > 1) {
+  a.cu_blocks = nullptr;
+  a.balanced = use_balanced(p, sp) ? 1 : 0;
+  a.num_wgs = decode_wgs(p->num_kv_heads);
+  a.waves_per_wg = decode_waves_per_wg(p->num_kv_heads);
+  a.min_blocks_per_wave = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 128) / 32);
+  a.forced_blocks_per_wave = 0;
+  if (p->num_splits > 0) {  // the caller pins the partition: about num_splits pieces for the longest row
+    const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
+                                       p->cu_kv_lens != nullptr);
+    a.forced_blocks_per_wave = (int32_t)std::max<int64_t>(1, ((bound + 31) / 32 + p->num_splits - 1) / p->num_splits);
+  }
+  if (a.balanced) {
+    const size_t need = rpa_workspace_bytes(p);
+    if (!p->workspace || p->workspace_bytes < need)
+      return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
+    a.ws_o = static_cast<float*>(p->workspace);
+    a.ws_ml = a.ws_o + (size_t)a.num_wgs * a.waves_per_wg * 2 * 16 * p->head_dim;
+    a.cu_blocks = reinterpret_cast<int32_t*>(a.ws_ml + (size_t)a.num_wgs * a.waves_per_wg * 2 * 16 * 2);
+  } else if (sp.splits > 1) {
     const size_t need = rpa_workspace_bytes(p);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);

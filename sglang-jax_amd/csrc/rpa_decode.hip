@@ -247,28 +247,20 @@ __device__ __forceinline__ int first_block_token(int kv_len, int window) {
   return t_lo & ~(kBlk - 1);
 }
 
-// grid = (max_splits, decode rows, head groups * row groups); block = NW waves.
-template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
-__global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const DecodeArgs a) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int nw = blockDim.x >> 6;
-  const int c = lane & 15, g = lane >> 4;
-  const int seq = blockIdx.y;
-  const int split = blockIdx.x;
-  const int head_groups = (a.Hkv + nw - 1) / nw;
-  const int hg = blockIdx.z % head_groups;
-  const int rg = blockIdx.z / head_groups;
-  const int hk = hg * nw + wave;
-  if (hk >= a.Hkv) return;
+// Where a wave leaves the result of one piece of work: the finished bf16 rows in `out`, or
+// unnormalised partial rows plus (max, sum) in the workspace, slot `base` + query head
+// (fixed split plan) or `base` + row inside the group of 16 (balanced plan).
+struct PartDest {
+  bool final_rows;
+  bool by_head;
+  int64_t base;
+};
 
-  const int kv_len = a.pt.kv_lens[seq];
-  const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
-  const int t0 = t_lo & ~(kBlk - 1);
-  const int t_begin = t0 + split * a.chunk;
-  if (t_begin >= kv_len) return;
-  // the last split runs to kv_len even if the host's length bound was too small
-  const int t_end = (split == a.max_splits - 1) ? kv_len : min(kv_len, t_begin + a.chunk);
+// One wave, one (sequence, kv head, group of 16 query heads), tokens [t_begin, t_end).
+template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
+__device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int hk, int rg, int kv_len, int t_lo,
+                                               int t_begin, int t_end, const PartDest dest, int lane) {
+  const int c = lane & 15, g = lane >> 4;
   const int nblk = (t_end - t_begin + kBlk - 1) / kBlk;
 
   SeqView sv;
@@ -352,7 +344,7 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const Decode
     const int row = row0 + mt * 16 + c;
     if (row >= a.G) continue;
     const int head = hk * a.G + row;
-    if (a.max_splits == 1) {
+    if (dest.final_rows) {
       const float inv = a.sm.sink ? vs * sink_inverse(m[mt], lt, a.sm.sink[head]) : vs / lt;
       uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 128 + g * 32;
 #pragma unroll
@@ -364,7 +356,7 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const Decode
         st16(op + r * 8, w);
       }
     } else {
-      const int64_t slot = ((int64_t)seq * a.max_splits + split) * a.Hq + head;
+      const int64_t slot = dest.base + (dest.by_head ? head : row - row0);
       float* wo = a.ws_o + slot * 128 + g * 32;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -379,6 +371,236 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const Decode
       }
     }
   }
+}
+
+// ---- fixed split plan: grid = (max_splits, decode rows, head groups * row groups); block = NW waves
+template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
+__global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const DecodeArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int seq = blockIdx.y;
+  const int split = blockIdx.x;
+  const int head_groups = (a.Hkv + nw - 1) / nw;
+  const int hg = blockIdx.z % head_groups;
+  const int rg = blockIdx.z / head_groups;
+  const int hk = hg * nw + wave;
+  if (hk >= a.Hkv) return;
+
+  const int kv_len = a.pt.kv_lens[seq];
+  const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
+  const int t0 = t_lo & ~(kBlk - 1);
+  const int t_begin = t0 + split * a.chunk;
+  if (t_begin >= kv_len) return;
+  // the last split runs to kv_len even if the host's length bound was too small
+  const int t_end = (split == a.max_splits - 1) ? kv_len : min(kv_len, t_begin + a.chunk);
+  PartDest dest;
+  dest.final_rows = a.max_splits == 1;
+  dest.by_head = true;
+  dest.base = ((int64_t)seq * a.max_splits + split) * a.Hq;
+  decode_segment<MT, FP8, UNIFORM_PAGE, CAP>(a, seq, hk, rg, kv_len, t_lo, t_begin, t_end, dest, lane);
+}
+
+// ---- balanced plan ------------------------------------------------------------------------
+// All 32-token blocks of the batch are laid out in one line -- sequence by sequence, inside a
+// sequence unit by unit, inside a unit block by block -- and workgroup j takes blocks
+// [j * pw, (j + 1) * pw): every workgroup streams the same number of KV bytes whatever the
+// ragged lengths are, and nothing about the lengths has to be known on the host.  A unit is a
+// group of NW neighbouring kv heads (x a group of 16 query heads): the NW waves of a workgroup
+// walk the same tokens of neighbouring heads, whose rows are adjacent in the head-interleaved
+// cache.  A workgroup crosses at most a few unit borders; units it covers completely are
+// finished in place, the cut ones (at most its first and its last) leave partial rows in the
+// workspace slots 2w and 2w + 1 of its waves w.
+__device__ __forceinline__ int seq_blocks(int kv_len, int window) {
+  return kv_len > 0 ? (kv_len - first_block_token(kv_len, window) + kBlk - 1) / kBlk : 0;
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int n = __shfl_up(v, off);
+    if (lane >= off) v += n;
+  }
+  return v;
+}
+
+// Linear block indices are 32-bit: a batch holds fewer than 2^31 (32-token block, unit) pairs.
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// total number of blocks of sequences [0, upto) -- all lanes of the wave must call it
+__device__ __forceinline__ int blocks_before(const DecodeArgs& a, int upto, int lane) {
+  int total = 0;
+  for (int s0 = 0; s0 < upto; s0 += 64) {
+    const int s = s0 + lane;
+    int nb = (s < upto) ? seq_blocks(a.pt.kv_lens[s], a.sm.window) : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) nb += __shfl_xor(nb, off);
+    total += nb;
+  }
+  return uniform(total);
+}
+
+__device__ __forceinline__ int blocks_per_wave(const DecodeArgs& a, int total_blocks) {
+  // never fewer than the even share: the grid has exactly num_wgs workgroups
+  const int even = (total_blocks + a.num_wgs - 1) / a.num_wgs;
+  const int floor_ = a.forced_blocks_per_wave > 0 ? a.forced_blocks_per_wave : a.min_blocks_per_wave;
+  return max(floor_, even);
+}
+
+// sequence that holds linear block x (x < total): first s with (blocks of [0, s]) * units > x
+__device__ __forceinline__ void locate_block(const DecodeArgs& a, int x, int units, int lane, int& seq,
+                                             int& seq_first_block) {
+  int base = 0;
+  seq = a.num_rows - 1;
+  seq_first_block = 0;
+  for (int s0 = 0; s0 < a.num_rows; s0 += 64) {
+    const int s = s0 + lane;
+    const int nb = (s < a.num_rows) ? seq_blocks(a.pt.kv_lens[s], a.sm.window) : 0;
+    const int incl = wave_inclusive_scan(nb, lane);
+    const uint64_t hit = __builtin_amdgcn_ballot_w64((base + incl) * units > x);
+    if (hit != 0) {
+      const int first = __builtin_ctzll(hit);
+      seq = s0 + first;
+      seq_first_block = uniform((base + __shfl(incl - nb, first)) * units);
+      return;
+    }
+    base += uniform(__shfl(incl, 63));
+  }
+}
+
+// grid = num_wgs workgroups of NW = waves_per_wg waves
+template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
+__global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const DecodeArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int nw = a.waves_per_wg;
+  const int wg = blockIdx.x;
+  const int w = wg * nw + wave;
+  const int row_groups = (a.G + 15) / 16;
+  const int head_groups = (a.Hkv + nw - 1) / nw;
+  const int units = head_groups * row_groups;
+  const int total = blocks_before(a, a.num_rows, lane) * units;
+  const int pw = blocks_per_wave(a, total);
+  if (wg == 0 && wave == 0) {
+    // the merge pass looks its sequences up in this prefix sum instead of scanning again
+    int base = 0;
+    for (int s0 = 0; s0 < a.num_rows; s0 += 64) {
+      const int s = s0 + lane;
+      const int nb = (s < a.num_rows) ? seq_blocks(a.pt.kv_lens[s], a.sm.window) : 0;
+      const int incl = wave_inclusive_scan(nb, lane);
+      if (s < a.num_rows) a.cu_blocks[s + 1] = base + incl;
+      base += uniform(__shfl(incl, 63));
+    }
+    if (lane == 0) a.cu_blocks[0] = 0;
+  }
+  if ((int64_t)wg * pw >= total) return;
+  int x = wg * pw;
+  const int x_end = min(total, x + pw);
+  const int x_first = x;
+
+  int seq, seq_first;
+  locate_block(a, x, units, lane, seq, seq_first);
+  seq = uniform(seq);
+  int kv_len = scalar_load_i32(a.pt.kv_lens + seq);
+  int nb = seq_blocks(kv_len, a.sm.window);
+  while (x < x_end) {
+    const int r = x - seq_first;
+    const int unit = r / nb;
+    const int blk = r - unit * nb;
+    const int take = min(nb - blk, x_end - x);
+    const int hg = unit / row_groups, rg = unit - hg * row_groups;
+    const int hk = hg * nw + wave;
+    const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
+    const int t0 = t_lo & ~(kBlk - 1);
+    PartDest dest;
+    dest.final_rows = (blk == 0) && (take == nb);
+    dest.by_head = false;
+    dest.base = ((int64_t)w * 2 + (x == x_first ? 0 : 1)) * 16;
+    if (hk < a.Hkv)
+      decode_segment<MT, FP8, UNIFORM_PAGE, CAP>(a, seq, hk, rg, kv_len, t_lo, t0 + blk * kBlk,
+                                                 min(kv_len, t0 + (blk + take) * kBlk), dest, lane);
+    x += take;
+    if (x < x_end && blk + take == nb && unit == units - 1) {
+      // next sequence that has any block (x < total guarantees there is one)
+      seq_first += nb * units;
+      do {
+        ++seq;
+        kv_len = scalar_load_i32(a.pt.kv_lens + seq);
+        nb = seq_blocks(kv_len, a.sm.window);
+      } while (nb == 0);
+    }
+  }
+}
+
+// Merge the partial rows of the balanced plan.  grid = (Hq, decode rows); block = one wave.
+__global__ __launch_bounds__(64) void rpa_combine_balanced_kernel(const DecodeArgs a) {
+  const int head = blockIdx.x;
+  const int seq = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int nw = a.waves_per_wg;
+  const int row_groups = (a.G + 15) / 16;
+  const int units = ((a.Hkv + nw - 1) / nw) * row_groups;
+  const int nb = seq_blocks(a.pt.kv_lens[seq], a.sm.window);
+  if (nb == 0) return;
+  const int before = scalar_load_i32(a.cu_blocks + seq);
+  const int total = scalar_load_i32(a.cu_blocks + a.num_rows) * units;
+  const int pw = blocks_per_wave(a, total);
+  const int hk = head / a.G, row = head - hk * a.G;
+  const int unit = (hk / nw) * row_groups + row / 16;
+  const int wv = hk % nw;
+  const int first_block = before * units + unit * nb;
+  const int w_first = first_block / pw, w_last = (first_block + nb - 1) / pw;
+  if (w_first == w_last) return;  // one wave covered the unit and wrote the finished rows
+  const int n = w_last - w_first + 1;
+  const int r16 = row & 15;
+  auto slot_of = [&](int j) -> int64_t {
+    const int wj = w_first + j;  // workgroup
+    // a workgroup's first piece of work goes to slot 0 of its waves: that is this unit iff it starts inside it
+    const int part = ((int64_t)wj * pw >= first_block) ? 0 : 1;
+    return (((int64_t)wj * nw + wv) * 2 + part) * 16 + r16;
+  };
+  const int d = lane * 2;
+  float mstar = -INFINITY;
+  for (int j0 = 0; j0 < n; j0 += 64) {
+    const int j = j0 + lane;
+    float mj = (j < n) ? a.ws_ml[slot_of(j) * 2] : -INFINITY;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mj = fmaxf(mj, __shfl_xor(mj, off));
+    mstar = fmaxf(mstar, mj);
+  }
+  float den = 0.f, o0 = 0.f, o1 = 0.f;
+  for (int j0 = 0; j0 < n; j0 += 64) {
+    const int j = j0 + lane;
+    float wj = 0.f, lj = 0.f;
+    if (j < n) {
+      const int64_t slot = slot_of(j);
+      wj = fast_exp2(a.ws_ml[slot * 2] - mstar);
+      lj = a.ws_ml[slot * 2 + 1] * wj;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) lj += __shfl_xor(lj, off);
+    den += lj;
+    const int cnt = min(64, n - j0);
+    for (int jj = 0; jj < cnt; jj += 8) {
+      f32x2_t o[8];
+      float wv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int js = min(jj + u, cnt - 1);
+        wv[u] = (jj + u < cnt) ? __shfl(wj, js) : 0.f;
+        o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + slot_of(j0 + js) * 128 + d);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        o0 += o[u][0] * wv[u];
+        o1 += o[u][1] * wv[u];
+      }
+    }
+  }
+  const float inv = a.sm.sink ? sink_inverse(mstar, den, a.sm.sink[head]) : 1.0f / den;
+  const int tq = a.pt.cu_q_lens[seq];
+  uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * 128 + d);
+  *op = pack_bf16x2(o0 * inv, o1 * inv);
 }
 
 // Merge the split partials: out = sum_j o_j 2^(m_j - m*) / sum_j l_j 2^(m_j - m*).
@@ -494,7 +716,8 @@ __global__ __launch_bounds__(256) void rpa_kv_write_kernel(const KvWriteArgs a) 
 
 template <bool FP8, bool UNIFORM, bool CAP>
 void launch_decode_variant(const DecodeArgs& a, dim3 grid, dim3 block, hipStream_t st) {
-  hipLaunchKernelGGL((rpa_decode_splitkv_kernel<1, FP8, UNIFORM, CAP>), grid, block, 0, st, a);
+  if (a.balanced) hipLaunchKernelGGL((rpa_decode_balanced_kernel<1, FP8, UNIFORM, CAP>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((rpa_decode_splitkv_kernel<1, FP8, UNIFORM, CAP>), grid, block, 0, st, a);
 }
 
 hipError_t launch_decode_mt(const DecodeArgs& a, dim3 grid, dim3 block, bool uniform, hipStream_t st) {
@@ -524,6 +747,12 @@ hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream) {
   // more than 16 query heads per kv head: further groups of 16 re-walk the KV (rare: MQA-like shapes)
   const int row_groups = (a.G + 15) / 16;
   const bool uniform = (a.pt.page_size % kBlk) == 0;
+  if (a.balanced) {
+    hipError_t e = launch_decode_mt(a, dim3(a.num_wgs), dim3(a.waves_per_wg * 64), uniform, stream);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(rpa_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
+    return hipGetLastError();
+  }
   dim3 grid(a.max_splits, a.num_rows, head_groups * row_groups);
   dim3 block(nw * 64);
   hipError_t e = launch_decode_mt(a, grid, block, uniform, stream);

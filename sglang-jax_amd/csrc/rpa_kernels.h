@@ -53,9 +53,17 @@ struct DecodeArgs {
   float* ws_ml;  // [num_rows, max_splits, Hq, 2]  (running max in log2 units, sum)
   int32_t num_rows;  // decode sequences
   int32_t Hq, Hkv, G;
-  int32_t chunk;       // kv tokens per split (multiple of 32)
-  int32_t max_splits;  // grid.x
+  int32_t chunk;       // fixed plan: kv tokens per split (multiple of 32)
+  int32_t max_splits;  // fixed plan: grid.x
   int32_t fp8;
+  // balanced plan: every wave takes the same number of 32-token blocks of the whole batch;
+  // ws_o / ws_ml hold 2 * num_wgs * waves_per_wg groups of 16 rows
+  int32_t balanced;
+  int32_t num_wgs;       // workgroups of the balanced grid
+  int32_t waves_per_wg;  // neighbouring kv heads walked together
+  int32_t min_blocks_per_wave;
+  int32_t forced_blocks_per_wave;  // > 0: tests pin the partition
+  int32_t* cu_blocks;              // [num_rows + 1] prefix sum of 32-token blocks, written by the kernel
 };
 
 struct PrefillArgs {

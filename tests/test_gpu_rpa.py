@@ -416,3 +416,29 @@ def test_custom_mask_and_no_mask(pkg, wl, gpu, P):
     torch.testing.assert_close(got3.float(), oracle_out(b).float(), **BF16_TOL)
     say("case no mask")
     torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=0).float(), oracle_out(b, causal=False).float(), **BF16_TOL)
+
+
+# ------------------------------------------------------------------ balanced decode plan
+@pytest.mark.parametrize("Hq,Hkv,window,kv_dtype", [(32, 8, None, torch.bfloat16), (96, 3, None, torch.bfloat16),
+                                                    (16, 4, 700, torch.bfloat16), (64, 8, None, torch.float8_e4m3fn)])
+def test_balanced_decode_plan_on_ragged_batches(pkg, wl, gpu, Hq, Hkv, window, kv_dtype):
+    """Many ragged decode rows: the plan that deals the 32-token blocks
+    of the whole batch evenly over the workgroups -- cutting sequences wherever a share ends --
+    against the oracle and against the single-piece run.  96/3 heads: two groups of 16 query
+    heads per kv head and an idle wave in the last workgroup of neighbouring kv heads."""
+    rng = np.random.default_rng(91)
+    kv_lens = [int(x) for x in rng.integers(1, 6000, size=90)]
+    kv_lens[7] = 33
+    kv_lens[40] = 4096
+    say(f"balanced plan Hq={Hq} Hkv={Hkv} window={window} {kv_dtype}")
+    b = wl.make_batch("balanced", [1] * len(kv_lens), kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=128,
+                      page_size=64, seed=92, sliding_window=window, kv_dtype=kv_dtype)
+    want = oracle_out(b)
+    tol = FP8_TOL if kv_dtype != torch.bfloat16 else BF16_TOL
+    auto = gpu_out(pkg, b, gpu)  # large ragged batch: the balanced plan
+    one = gpu_out(pkg, b, gpu, num_splits=1)  # every row in one piece, no merge pass
+    torch.testing.assert_close(auto.float(), want.float(), **tol)
+    torch.testing.assert_close(one.float(), want.float(), **tol)
+    torch.testing.assert_close(auto.float(), one.float(), rtol=1e-2, atol=4e-3)
+    for ns in (3, 50):
+        torch.testing.assert_close(gpu_out(pkg, b, gpu, num_splits=ns).float(), one.float(), rtol=1e-2, atol=4e-3)
