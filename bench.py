@@ -38,6 +38,17 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch (read + write) of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE scaled by a 1 GiB device copy (profiles/hbm_traffic_pmc.txt).  Counter runs cannot be
 # taken inside this process, so these are the figures of the committed profile, not live ones.
+# kernel that streams the KV bytes of each workload's decode rows: ragged batches that need
+# splitting take the balanced plan, equal-length and tiny ones the fixed split plan
+DECODE_KERNEL = {
+    "c1": "rpa_decode_splitkv_kernel",
+    "c2": "rpa_decode_balanced_kernel",
+    "c3": "rpa_decode_splitkv_kernel",
+    "c4": "rpa_decode_balanced_kernel",
+    "c4swa": "rpa_decode_balanced_kernel",
+    "c5": "rpa_mla_balanced_kernel",
+}
+
 MEASURED_TRAFFIC_BYTES = {
     ("c2", "rpa_prefill_async_kernel"): 359.6e6 + 77.3e6,
     ("c2", "rpa_decode_splitkv_kernel"): 501.5e6 + 3.5e6,
@@ -226,7 +237,7 @@ def main():
     dec_gbps = main_res.get("decode_gbps")
     pre_tflops = main_res.get("prefill_tflops")
     # dominant kernel of the workload (largest average launch time inside the timed region)
-    dec_kernel = "rpa_mla_decode_kernel" if args.config == "c5" else "rpa_decode_splitkv_kernel"
+    dec_kernel = DECODE_KERNEL[args.config]
     roofline_decode = None
     if dec_gbps is not None:
         roofline_decode = {"kernel": dec_kernel + (" + combine" if args.config != "c1" else ""), "bound": "hbm",

@@ -466,16 +466,37 @@ static int mla_validate(const RpaMlaParams* p) {
   return RPA_OK;
 }
 
-static size_t mla_workspace(const RpaMlaParams* p, int64_t rows) {
+static int mla_wgs() { return std::max(1, env_int("RPA_MLA_WG_CAPACITY", wave_capacity() / 8)); }
+
+// same criteria as the MHA decode path: ragged sequence rows that need splitting
+static bool mla_use_balanced(const RpaMlaParams* p, const SplitPlan& fixed, bool token_rows) {
+  static const bool on = env_int("RPA_MLA_BALANCED", 1) != 0;
+  if (!on || token_rows || fixed.splits <= 1) return false;
+  if (p->num_splits > 0) return true;
+  const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
+                                     p->cu_kv_lens != nullptr);
+  const int64_t units = (p->num_q_heads + 127) / 128;
+  const int64_t min_tiles = std::max(1, env_int("RPA_MLA_MIN_CHUNK", 256) / 32);
+  if ((int64_t)p->num_seqs * ((bound + 31) / 32) * units <= (int64_t)mla_wgs() * min_tiles) return false;
+  const bool equal_lengths = p->sum_kv_len > 0 && p->max_kv_len > 0 &&
+                             p->sum_kv_len == (int64_t)p->num_seqs * p->max_kv_len;
+  return !equal_lengths;
+}
+
+static size_t mla_workspace(const RpaMlaParams* p, int64_t rows, bool token_rows) {
   if (!p || p->num_seqs <= 0 || rows <= 0) return 0;
   const SplitPlan sp = mla_plan(p, rows);
+  if (mla_use_balanced(p, sp, token_rows))
+    return (size_t)mla_wgs() * 2 * 128 * (p->lkv_dim + 2) * sizeof(float) + ((size_t)p->num_seqs + 1) * sizeof(int32_t);
   if (sp.splits <= 1) return 0;
   return (size_t)rows * sp.splits * p->num_q_heads * (p->lkv_dim + 2) * sizeof(float);
 }
 
-size_t rpa_mla_workspace_bytes(const RpaMlaParams* p) { return mla_workspace(p, p ? p->num_seqs : 0); }
+size_t rpa_mla_workspace_bytes(const RpaMlaParams* p) { return mla_workspace(p, p ? p->num_seqs : 0, false); }
 
-size_t rpa_mla_attention_workspace_bytes(const RpaMlaParams* p) { return mla_workspace(p, p ? p->num_tokens : 0); }
+size_t rpa_mla_attention_workspace_bytes(const RpaMlaParams* p) {
+  return mla_workspace(p, p ? p->num_tokens : 0, true);
+}
 
 static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   int rc = mla_validate(p);
@@ -508,8 +529,25 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   a.max_splits = sp.splits;
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
-  if (sp.splits > 1) {
-    const size_t need = mla_workspace(p, rows);
+  a.cu_tiles = nullptr;
+  a.balanced = mla_use_balanced(p, sp, token_rows) ? 1 : 0;
+  a.num_wgs = mla_wgs();
+  a.min_tiles_per_wg = std::max(1, env_int("RPA_MLA_MIN_CHUNK", 256) / 32);
+  a.forced_tiles_per_wg = 0;
+  if (p->num_splits > 0) {
+    const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
+                                       p->cu_kv_lens != nullptr);
+    a.forced_tiles_per_wg = (int32_t)std::max<int64_t>(1, ((bound + 31) / 32 + p->num_splits - 1) / p->num_splits);
+  }
+  if (a.balanced) {
+    const size_t need = mla_workspace(p, rows, token_rows);
+    if (!p->workspace || p->workspace_bytes < need)
+      return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
+    a.ws_o = static_cast<float*>(p->workspace);
+    a.ws_ml = a.ws_o + (size_t)a.num_wgs * 2 * 128 * p->lkv_dim;
+    a.cu_tiles = reinterpret_cast<int32_t*>(a.ws_ml + (size_t)a.num_wgs * 2 * 128 * 2);
+  } else if (sp.splits > 1) {
+    const size_t need = mla_workspace(p, rows, token_rows);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
     a.ws_o = static_cast<float*>(p->workspace);

@@ -120,6 +120,13 @@ struct MlaDecodeArgs {
   int32_t rope_offset;  // elements
   int32_t chunk;
   int32_t max_splits;
+  // balanced plan (sequence rows only): the workgroups share the 32-token tiles of the batch
+  // evenly; ws_o / ws_ml hold 2 * num_wgs groups of 128 heads
+  int32_t balanced;
+  int32_t num_wgs;
+  int32_t min_tiles_per_wg;
+  int32_t forced_tiles_per_wg;
+  int32_t* cu_tiles;  // [num_rows + 1] prefix sum of tiles, written by the kernel
 };
 
 struct MlaWriteArgs {

@@ -150,33 +150,28 @@ __device__ __forceinline__ MlaRow mla_row(const MlaDecodeArgs& a, int row) {
   return r;
 }
 
-// grid = (max_splits, rows, head groups of 128); block = 512 threads.
-template <bool UNIFORM, bool CAP>
-__global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeArgs a) {
-  // three separate arrays: lets the compiler see that a copy into one slot does not alias the
-  // reads of another, so it does not drain the vector-memory queue before LDS reads
-  __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
-  __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
-  __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
+// Where a workgroup leaves the result of one piece of work: finished bf16 rows in `out`, or
+// unnormalised partial rows plus (max, sum) in workspace slot `base` + head.
+struct MlaDest {
+  bool final_rows;
+  int64_t base;
+};
 
+// One workgroup, one row, one group of 128 heads, tokens [t_begin, t_end).  Every wave of the
+// workgroup calls it with the same arguments; all LDS reads of an earlier call are behind a
+// barrier when it returns.
+template <bool UNIFORM, bool CAP>
+__device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
+                                            int t_begin, int t_end, const MlaDest dest, char* slot0, char* slot1,
+                                            char* slot2) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, g = lane >> 4;
-  const int row_id = blockIdx.y, split = blockIdx.x;
-  const int head0 = blockIdx.z * 128 + wave * 16;
+  const int head0 = head_base + wave * 16;
   const bool wave_on = head0 < a.Hq;
-
-  const MlaRow mr = mla_row(a, row_id);
-  if (!mr.valid) return;
   const int seq = mr.seq;
   const int kv_len = mr.kv_len;
-  if (kv_len <= 0) return;
-  const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
-  const int t0 = t_lo & ~(kTok - 1);
-  const int t_begin = t0 + split * a.chunk;
-  if (t_begin >= kv_len) return;
-  const int t_end = (split == a.max_splits - 1) ? kv_len : min(kv_len, t_begin + a.chunk);
 
   Src src;
   src.page_size = a.pt.page_size;
@@ -326,7 +321,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   l += __shfl_xor(l, 32);
   const int head = head0 + c;
   if (!wave_on || head >= a.Hq) return;
-  if (a.max_splits == 1) {
+  if (dest.final_rows) {
     const float inv = 1.0f / l;
     uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 512 + g * 4;
 #pragma unroll
@@ -335,7 +330,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
       *reinterpret_cast<u32x2_t*>(op + j * 16) = w;
     }
   } else {
-    const int64_t slot = ((int64_t)row_id * a.max_splits + split) * a.Hq + head;
+    const int64_t slot = dest.base + head;
     float* wo = a.ws_o + slot * 512 + g * 4;
 #pragma unroll
     for (int j = 0; j < 32; ++j) *reinterpret_cast<f32x4_t*>(wo + j * 16) = acc[j];
@@ -344,6 +339,174 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
       a.ws_ml[slot * 2 + 1] = l;
     }
   }
+}
+
+// ---- fixed split plan: grid = (max_splits, rows, head groups of 128); block = 512 threads
+template <bool UNIFORM, bool CAP>
+__global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeArgs a) {
+  // three separate arrays: lets the compiler see that a copy into one slot does not alias the
+  // reads of another, so it does not drain the vector-memory queue before LDS reads
+  __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
+  const int row_id = blockIdx.y, split = blockIdx.x;
+  const MlaRow mr = mla_row(a, row_id);
+  if (!mr.valid) return;
+  const int kv_len = mr.kv_len;
+  if (kv_len <= 0) return;
+  const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
+  const int t0 = t_lo & ~(kTok - 1);
+  const int t_begin = t0 + split * a.chunk;
+  if (t_begin >= kv_len) return;
+  const int t_end = (split == a.max_splits - 1) ? kv_len : min(kv_len, t_begin + a.chunk);
+  MlaDest dest;
+  dest.final_rows = a.max_splits == 1;
+  dest.base = ((int64_t)row_id * a.max_splits + split) * a.Hq;
+  mla_segment<UNIFORM, CAP>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2);
+}
+
+// ---- balanced plan (one row per sequence): the 32-token tiles of the whole batch, sequence by
+// sequence and inside a sequence head group by head group, are dealt evenly to the workgroups;
+// workgroup j takes tiles [j * pw, (j + 1) * pw).  Pieces that are whole rows are finished in
+// place, cut ones (at most the first and the last of a workgroup) leave partial rows in the
+// workspace slots 2j and 2j + 1 (128 heads each).
+__device__ __forceinline__ int mla_tiles(int kv_len, int window) {
+  if (kv_len <= 0) return 0;
+  const int t_lo = (window > 0) ? max(0, kv_len - window) : 0;
+  return (kv_len - (t_lo & ~(kTok - 1)) + kTok - 1) / kTok;
+}
+
+__device__ __forceinline__ int mla_tiles_per_wg(const MlaDecodeArgs& a, int total) {
+  const int even = (total + a.num_wgs - 1) / a.num_wgs;  // the grid has exactly num_wgs workgroups
+  return max(a.forced_tiles_per_wg > 0 ? a.forced_tiles_per_wg : a.min_tiles_per_wg, even);
+}
+
+template <bool UNIFORM, bool CAP>
+__global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecodeArgs a) {
+  __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
+  const int lane = threadIdx.x & 63;
+  const int wg = blockIdx.x;
+  const int units = (a.Hq + 127) / 128;
+  // prefix sums of tiles over the sequences: every wave scans (the result is wave-uniform)
+  int total = 0, seq = -1, seq_first = 0;
+  {
+    // first pass: total; second pass (below) locates this workgroup's first tile
+    for (int s0 = 0; s0 < a.num_rows; s0 += 64) {
+      const int s = s0 + lane;
+      int nt = (s < a.num_rows) ? mla_tiles(a.pt.kv_lens[s], a.sm.window) : 0;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) nt += __shfl_xor(nt, off);
+      total += nt;
+    }
+    total = __builtin_amdgcn_readfirstlane(total) * units;
+  }
+  const int pw = mla_tiles_per_wg(a, total);
+  if (wg == 0 && threadIdx.x < 64) {
+    int base = 0;
+    for (int s0 = 0; s0 < a.num_rows; s0 += 64) {
+      const int s = s0 + lane;
+      const int nt = (s < a.num_rows) ? mla_tiles(a.pt.kv_lens[s], a.sm.window) : 0;
+      int incl = nt;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int n = __shfl_up(incl, off);
+        if (lane >= off) incl += n;
+      }
+      if (s < a.num_rows) a.cu_tiles[s + 1] = base + incl;
+      base += __builtin_amdgcn_readfirstlane(__shfl(incl, 63));
+    }
+    if (lane == 0) a.cu_tiles[0] = 0;
+  }
+  if ((int64_t)wg * pw >= total) return;
+  int x = wg * pw;
+  const int x_end = min(total, x + pw);
+  const int x_first = x;
+  {
+    int base = 0;
+    for (int s0 = 0; s0 < a.num_rows && seq < 0; s0 += 64) {
+      const int s = s0 + lane;
+      const int nt = (s < a.num_rows) ? mla_tiles(a.pt.kv_lens[s], a.sm.window) : 0;
+      int incl = nt;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int n = __shfl_up(incl, off);
+        if (lane >= off) incl += n;
+      }
+      const uint64_t hit = __builtin_amdgcn_ballot_w64((base + incl) * units > x);
+      if (hit != 0) {
+        const int first = __builtin_ctzll(hit);
+        seq = s0 + first;
+        seq_first = __builtin_amdgcn_readfirstlane((base + __shfl(incl - nt, first)) * units);
+      } else {
+        base += __builtin_amdgcn_readfirstlane(__shfl(incl, 63));
+      }
+    }
+    seq = __builtin_amdgcn_readfirstlane(seq);
+  }
+  int kv_len = scalar_load_i32(a.pt.kv_lens + seq);
+  int nt = mla_tiles(kv_len, a.sm.window);
+  while (x < x_end) {
+    const int r = x - seq_first;
+    const int unit = r / nt;
+    const int tile = r - unit * nt;
+    const int take = min(nt - tile, x_end - x);
+    const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
+    const int t0 = t_lo & ~(kTok - 1);
+    MlaRow mr;
+    mr.seq = seq;
+    mr.kv_len = kv_len;
+    mr.tq = scalar_load_i32(a.pt.cu_q_lens + seq);
+    mr.valid = true;
+    MlaDest dest;
+    dest.final_rows = (tile == 0) && (take == nt);
+    dest.base = ((int64_t)wg * 2 + (x == x_first ? 0 : 1)) * 128 - unit * 128;  // + head
+    mla_segment<UNIFORM, CAP>(a, mr, unit * 128, t_lo, t0 + tile * kTok, min(kv_len, t0 + (tile + take) * kTok),
+                              dest, slot0, slot1, slot2);
+    x += take;
+    if (x < x_end && tile + take == nt && unit == units - 1) {
+      seq_first += nt * units;
+      do {
+        ++seq;
+        kv_len = scalar_load_i32(a.pt.kv_lens + seq);
+        nt = mla_tiles(kv_len, a.sm.window);
+      } while (nt == 0);
+    }
+  }
+}
+
+// Merge of the balanced plan.  grid = (Hq, rows); block = 128 threads, 4 dims each.
+__global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const MlaDecodeArgs a) {
+  const int head = blockIdx.x, seq = blockIdx.y;
+  const int nt = mla_tiles(a.pt.kv_lens[seq], a.sm.window);
+  if (nt == 0) return;
+  const int units = (a.Hq + 127) / 128;
+  const int total = a.cu_tiles[a.num_rows] * units;
+  const int pw = mla_tiles_per_wg(a, total);
+  const int unit = head >> 7;
+  const int first_tile = a.cu_tiles[seq] * units + unit * nt;
+  const int w_first = first_tile / pw, w_last = (first_tile + nt - 1) / pw;
+  if (w_first == w_last) return;  // one workgroup covered the row and wrote the finished output
+  auto slot_of = [&](int wj) -> int64_t {
+    const int part = ((int64_t)wj * pw >= first_tile) ? 0 : 1;
+    return ((int64_t)wj * 2 + part) * 128 + (head & 127);
+  };
+  float mstar = -INFINITY;
+  for (int wj = w_first; wj <= w_last; ++wj) mstar = fmaxf(mstar, a.ws_ml[slot_of(wj) * 2]);
+  float den = 0.f;
+  f32x4_t o = {0.f, 0.f, 0.f, 0.f};
+  const int d = threadIdx.x * 4;
+  for (int wj = w_first; wj <= w_last; ++wj) {
+    const int64_t slot = slot_of(wj);
+    const float w = fast_exp2(a.ws_ml[slot * 2] - mstar);
+    den += a.ws_ml[slot * 2 + 1] * w;
+    o += *reinterpret_cast<const f32x4_t*>(a.ws_o + slot * 512 + d) * w;
+  }
+  const float inv = 1.0f / den;
+  const int tq = a.pt.cu_q_lens[seq];
+  u32x2_t w = {pack_bf16x2(o[0] * inv, o[1] * inv), pack_bf16x2(o[2] * inv, o[3] * inv)};
+  *reinterpret_cast<u32x2_t*>(a.out + ((int64_t)tq * a.Hq + head) * 512 + d) = w;
 }
 
 // grid = (Hq, rows); block = 128 threads, 4 dims each.
@@ -409,6 +572,20 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   const dim3 grid(a.max_splits, a.num_rows, head_groups), block(512);
   const bool uniform = (a.pt.page_size % kTok) == 0;
   const bool cap = a.sm.soft_cap != 0.f;
+  if (a.balanced) {
+    const dim3 bgrid(a.num_wgs);
+    if (uniform) {
+      if (cap) hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, true>), bgrid, block, 0, stream, a);
+      else hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, false>), bgrid, block, 0, stream, a);
+    } else {
+      if (cap) hipLaunchKernelGGL((rpa_mla_balanced_kernel<false, true>), bgrid, block, 0, stream, a);
+      else hipLaunchKernelGGL((rpa_mla_balanced_kernel<false, false>), bgrid, block, 0, stream, a);
+    }
+    hipError_t eb = hipGetLastError();
+    if (eb != hipSuccess) return eb;
+    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+    return hipGetLastError();
+  }
   if (uniform) {
     if (cap) hipLaunchKernelGGL((rpa_mla_decode_kernel<true, true>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((rpa_mla_decode_kernel<true, false>), grid, block, 0, stream, a);
