@@ -45,7 +45,7 @@ DECODE_KERNEL = {
     "c2": "rpa_decode_balanced_kernel",
     "c3": "rpa_decode_splitkv_kernel",
     "c4": "rpa_decode_balanced_kernel",
-    "c4swa": "rpa_decode_balanced_kernel",
+    "c4swa": "rpa_decode_splitkv_kernel",
     "c5": "rpa_mla_balanced_kernel",
 }
 

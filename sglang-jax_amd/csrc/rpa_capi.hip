@@ -190,7 +190,11 @@ bool use_balanced(const RpaParams* p, const SplitPlan& fixed) {
     return false;
   const bool equal_lengths = p->sum_decode_kv_len > 0 && p->max_kv_len > 0 &&
                              p->sum_decode_kv_len == (int64_t)p->decode_end * p->max_kv_len;
-  return !equal_lengths;
+  if (equal_lengths) return false;
+  // a sliding window clips every longer row to the same length: once the mean length reaches
+  // the window most rows are clipped and the batch is as good as uniform
+  if (p->sliding_window > 0 && p->sum_decode_kv_len >= (int64_t)p->decode_end * p->sliding_window) return false;
+  return true;
 }
 
 int decode_waves_per_wg(int num_kv_heads) {

@@ -104,12 +104,17 @@ __device__ __forceinline__ f32x2_t fp8x2_to_f32(uint32_t w, bool hi) {
   return hi ? __builtin_amdgcn_cvt_pk_f32_fp8(w, true) : __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
 }
 
+// Two fp8-e4m3 bytes (low or high half of `w`) -> two bf16 in one dword, one instruction
+// (v_cvt_scalef32_pk_bf16_fp8 with scale 1; exact: e4m3 fits bf16).
+__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
+  const bf16x2_t r = hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)
+                        : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
 // Four fp8-e4m3 bytes -> four bf16 packed in two dwords (exact: e4m3 fits bf16).
 __device__ __forceinline__ u32x2_t fp8x4_to_bf16x4(uint32_t w) {
-  f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
-  f32x2_t b = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
-  u32x2_t r = {pack_bf16x2(a[0], a[1]), pack_bf16x2(b[0], b[1])};
-  return r;
+  return u32x2_t{fp8x2_to_bf16x2(w, false), fp8x2_to_bf16x2(w, true)};
 }
 
 }  // namespace rpa

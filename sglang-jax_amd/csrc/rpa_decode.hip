@@ -156,20 +156,20 @@ __device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_
   // ---- V^T operands (A of O^T = V^T P^T), one per output dim j of the lane's 8-dim chunk ----
   u32x4_t vA[8];
   if constexpr (FP8) {
-    float f[8][8];
+    // r.v[i] = 8 fp8 (dims 8c .. 8c+7) of token slot i.  A byte permute first pairs the bytes of
+    // two neighbouring tokens for two dims (t0 d, t1 d, t0 d+1, t1 d+1), then each half converts
+    // straight to a bf16 pair: 3 instructions per 4 values.
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const f32x2_t a0 = __builtin_amdgcn_cvt_pk_f32_fp8(r.v[i][0], false);
-      const f32x2_t a1 = __builtin_amdgcn_cvt_pk_f32_fp8(r.v[i][0], true);
-      const f32x2_t a2 = __builtin_amdgcn_cvt_pk_f32_fp8(r.v[i][1], false);
-      const f32x2_t a3 = __builtin_amdgcn_cvt_pk_f32_fp8(r.v[i][1], true);
-      f[i][0] = a0[0]; f[i][1] = a0[1]; f[i][2] = a1[0]; f[i][3] = a1[1];
-      f[i][4] = a2[0]; f[i][5] = a2[1]; f[i][6] = a3[0]; f[i][7] = a3[1];
-    }
+    for (int tp = 0; tp < 4; ++tp)
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      vA[j] = u32x4_t{pack_bf16x2(f[0][j], f[1][j]), pack_bf16x2(f[2][j], f[3][j]),
-                      pack_bf16x2(f[4][j], f[5][j]), pack_bf16x2(f[6][j], f[7][j])};
+      for (int dp = 0; dp < 4; ++dp) {
+        const uint32_t lo_tok = r.v[2 * tp][dp >> 1], hi_tok = r.v[2 * tp + 1][dp >> 1];
+        // selector bytes: 0-3 pick from lo_tok (second operand), 4-7 from hi_tok (first operand)
+        const uint32_t sel = (dp & 1) ? 0x07030602u : 0x05010400u;
+        const uint32_t mixed = __builtin_amdgcn_perm(hi_tok, lo_tok, sel);
+        vA[2 * dp][tp] = fp8x2_to_bf16x2(mixed, false);
+        vA[2 * dp + 1][tp] = fp8x2_to_bf16x2(mixed, true);
+      }
   } else {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
