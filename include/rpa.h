@@ -50,7 +50,12 @@ typedef enum RpaKvDtype {
   RPA_KV_FP8_E4M3 = 1 /* OCP e4m3fn, max 448 */
 } RpaKvDtype;
 
-typedef enum RpaMaskMode {
+typedef enum RpaSoftmaxDtype {
+  RPA_SOFTMAX_F32 = 0,
+  RPA_SOFTMAX_BF16 = 1
+} RpaSoftmaxDtype;
+
+enum RpaMaskMode {
   RPA_MASK_CAUSAL = 0, /* query j of a sequence sees tokens <= kv_len - q_len + j */
   RPA_MASK_CUSTOM = 1, /* causal = 0 with custom_mask (speculative tree verification) */
   RPA_MASK_NONE = 2    /* causal = 0 without a mask: every query sees all kv_len tokens */
@@ -122,6 +127,12 @@ typedef struct RpaParams {
   int32_t mask_mode;            /* RpaMaskMode */
   int32_t mask_rows_page_aligned; /* custom mask row_width_i: 0 => kv_len_i, 1 => kv_len_i rounded up to
                                    pages (cu_kv_lens delta; mask_aligned_to_cu_kv, :1791-1806) */
+  int32_t softmax_dtype;        /* RpaSoftmaxDtype: the masked logits (and the sink) are rounded to this type
+                                   before the softmax (:181-186, kernel :522-523); maxima, exponentials and
+                                   sums stay f32 */
+  float q_scale;                /* > 0: queries are divided by it and rounded to the cache's element type
+                                   (fp8 saturating at +-448) before the first product, the logits multiplied
+                                   by it (kernel :463-478); 0 => off */
 } RpaParams;
 
 /*

@@ -214,6 +214,21 @@ def ref_ragged_paged_attention(
     return torch.cat(outputs, dim=0)  # rpa_v3:202
 
 
+def quantise_queries(q: torch.Tensor, q_scale: float, kv_dtype: torch.dtype) -> torch.Tensor:
+    """Query quantisation of the reference's kernel, rpa_v3:463-470 (the pure-jnp
+    function has no q_scale; the logits are then multiplied by q_scale, :477-478,
+    which a caller of this oracle folds into sm_scale).  ``q / q_scale`` is a bf16
+    array there (a bf16 array divided by a Python float keeps its type); it is
+    clipped to the finite range of the cache's element type and cast to it.
+    Returned in q's dtype (every e4m3 value is a bf16 value).  Parity unpinned by
+    reference-held data; pinned by grid membership, range and idempotence."""
+    x = q / q_scale
+    if kv_dtype.is_floating_point:
+        info = torch.finfo(kv_dtype)
+        x = torch.clamp(x.to(torch.float32), min=float(info.min), max=float(info.max)).to(q.dtype)
+    return x.to(kv_dtype).to(q.dtype)
+
+
 def split_fused_cache(kv_pages_fused: torch.Tensor):
     """rpa_v1:74-76: heads are stored K0,V0,K1,V1,...; K = [:, :, 0::2], V = [:, :, 1::2]."""
     return kv_pages_fused[:, :, 0::2, :], kv_pages_fused[:, :, 1::2, :]

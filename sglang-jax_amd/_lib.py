@@ -92,10 +92,13 @@ class RpaParams(ctypes.Structure):
         ("xai_temperature_len", ctypes.c_float),
         ("mask_mode", ctypes.c_int32),
         ("mask_rows_page_aligned", ctypes.c_int32),
+        ("softmax_dtype", ctypes.c_int32),
+        ("q_scale", ctypes.c_float),
     ]
 
 
 MASK_CAUSAL, MASK_CUSTOM, MASK_NONE = 0, 1, 2
+SOFTMAX_F32, SOFTMAX_BF16 = 0, 1
 
 
 class RpaMlaParams(ctypes.Structure):

@@ -77,6 +77,8 @@ rpa::SoftmaxOpts softmax_opts(float sm_scale, float soft_cap, float mask_value, 
   s.mask_rows_page_aligned = 0;
   s.custom_mask = nullptr;
   s.cu_mask_lens = nullptr;
+  s.round_logits = 0;
+  s.q_scale = 0.f;
   return s;
 }
 
@@ -88,6 +90,8 @@ rpa::SoftmaxOpts softmax_opts(const RpaParams* p) {
   s.mask_rows_page_aligned = p->mask_rows_page_aligned;
   s.custom_mask = p->custom_mask;
   s.cu_mask_lens = p->cu_mask_lens;
+  s.round_logits = p->softmax_dtype == RPA_SOFTMAX_BF16 ? 1 : 0;
+  s.q_scale = p->q_scale;
   return s;
 }
 
@@ -255,6 +259,10 @@ int rpa_validate(const RpaParams* p) {
     return fail(RPA_EINVAL_NULL, "RPA_MASK_CUSTOM needs custom_mask and cu_mask_lens");
   if (p->mask_mode == RPA_MASK_CUSTOM && p->mask_rows_page_aligned && !p->cu_kv_lens)
     return fail(RPA_EINVAL_NULL, "page-aligned mask rows need cu_kv_lens");
+  if (p->softmax_dtype != RPA_SOFTMAX_F32 && p->softmax_dtype != RPA_SOFTMAX_BF16)
+    return fail(RPA_EINVAL_DTYPE, "softmax_dtype=%d is not an RpaSoftmaxDtype", p->softmax_dtype);
+  if (p->q_scale < 0.0f || std::isnan(p->q_scale))
+    return fail(RPA_EINVAL_SHAPE, "q_scale=%g must be positive (0 = off)", p->q_scale);
   if (p->xai_temperature_len < 0.0f || std::isnan(p->xai_temperature_len))
     return fail(RPA_EINVAL_SHAPE, "xai_temperature_len=%g must be positive", p->xai_temperature_len);
   return RPA_OK;

@@ -61,6 +61,36 @@ __device__ __forceinline__ float xai_factor(int qpos, float xai_len) {
   return ((float)qpos > xai_len) ? __log2f((float)qpos) / __log2f(xai_len) : 1.0f;
 }
 
+__device__ __forceinline__ float bf16_round(float x) { return bf16_lo_to_f32(pack_bf16x2(x, 0.f)); }
+
+// the sink logit of a query head, rounded like the other logits when rounding is on
+__device__ __forceinline__ float sink_logit(const float* sink, int round_logits, int head) {
+  const float s = sink[head];
+  return round_logits ? bf16_round(s) : s;
+}
+
+// Queries divided by q_scale and rounded to the cache's element type
+// (ragged_paged_attention_v3.py:463-470: the quotient is a bf16 array, clipped to the fp8
+// range and cast when the cache holds fp8).  Eight bf16 values in, eight out.
+__device__ __forceinline__ u32x4_t requantise_q(u32x4_t q, float q_scale, bool to_fp8) {
+  u32x4_t r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float lo = bf16_round(bf16_lo_to_f32(q[i]) / q_scale);
+    float hi = bf16_round(bf16_hi_to_f32(q[i]) / q_scale);
+    if (to_fp8) {
+      lo = fminf(fmaxf(lo, -448.0f), 448.0f);
+      hi = fminf(fmaxf(hi, -448.0f), 448.0f);
+      const uint32_t b = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(lo, hi, 0, false);
+      const f32x2_t f = __builtin_amdgcn_cvt_pk_f32_fp8(b, false);
+      lo = f[0];
+      hi = f[1];
+    }
+    r[i] = pack_bf16x2(lo, hi);
+  }
+  return r;
+}
+
 // Softmax denominator with an attention sink: given the running maximum m2 (log2 units), the
 // sum l of 2^(x - m2) and a sink logit (natural units), returns the factor that turns the
 // unnormalised output into out = sum p v / (sum p + e^sink)

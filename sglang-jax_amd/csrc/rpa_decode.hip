@@ -125,7 +125,8 @@ struct ScoreOpts {
   float scale;      // sm_scale * k_scale            (soft-cap path)
   float scale2;     // sm_scale * k_scale * log2(e)  (plain path)
   float cap, inv_cap;
-  float post;       // log2(e) * temperature factor, applied after the soft cap
+  float temp;       // temperature factor                (soft-cap path; the plain path folds it into scale2)
+  bool round_bf16;  // logits rounded to bf16 before the softmax (soft-cap path)
   float mask2;      // mask value in log2 units (finite)
   int t_lo;         // first visible token (sliding window), 0 otherwise
   int kv_len;
@@ -195,8 +196,16 @@ __device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       float v = s[i >> 2][i & 3];
-      if constexpr (CAP) v = soft_cap_f(v * so.scale, so.cap, so.inv_cap) * so.post;
-      else v = v * so.scale2;
+      if constexpr (CAP) {
+        // the general path: soft cap (if any), temperature, rounding of the logit (if asked)
+        v = v * so.scale;
+        if (so.cap != 0.f) v = soft_cap_f(v, so.cap, so.inv_cap);
+        v = v * so.temp;
+        if (so.round_bf16) v = bf16_round(v);
+        v = v * kLog2e;
+      } else {
+        v = v * so.scale2;
+      }
       x[i] = v;
     }
     if (need_mask) {
@@ -285,6 +294,7 @@ __device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int
     for (int st = 0; st < 4; ++st) {
       const int d0 = FP8 ? (g * 32 + st * 8) : (st * 32 + g * 8);
       qB[mt][st] = (row < a.G) ? ld16(qp + d0) : u32x4_t{0u, 0u, 0u, 0u};
+      if (a.sm.q_scale > 0.f) qB[mt][st] = requantise_q(qB[mt][st], a.sm.q_scale, FP8);
     }
   }
 
@@ -292,9 +302,10 @@ __device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int
   const float ks = a.k_scale ? a.k_scale[hk] : 1.0f;
   // the one query of a decode row sits at position kv_len - 1
   const float temp = xai_factor(kv_len - 1, a.sm.xai_len);
-  so.scale = a.sm.sm_scale * ks;
+  so.scale = a.sm.sm_scale * ks * (a.sm.q_scale > 0.f ? a.sm.q_scale : 1.0f);
   so.scale2 = so.scale * kLog2e * temp;
-  so.post = kLog2e * temp;
+  so.temp = temp;
+  so.round_bf16 = a.sm.round_logits != 0;
   so.cap = a.sm.soft_cap;
   so.inv_cap = (so.cap != 0.f) ? 1.0f / so.cap : 0.f;
   so.mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
@@ -345,7 +356,7 @@ __device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int
     if (row >= a.G) continue;
     const int head = hk * a.G + row;
     if (dest.final_rows) {
-      const float inv = a.sm.sink ? vs * sink_inverse(m[mt], lt, a.sm.sink[head]) : vs / lt;
+      const float inv = a.sm.sink ? vs * sink_inverse(m[mt], lt, sink_logit(a.sm.sink, a.sm.round_logits, head)) : vs / lt;
       uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 128 + g * 32;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -597,7 +608,7 @@ __global__ __launch_bounds__(64) void rpa_combine_balanced_kernel(const DecodeAr
       }
     }
   }
-  const float inv = a.sm.sink ? sink_inverse(mstar, den, a.sm.sink[head]) : 1.0f / den;
+  const float inv = a.sm.sink ? sink_inverse(mstar, den, sink_logit(a.sm.sink, a.sm.round_logits, head)) : 1.0f / den;
   const int tq = a.pt.cu_q_lens[seq];
   uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * 128 + d);
   *op = pack_bf16x2(o0 * inv, o1 * inv);
@@ -655,7 +666,7 @@ __global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a) {
       }
     }
   }
-  const float inv = a.sm.sink ? sink_inverse(mstar, den, a.sm.sink[head]) : 1.0f / den;
+  const float inv = a.sm.sink ? sink_inverse(mstar, den, sink_logit(a.sm.sink, a.sm.round_logits, head)) : 1.0f / den;
   const int tq = a.pt.cu_q_lens[seq];
   uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * 128 + d);
   *op = pack_bf16x2(o0 * inv, o1 * inv);
@@ -721,7 +732,8 @@ void launch_decode_variant(const DecodeArgs& a, dim3 grid, dim3 block, hipStream
 }
 
 hipError_t launch_decode_mt(const DecodeArgs& a, dim3 grid, dim3 block, bool uniform, hipStream_t st) {
-  const bool cap = a.sm.soft_cap != 0.f;
+  // soft cap and logit rounding share the general score path
+  const bool cap = a.sm.soft_cap != 0.f || a.sm.round_logits != 0;
   const int key = (a.fp8 ? 4 : 0) | (uniform ? 2 : 0) | (cap ? 1 : 0);
   switch (key) {
     case 0: launch_decode_variant<false, false, false>(a, grid, block, st); break;

@@ -39,6 +39,8 @@ struct SoftmaxOpts {
   int32_t mask_rows_page_aligned;
   const int32_t* custom_mask;
   const int32_t* cu_mask_lens;
+  int32_t round_logits;  // 1: masked logits and the sink are rounded to bf16 before the softmax
+  float q_scale;         // > 0: queries are divided by it and rounded to the cache's element type; 0 => off
 };
 
 struct DecodeArgs {

@@ -148,7 +148,8 @@ template <bool CAP>
 struct Softmax {
   float scale, cap, inv_cap;
   float sc2;   // raw score -> log2 units inside the exponent (per row: carries the temperature factor)
-  float post;  // soft-cap path: log2(e) * temperature factor
+  float temp;  // soft-cap path: temperature factor
+  bool round_bf16;  // soft-cap path: logits rounded to bf16 before the softmax
 };
 
 // Online-softmax update of one 64-token tile.  On entry S holds raw scores (MFMA units); on
@@ -215,7 +216,14 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4],
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) S[mt][v] = soft_cap_f(S[mt][v] * sm.scale, sm.cap, sm.inv_cap) * sm.post;
+      for (int v = 0; v < 16; ++v) {
+        // the general path: soft cap (if any), temperature, rounding of the logit (if asked)
+        float x = S[mt][v] * sm.scale;
+        if (sm.cap != 0.f) x = soft_cap_f(x, sm.cap, sm.inv_cap);
+        x = x * sm.temp;
+        if (sm.round_bf16) x = bf16_round(x);
+        S[mt][v] = x * kLog2e;
+      }
   }
   if (need_mask) {
 #pragma unroll
@@ -268,7 +276,7 @@ __device__ __forceinline__ void write_rows(const PrefillArgs& a, const Work& w, 
   l += __shfl_xor(l, 32);
   if (!wr.active || wr.row >= w.q_len) return;
   const float vs = a.v_scale ? a.v_scale[w.hk] : 1.0f;
-  const float inv = a.sm.sink ? vs * sink_inverse(m2, l, a.sm.sink[w.head]) : vs / l;
+  const float inv = a.sm.sink ? vs * sink_inverse(m2, l, sink_logit(a.sm.sink, a.sm.round_logits, w.head)) : vs / l;
   uint16_t* op = a.out + ((int64_t)(w.qg0 + wr.row) * a.Hq + w.head) * 128 + 4 * h;
 #pragma unroll
   for (int d = 0; d < 4; ++d)
@@ -399,15 +407,21 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
     const uint16_t* qp = a.q + ((int64_t)(w.qg0 + rr) * a.Hq + w.head) * 128 + h * 8;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qB[ks] = ld16(qp + ks * 16);
+    if (EXT && a.sm.q_scale > 0.f) {
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) qB[ks] = requantise_q(qB[ks], a.sm.q_scale, false);
+    }
   }
   Softmax<CAP> sm;
-  sm.scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f);
+  sm.scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f) *
+             ((EXT && a.sm.q_scale > 0.f) ? a.sm.q_scale : 1.0f);
   sm.cap = a.sm.soft_cap;
   sm.inv_cap = (sm.cap != 0.f) ? 1.0f / sm.cap : 0.f;
   {
     const float temp = EXT ? xai_factor(wr.qpos, a.sm.xai_len) : 1.0f;  // per query row
     sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e * temp;
-    sm.post = kLog2e * temp;
+    sm.temp = temp;
+    sm.round_bf16 = a.sm.round_logits != 0;
   }
 
   f32x16_t O[4];
@@ -654,15 +668,21 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
     const uint16_t* qp = a.q + ((int64_t)(w.qg0 + rr) * a.Hq + w.head) * 128 + h * 8;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qB[ks] = ld16(qp + ks * 16);
+    if (EXT && a.sm.q_scale > 0.f) {
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) qB[ks] = requantise_q(qB[ks], a.sm.q_scale, FP8);
+    }
   }
   Softmax<CAP> sm;
-  sm.scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f);
+  sm.scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f) *
+             ((EXT && a.sm.q_scale > 0.f) ? a.sm.q_scale : 1.0f);
   sm.cap = a.sm.soft_cap;
   sm.inv_cap = (sm.cap != 0.f) ? 1.0f / sm.cap : 0.f;
   {
     const float temp = EXT ? xai_factor(wr.qpos, a.sm.xai_len) : 1.0f;  // per query row
     sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e * temp;
-    sm.post = kLog2e * temp;
+    sm.temp = temp;
+    sm.round_bf16 = a.sm.round_logits != 0;
   }
 
   f32x16_t O[4];
@@ -742,11 +762,12 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const int64_t grid = (units >= 8 ? ((units + 7) / 8) * 8 : units) * a.G * tiles;
   if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
   const bool uniform = (a.pt.page_size % kBN) == 0;
-  const bool cap = a.sm.soft_cap != 0.f;
+  // soft cap and logit rounding share the general score path
+  const bool cap = a.sm.soft_cap != 0.f || a.sm.round_logits != 0;
   static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
   const bool staged = a.fp8 || force_staged;
   const dim3 g((unsigned)grid), blk(256);
-  const bool ext = a.sm.xai_len > 0.f || a.sm.mask_mode != 0;
+  const bool ext = a.sm.xai_len > 0.f || a.sm.mask_mode != 0 || a.sm.q_scale > 0.f;
 #define RPA_STAGED(F, U, C, E) \
   hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C, E>), g, blk, 0, stream, a, tiles, nseq)
 #define RPA_ASYNC(U, C, E) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E>), g, blk, 0, stream, a, tiles, nseq)

@@ -189,7 +189,7 @@ class RpaCall:
                  sm_scale, sliding_window=None, soft_cap=None, mask_value=DEFAULT_MASK_VALUE, k_scale=None,
                  v_scale=None, max_kv_len=0, max_q_len=0, num_splits=0, out=None, sum_decode_kv_len=0,
                  attention_sink=None, xai_temperature_len=None, causal=True, custom_mask=None,
-                 mask_aligned_to_cu_kv=False):
+                 mask_aligned_to_cu_kv=False, softmax_dtype=None, q_scale=None):
         self.lib = _lib.load()
         self.device = queries.device
         fused = v_pages is None
@@ -231,6 +231,20 @@ class RpaCall:
             if not xai_temperature_len > 0:
                 raise ValueError(f"xai_temperature_len={xai_temperature_len} must be positive.")
             p.xai_temperature_len = float(xai_temperature_len)
+        # ---- softmax_dtype (rpa_v3:181-186, kernel :522-523): logits rounded to it before the softmax
+        if softmax_dtype in (None, torch.float32):
+            p.softmax_dtype = _lib.SOFTMAX_F32
+        elif softmax_dtype == torch.bfloat16:
+            p.softmax_dtype = _lib.SOFTMAX_BF16
+        elif isinstance(softmax_dtype, torch.dtype) and softmax_dtype.is_floating_point:
+            raise NotImplementedError(f"softmax_dtype={softmax_dtype}: only float32 and bfloat16 are built")
+        else:
+            raise ValueError(f"Expected softmax_dtype to be a floating point dtype, got {softmax_dtype}")
+        # ---- q_scale (kernel rpa_v3:463-478): queries quantised to the cache's element type
+        if q_scale is not None:
+            if not q_scale > 0:
+                raise ValueError(f"q_scale={q_scale} must be positive.")
+            p.q_scale = float(q_scale)
         # ---- mask mode (rpa_v3:152-165): causal, the caller's flat mask, or none
         self.mask = self.cu_mask = None
         if causal:
@@ -346,9 +360,6 @@ def ragged_paged_attention(
     static_validate_inputs(queries, keys, values, kv_cache_fused, kv_lens_d, page_d, cu_q_d, cu_kv_d, dist_t,
                            causal=causal, sliding_window=sliding_window, soft_cap=soft_cap,
                            chunk_prefill_size=chunk_prefill_size, skip_kv_mask=skip_kv_mask)
-    for name, val in (("softmax_dtype", softmax_dtype), ("q_scale", q_scale)):
-        if val is not None:
-            raise NotImplementedError(f"{name} is not built")
     if kv_cache_fused.dim() == 5:  # reference's packed view [pages, P, 2Hkv/pack, pack, D]
         s = kv_cache_fused.shape
         kv_cache_fused = kv_cache_fused.view(s[0], s[1], s[2] * s[3], s[4])
@@ -376,7 +387,8 @@ def ragged_paged_attention(
                    max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits,
                    sum_decode_kv_len=_host_decode_sum(host_kv_lens if host_kv_lens is not None else kv_lens, i),
                    attention_sink=attention_sink, xai_temperature_len=xai_temperature_len, causal=bool(causal),
-                   custom_mask=custom_mask, mask_aligned_to_cu_kv=mask_aligned_to_cu_kv)
+                   custom_mask=custom_mask, mask_aligned_to_cu_kv=mask_aligned_to_cu_kv,
+                   softmax_dtype=softmax_dtype, q_scale=q_scale)
     if validate_values:
         dynamic_validate_inputs(call.params, kv_lens_d.cpu().numpy(), page_d.cpu().numpy(), cu_q_d.cpu().numpy(),
                                 cu_kv_d.cpu().numpy(), dist.astype(np.int32))
@@ -420,8 +432,6 @@ def ragged_paged_attention_ref_surface(
     how many leading sequences are single-token rows (0 is always valid: the
     flash kernel handles q_len == 1 too)."""
     _require_gpu(queries, "queries")
-    if softmax_dtype is not None:
-        raise NotImplementedError("softmax_dtype is not built")
     if sliding_window is not None and sliding_window <= 0:
         raise ValueError(f"sliding_window={sliding_window} must be positive.")
     if soft_cap is not None and soft_cap == 0.0:
@@ -445,7 +455,8 @@ def ragged_paged_attention_ref_surface(
                    max_kv_len=max_kv_len if max_kv_len is not None else _host_max(kv_lens),
                    max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits,
                    sum_decode_kv_len=_host_decode_sum(kv_lens, decode_end), attention_sink=attention_sink,
-                   xai_temperature_len=xai_temperature_len, causal=bool(causal), custom_mask=custom_mask)
+                   xai_temperature_len=xai_temperature_len, causal=bool(causal), custom_mask=custom_mask,
+                   softmax_dtype=softmax_dtype)
     call.attention()
     return call.out
 

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol(pkg):
 
 def test_struct_layout_matches_header(pkg):
     # 11 pointers + size_t + 15 int32 + 3 float + int64
-    assert ctypes.sizeof(pkg._lib.RpaParams) == 12 * 8 + 18 * 4 + 8 + 3 * 8 + 3 * 4 + 4  # + tail padding
+    assert ctypes.sizeof(pkg._lib.RpaParams) == 12 * 8 + 18 * 4 + 8 + 3 * 8 + 5 * 4 + 4  # + tail padding
     assert ctypes.sizeof(pkg._lib.RpaMlaParams) == 10 * 8 + 13 * 4 + 3 * 4 + 8
 
 

@@ -380,6 +380,49 @@ def test_xai_temperature(pkg, wl, gpu, cap):
     assert torch.equal(gpu_out(pkg, b, gpu, xai_temperature_len=8192.0), gpu_out(pkg, b, gpu))
 
 
+@pytest.mark.parametrize("cap,use_sink", [(None, False), (20.0, True)])
+def test_softmax_dtype_bfloat16(pkg, wl, gpu, cap, use_sink):
+    """Masked logits (and the sink) rounded to bf16 before the softmax
+    (ragged_paged_attention_v3.py:181-186; kernel :522-523).  float32 is the default path."""
+    q_lens, kv_lens, b = options_batch(wl, "smdt", 74)
+    b.soft_cap = cap
+    kw = {}
+    if use_sink:
+        kw["attention_sink"] = torch.from_numpy(np.random.RandomState(456).randn(16).astype(np.float32)) * 2.0
+    say(f"case softmax_dtype cap={cap} sink={use_sink}")
+    want = oracle_out(b, softmax_dtype=torch.bfloat16, **kw)
+    got = gpu_out(pkg, b, gpu, softmax_dtype=torch.bfloat16, **kw)
+    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    assert torch.equal(gpu_out(pkg, b, gpu, softmax_dtype=torch.float32, **kw), gpu_out(pkg, b, gpu, **kw))
+    with pytest.raises(NotImplementedError):
+        gpu_out(pkg, b, gpu, softmax_dtype=torch.float16)
+    with pytest.raises(ValueError):
+        gpu_out(pkg, b, gpu, softmax_dtype=torch.int32)
+
+
+@pytest.mark.parametrize("kv_dtype", [torch.bfloat16, torch.float8_e4m3fn])
+def test_q_scale_quantises_queries_to_the_cache_type(pkg, wl, gpu, kv_dtype):
+    """q / q_scale rounded to the cache's element type, logits multiplied by q_scale (kernel,
+    ragged_paged_attention_v3.py:463-478).  The oracle gets the quantised queries and
+    sm_scale * q_scale, which is the same arithmetic."""
+    from oracle.ref_rpa import quantise_queries
+    q_lens, kv_lens = [1, 1, 1, 40, 130], [5, 700, 1025, 40, 300]
+    b = wl.make_batch("qscale", q_lens, kv_lens, num_q_heads=16, num_kv_heads=4, head_dim=128, page_size=64,
+                      seed=75, kv_dtype=kv_dtype)
+    q_scale = 0.37
+    say(f"case q_scale kv_dtype={kv_dtype}")
+    got = gpu_out(pkg, b, gpu, q_scale=q_scale)
+    q_orig, sm_orig = b.q, b.sm_scale
+    b.q, b.sm_scale = quantise_queries(b.q, q_scale, kv_dtype), sm_orig * q_scale
+    want = oracle_out(b)
+    b.q, b.sm_scale = q_orig, sm_orig
+    torch.testing.assert_close(got.float(), want.float(), **(FP8_TOL if kv_dtype != torch.bfloat16 else BF16_TOL))
+    # and the kernels compute exactly what they compute on pre-quantised queries
+    b.q, b.sm_scale = quantise_queries(q_orig, q_scale, kv_dtype), sm_orig * q_scale
+    same = gpu_out(pkg, b, gpu)
+    torch.testing.assert_close(got.float(), same.float(), rtol=8e-3, atol=1e-3)
+
+
 def flat_mask(masks):
     return torch.from_numpy(np.concatenate([m.reshape(-1) for m in masks]).astype(np.int32))
 

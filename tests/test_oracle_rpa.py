@@ -402,3 +402,54 @@ def test_custom_mask_special_cases_and_brute_force():
                 want = (w / w.sum()) @ vv[keep, h // 2]
                 np.testing.assert_allclose(out[o + j, h], want, rtol=2e-5, atol=2e-6)
         o += ql
+
+
+def test_query_quantisation_lands_on_the_cache_grid():
+    """rpa_v3:463-470.  Pins: results are values of the cache's element type, inside its finite
+    range, unchanged by a second pass at scale 1, and equal to the input when that is already
+    on the grid; the clip makes 1e4 / 2 saturate at 448 instead of overflowing e4m3."""
+    from oracle.ref_rpa import quantise_queries
+    g = torch.Generator().manual_seed(5)
+    q = (torch.randn(64, 4, 128, generator=g) * 3).to(torch.bfloat16)
+    q[0, 0, 0] = 1.0e4
+    x = quantise_queries(q, 2.0, torch.float8_e4m3fn)
+    assert x.dtype == torch.bfloat16 and float(x.abs().max()) == 448.0
+    assert torch.equal(x.to(torch.float8_e4m3fn).to(torch.bfloat16), x)
+    assert torch.equal(quantise_queries(x, 1.0, torch.float8_e4m3fn), x)
+    # nearest grid point: error at most half a grid step (2^-4 relative for 3 mantissa bits)
+    ref = (q.float() / 2.0).clamp(-448, 448)
+    big = ref.abs() > 2.0 ** -6  # normal range of e4m3
+    assert float(((x.float() - ref).abs()[big] / ref.abs()[big]).max()) <= 2.0 ** -4 + 2.0 ** -8
+    # a bf16 cache: the quotient rounded to bf16, nothing else
+    y = quantise_queries(q, 3.0, torch.bfloat16)
+    assert torch.equal(y, (q.float() / 3.0).to(torch.bfloat16))
+
+
+def test_softmax_dtype_rounds_logits_and_probabilities():
+    """rpa_v3:181-199 with softmax_dtype = bfloat16: the masked logits become bf16 values and so do
+    the probabilities that multiply V.  Checked against a float64 loop with the two roundings done
+    by hand, and against the f32 softmax, from which it may differ by bf16 rounding only.  The
+    reduction order inside jax's bf16 softmax is not reproducible here: parity unpinned below
+    one bf16 ulp of the probabilities."""
+    c = make_case([3, 1], [9, 17], Hq=4, Hkv=2, D=8, P=4, seed=21)
+    base = run(c, sm_scale=0.5)
+    rnd = run(c, sm_scale=0.5, softmax_dtype=torch.bfloat16)
+    torch.testing.assert_close(rnd.float(), base.float(), rtol=2e-2, atol=2e-2)
+
+    def bf(x):
+        return float(torch.tensor(x, dtype=torch.float32).to(torch.bfloat16))
+
+    o = 0
+    for i, (ql, kv) in enumerate([(3, 9), (1, 17)]):
+        k, v = gathered(c, i)
+        for j in range(ql):
+            for h in range(4):
+                qv = c["q"][o + j, h].double()
+                vis = range(kv - ql + j + 1)
+                logit = [bf(float((qv * k[t, h // 2].double()).sum()) * 0.5) for t in vis]
+                mx = max(logit)
+                e = [math.exp(x - mx) for x in logit]
+                p = [bf(x / sum(e)) for x in e]
+                want = sum(pt * v[t, h // 2].double() for pt, t in zip(p, vis))
+                torch.testing.assert_close(rnd[o + j, h].double(), want, rtol=2e-2, atol=2e-2)
+        o += ql
