@@ -419,6 +419,7 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   a.Hkv = p->num_kv_heads;
   a.G = p->num_q_heads / p->num_kv_heads;
   a.max_q_len = p->max_q_len > 0 ? p->max_q_len : p->num_tokens;
+  a.max_kv_len = p->max_kv_len > 0 ? p->max_kv_len : 0;
   a.fp8 = p->kv_dtype == RPA_KV_FP8_E4M3;
   return check_hip(rpa::launch_prefill(a, static_cast<hipStream_t>(stream)), "rpa_prefill");
 }

@@ -79,6 +79,7 @@ struct PrefillArgs {
   int32_t seq_begin, seq_end;  // sequences [seq_begin, seq_end)
   int32_t Hq, Hkv, G;
   int32_t max_q_len;
+  int32_t max_kv_len;  // host bound on kv_len of these sequences, 0 = unknown
   int32_t fp8;
 };
 

@@ -86,14 +86,17 @@ __device__ __forceinline__ int64_t row_offset(const TileSrc& s, const KvAddr& kv
 // A unit is one (sequence, kv head): its G query heads and all their query tiles read the
 // same K/V, so a unit stays on one XCD (one L2).  Hardware deals workgroup n to XCD n % 8;
 // XCD x owns units x, x+8, ...: units of one sequence cost the same, so the XCDs stay
-// balanced whatever the ragged lengths are.  Inside an XCD, late (long, causal) query
-// tiles of every unit are issued first and the G heads of a unit sit next to each other.
+// balanced whatever the ragged lengths are.  Inside an XCD the G heads of a unit sit next to
+// each other and the most expensive query tiles are issued first, so that the last workgroups
+// to start are short ones.  A causal tile costs what its last row sees: with a bound on kv_len
+// from the host, tiles are ordered by level = tile index + ceil(prefix / tile rows), i.e. by
+// that extent across sequences; without one, by position inside their own sequence.
 struct Work {
   int seq, hk, head, q_start, qg0, q_len, kv_len, prefix;
   bool valid;
 };
 
-__device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int nseq) {
+__device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int nseq, bool by_level) {
   Work w;
   w.valid = false;
   const int units = nseq * a.Hkv;
@@ -120,10 +123,12 @@ __device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int n
   w.seq = a.seq_begin + si;
   w.qg0 = a.pt.cu_q_lens[w.seq];
   w.q_len = a.pt.cu_q_lens[w.seq + 1] - w.qg0;
-  w.q_start = (tiles - 1 - tile_rev) * kBM;
-  if (w.q_start >= w.q_len) return w;
   w.kv_len = a.pt.kv_lens[w.seq];
   w.prefix = w.kv_len - w.q_len;
+  int tile = tiles - 1 - tile_rev;
+  if (by_level) tile -= (max(w.prefix, 0) + kBM - 1) / kBM;
+  w.q_start = tile * kBM;
+  if (tile < 0 || w.q_start >= w.q_len) return w;
   w.valid = true;
   return w;
 }
@@ -374,7 +379,7 @@ __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const 
 // EXT compiles in the rarely used options (temperature factor, custom mask / no mask); the
 // plain causal instantiation keeps its scale in a scalar register and its mask test to one compare.
 template <bool UNIFORM, bool CAP, bool EXT>
-__global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const PrefillArgs a, int tiles, int nseq) {
+__global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const PrefillArgs a, int tiles, int nseq, bool by_level) {
   // Four separate arrays (not one indexed array): the compiler can then prove that the
   // asynchronous copy into one ring slot does not alias the LDS reads of the other slot and
   // does not drain the vector-memory queue in the middle of a tile.
@@ -383,7 +388,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
   __shared__ __attribute__((aligned(1024))) char lds_v0[kTileB];
   __shared__ __attribute__((aligned(1024))) char lds_v1[kTileB];
 
-  const Work w = decompose(a, tiles, nseq);
+  const Work w = decompose(a, tiles, nseq, by_level);
   if (!w.valid) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -641,11 +646,11 @@ __device__ __forceinline__ void tile_lstore(const Stage<FP8>& st, char* lds_k, c
 }
 
 template <bool FP8, bool UNIFORM, bool CAP, bool EXT>
-__global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const PrefillArgs a, int tiles, int nseq) {
+__global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const PrefillArgs a, int tiles, int nseq, bool by_level) {
   __shared__ __attribute__((aligned(16))) char lds_k_buf[2][kBN * kKPitch];
   __shared__ __attribute__((aligned(16))) char lds_v_buf[2][128 * kVPitch];
 
-  const Work w = decompose(a, tiles, nseq);
+  const Work w = decompose(a, tiles, nseq, by_level);
   if (!w.valid) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -757,7 +762,13 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
 hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const int nseq = a.seq_end - a.seq_begin;
   if (nseq <= 0 || a.max_q_len <= 0) return hipSuccess;
-  const int tiles = (a.max_q_len + kBM - 1) / kBM;
+  int tiles = (a.max_q_len + kBM - 1) / kBM;
+  // levels 0 .. ceil(max_kv_len / rows): only worth their empty workgroups when prefixes are
+  // not much longer than the chunks (else every tile of a sequence costs about the same anyway)
+  static const bool level_order = [] { const char* v = getenv("RPA_PREFILL_LEVEL_ORDER"); return !(v && *v == '0'); }();
+  const int levels = a.max_kv_len > 0 ? (a.max_kv_len + kBM - 1) / kBM + 1 : 0;
+  const bool by_level = level_order && a.sm.mask_mode == 0 && levels > tiles && levels <= 2 * tiles + 2;
+  if (by_level) tiles = levels;
   const int64_t units = (int64_t)nseq * a.Hkv;
   const int64_t grid = (units >= 8 ? ((units + 7) / 8) * 8 : units) * a.G * tiles;
   if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
@@ -769,8 +780,8 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const dim3 g((unsigned)grid), blk(256);
   const bool ext = a.sm.xai_len > 0.f || a.sm.mask_mode != 0 || a.sm.q_scale > 0.f;
 #define RPA_STAGED(F, U, C, E) \
-  hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C, E>), g, blk, 0, stream, a, tiles, nseq)
-#define RPA_ASYNC(U, C, E) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E>), g, blk, 0, stream, a, tiles, nseq)
+  hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
+#define RPA_ASYNC(U, C, E) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_PICK(M, ...)                                            \
   switch ((uniform ? 4 : 0) | (cap ? 2 : 0) | (ext ? 1 : 0)) {        \
     case 0: M(__VA_ARGS__ false, false, false); break;              \
