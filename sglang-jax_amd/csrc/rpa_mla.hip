@@ -15,12 +15,14 @@
 // Partials (unnormalised O, running max, sum) go to the workspace and are merged
 // by rpa_mla_combine_kernel; with a single split the output is written directly.
 //
-// LDS layout of a tile: row r (token) at r * 1168 bytes = 73 chunks of 16 bytes, the last one
-// padding.  1168 bytes = 292 dwords = 36 (mod 64 banks): the 16 rows of a b128 operand read
-// start at 16 distinct multiples of 4 banks, and the 8 even (or 8 odd) rows of a transposing
-// read at 8 distinct 8-bank windows -- no bank conflicts and no address swizzle, so every LDS
-// address is a per-lane base plus a compile-time offset.  MFMA row m of a score tile is token
-// 16b + 2(m & 7) + (m >> 3), which puts even tokens in lane groups 0-1 and odd ones in 2-3.
+// LDS layout of a tile: row r (token) at r * 1184 bytes = 74 chunks of 16 bytes, the last two
+// padding.  Measured on gfx950 (256 WGs of 8 waves reading one pattern): a ds_read_b128 whose 16
+// lanes of a group read the same column of 16 rows runs at the full rate (3.7 clk per wave
+// instruction, like 64 contiguous chunks) when the pitch is 74 or 78 chunks and at half of it
+// (7.3 clk) for 73, 75, 76, 77, 79 and 81 chunks, whatever the order of the rows; the
+// transposing b64 read of 4 consecutive rows x 32 bytes is full rate (2.6 clk) at 74 chunks
+// too.  So no address swizzle and no row permutation: MFMA row m of a score tile is token
+// 16b + m, and every LDS address is a per-lane base plus a compile-time offset.
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
@@ -30,9 +32,9 @@ namespace rpa {
 namespace {
 
 constexpr int kTok = 32;                 // tokens per tile
-constexpr int kRowB = 1168;              // latent row in LDS: 576 bf16 + 16 bytes of padding
-constexpr int kChunks = 73;              // 16-byte chunks per row (72 data + 1 pad)
-constexpr int kSlotB = 40 * 1024;        // one ring slot: 40 copy blocks of 64 chunks (36.5 used)
+constexpr int kRowB = 1184;              // latent row in LDS: 576 bf16 + 32 bytes of padding
+constexpr int kChunks = 74;              // 16-byte chunks per row (72 data + 2 pad)
+constexpr int kSlotB = 40 * 1024;        // one ring slot: 40 copy blocks of 64 chunks (37 used)
 constexpr int kCopiesPerWave = 5;        // every wave issues 5 copy instructions per tile
 
 __device__ __forceinline__ u32x4_t lds_ld16(const char* p) { return *reinterpret_cast<const u32x4_t*>(p); }
@@ -46,7 +48,7 @@ __device__ __forceinline__ u32x2_t lds_tr16(const char* p) {
 
 // token (inside a tile) behind slot i = 4b + r of lane group g in the S^T result registers
 __device__ __forceinline__ int tok_of(int g, int i) {
-  return 16 * (i >> 2) + 8 * (g & 1) + 2 * (i & 3) + (g >> 1);
+  return 16 * (i >> 2) + 4 * g + (i & 3);
 }
 
 struct Src {
@@ -61,14 +63,14 @@ __device__ __forceinline__ int page_slot(const Src& s, int tok) {
   return s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
 }
 
-// A lane's 5 chunks of a tile: position p = 64*(5*wave + n) + lane; row p / 73, chunk
-// column p % 73.  The pad column and positions >= 32*73 copy the tile's first chunk.
+// A lane's 5 chunks of a tile: position p = 64*(5*wave + n) + lane; row p / 74, chunk
+// column p % 74.  The pad columns and positions >= 32*74 copy the tile's first chunk.
 __device__ __forceinline__ void chunk_of(const Src& s, int wave, int lane, int n, int& row, int& inner) {
   int p = (wave * kCopiesPerWave + n) * 64 + lane;
   if (p >= kTok * kChunks) p = 0;
   row = p / kChunks;
   int j = p - row * kChunks;
-  if (j == kChunks - 1) { row = 0; j = 0; }
+  if (j >= 72) { row = 0; j = 0; }
   inner = j < 64 ? j * 16 : s.rope_byte + (j - 64) * 16;
 }
 
@@ -211,11 +213,11 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   const float mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
 
   // ---- LDS operand addresses (bytes inside a slot) ----
-  // K operand of score tile b, k-step ks: row 16b + 2(c & 7) + (c >> 3), bytes 64ks + 16g
-  const int k_off = (2 * (c & 7) + (c >> 3)) * kRowB + g * 16;
-  // V^T operand of dim chunk j: source lane r = c points at token 8(g & 1) + 2(r >> 2) + (g >> 1)
+  // K operand of score tile b, k-step ks: row 16b + c, bytes 64ks + 16g
+  const int k_off = c * kRowB + g * 16;
+  // V^T operand of dim chunk j: source lane r = c points at token 4g + (r >> 2)
   // (+16 for the second half of the k-step), dims 16j + 4(r & 3)
-  const int v_off = (8 * (g & 1) + 2 * (c >> 2) + (g >> 1)) * kRowB + (c & 3) * 8;
+  const int v_off = (4 * g + (c >> 2)) * kRowB + (c & 3) * 8;
 
   f32x4_t acc[32];
 #pragma unroll
