@@ -12,6 +12,7 @@ from .backend import (  # noqa: F401
     MLAAttentionBackend,
     build_forward_metadata,
 )
+from .dsa import compute_topk_pages, sparse_mla_page_level, sparse_mla_via_dense  # noqa: F401
 from .mla import mla_ragged_paged_attention  # noqa: F401
 from .ragged_paged_attention import (  # noqa: F401
     DEFAULT_MASK_VALUE,
