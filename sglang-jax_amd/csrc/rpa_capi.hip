@@ -215,6 +215,27 @@ int check_hip(hipError_t e, const char* what) {
   return fail(RPA_EHIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+// head_dim 256: every query token of sequences [seq_begin, seq_end) is a row of the row kernel
+int rows256(const RpaParams* p, int seq_begin, int seq_end, void* stream) {
+  if (seq_end <= seq_begin) return RPA_OK;
+  rpa::DecodeArgs a = {};
+  a.q = static_cast<const uint16_t*>(p->q);
+  a.out = static_cast<uint16_t*>(p->out);
+  a.kv = kv_addr(p);
+  a.pt = page_table(p);
+  a.sm = softmax_opts(p);
+  a.k_scale = p->k_scale;
+  a.v_scale = p->v_scale;
+  a.num_rows = seq_end;
+  a.Hq = p->num_q_heads;
+  a.Hkv = p->num_kv_heads;
+  a.G = p->num_q_heads / p->num_kv_heads;
+  a.fp8 = p->kv_dtype == RPA_KV_FP8_E4M3;
+  // decode rows are one token each; other sequences are bounded by the tokens of the call
+  const int rows = (seq_end <= p->decode_end) ? (seq_end - seq_begin) : p->num_tokens;
+  return check_hip(rpa::launch_rows256(a, seq_begin, seq_end, rows, static_cast<hipStream_t>(stream)), "rpa rows256");
+}
+
 }  // namespace
 
 extern "C" {
@@ -233,8 +254,12 @@ int rpa_validate(const RpaParams* p) {
   if (p->num_q_heads % p->num_kv_heads != 0)
     return fail(RPA_EINVAL_HEADS, "expected num_q_heads=%d to be divisible by num_kv_heads=%d",
                 p->num_q_heads, p->num_kv_heads);
-  if (p->head_dim != 128)
-    return fail(RPA_EUNSUPPORTED, "head_dim=%d: only 128 is built", p->head_dim);
+  if (p->head_dim != 128 && p->head_dim != 256)
+    return fail(RPA_EUNSUPPORTED, "head_dim=%d: 128 and 256 are built", p->head_dim);
+  if (p->head_dim == 256 && (p->mask_mode == RPA_MASK_CUSTOM || p->q_scale > 0.0f))
+    return fail(RPA_EUNSUPPORTED, "head_dim=256: custom masks and q_scale are not built");
+  if (p->head_dim == 256 && p->num_tokens > 65535)
+    return fail(RPA_EUNSUPPORTED, "head_dim=256: at most 65535 tokens per call, got %d", p->num_tokens);
   if (p->kv_dtype != RPA_KV_BF16 && p->kv_dtype != RPA_KV_FP8_E4M3)
     return fail(RPA_EINVAL_DTYPE, "kv_dtype=%d is not a floating point cache dtype", p->kv_dtype);
   if (p->layout != RPA_LAYOUT_FUSED && p->layout != RPA_LAYOUT_SPLIT)
@@ -322,6 +347,7 @@ int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t*
 
 size_t rpa_workspace_bytes(const RpaParams* p) {
   if (!p || p->decode_end <= 0) return 0;
+  if (p->head_dim == 256) return 0;  // the 256-dim kernel does not split sequences
   const SplitPlan sp = decode_plan(p);
   if (use_balanced(p, sp))
     return (size_t)decode_wgs(p->num_kv_heads) * decode_waves_per_wg(p->num_kv_heads) * 2 * 16 * (p->head_dim + 2) *
@@ -355,6 +381,7 @@ int rpa_decode(const RpaParams* p, void* stream) {
   if (rc != RPA_OK) return rc;
   if (p->decode_end <= 0) return RPA_OK;
   if (p->mask_mode == RPA_MASK_CUSTOM) return RPA_OK;  // masked rows all go through the prefill kernel
+  if (p->head_dim == 256) return rows256(p, 0, p->decode_end, stream);
   const SplitPlan sp = decode_plan(p);
   rpa::DecodeArgs a;
   a.q = static_cast<const uint16_t*>(p->q);
@@ -405,6 +432,7 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   int rc = rpa_validate(p);
   if (rc != RPA_OK) return rc;
   if (p->num_seqs <= p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) return RPA_OK;
+  if (p->head_dim == 256) return rows256(p, p->decode_end, p->num_seqs, stream);
   rpa::PrefillArgs a;
   a.q = static_cast<const uint16_t*>(p->q);
   a.out = static_cast<uint16_t*>(p->out);

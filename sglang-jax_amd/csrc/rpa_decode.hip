@@ -132,12 +132,9 @@ struct ScoreOpts {
   int kv_len;
 };
 
-template <int MT, bool FP8, bool CAP>
-__device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_t (&qB)[MT][4],
-                                              f32x4_t (&acc)[MT][8], float (&m)[MT], float (&l)[MT],
-                                              const ScoreOpts& so, int tb, int g) {
-  // ---- K operands (A of S^T = K Q^T) ----
-  u32x4_t kA[2][4];
+// K operands (A of S^T = K Q^T) of one 32-token block: [token half][k step]
+template <bool FP8>
+__device__ __forceinline__ void k_operands(const KvRegs<FP8>& r, u32x4_t (&kA)[2][4]) {
 #pragma unroll
   for (int b = 0; b < 2; ++b) {
     if constexpr (FP8) {
@@ -154,8 +151,11 @@ __device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_
       for (int st = 0; st < 4; ++st) kA[b][st] = r.k[b][st];
     }
   }
-  // ---- V^T operands (A of O^T = V^T P^T), one per output dim j of the lane's 8-dim chunk ----
-  u32x4_t vA[8];
+}
+
+// V^T operands (A of O^T = V^T P^T), one per output dim j of the lane's 8-dim chunk
+template <bool FP8>
+__device__ __forceinline__ void v_operands(const KvRegs<FP8>& r, u32x4_t (&vA)[8]) {
   if constexpr (FP8) {
     // r.v[i] = 8 fp8 (dims 8c .. 8c+7) of token slot i.  A byte permute first pairs the bytes of
     // two neighbouring tokens for two dims (t0 d, t1 d, t0 d+1, t1 d+1), then each half converts
@@ -182,6 +182,16 @@ __device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_
                       __builtin_amdgcn_perm(r.v[7][jj], r.v[6][jj], sel)};
     }
   }
+}
+
+template <int MT, bool FP8, bool CAP>
+__device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_t (&qB)[MT][4],
+                                              f32x4_t (&acc)[MT][8], float (&m)[MT], float (&l)[MT],
+                                              const ScoreOpts& so, int tb, int g) {
+  u32x4_t kA[2][4];
+  k_operands<FP8>(r, kA);
+  u32x4_t vA[8];
+  v_operands<FP8>(r, vA);
   const bool need_mask = (tb + kBlk > so.kv_len) || (tb < so.t_lo);
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -614,6 +624,156 @@ __global__ __launch_bounds__(64) void rpa_combine_balanced_kernel(const DecodeAr
   *op = pack_bf16x2(o0 * inv, o1 * inv);
 }
 
+// ---- head_dim 256 ---------------------------------------------------------------------------
+// One wave per (query token, kv head, group of 16 query heads): a query token of a chunk is a
+// decode row over the first kv_len - q_len + j + 1 tokens, so one kernel serves decode rows and
+// prefill chunks alike.  The two 128-dim halves of a head reuse the register layouts and the
+// loads of the 128-dim kernel (a half is 128 contiguous elements of the head's row); scores sum
+// over both halves, each half has its own accumulators.  No split over tokens, no prefetch
+// ahead of the block being consumed, and a chunk's tokens each stream the prefix again: this
+// path exists so that 256-dim heads work, it is not tuned.
+__device__ __forceinline__ int owner_of_token(const int32_t* cu_q_lens, int num_seqs, int tok) {
+  int lo = 0, hi = num_seqs;  // last i with cu_q_lens[i] <= tok (zero-length sequences are skipped)
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu_q_lens[mid] <= tok) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// grid = (row groups of 16 query heads, Hkv, token rows); block = one wave
+template <bool FP8, bool UNIFORM_PAGE>
+__global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int seq_begin, int seq_end) {
+  const int lane = threadIdx.x;
+  const int c = lane & 15, g = lane >> 4;
+  const int rg = blockIdx.x, hk = blockIdx.y;
+  const int tok_row = blockIdx.z + a.pt.cu_q_lens[seq_begin];
+  if (tok_row >= a.pt.cu_q_lens[seq_end]) return;
+  const int seq = owner_of_token(a.pt.cu_q_lens, seq_end, tok_row);
+  const int q0 = a.pt.cu_q_lens[seq];
+  const int q_len = a.pt.cu_q_lens[seq + 1] - q0;
+  const int kv_len = a.pt.kv_lens[seq];
+  const int qpos = kv_len - q_len + (tok_row - q0);
+  // tokens this row sees: [t_lo, t_hi)
+  const int t_hi = (a.sm.mask_mode == 0) ? qpos + 1 : kv_len;
+  if (t_hi <= 0) return;
+  const int t_lo = (a.sm.window > 0) ? max(0, qpos - a.sm.window + 1) : 0;
+
+  SeqView sv;
+  sv.page_size = a.pt.page_size;
+  sv.page_shift = ((sv.page_size & (sv.page_size - 1)) == 0) ? (31 - __builtin_clz(sv.page_size)) : -1;
+  sv.last_tok = t_hi - 1;
+  sv.pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[seq] / a.pt.page_size)
+                                                  : (int64_t)seq * a.pt.pages_per_seq);
+  constexpr int kHalfB = FP8 ? 128 : 256;  // bytes of 128 cached elements
+  const char* kh = a.kv.k_base + (int64_t)hk * a.kv.head_stride;
+  const char* vh = a.kv.v_base + (int64_t)hk * a.kv.head_stride;
+
+  // ---- Q^T operands: column c = query head (16 rg + c) of this kv head, both halves ----
+  const int row = rg * 16 + c;
+  u32x4_t qB[2][4];
+  {
+    const uint16_t* qp = a.q + ((int64_t)tok_row * a.Hq + (int64_t)hk * a.G + min(row, a.G - 1)) * 256;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const int d0 = hf * 128 + (FP8 ? (g * 32 + st * 8) : (st * 32 + g * 8));
+        qB[hf][st] = ld16(qp + d0);
+      }
+  }
+  const float scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[hk] : 1.0f);
+  const float temp = xai_factor(qpos, a.sm.xai_len);
+  const float cap = a.sm.soft_cap;
+  const float inv_cap = (cap != 0.f) ? 1.0f / cap : 0.f;
+  const float mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
+  const bool round_bf16 = a.sm.round_logits != 0;
+
+  f32x4_t acc[2][8];
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[hf][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int tb = t_lo & ~(kBlk - 1); tb < t_hi; tb += kBlk) {
+    int page = 0;
+    if constexpr (UNIFORM_PAGE) page = __builtin_amdgcn_readfirstlane(sv.pages[page_slot_of(sv, tb)]);
+    KvRegs<FP8> r0, r1;
+    load_block<FP8, UNIFORM_PAGE>(r0, sv, a.kv, kh, vh, tb, page, c, g);
+    load_block<FP8, UNIFORM_PAGE>(r1, sv, a.kv, kh + kHalfB, vh + kHalfB, tb, page, c, g);
+    f32x4_t s[2];
+    {
+      u32x4_t kA[2][4];
+      k_operands<FP8>(r0, kA);
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        s[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int st = 0; st < 4; ++st) s[b] = mfma16(kA[b][st], qB[0][st], s[b]);
+      }
+      k_operands<FP8>(r1, kA);
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int st = 0; st < 4; ++st) s[b] = mfma16(kA[b][st], qB[1][st], s[b]);
+    }
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float v = s[i >> 2][i & 3] * scale;
+      if (cap != 0.f) v = soft_cap_f(v, cap, inv_cap);
+      v = v * temp;
+      if (round_bf16) v = bf16_round(v);
+      v = v * kLog2e;
+      const int tok = tb + tok_slot(g, i);
+      x[i] = (tok >= t_hi || tok < t_lo) ? mask2 : v;
+    }
+    float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = fast_exp2(m - m_new);
+    float p[8], ps = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      p[i] = fast_exp2(x[i] - m_new);
+      ps += p[i];
+    }
+    l = l * alpha + ps;
+    m = m_new;
+    const u32x4_t pB = u32x4_t{pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
+                               pack_bf16x2(p[6], p[7])};
+    {
+      u32x4_t vA[8];
+      v_operands<FP8>(r0, vA);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[0][j] = mfma16(vA[j], pB, acc[0][j] * alpha);
+      v_operands<FP8>(r1, vA);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[1][j] = mfma16(vA[j], pB, acc[1][j] * alpha);
+    }
+  }
+
+  // ---- epilogue: lane (c, g) holds q row c, dims 128 hf + 32g + 8r + j in acc[hf][j][r] ----
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+  if (row >= a.G) return;
+  const int head = hk * a.G + row;
+  const float vs = a.v_scale ? a.v_scale[hk] : 1.0f;
+  const float inv = a.sm.sink ? vs * sink_inverse(m, l, sink_logit(a.sm.sink, a.sm.round_logits, head)) : vs / l;
+  uint16_t* op = a.out + ((int64_t)tok_row * a.Hq + head) * 256 + g * 32;
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      u32x4_t w;
+#pragma unroll
+      for (int jp = 0; jp < 4; ++jp) w[jp] = pack_bf16x2(acc[hf][2 * jp][r] * inv, acc[hf][2 * jp + 1][r] * inv);
+      st16(op + hf * 128 + r * 8, w);
+    }
+}
+
 // Merge the split partials: out = sum_j o_j 2^(m_j - m*) / sum_j l_j 2^(m_j - m*).
 // grid = (Hq, decode rows); block = one wave, 2 dims per lane (D = 128).  Lane j
 // first fetches (m_j, l_j) of split j, the wave reduces m* and the denominator
@@ -781,6 +941,21 @@ hipError_t launch_gather(const GatherArgs& a, hipStream_t stream) {
   const int64_t total = (int64_t)a.max_tokens * (a.row_bytes / 16);
   const int blocks = (int)((total + 255) / 256);
   hipLaunchKernelGGL(rpa_gather_kernel, dim3(blocks), dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int max_token_rows, hipStream_t stream) {
+  if (seq_end <= seq_begin || max_token_rows <= 0) return hipSuccess;
+  if (max_token_rows > 65535) return hipErrorInvalidValue;  // grid.z
+  const dim3 grid((a.G + 15) / 16, a.Hkv, max_token_rows), block(64);
+  const bool uniform = (a.pt.page_size % kBlk) == 0;
+  if (a.fp8) {
+    if (uniform) hipLaunchKernelGGL((rpa_rows256_kernel<true, true>), grid, block, 0, stream, a, seq_begin, seq_end);
+    else hipLaunchKernelGGL((rpa_rows256_kernel<true, false>), grid, block, 0, stream, a, seq_begin, seq_end);
+  } else {
+    if (uniform) hipLaunchKernelGGL((rpa_rows256_kernel<false, true>), grid, block, 0, stream, a, seq_begin, seq_end);
+    else hipLaunchKernelGGL((rpa_rows256_kernel<false, false>), grid, block, 0, stream, a, seq_begin, seq_end);
+  }
   return hipGetLastError();
 }
 

@@ -146,6 +146,9 @@ struct MlaWriteArgs {
 hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream);
 hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream);
 hipError_t launch_gather(const GatherArgs& a, hipStream_t stream);
+// head_dim 256: every query token of sequences [seq_begin, seq_end) as a row of its own; at most
+// max_token_rows tokens (a host bound) are covered
+hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int max_token_rows, hipStream_t stream);
 hipError_t launch_kv_write(const KvWriteArgs& a, hipStream_t stream);
 hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream);
 hipError_t launch_mla_kv_write(const MlaWriteArgs& a, hipStream_t stream);

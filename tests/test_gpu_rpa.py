@@ -485,3 +485,68 @@ def test_balanced_decode_plan_on_ragged_batches(pkg, wl, gpu, Hq, Hkv, window, k
     torch.testing.assert_close(auto.float(), one.float(), rtol=1e-2, atol=4e-3)
     for ns in (3, 50):
         torch.testing.assert_close(gpu_out(pkg, b, gpu, num_splits=ns).float(), one.float(), rtol=1e-2, atol=4e-3)
+
+
+# ------------------------------------------------------------------ head_dim 256
+def batch256(wl, name, q_lens, kv_lens, seed, Hq=8, Hkv=2, P=16, **mk):
+    return wl.make_batch(name, q_lens, kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=256, page_size=P,
+                         seed=seed, **mk)
+
+
+@pytest.mark.parametrize("Hq,Hkv,P", [(8, 2, 16), (32, 1, 64), (4, 4, 1), (40, 2, 24)])
+def test_head_dim_256_decode_and_prefill(pkg, wl, gpu, Hq, Hkv, P):
+    """256-wide heads (reference: head_dim padded to a multiple of 128, util.py:7-18) through the
+    row kernel: decode rows, chunks with and without a prefix, one-token sequences."""
+    q_lens = [1, 1, 1, 5, 33, 64, 1]
+    kv_lens = [1, 70, 257, 5, 100, 64, 31]
+    say(f"case d256 Hq={Hq} Hkv={Hkv} P={P}")
+    b = batch256(wl, "d256", q_lens, kv_lens, 91, Hq=Hq, Hkv=Hkv, P=P)
+    want = oracle_out(b)
+    got = gpu_out(pkg, b, gpu)
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+
+
+@pytest.mark.parametrize("window,cap,kv_dtype", [(40, None, torch.bfloat16), (None, 20.0, torch.bfloat16),
+                                                 (40, 20.0, torch.float8_e4m3fn), (None, None, torch.float8_e4m3fn)])
+def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
+    q_lens, kv_lens = [1, 1, 20, 50], [90, 300, 20, 130]
+    b = batch256(wl, "d256o", q_lens, kv_lens, 92, Hq=16, Hkv=4, P=32, kv_dtype=kv_dtype, sliding_window=window,
+                 soft_cap=cap)
+    sink = torch.from_numpy(np.random.RandomState(789).randn(16).astype(np.float32))
+    say(f"case d256 options window={window} cap={cap} {kv_dtype}")
+    tol = BF16_TOL if kv_dtype == torch.bfloat16 else FP8_TOL
+    for kw in ({}, {"attention_sink": sink}, {"xai_temperature_len": 64.0}, {"softmax_dtype": torch.bfloat16}):
+        torch.testing.assert_close(gpu_out(pkg, b, gpu, **kw).float(), oracle_out(b, **kw).float(), **tol)
+    # full attention (causal = 0 without a mask)
+    torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=False).float(), oracle_out(b, causal=False).float(), **tol)
+    with pytest.raises(ValueError, match="custom masks"):
+        gpu_out(pkg, b, gpu, causal=False, custom_mask=torch.ones(1, dtype=torch.int32))
+
+
+def test_head_dim_256_cache_write_and_gather(pkg, wl, gpu):
+    """The new-token write and the page gather take any head width (bit-exact)."""
+    q_lens, kv_lens = [1, 7], [33, 40]
+    b = batch256(wl, "d256w", q_lens, kv_lens, 93, Hq=4, Hkv=2, P=16)
+    g = b.to(gpu)
+    T = sum(q_lens)
+    keys = torch.randn(T, 2, 256, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    vals = torch.randn(T, 2, 256, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+    dist = b.distribution.cpu().numpy()
+    out, cache = pkg.ragged_paged_attention(
+        g.q, keys.to(gpu), vals.to(gpu), g.kv_cache.clone(), g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+        dist, None, sm_scale=b.sm_scale, max_kv_len=max(kv_lens), max_q_len=max(q_lens))
+    torch.cuda.synchronize()
+    from oracle.ref_rpa import merge_kv
+    want_cache = b.kv_cache.clone()
+    o = t = 0
+    for ql, kv in zip(q_lens, kv_lens):
+        for j in range(ql):
+            pos = kv - ql + j
+            page = int(b.page_indices[o + pos // 16])
+            want_cache[page, pos % 16] = merge_kv(keys[t : t + 1], vals[t : t + 1])[0]
+            t += 1
+        o += -(-kv // 16)
+    assert torch.equal(cache.cpu(), want_cache)
+    b.kv_cache = want_cache
+    torch.testing.assert_close(out[:T].cpu().float(), oracle_out(b).float(), **BF16_TOL)
