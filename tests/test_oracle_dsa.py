@@ -75,3 +75,15 @@ def test_page_lists_by_hand():
         page_size=8, pages_per_seq=6, k_pages_max=4, sentinel_page=99)
     assert kv_len.tolist() == [2 * 8 + 4 + 1, 0 * 8 + 0 + 1]
     assert pages.tolist() == [[50, 52, 54, 99], [99, 99, 99, 99]]
+
+
+def test_device_page_lists_agree_with_the_loops_on_cpu_tensors(pkg):
+    """compute_topk_pages is plain tensor code: it runs on CPU tensors too and must reproduce the
+    per-row loops, including rows with more touched pages than k_pages_max and empty rows."""
+    rng = np.random.default_rng(9)
+    topk = rng.integers(-1, 900, size=(7, 40)).astype(np.int32)
+    topk[3] = -1
+    for P, kp in ((16, 8), (64, 64), (1, 5)):
+        pps = -(-900 // P)
+        got = pkg.compute_topk_pages(torch.from_numpy(topk), page_size=P, pages_per_seq=pps, k_pages_max=kp)
+        assert np.array_equal(got.numpy(), topk_pages_ref(topk, P, pps, kp))
