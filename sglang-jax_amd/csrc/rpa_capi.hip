@@ -258,8 +258,6 @@ int rpa_validate(const RpaParams* p) {
     return fail(RPA_EUNSUPPORTED, "head_dim=%d: 128 and 256 are built", p->head_dim);
   if (p->head_dim == 256 && (p->mask_mode == RPA_MASK_CUSTOM || p->q_scale > 0.0f))
     return fail(RPA_EUNSUPPORTED, "head_dim=256: custom masks and q_scale are not built");
-  if (p->head_dim == 256 && p->num_tokens > 65535)
-    return fail(RPA_EUNSUPPORTED, "head_dim=256: at most 65535 tokens per call, got %d", p->num_tokens);
   if (p->kv_dtype != RPA_KV_BF16 && p->kv_dtype != RPA_KV_FP8_E4M3)
     return fail(RPA_EINVAL_DTYPE, "kv_dtype=%d is not a floating point cache dtype", p->kv_dtype);
   if (p->layout != RPA_LAYOUT_FUSED && p->layout != RPA_LAYOUT_SPLIT)
@@ -382,6 +380,8 @@ int rpa_decode(const RpaParams* p, void* stream) {
   if (p->decode_end <= 0) return RPA_OK;
   if (p->mask_mode == RPA_MASK_CUSTOM) return RPA_OK;  // masked rows all go through the prefill kernel
   if (p->head_dim == 256) return rows256(p, 0, p->decode_end, stream);
+  if (p->decode_end > 65535)  // rows sit on the second grid dimension
+    return fail(RPA_EUNSUPPORTED, "at most 65535 decode rows per call, got %d", p->decode_end);
   const SplitPlan sp = decode_plan(p);
   rpa::DecodeArgs a;
   a.q = static_cast<const uint16_t*>(p->q);
@@ -547,6 +547,9 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
     return fail(RPA_EINVAL_SHAPE, "decode rows=%d exceed tokens=%d", p->num_seqs, p->num_tokens);
   const int64_t rows = token_rows ? p->num_tokens : p->num_seqs;
   if (rows <= 0) return RPA_OK;
+  if (rows > 65535)  // rows sit on the second grid dimension
+    return fail(RPA_EUNSUPPORTED, "MLA: at most 65535 rows (%s) per call, got %lld",
+                token_rows ? "query tokens" : "sequences", (long long)rows);
   const SplitPlan sp = mla_plan(p, rows);
   rpa::MlaDecodeArgs a;
   a.ql_nope = static_cast<const uint16_t*>(p->ql_nope);

@@ -641,13 +641,13 @@ __device__ __forceinline__ int owner_of_token(const int32_t* cu_q_lens, int num_
   return lo;
 }
 
-// grid = (row groups of 16 query heads, Hkv, token rows); block = one wave
+// grid = (token rows, Hkv, row groups of 16 query heads); block = one wave
 template <bool FP8, bool UNIFORM_PAGE>
 __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int seq_begin, int seq_end) {
   const int lane = threadIdx.x;
   const int c = lane & 15, g = lane >> 4;
-  const int rg = blockIdx.x, hk = blockIdx.y;
-  const int tok_row = blockIdx.z + a.pt.cu_q_lens[seq_begin];
+  const int rg = blockIdx.z, hk = blockIdx.y;
+  const int tok_row = blockIdx.x + a.pt.cu_q_lens[seq_begin];
   if (tok_row >= a.pt.cu_q_lens[seq_end]) return;
   const int seq = owner_of_token(a.pt.cu_q_lens, seq_end, tok_row);
   const int q0 = a.pt.cu_q_lens[seq];
@@ -946,8 +946,8 @@ hipError_t launch_gather(const GatherArgs& a, hipStream_t stream) {
 
 hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int max_token_rows, hipStream_t stream) {
   if (seq_end <= seq_begin || max_token_rows <= 0) return hipSuccess;
-  if (max_token_rows > 65535) return hipErrorInvalidValue;  // grid.z
-  const dim3 grid((a.G + 15) / 16, a.Hkv, max_token_rows), block(64);
+  if (a.Hkv > 65535) return hipErrorInvalidValue;  // grid.y
+  const dim3 grid(max_token_rows, a.Hkv, (a.G + 15) / 16), block(64);
   const bool uniform = (a.pt.page_size % kBlk) == 0;
   if (a.fp8) {
     if (uniform) hipLaunchKernelGGL((rpa_rows256_kernel<true, true>), grid, block, 0, stream, a, seq_begin, seq_end);
