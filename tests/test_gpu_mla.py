@@ -180,3 +180,30 @@ def test_mla_new_rows_are_written_into_the_cache(pkg, wl, gpu, padded):
     torch.cuda.synchronize()
     assert torch.equal(got_cache.cpu().view(torch.int16), cache.view(torch.int16))
     torch.testing.assert_close(out.cpu()[:T].float(), want.float(), **TOL)
+
+
+def test_c5_full_size_page_permutation_invariance(pkg, wl, gpu):
+    """DeepSeek-V3 decode configuration at full size, no oracle: the output must not depend, bit
+    for bit, on where pages physically live, and the split plans must agree with a single pass."""
+    b = wl.config_c5(device=gpu)
+    n = int(b.distribution[2])
+    kw = dict(sm_scale=b.sm_scale, max_kv_len=int(max(b.meta["kv_lens"])))
+
+    def run(x, **extra):
+        out, _ = pkg.mla_ragged_paged_attention(x.ql_nope, x.q_pe, None, None, x.cache_kv, x.kv_lens, x.page_indices,
+                                                x.cu_q_lens, x.cu_kv_lens, (n, n, n), **kw, **extra)
+        torch.cuda.synchronize()
+        return out
+
+    a = run(b)
+    assert torch.isfinite(a.float()).all()
+    pool = b.cache_kv.shape[0]
+    perm = torch.randperm(pool, generator=torch.Generator().manual_seed(11)).to(gpu)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(pool, device=gpu)
+    c = b.to(gpu)
+    c.cache_kv = b.cache_kv[perm]  # new page j holds old page perm[j]
+    c.page_indices = inv[b.page_indices.long()].to(torch.int32)
+    assert torch.equal(a.view(torch.int16), run(c).view(torch.int16))
+    one = run(b, num_splits=1)
+    torch.testing.assert_close(a.float(), one.float(), rtol=1e-2, atol=4e-3)

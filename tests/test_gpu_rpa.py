@@ -313,15 +313,16 @@ def _permute_pages(b, seed):
     return c
 
 
-@pytest.mark.parametrize("name", ["config_c3", "config_c2"])
+@pytest.mark.parametrize("name", ["config_c3", "config_c2", "config_c4"])
 def test_full_size_page_permutation_invariance(pkg, wl, gpu, name):
     """Full benchmark size, no oracle: the output must not depend, bit for bit, on
     where pages physically live, and split-KV must agree with a single pass."""
-    scale = 1.0 if name == "config_c2" else 0.25  # C3 at 8192 tokens x 16 seqs = 0.5 GiB pool
+    scale = 0.25 if name == "config_c3" else 1.0  # C3 at 8192 tokens x 16 seqs = 0.5 GiB pool
     b = getattr(wl, name)(device=gpu, scale=scale)
     q_lens = b.q_lens()
     n = int(b.distribution[2])
-    kw = dict(sm_scale=b.sm_scale, max_kv_len=int(max(b.meta["kv_lens"])), max_q_len=int(q_lens[:n].max()))
+    kw = dict(sm_scale=b.sm_scale, max_kv_len=int(max(b.meta["kv_lens"])), max_q_len=int(q_lens[:n].max()),
+              k_scale=b.k_scale, v_scale=b.v_scale)
     dist = b.distribution.cpu().numpy()
 
     def run(x, **extra):
