@@ -551,3 +551,86 @@ def test_head_dim_256_cache_write_and_gather(pkg, wl, gpu):
     assert torch.equal(cache.cpu(), want_cache)
     b.kv_cache = want_cache
     torch.testing.assert_close(out[:T].cpu().float(), oracle_out(b).float(), **BF16_TOL)
+
+
+# ------------------------------------------------------------------ a captured step
+def test_a_captured_step_replays_with_new_lengths_and_page_tables(pkg, wl, gpu):
+    """One serving step -- cache write of the new tokens, decode rows, prefill chunks -- captured
+    in a HIP graph once and replayed on other queries, lengths and page tables of the same bounds:
+    the library reads lengths and page ids on the device and allocates nothing, so a replay must
+    match the oracle every time (checked on three replays with eager launches in between)."""
+    import importlib
+    RpaCall = importlib.import_module("sglang_jax_amd.ragged_paged_attention").RpaCall
+    P, Hq, Hkv = 16, 16, 4
+    q_lens = [1, 1, 1, 40, 100]
+    cases = [[50, 700, 128, 40, 300], [64, 33, 1000, 90, 100]]
+    batches = [wl.make_batch("graph", q_lens, kv, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=128, page_size=P,
+                             seed=95 + i) for i, kv in enumerate(cases)]
+    T, S = sum(q_lens), len(q_lens)
+    pool = max(b.kv_cache.shape[0] for b in batches)
+    n_pages = max(b.page_indices.numel() for b in batches)
+    st = dict(
+        q=torch.zeros(T, Hq, 128, dtype=torch.bfloat16, device=gpu),
+        cache=torch.zeros(pool, P, 2 * Hkv, 128, dtype=torch.bfloat16, device=gpu),
+        kv_lens=torch.zeros(S, dtype=torch.int32, device=gpu),
+        pages=torch.zeros(n_pages, dtype=torch.int32, device=gpu),
+        cu_q=batches[0].cu_q_lens.to(gpu),
+        cu_kv=torch.zeros(S + 1, dtype=torch.int32, device=gpu),
+        keys=torch.zeros(T, Hkv, 128, dtype=torch.bfloat16, device=gpu),
+        vals=torch.zeros(T, Hkv, 128, dtype=torch.bfloat16, device=gpu),
+    )
+
+    def stage(b):
+        """The batch into the static buffers; its newest rows leave the cache and arrive as keys / values."""
+        cache = b.kv_cache.clone()
+        k_pages, v_pages = split_fused_cache(cache)
+        keys = torch.zeros(T, Hkv, 128, dtype=torch.bfloat16)
+        vals = torch.zeros_like(keys)
+        o = t = 0
+        for ql, kv in zip(q_lens, b.meta["kv_lens"]):
+            for j in range(ql):
+                pos = int(kv) - ql + j
+                page = int(b.page_indices[o + pos // P])
+                keys[t], vals[t] = k_pages[page, pos % P], v_pages[page, pos % P]
+                cache[page, pos % P] = float("nan")
+                t += 1
+            o += -(-int(kv) // P)
+        st["q"].copy_(b.q)
+        st["cache"].zero_()
+        st["cache"][: cache.shape[0]].copy_(cache)
+        st["kv_lens"].copy_(b.kv_lens)
+        st["pages"].zero_()
+        st["pages"][: b.page_indices.numel()].copy_(b.page_indices)
+        st["cu_kv"].copy_(b.cu_kv_lens)
+        st["keys"].copy_(keys)
+        st["vals"].copy_(vals)
+
+    call = RpaCall(st["q"], st["cache"], None, st["kv_lens"], st["pages"], st["cu_q"], st["cu_kv"], num_seqs=S,
+                   decode_end=3, sm_scale=batches[0].sm_scale, max_kv_len=1024, max_q_len=max(q_lens))
+
+    def step():
+        call.kv_write(st["keys"], st["vals"])
+        call.attention()
+
+    stage(batches[0])
+    side = torch.cuda.Stream(device=gpu)
+    side.wait_stream(torch.cuda.current_stream(gpu))
+    with torch.cuda.stream(side):
+        step()  # warm-up outside the capture
+    torch.cuda.current_stream(gpu).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for which in (0, 1, 0):
+        b = batches[which]
+        say(f"case captured step, batch {which}")
+        stage(b)
+        call.out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        torch.testing.assert_close(call.out[:T].cpu().float(), oracle_out(b).float(), **BF16_TOL)
+        assert torch.equal(st["cache"][: b.kv_cache.shape[0]].cpu(), b.kv_cache)  # the new rows are back in place
+        # eager work between the replays
+        other = batches[1 - which]
+        torch.testing.assert_close(gpu_out(pkg, other, gpu).float(), oracle_out(other).float(), **BF16_TOL)
