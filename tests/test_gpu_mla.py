@@ -207,3 +207,32 @@ def test_c5_full_size_page_permutation_invariance(pkg, wl, gpu):
     assert torch.equal(a.view(torch.int16), run(c).view(torch.int16))
     one = run(b, num_splits=1)
     torch.testing.assert_close(a.float(), one.float(), rtol=1e-2, atol=4e-3)
+
+
+@pytest.mark.parametrize("seed", list(range(8)))
+def test_random_mla_batches_against_oracle(pkg, wl, gpu, seed):
+    """Seeded random decode and mixed batches, head counts, page sizes, window and soft cap."""
+    import numpy as np
+    rng = np.random.default_rng(3000 + seed)
+    Hq = int(rng.choice([16, 48, 128, 160]))
+    P = int(rng.choice([8, 16, 32, 64]))
+    n_dec, n_pre = int(rng.integers(0, 6)), int(rng.integers(0, 3))
+    if seed % 2 == 0:
+        n_pre = 0  # decode batches take the one-row-per-sequence entry point
+    if n_dec + n_pre == 0:
+        n_dec = 2
+    kv_dec = rng.integers(1, 2500, size=n_dec)
+    q_pre = rng.integers(2, 60, size=n_pre)
+    kv_pre = q_pre + rng.integers(0, 400, size=n_pre)
+    q_lens = [1] * n_dec + [int(x) for x in q_pre]
+    kv_lens = [int(x) for x in kv_dec] + [int(x) for x in kv_pre]
+    window = int(rng.integers(1, 300)) if rng.integers(0, 3) == 0 else None
+    cap = 30.0 if rng.integers(0, 3) == 0 else None
+    say(f"mla random seed={seed} Hq={Hq} P={P} q={q_lens} kv={kv_lens} window={window} cap={cap}")
+    b = wl.make_mla_batch("mla_rand", q_lens, kv_lens, num_q_heads=Hq, lkv_dim=512, rope_dim=64, page_size=P,
+                          seed=4000 + seed, sliding_window=window, soft_cap=cap)
+    want = oracle(b)
+    got = run_gpu(pkg, b, gpu)
+    T = sum(q_lens)
+    assert torch.isfinite(got[:T].float()).all()
+    torch.testing.assert_close(got[:T].float(), want.float(), **TOL)

@@ -634,3 +634,36 @@ def test_a_captured_step_replays_with_new_lengths_and_page_tables(pkg, wl, gpu):
         # eager work between the replays
         other = batches[1 - which]
         torch.testing.assert_close(gpu_out(pkg, other, gpu).float(), oracle_out(other).float(), **BF16_TOL)
+
+
+# ------------------------------------------------------------------ random shapes
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_random_batches_against_oracle(pkg, wl, gpu, seed):
+    """Seeded random mixes of decode rows and chunks, head shapes, page sizes, window, soft cap, sink
+    and cache type; every combination must match the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    G = int(rng.choice([1, 2, 4, 8, 16]))
+    P = int(rng.choice([1, 4, 16, 32, 64, 128]))
+    n_dec, n_pre = int(rng.integers(0, 6)), int(rng.integers(0, 4))
+    if n_dec + n_pre == 0:
+        n_dec = 1
+    kv_dec = rng.integers(1, 1500, size=n_dec)
+    q_pre = rng.integers(2, 200, size=n_pre)
+    kv_pre = q_pre + rng.integers(0, 600, size=n_pre) * rng.integers(0, 2, size=n_pre)
+    q_lens = [1] * n_dec + [int(x) for x in q_pre]
+    kv_lens = [int(x) for x in kv_dec] + [int(x) for x in kv_pre]
+    fp8 = bool(rng.integers(0, 2))
+    window = int(rng.integers(1, 400)) if rng.integers(0, 3) == 0 else None
+    cap = float(rng.choice([10.0, 30.0])) if rng.integers(0, 3) == 0 else None
+    kw = {}
+    if rng.integers(0, 3) == 0:
+        kw["attention_sink"] = torch.from_numpy(rng.standard_normal(Hkv * G).astype(np.float32))
+    say(f"case random seed={seed} Hkv={Hkv} G={G} P={P} q={q_lens} kv={kv_lens} fp8={fp8} window={window} cap={cap} {list(kw)}")
+    b = wl.make_batch("rand", q_lens, kv_lens, num_q_heads=Hkv * G, num_kv_heads=Hkv, head_dim=128, page_size=P,
+                      seed=2000 + seed, kv_dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16,
+                      sliding_window=window, soft_cap=cap)
+    want = oracle_out(b, **kw)
+    got = gpu_out(pkg, b, gpu, **kw)
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got.float(), want.float(), **(FP8_TOL if fp8 else BF16_TOL))
