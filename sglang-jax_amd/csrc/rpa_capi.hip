@@ -165,7 +165,7 @@ SplitPlan decode_plan(const RpaParams* p) {
   int64_t work = p->sum_decode_kv_len > 0 ? p->sum_decode_kv_len * per_row : 0;
   if (p->sliding_window > 0) work = 0;  // visible lengths are not the raw lengths
   return plan_splits(bound, p->sliding_window, units, work, p->num_splits,
-                     env_int("RPA_DECODE_MIN_CHUNK", 128), env_int("RPA_DECODE_WAVE_CAPACITY", wave_capacity()));
+                     env_int("RPA_DECODE_MIN_CHUNK", 64), env_int("RPA_DECODE_WAVE_CAPACITY", wave_capacity()));
 }
 
 // Balanced decode plan: a fixed number of waves (every wave slot of the GPU once) share the
@@ -189,7 +189,7 @@ bool use_balanced(const RpaParams* p, const SplitPlan& fixed) {
                                      p->cu_kv_lens != nullptr);
   const int nw = decode_waves_per_wg(p->num_kv_heads);
   const int64_t units = (int64_t)((p->num_kv_heads + nw - 1) / nw) * ((p->num_q_heads / p->num_kv_heads + 15) / 16);
-  const int64_t min_blocks = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 128) / 32);
+  const int64_t min_blocks = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 64) / 32);
   if ((int64_t)p->decode_end * ((bound + 31) / 32) * units <= (int64_t)decode_wgs(p->num_kv_heads) * min_blocks)
     return false;
   const bool equal_lengths = p->sum_decode_kv_len > 0 && p->max_kv_len > 0 &&
@@ -404,7 +404,7 @@ int rpa_decode(const RpaParams* p, void* stream) {
   a.balanced = use_balanced(p, sp) ? 1 : 0;
   a.num_wgs = decode_wgs(p->num_kv_heads);
   a.waves_per_wg = decode_waves_per_wg(p->num_kv_heads);
-  a.min_blocks_per_wave = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 128) / 32);
+  a.min_blocks_per_wave = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 64) / 32);
   a.forced_blocks_per_wave = 0;
   if (p->num_splits > 0) {  // the caller pins the partition: about num_splits pieces for the longest row
     const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
