@@ -275,27 +275,11 @@ struct PartDest {
   int64_t base;
 };
 
-// One wave, one (sequence, kv head, group of 16 query heads), tokens [t_begin, t_end).
-template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
-__device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int hk, int rg, int kv_len, int t_lo,
-                                               int t_begin, int t_end, const PartDest dest, int lane) {
-  const int c = lane & 15, g = lane >> 4;
-  const int nblk = (t_end - t_begin + kBlk - 1) / kBlk;
-
-  SeqView sv;
-  sv.page_size = a.pt.page_size;
-  sv.page_shift = ((sv.page_size & (sv.page_size - 1)) == 0) ? (31 - __builtin_clz(sv.page_size)) : -1;
-  sv.last_tok = kv_len - 1;
-  sv.pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[seq] / a.pt.page_size)
-                                                  : (int64_t)seq * a.pt.pages_per_seq);
-
-  const char* kh = a.kv.k_base + (int64_t)hk * a.kv.head_stride;
-  const char* vh = a.kv.v_base + (int64_t)hk * a.kv.head_stride;
-
-  // ---- Q^T operands: column c = query head (row0 + 16*mt + c) of this kv head ----
-  const int tq = a.pt.cu_q_lens[seq];
-  const int row0 = rg * 16 * MT;
-  u32x4_t qB[MT][4];
+// Q^T operands of one (query token, kv head, group of 16 query heads): column c = query head
+// row0 + 16*mt + c of the kv head, zero beyond the G real ones.
+template <int MT, bool FP8>
+__device__ __forceinline__ void load_queries(const DecodeArgs& a, int tq, int hk, int row0, int c, int g,
+                                             u32x4_t (&qB)[MT][4]) {
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int row = row0 + mt * 16 + c;
@@ -304,58 +288,26 @@ __device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int
     for (int st = 0; st < 4; ++st) {
       const int d0 = FP8 ? (g * 32 + st * 8) : (st * 32 + g * 8);
       qB[mt][st] = (row < a.G) ? ld16(qp + d0) : u32x4_t{0u, 0u, 0u, 0u};
-      if (a.sm.q_scale > 0.f) qB[mt][st] = requantise_q(qB[mt][st], a.sm.q_scale, FP8);
     }
   }
+}
 
-  ScoreOpts so;
-  const float ks = a.k_scale ? a.k_scale[hk] : 1.0f;
-  // the one query of a decode row sits at position kv_len - 1
-  const float temp = xai_factor(kv_len - 1, a.sm.xai_len);
-  so.scale = a.sm.sm_scale * ks * (a.sm.q_scale > 0.f ? a.sm.q_scale : 1.0f);
-  so.scale2 = so.scale * kLog2e * temp;
-  so.temp = temp;
-  so.round_bf16 = a.sm.round_logits != 0;
-  so.cap = a.sm.soft_cap;
-  so.inv_cap = (so.cap != 0.f) ? 1.0f / so.cap : 0.f;
-  so.mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
-  so.t_lo = t_lo;
-  so.kv_len = kv_len;
-
-  f32x4_t acc[MT][8];
-  float m[MT], l[MT];
+template <int MT, bool FP8>
+__device__ __forceinline__ void requantise_queries(const DecodeArgs& a, u32x4_t (&qB)[MT][4]) {
+  if (a.sm.q_scale > 0.f) {
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    m[mt] = -INFINITY;
-    l[mt] = 0.f;
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[mt][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int st = 0; st < 4; ++st) qB[mt][st] = requantise_q(qB[mt][st], a.sm.q_scale, FP8);
   }
+}
 
-  // ---- software pipeline: the loads of block i+1 are in flight while block i is consumed.
-  // The prefetch is unconditional (past the end it re-reads the last block) so that the
-  // number of outstanding loads is the same on every path and the waits stay partial; the
-  // page id of block i+2 is fetched while block i is consumed.
-  const int t_last = t_begin + (nblk - 1) * kBlk;
-  auto block_tok = [&](int b) { return min(t_begin + b * kBlk, t_last); };
-  auto page_of = [&](int tb) -> int {
-    if constexpr (UNIFORM_PAGE) return __builtin_amdgcn_readfirstlane(sv.pages[page_slot_of(sv, tb)]);
-    else return 0;
-  };
-  KvRegs<FP8> ra, rb;
-  int pg_next = page_of(block_tok(1));
-  load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, t_begin, page_of(t_begin), c, g);
-  for (int blk = 0; blk < nblk; blk += 2) {
-    load_block<FP8, UNIFORM_PAGE>(rb, sv, a.kv, kh, vh, block_tok(blk + 1), pg_next, c, g);
-    pg_next = page_of(block_tok(blk + 2));
-    compute_block<MT, FP8, CAP>(ra, qB, acc, m, l, so, t_begin + blk * kBlk, g);
-    if (blk + 1 >= nblk) break;
-    load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, block_tok(blk + 2), pg_next, c, g);
-    pg_next = page_of(block_tok(blk + 3));
-    compute_block<MT, FP8, CAP>(rb, qB, acc, m, l, so, t_begin + (blk + 1) * kBlk, g);
-  }
-
-  // ---- epilogue: lane (c, g) holds q row c, dims 32g + 8r + j in acc[mt][j][r] ----
+// Leave the result of one piece of work: lane (c, g) holds q row c, dims 32g + 8r + j in
+// acc[mt][j][r].
+template <int MT>
+__device__ __forceinline__ void write_rows(const DecodeArgs& a, const f32x4_t (&acc)[MT][8], const float (&m)[MT],
+                                           const float (&l)[MT], int tq, int hk, int row0, const PartDest dest,
+                                           int c, int g) {
   const float vs = a.v_scale ? a.v_scale[hk] : 1.0f;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -392,6 +344,84 @@ __device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int
       }
     }
   }
+}
+
+// One wave, one (sequence, kv head, group of 16 query heads), tokens [t_begin, t_end).
+template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
+__device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int hk, int rg, int kv_len, int t_lo,
+                                               int t_begin, int t_end, const PartDest dest, int lane) {
+  const int c = lane & 15, g = lane >> 4;
+  const int nblk = (t_end - t_begin + kBlk - 1) / kBlk;
+
+  SeqView sv;
+  sv.page_size = a.pt.page_size;
+  sv.page_shift = ((sv.page_size & (sv.page_size - 1)) == 0) ? (31 - __builtin_clz(sv.page_size)) : -1;
+  sv.last_tok = kv_len - 1;
+  // Sequence metadata and page ids go through the scalar cache: nothing writes them while the
+  // kernel runs, and a scalar load is not counted by vmcnt, so waiting for a page id never
+  // drains the block prefetch issued just before it.
+  seq = __builtin_amdgcn_readfirstlane(seq);
+  sv.pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (scalar_load_i32(a.pt.cu_kv_lens + seq) / a.pt.page_size)
+                                                  : (int64_t)seq * a.pt.pages_per_seq);
+
+  const char* kh = a.kv.k_base + (int64_t)hk * a.kv.head_stride;
+  const char* vh = a.kv.v_base + (int64_t)hk * a.kv.head_stride;
+
+  // ---- Q^T operands: column c = query head (row0 + 16*mt + c) of this kv head ----
+  const int tq = scalar_load_i32(a.pt.cu_q_lens + seq);
+  const int row0 = rg * 16 * MT;
+  u32x4_t qB[MT][4];
+  load_queries<MT, FP8>(a, tq, hk, row0, c, g, qB);
+  requantise_queries<MT, FP8>(a, qB);
+
+  ScoreOpts so;
+  const float ks = a.k_scale ? a.k_scale[hk] : 1.0f;
+  // the one query of a decode row sits at position kv_len - 1
+  const float temp = xai_factor(kv_len - 1, a.sm.xai_len);
+  so.scale = a.sm.sm_scale * ks * (a.sm.q_scale > 0.f ? a.sm.q_scale : 1.0f);
+  so.scale2 = so.scale * kLog2e * temp;
+  so.temp = temp;
+  so.round_bf16 = a.sm.round_logits != 0;
+  so.cap = a.sm.soft_cap;
+  so.inv_cap = (so.cap != 0.f) ? 1.0f / so.cap : 0.f;
+  so.mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
+  so.t_lo = t_lo;
+  so.kv_len = kv_len;
+
+  f32x4_t acc[MT][8];
+  float m[MT], l[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    m[mt] = -INFINITY;
+    l[mt] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[mt][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // ---- software pipeline: the loads of block i+1 are in flight while block i is consumed.
+  // The prefetch is unconditional (past the end it re-reads the last block) so that the
+  // number of outstanding loads is the same on every path and the waits stay partial; the
+  // page id of block i+2 is fetched while block i is consumed.
+  const int t_last = t_begin + (nblk - 1) * kBlk;
+  auto block_tok = [&](int b) { return min(t_begin + b * kBlk, t_last); };
+  auto page_of = [&](int tb) -> int {
+    if constexpr (UNIFORM_PAGE) return scalar_load_i32(sv.pages + __builtin_amdgcn_readfirstlane(page_slot_of(sv, tb)));
+    else return 0;
+  };
+  KvRegs<FP8> ra, rb;
+  int pg_next = page_of(block_tok(1));
+  load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, t_begin, page_of(t_begin), c, g);
+  for (int blk = 0; blk < nblk; blk += 2) {
+    load_block<FP8, UNIFORM_PAGE>(rb, sv, a.kv, kh, vh, block_tok(blk + 1), pg_next, c, g);
+    pg_next = page_of(block_tok(blk + 2));
+    compute_block<MT, FP8, CAP>(ra, qB, acc, m, l, so, t_begin + blk * kBlk, g);
+    if (blk + 1 >= nblk) break;
+    load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, block_tok(blk + 2), pg_next, c, g);
+    pg_next = page_of(block_tok(blk + 3));
+    compute_block<MT, FP8, CAP>(rb, qB, acc, m, l, so, t_begin + (blk + 1) * kBlk, g);
+  }
+
+  write_rows<MT>(a, acc, m, l, tq, hk, row0, dest, c, g);
 }
 
 // ---- fixed split plan: grid = (max_splits, decode rows, head groups * row groups); block = NW waves
@@ -489,23 +519,118 @@ __device__ __forceinline__ void locate_block(const DecodeArgs& a, int x, int uni
   }
 }
 
-// grid = num_wgs workgroups of NW = waves_per_wg waves
+// Wave-uniform facts of one decode row.
+struct RowMeta {
+  int seq;
+  int kv_len;
+  int nb;         // its 32-token blocks (0: nothing to read)
+  int64_t page0;  // index of its first page id in page_indices
+  int tq;         // its query token
+};
+
+struct RowLoads {  // the three words of a row, as loaded
+  int kv_len, cu_kv, tq;
+};
+
+__device__ __forceinline__ RowLoads row_issue_scalar(const DecodeArgs& a, int seq) {
+  RowLoads r;
+  r.kv_len = scalar_load_i32(a.pt.kv_lens + seq);
+  r.cu_kv = a.pt.cu_kv_lens ? scalar_load_i32(a.pt.cu_kv_lens + seq) : 0;
+  r.tq = scalar_load_i32(a.pt.cu_q_lens + seq);
+  return r;
+}
+
+__device__ __forceinline__ RowMeta row_resolve(const DecodeArgs& a, int seq, const RowLoads& r) {
+  RowMeta m;
+  m.seq = seq;
+  m.kv_len = r.kv_len;
+  m.nb = seq_blocks(r.kv_len, a.sm.window);
+  m.page0 = a.pt.cu_kv_lens ? (int64_t)(r.cu_kv / a.pt.page_size) : (int64_t)seq * a.pt.pages_per_seq;
+  m.tq = r.tq;
+  return m;
+}
+
+// A window of 64 consecutive page ids of a row, copied asynchronously into the wave's own LDS
+// slice (global_load_lds_dword, no register in between) and looked up with a uniform LDS read:
+// the steady state of a wave issues no small dependent global loads at all, and because no
+// register ever waits for the copy, the compiler never drains the vector-memory queue for it.
+// The copy is issued as inline assembly and its completion is the caller's business: loads
+// complete in order, so it has landed once any load issued after it has been waited for.
+struct PageWindow {
+  int32_t* lds;  // 64 ids of this wave
+  int first;     // slot of entry 0
+};
+
+__device__ __forceinline__ void request_window(const DecodeArgs& a, const RowMeta& row, PageWindow& w,
+                                               int first_slot, int page_shift, int lane) {
+  w.first = first_slot;
+  const int last_tok = max(row.kv_len - 1, 0);
+  const int last_slot = page_shift >= 0 ? (last_tok >> page_shift) : (last_tok / a.pt.page_size);
+  const int32_t* src = a.pt.page_indices + row.page0 + min(first_slot + lane, last_slot);
+  typedef const __attribute__((address_space(3))) char* lds_ptr_t;
+  const uint32_t m0v = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)w.lds));
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(m0v), "v"(src) : "memory", "m0");
+}
+
+__device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// One piece of work of a wave: tokens of one (row, kv head, group of 16 query heads).
+struct Piece {
+  RowMeta row;
+  int hk, rg;
+  int t_lo;     // first visible token (sliding window)
+  int t_first;  // first token of the piece (a multiple of 32 past the window's first block)
+  int nblk;     // its 32-token blocks
+  bool final_rows;
+};
+
+// grid = num_wgs workgroups of NW = waves_per_wg waves.
+//
+// A wave treats its share as one stream of blocks: the block prefetched behind the last block of
+// a piece is the first block of the next piece, the next row's lengths are fetched as scalar
+// loads while the current piece streams, its page ids arrive as one window load and its queries
+// are requested right behind that first block.  A piece border costs no round trip to memory,
+// and neither does a block: under load a small dependent load waits behind megabytes of queued
+// KV traffic (10 us and more), so there are none after the first block.
 template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
 __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const DecodeArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
+  const int c = lane & 15, g = lane >> 4;
   const int nw = a.waves_per_wg;
   const int wg = blockIdx.x;
   const int w = wg * nw + wave;
   const int row_groups = (a.G + 15) / 16;
   const int head_groups = (a.Hkv + nw - 1) / nw;
   const int units = head_groups * row_groups;
-  const int total = blocks_before(a, a.num_rows, lane) * units;
+  const int page_size = a.pt.page_size;
+  const int page_shift = ((page_size & (page_size - 1)) == 0) ? (31 - __builtin_clz(page_size)) : -1;
+
+  // ---- one pass over the rows: lengths, page offsets and query tokens of rows 0..63 stay in
+  // registers (most batches end there), the rest only adds to the total
+  int kv0 = 0, cu0 = 0, tq0 = 0;
+  if (lane < a.num_rows) {
+    kv0 = a.pt.kv_lens[lane];
+    cu0 = a.pt.cu_kv_lens ? a.pt.cu_kv_lens[lane] : 0;
+    tq0 = a.pt.cu_q_lens[lane];
+  }
+  const int nb0 = seq_blocks(kv0, a.sm.window);
+  const int incl0 = wave_inclusive_scan(nb0, lane);
+  int total_rows = uniform(__shfl(incl0, 63));
+  for (int s0 = 64; s0 < a.num_rows; s0 += 64) {
+    const int s = s0 + lane;
+    int nb = (s < a.num_rows) ? seq_blocks(a.pt.kv_lens[s], a.sm.window) : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) nb += __shfl_xor(nb, off);
+    total_rows += uniform(nb);
+  }
+  const int total = total_rows * units;
   const int pw = blocks_per_wave(a, total);
   if (wg == 0 && wave == 0) {
-    // the merge pass looks its sequences up in this prefix sum instead of scanning again
-    int base = 0;
-    for (int s0 = 0; s0 < a.num_rows; s0 += 64) {
+    // the merge pass looks its rows up in this prefix sum instead of scanning again
+    if (lane < a.num_rows) a.cu_blocks[lane + 1] = incl0;
+    int base = uniform(__shfl(incl0, 63));
+    for (int s0 = 64; s0 < a.num_rows; s0 += 64) {
       const int s = s0 + lane;
       const int nb = (s < a.num_rows) ? seq_blocks(a.pt.kv_lens[s], a.sm.window) : 0;
       const int incl = wave_inclusive_scan(nb, lane);
@@ -519,37 +644,208 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
   const int x_end = min(total, x + pw);
   const int x_first = x;
 
-  int seq, seq_first;
-  locate_block(a, x, units, lane, seq, seq_first);
-  seq = uniform(seq);
-  int kv_len = scalar_load_i32(a.pt.kv_lens + seq);
-  int nb = seq_blocks(kv_len, a.sm.window);
-  while (x < x_end) {
-    const int r = x - seq_first;
-    const int unit = r / nb;
-    const int blk = r - unit * nb;
-    const int take = min(nb - blk, x_end - x);
-    const int hg = unit / row_groups, rg = unit - hg * row_groups;
-    const int hk = hg * nw + wave;
-    const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
-    const int t0 = t_lo & ~(kBlk - 1);
-    PartDest dest;
-    dest.final_rows = (blk == 0) && (take == nb);
-    dest.by_head = false;
-    dest.base = ((int64_t)w * 2 + (x == x_first ? 0 : 1)) * 16;
-    if (hk < a.Hkv)
-      decode_segment<MT, FP8, UNIFORM_PAGE, CAP>(a, seq, hk, rg, kv_len, t_lo, t0 + blk * kBlk,
-                                                 min(kv_len, t0 + (blk + take) * kBlk), dest, lane);
-    x += take;
-    if (x < x_end && blk + take == nb && unit == units - 1) {
-      // next sequence that has any block (x < total guarantees there is one)
-      seq_first += nb * units;
-      do {
-        ++seq;
-        kv_len = scalar_load_i32(a.pt.kv_lens + seq);
-        nb = seq_blocks(kv_len, a.sm.window);
-      } while (nb == 0);
+  // ---- the row that holds block x
+  RowMeta row;
+  int row_first;  // linear index of the row's first block
+  {
+    const uint64_t hit = __builtin_amdgcn_ballot_w64(incl0 * units > x);
+    if (hit != 0) {
+      const int first = __builtin_ctzll(hit);
+      RowLoads rl;
+      rl.kv_len = __builtin_amdgcn_readlane(kv0, first);
+      rl.cu_kv = __builtin_amdgcn_readlane(cu0, first);
+      rl.tq = __builtin_amdgcn_readlane(tq0, first);
+      row = row_resolve(a, first, rl);
+      row_first = uniform(__builtin_amdgcn_readlane(incl0 - nb0, first) * units);
+    } else {
+      int seq;
+      locate_block(a, x, units, lane, seq, row_first);
+      seq = uniform(seq);
+      row = row_resolve(a, seq, row_issue_scalar(a, seq));
     }
+  }
+
+  auto make_piece = [&](const RowMeta& r, int unit, int blk, int take) {
+    Piece p;
+    p.row = r;
+    const int hg = unit / row_groups;
+    p.rg = unit - hg * row_groups;
+    // a head group may reach past the last kv head: such a wave repeats the last head and its
+    // result is dropped
+    p.hk = hg * nw + wave;
+    p.t_lo = (a.sm.window > 0) ? max(0, r.kv_len - a.sm.window) : 0;
+    p.t_first = (p.t_lo & ~(kBlk - 1)) + blk * kBlk;
+    p.nblk = take;
+    p.final_rows = (blk == 0) && (take == r.nb);
+    return p;
+  };
+  auto view_of = [&](const RowMeta& r) {
+    SeqView sv;
+    sv.page_size = page_size;
+    sv.page_shift = page_shift;
+    sv.last_tok = r.kv_len - 1;
+    sv.pages = a.pt.page_indices + r.page0;
+    return sv;
+  };
+  auto slot_of_tok = [&](int tok) { return page_shift >= 0 ? (tok >> page_shift) : (tok / page_size); };
+  auto page_in = [&](const PageWindow& pwn, int tok) -> int {
+    if constexpr (UNIFORM_PAGE) return uniform(pwn.lds[uniform(slot_of_tok(tok) - pwn.first)]);
+    else return 0;
+  };
+
+  Piece cur;
+  {
+    const int r = x - row_first;
+    const int unit = r / row.nb;
+    const int blk = r - unit * row.nb;
+    cur = make_piece(row, unit, blk, min(row.nb - blk, x_end - x));
+  }
+  int cur_unit = (x - row_first) / row.nb;
+  __shared__ int32_t lds_windows[4][2][64];  // [wave][current / next piece][entry]
+  PageWindow win = {lds_windows[wave][0], 0};
+  PageWindow nwin = {lds_windows[wave][1], 0};
+  if constexpr (UNIFORM_PAGE) request_window(a, cur.row, win, slot_of_tok(cur.t_first), page_shift, lane);
+  u32x4_t qB[MT][4];
+  load_queries<MT, FP8>(a, cur.row.tq, min(cur.hk, a.Hkv - 1), cur.rg * 16 * MT, c, g, qB);
+  if constexpr (UNIFORM_PAGE) wait_all_loads();  // the window (and the queries behind it)
+
+  KvRegs<FP8> ra, rb;
+  bool in_b = false;  // which register set holds the block about to be consumed
+  {
+    const SeqView sv = view_of(cur.row);
+    const int hk = min(cur.hk, a.Hkv - 1);
+    load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, a.kv.k_base + (int64_t)hk * a.kv.head_stride,
+                                  a.kv.v_base + (int64_t)hk * a.kv.head_stride, cur.t_first,
+                                  page_in(win, cur.t_first), c, g);
+  }
+
+  for (;;) {
+    // ---- this piece
+    const int hk = min(cur.hk, a.Hkv - 1);
+    const SeqView sv = view_of(cur.row);
+    const char* kh = a.kv.k_base + (int64_t)hk * a.kv.head_stride;
+    const char* vh = a.kv.v_base + (int64_t)hk * a.kv.head_stride;
+    requantise_queries<MT, FP8>(a, qB);
+    ScoreOpts so;
+    {
+      const float ks = a.k_scale ? a.k_scale[hk] : 1.0f;
+      const float temp = xai_factor(cur.row.kv_len - 1, a.sm.xai_len);  // the one query sits at kv_len - 1
+      so.scale = a.sm.sm_scale * ks * (a.sm.q_scale > 0.f ? a.sm.q_scale : 1.0f);
+      so.scale2 = so.scale * kLog2e * temp;
+      so.temp = temp;
+      so.round_bf16 = a.sm.round_logits != 0;
+      so.cap = a.sm.soft_cap;
+      so.inv_cap = (so.cap != 0.f) ? 1.0f / so.cap : 0.f;
+      so.mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
+      so.t_lo = cur.t_lo;
+      so.kv_len = cur.row.kv_len;
+    }
+    f32x4_t acc[MT][8];
+    float m[MT], l[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      m[mt] = -INFINITY;
+      l[mt] = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[mt][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // ---- the piece after it: the next unit of the same row, or the first unit of the next row
+    // that has any block (has_next guarantees there is one)
+    const bool has_next = x + cur.nblk < x_end;
+    const bool next_row = has_next && (cur_unit == units - 1);
+    int nseq = cur.row.seq + 1;
+    RowLoads nl = {0, 0, 0};
+    if (next_row) nl = row_issue_scalar(a, nseq);
+    Piece nxt = cur;
+    SeqView nsv = sv;
+    const char* nkh = kh;
+    const char* nvh = vh;
+    // resolved one block into the piece when it has more than one block, at once otherwise
+    const int resolve_at = (cur.nblk > 1) ? 1 : 0;
+
+    auto step = [&](int i, const KvRegs<FP8>& use, KvRegs<FP8>& fill) __attribute__((always_inline)) {
+      if (has_next && i == resolve_at) {
+        RowMeta nrow = cur.row;
+        int nunit = cur_unit + 1;
+        if (next_row) {
+          nrow = row_resolve(a, nseq, nl);
+          while (nrow.nb == 0) {  // rows without tokens (padding)
+            ++nseq;
+            nrow = row_resolve(a, nseq, row_issue_scalar(a, nseq));
+          }
+          nunit = 0;
+        }
+        const int x_next = x + cur.nblk;
+        nxt = make_piece(nrow, nunit, 0, min(nrow.nb, x_end - x_next));
+        if constexpr (UNIFORM_PAGE) request_window(a, nrow, nwin, slot_of_tok(nxt.t_first), page_shift, lane);
+        nsv = view_of(nrow);
+        const int nhk = min(nxt.hk, a.Hkv - 1);
+        nkh = a.kv.k_base + (int64_t)nhk * a.kv.head_stride;
+        nvh = a.kv.v_base + (int64_t)nhk * a.kv.head_stride;
+      }
+      const int tb = cur.t_first + i * kBlk;
+      const bool last = (i + 1 == cur.nblk);
+      // the block to request now: the next one of this piece, the first one of the next piece,
+      // or (nothing left) this block again, so that every path has the same loads in flight
+      if constexpr (UNIFORM_PAGE) {
+        if (!last && slot_of_tok(tb + kBlk) - win.first >= 64) {  // every 64 pages
+          request_window(a, cur.row, win, slot_of_tok(tb + kBlk), page_shift, lane);
+          wait_all_loads();
+        }
+      }
+      // real branches, not selects: looking a page up in the next piece's window must not make
+      // every block wait for that window
+      if (last && has_next) {
+        // The next piece's window was requested at block resolve_at, in front of that block's
+        // prefetch.  Two blocks later a wait for younger loads has passed; earlier it has not.
+        if (UNIFORM_PAGE && i <= resolve_at + 1) wait_all_loads();
+        load_block<FP8, UNIFORM_PAGE>(fill, nsv, a.kv, nkh, nvh, nxt.t_first, page_in(nwin, nxt.t_first), c, g);
+      } else {
+        const int ptb = last ? tb : tb + kBlk;
+        load_block<FP8, UNIFORM_PAGE>(fill, sv, a.kv, kh, vh, ptb, page_in(win, ptb), c, g);
+      }
+      compute_block<MT, FP8, CAP>(use, qB, acc, m, l, so, tb, g);
+    };
+    // the piece's first block sits in ra or in rb, wherever the piece before it ended
+    {
+      int i = 0;
+      bool skip_a = in_b;
+      for (;;) {
+        if (!skip_a) {
+          step(i, ra, rb);
+          if (++i == cur.nblk) {
+            in_b = true;
+            break;
+          }
+        }
+        skip_a = false;
+        step(i, rb, ra);
+        if (++i == cur.nblk) {
+          in_b = false;
+          break;
+        }
+      }
+    }
+
+    if (cur.hk < a.Hkv) {
+      PartDest dest;
+      dest.final_rows = cur.final_rows;
+      dest.by_head = false;
+      dest.base = ((int64_t)w * 2 + (x == x_first ? 0 : 1)) * 16;
+      write_rows<MT>(a, acc, m, l, cur.row.tq, hk, cur.rg * 16 * MT, dest, c, g);
+    }
+    if (!has_next) break;
+    x += cur.nblk;
+    cur_unit = next_row ? 0 : cur_unit + 1;
+    cur = nxt;
+    {  // the two LDS windows trade places
+      const PageWindow t = win;
+      win = nwin;
+      nwin = t;
+    }
+    // the queries queue up right behind the piece's first block, which is already on its way
+    load_queries<MT, FP8>(a, cur.row.tq, min(cur.hk, a.Hkv - 1), cur.rg * 16 * MT, c, g, qB);
   }
 }
 

@@ -488,6 +488,28 @@ def test_balanced_decode_plan_on_ragged_batches(pkg, wl, gpu, Hq, Hkv, window, k
         torch.testing.assert_close(gpu_out(pkg, b, gpu, num_splits=ns).float(), one.float(), rtol=1e-2, atol=4e-3)
 
 
+def test_balanced_plan_long_shares_and_tiny_rows(pkg, wl, gpu, monkeypatch):
+    """Eight workgroups for the whole batch (the wave capacity is an environment knob): a share is
+    131 blocks, so one wave walks more than 64 pages of a long row (its page-id window is
+    refilled on the way) and another crosses rows of 1, 33, 64 and 70 tokens in one go (pieces
+    of one to three blocks, each prefetched behind the piece before it)."""
+    monkeypatch.setenv("RPA_DECODE_WAVE_CAPACITY", "16")
+    kv_lens = [9000, 5000, 70, 1, 12000, 64, 33, 7000]
+    for Hq, Hkv, kv_dtype, window in ((8, 2, torch.bfloat16, None), (16, 2, torch.float8_e4m3fn, None),
+                                      (8, 2, torch.bfloat16, 5000)):
+        say(f"long shares Hq={Hq} Hkv={Hkv} {kv_dtype} window={window}")
+        b = wl.make_batch("long_shares", [1] * len(kv_lens), kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=128,
+                          page_size=64, seed=95, kv_dtype=kv_dtype, sliding_window=window)
+        want = oracle_out(b)
+        tol = FP8_TOL if kv_dtype != torch.bfloat16 else BF16_TOL
+        auto = gpu_out(pkg, b, gpu)
+        one = gpu_out(pkg, b, gpu, num_splits=1)
+        torch.testing.assert_close(auto.float(), want.float(), **tol)
+        torch.testing.assert_close(auto.float(), one.float(), rtol=1e-2, atol=4e-3)
+        again = gpu_out(pkg, b, gpu)
+        assert torch.equal(auto, again)
+
+
 # ------------------------------------------------------------------ head_dim 256
 def batch256(wl, name, q_lens, kv_lens, seed, Hq=8, Hkv=2, P=16, **mk):
     return wl.make_batch(name, q_lens, kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=256, page_size=P,
