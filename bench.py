@@ -50,9 +50,9 @@ DECODE_KERNEL = {
 }
 
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", "rpa_prefill_async_kernel"): 364.7e6 + 77.5e6,
-    ("c2", "rpa_decode_balanced_kernel"): 505.7e6 + 5.1e6,
-    ("c3", "rpa_decode_splitkv_kernel"): 2150.1e6 + 4.3e6,
+    ("c2", "rpa_prefill_async_kernel"): 362.7e6 + 77.5e6,
+    ("c2", "rpa_decode_balanced_kernel"): 504.3e6 + 5.1e6,
+    ("c3", "rpa_decode_splitkv_kernel"): 2149.9e6 + 4.3e6,
     ("c5", "rpa_mla_balanced_kernel"): 810.7e6 + 85.9e6,
 }
 
