@@ -5,8 +5,8 @@
 // workgroup of 8 waves owns one (sequence, kv split) and 128 heads (wave w owns
 // heads 16w..16w+15), so each latent row is fetched from HBM exactly once:
 //   global -> LDS   global_load_lds_dwordx4 copies 32-token tiles (rows of 72
-//                   16-byte chunks, row-major, XOR-swizzled) into a 3-slot ring,
-//                   two tiles ahead of the MFMAs; no staging registers
+//                   16-byte chunks, row-major) into a 4-slot ring,
+//                   three tiles ahead of the MFMAs; no staging registers
 //   S^T[tok, head] = K . Q^T       36 MFMA 16x16x32 per wave and tile, A = rows
 //                                  read with ds_read_b128, B = Q^T in registers
 //   online softmax, P rounded to bf16 (as the reference rounds it)
@@ -34,7 +34,8 @@ namespace {
 constexpr int kTok = 32;                 // tokens per tile
 constexpr int kRowB = 1184;              // latent row in LDS: 576 bf16 + 32 bytes of padding
 constexpr int kChunks = 74;              // 16-byte chunks per row (72 data + 2 pad)
-constexpr int kSlotB = 40 * 1024;        // one ring slot: 40 copy blocks of 64 chunks (37 used)
+constexpr int kUsedBlocks = 37;          // copy blocks of 64 chunks that hold a tile (32 rows x 74 chunks)
+constexpr int kSlotB = kUsedBlocks * 1024;  // one ring slot
 constexpr int kCopiesPerWave = 5;        // every wave issues 5 copy instructions per tile
 
 __device__ __forceinline__ u32x4_t lds_ld16(const char* p) { return *reinterpret_cast<const u32x4_t*>(p); }
@@ -64,10 +65,17 @@ __device__ __forceinline__ int page_slot(const Src& s, int tok) {
 }
 
 // A lane's 5 chunks of a tile: position p = 64*(5*wave + n) + lane; row p / 74, chunk
-// column p % 74.  The pad columns and positions >= 32*74 copy the tile's first chunk.
+// column p % 74.  The pad columns copy the tile's first chunk.
+// The 8 x 5 = 40 copy instructions of a tile cover 37 blocks: the last three repeat block 0
+// (same source, same destination, same bytes), so every wave has the same number of copies
+// in flight and the slot is exactly 37 KiB.
+__device__ __forceinline__ int copy_block(int wave, int n) {
+  const int blk = wave * kCopiesPerWave + n;
+  return blk < kUsedBlocks ? blk : 0;
+}
+
 __device__ __forceinline__ void chunk_of(const Src& s, int wave, int lane, int n, int& row, int& inner) {
-  int p = (wave * kCopiesPerWave + n) * 64 + lane;
-  if (p >= kTok * kChunks) p = 0;
+  const int p = copy_block(wave, n) * 64 + lane;
   row = p / kChunks;
   int j = p - row * kChunks;
   if (j >= 72) { row = 0; j = 0; }
@@ -91,7 +99,7 @@ __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* 
       for (int n = 0; n < kCopiesPerWave; ++n) {
         int row, inner;
         chunk_of(s, wave, ln, n, row, inner);
-        async_copy16(base + (uint32_t)(row * s.row_bytes + inner), slot + (wave * kCopiesPerWave + n) * 1024);
+        async_copy16(base + (uint32_t)(row * s.row_bytes + inner), slot + copy_block(wave, n) * 1024);
       }
       return;
     }
@@ -105,7 +113,7 @@ __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* 
     const int ps = page_slot(s, tok);
     const int pg = UNIFORM ? page : s.pages[ps];
     const char* src = cache + (int64_t)pg * s.page_stride + (int64_t)(tok - ps * s.page_size) * s.row_bytes + inner;
-    async_copy16(src, slot + (wave * kCopiesPerWave + n) * 1024);
+    async_copy16(src, slot + copy_block(wave, n) * 1024);
   }
 }
 
@@ -165,7 +173,7 @@ struct MlaDest {
 template <bool UNIFORM, bool CAP>
 __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
                                             int t_begin, int t_end, const MlaDest dest, char* slot0, char* slot1,
-                                            char* slot2) {
+                                            char* slot2, char* slot3) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -224,23 +232,25 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   for (int j = 0; j < 32; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  // ---- pipeline: copies run two tiles ahead of the MFMAs (3-slot ring) ----
-  int pg_next = page_of(t_begin + 2 * kTok);
+  // ---- pipeline: copies run three tiles ahead of the MFMAs (4-slot ring, 148 of the CU's 160 KiB:
+  // 111 KiB per CU in flight, which is what HBM latency under load asks for) ----
+  int pg_next = page_of(t_begin + 3 * kTok);
   copy_tile<UNIFORM>(slot0, src, a.cache, t_begin, wave, lane, page_of(t_begin));
   copy_tile<UNIFORM>(slot1, src, a.cache, t_begin + kTok, wave, lane, page_of(t_begin + kTok));
+  copy_tile<UNIFORM>(slot2, src, a.cache, t_begin + 2 * kTok, wave, lane, page_of(t_begin + 2 * kTok));
   // Touch every Q^T register here: the compiler then waits for the Q loads now, instead of
   // re-checking them with s_waitcnt vmcnt(0..4) inside the loop, where such a wait would also
   // drain the copy queue.
 #pragma unroll
   for (int ks = 0; ks < 18; ++ks) asm volatile("" ::"v"(qB[ks]));
-  // wait for the first tile (all but the 5 newest copies), then meet
-  __builtin_amdgcn_s_waitcnt(0x0F70 | kCopiesPerWave);
+  // wait for the first tile (all but the 10 newest copies), then meet
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kCopiesPerWave));
   __syncthreads();
 
   auto tile_step = [&](const char* cur, char* fill, int tb) {
     // `fill` held tile tb - 32, which every wave finished before the last barrier
-    copy_tile<UNIFORM>(fill, src, a.cache, tb + 2 * kTok, wave, lane, pg_next);
-    pg_next = page_of(tb + 3 * kTok);
+    copy_tile<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane, pg_next);
+    pg_next = page_of(tb + 4 * kTok);
     if (wave_on) {
       // two independent accumulator chains (token halves), issued alternately
       f32x4_t s[2];
@@ -299,22 +309,24 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
         if (j % 2 == 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // Tile tb + 32 has landed once at most the 5 copies of tile tb + 64 are outstanding.  A bare
+    // Tile tb + 32 has landed once at most the 10 copies of tiles tb + 64 and tb + 96 are outstanding.  A bare
     // s_barrier is used instead of __syncthreads(): the fence in the latter makes the compiler
     // wait for ALL outstanding copies, which would shorten the prefetch distance to one tile.
     // Every LDS read of this tile has returned (its MFMA consumed it) before the barrier, and
     // each wave has waited for its own share of the next tile, so no fence is needed.
-    __builtin_amdgcn_s_waitcnt(0x0F70 | kCopiesPerWave);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kCopiesPerWave));
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
-  for (int tb = t_begin; tb < t_end; tb += 3 * kTok) {
-    tile_step(slot0, slot2, tb);
+  for (int tb = t_begin; tb < t_end; tb += 4 * kTok) {
+    tile_step(slot0, slot3, tb);
     if (tb + kTok >= t_end) break;
     tile_step(slot1, slot0, tb + kTok);
     if (tb + 2 * kTok >= t_end) break;
     tile_step(slot2, slot1, tb + 2 * kTok);
+    if (tb + 3 * kTok >= t_end) break;
+    tile_step(slot3, slot2, tb + 3 * kTok);
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the copies issued past the end
 
@@ -351,6 +363,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot3[kSlotB];
   const int row_id = blockIdx.y, split = blockIdx.x;
   const MlaRow mr = mla_row(a, row_id);
   if (!mr.valid) return;
@@ -364,7 +377,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   MlaDest dest;
   dest.final_rows = a.max_splits == 1;
   dest.base = ((int64_t)row_id * a.max_splits + split) * a.Hq;
-  mla_segment<UNIFORM, CAP>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2);
+  mla_segment<UNIFORM, CAP>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
 }
 
 // ---- balanced plan (one row per sequence): the 32-token tiles of the whole batch, sequence by
@@ -388,6 +401,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
   __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot3[kSlotB];
   const int lane = threadIdx.x & 63;
   const int wg = blockIdx.x;
   const int units = (a.Hq + 127) / 128;
@@ -465,7 +479,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
     dest.final_rows = (tile == 0) && (take == nt);
     dest.base = ((int64_t)wg * 2 + (x == x_first ? 0 : 1)) * 128 - unit * 128;  // + head
     mla_segment<UNIFORM, CAP>(a, mr, unit * 128, t_lo, t0 + tile * kTok, min(kv_len, t0 + (tile + take) * kTok),
-                              dest, slot0, slot1, slot2);
+                              dest, slot0, slot1, slot2, slot3);
     x += take;
     if (x < x_end && tile + take == nt && unit == units - 1) {
       seq_first += nt * units;
