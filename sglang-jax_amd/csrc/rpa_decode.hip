@@ -849,6 +849,94 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
   }
 }
 
+// Merge the n partial rows of one (decode row, query head) and write the finished row.
+// slot_of(j) is the workspace slot of partial j.  One wave, 2 dims per lane.  Up to 16 partials
+// (nearly always) everything is requested at once -- the (max, sum) pairs by lanes 0..n-1, the
+// partial rows by all lanes, the row's query token before either -- so the merge costs one round
+// trip to memory instead of three dependent ones.
+template <int N, typename SlotOf>
+__device__ __forceinline__ void merge_few(const DecodeArgs& a, int n, int lane, SlotOf slot_of, float& mstar,
+                                          float& den, float& o0, float& o1) {
+  const int d = lane * 2;
+  float mj = -INFINITY, lj = 0.f;
+  if (lane < n) {
+    const int64_t slot = slot_of(lane);
+    mj = a.ws_ml[slot * 2];
+    lj = a.ws_ml[slot * 2 + 1];
+  }
+  f32x2_t o[N];
+#pragma unroll
+  for (int u = 0; u < N; ++u) o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + slot_of(min(u, n - 1)) * 128 + d);
+  mstar = mj;
+#pragma unroll
+  for (int off = N / 2; off > 0; off >>= 1) mstar = fmaxf(mstar, __shfl_xor(mstar, off));
+  mstar = __shfl(mstar, 0);
+  const float wj = (lane < n) ? fast_exp2(mj - mstar) : 0.f;
+  den = lj * wj;
+#pragma unroll
+  for (int off = N / 2; off > 0; off >>= 1) den += __shfl_xor(den, off);
+  den = __shfl(den, 0);
+  o0 = 0.f;
+  o1 = 0.f;
+#pragma unroll
+  for (int u = 0; u < N; ++u) {
+    const float wu = __shfl(wj, u);  // 0 beyond n: the repeated last row does not count
+    o0 += o[u][0] * wu;
+    o1 += o[u][1] * wu;
+  }
+}
+
+template <typename SlotOf>
+__device__ __forceinline__ void merge_rows(const DecodeArgs& a, int seq, int head, int n, int lane, SlotOf slot_of) {
+  const int d = lane * 2;
+  const int tq = scalar_load_i32(a.pt.cu_q_lens + seq);
+  float mstar = -INFINITY, den = 0.f, o0 = 0.f, o1 = 0.f;
+  if (n <= 8) {
+    merge_few<8>(a, n, lane, slot_of, mstar, den, o0, o1);
+  } else if (n <= 16) {
+    merge_few<16>(a, n, lane, slot_of, mstar, den, o0, o1);
+  } else {
+    for (int j0 = 0; j0 < n; j0 += 64) {
+      const int j = j0 + lane;
+      float mj = (j < n) ? a.ws_ml[slot_of(j) * 2] : -INFINITY;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) mj = fmaxf(mj, __shfl_xor(mj, off));
+      mstar = fmaxf(mstar, mj);
+    }
+    for (int j0 = 0; j0 < n; j0 += 64) {
+      const int j = j0 + lane;
+      float wj = 0.f, lj = 0.f;
+      if (j < n) {
+        const int64_t slot = slot_of(j);
+        wj = fast_exp2(a.ws_ml[slot * 2] - mstar);
+        lj = a.ws_ml[slot * 2 + 1] * wj;
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) lj += __shfl_xor(lj, off);
+      den += lj;
+      const int cnt = min(64, n - j0);
+      for (int jj = 0; jj < cnt; jj += 8) {
+        f32x2_t o[8];
+        float wv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int js = min(jj + u, cnt - 1);
+          wv[u] = (jj + u < cnt) ? __shfl(wj, js) : 0.f;
+          o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + slot_of(j0 + js) * 128 + d);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          o0 += o[u][0] * wv[u];
+          o1 += o[u][1] * wv[u];
+        }
+      }
+    }
+  }
+  const float inv = a.sm.sink ? sink_inverse(mstar, den, sink_logit(a.sm.sink, a.sm.round_logits, head)) : 1.0f / den;
+  uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * 128 + d);
+  *op = pack_bf16x2(o0 * inv, o1 * inv);
+}
+
 // Merge the partial rows of the balanced plan.  grid = (Hq, decode rows); block = one wave.
 __global__ __launch_bounds__(64) void rpa_combine_balanced_kernel(const DecodeArgs a) {
   const int head = blockIdx.x;
@@ -876,48 +964,7 @@ __global__ __launch_bounds__(64) void rpa_combine_balanced_kernel(const DecodeAr
     const int part = ((int64_t)wj * pw >= first_block) ? 0 : 1;
     return (((int64_t)wj * nw + wv) * 2 + part) * 16 + r16;
   };
-  const int d = lane * 2;
-  float mstar = -INFINITY;
-  for (int j0 = 0; j0 < n; j0 += 64) {
-    const int j = j0 + lane;
-    float mj = (j < n) ? a.ws_ml[slot_of(j) * 2] : -INFINITY;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mj = fmaxf(mj, __shfl_xor(mj, off));
-    mstar = fmaxf(mstar, mj);
-  }
-  float den = 0.f, o0 = 0.f, o1 = 0.f;
-  for (int j0 = 0; j0 < n; j0 += 64) {
-    const int j = j0 + lane;
-    float wj = 0.f, lj = 0.f;
-    if (j < n) {
-      const int64_t slot = slot_of(j);
-      wj = fast_exp2(a.ws_ml[slot * 2] - mstar);
-      lj = a.ws_ml[slot * 2 + 1] * wj;
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) lj += __shfl_xor(lj, off);
-    den += lj;
-    const int cnt = min(64, n - j0);
-    for (int jj = 0; jj < cnt; jj += 8) {
-      f32x2_t o[8];
-      float wv[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int js = min(jj + u, cnt - 1);
-        wv[u] = (jj + u < cnt) ? __shfl(wj, js) : 0.f;
-        o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + slot_of(j0 + js) * 128 + d);
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        o0 += o[u][0] * wv[u];
-        o1 += o[u][1] * wv[u];
-      }
-    }
-  }
-  const float inv = a.sm.sink ? sink_inverse(mstar, den, sink_logit(a.sm.sink, a.sm.round_logits, head)) : 1.0f / den;
-  const int tq = a.pt.cu_q_lens[seq];
-  uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * 128 + d);
-  *op = pack_bf16x2(o0 * inv, o1 * inv);
+  merge_rows(a, seq, head, n, lane, slot_of);
 }
 
 // ---- head_dim 256 ---------------------------------------------------------------------------
@@ -1084,48 +1131,7 @@ __global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a) {
   const int n = min(a.max_splits, (kv_len - t0 + a.chunk - 1) / a.chunk);
   if (n <= 0) return;
   const int64_t base = ((int64_t)seq * a.max_splits) * a.Hq + head;
-  const int d = lane * 2;
-  float mstar = -INFINITY;
-  for (int j0 = 0; j0 < n; j0 += 64) {
-    const int j = j0 + lane;
-    float mj = (j < n) ? a.ws_ml[(base + (int64_t)j * a.Hq) * 2] : -INFINITY;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mj = fmaxf(mj, __shfl_xor(mj, off));
-    mstar = fmaxf(mstar, mj);
-  }
-  float den = 0.f, o0 = 0.f, o1 = 0.f;
-  for (int j0 = 0; j0 < n; j0 += 64) {
-    const int j = j0 + lane;
-    float wj = 0.f, lj = 0.f;
-    if (j < n) {
-      const int64_t slot = base + (int64_t)j * a.Hq;
-      wj = fast_exp2(a.ws_ml[slot * 2] - mstar);
-      lj = a.ws_ml[slot * 2 + 1] * wj;
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) lj += __shfl_xor(lj, off);
-    den += lj;
-    const int cnt = min(64, n - j0);
-    for (int jj = 0; jj < cnt; jj += 8) {
-      f32x2_t o[8];
-      float w[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int js = min(jj + u, cnt - 1);
-        w[u] = (jj + u < cnt) ? __shfl(wj, js) : 0.f;
-        o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + (base + (int64_t)(j0 + js) * a.Hq) * 128 + d);
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        o0 += o[u][0] * w[u];
-        o1 += o[u][1] * w[u];
-      }
-    }
-  }
-  const float inv = a.sm.sink ? sink_inverse(mstar, den, sink_logit(a.sm.sink, a.sm.round_logits, head)) : 1.0f / den;
-  const int tq = a.pt.cu_q_lens[seq];
-  uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * 128 + d);
-  *op = pack_bf16x2(o0 * inv, o1 * inv);
+  merge_rows(a, seq, head, n, lane, [&](int j) -> int64_t { return base + (int64_t)j * a.Hq; });
 }
 
 // One thread copies one 16-byte piece of one gathered row.
