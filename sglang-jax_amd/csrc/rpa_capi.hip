@@ -156,6 +156,8 @@ SplitPlan plan_splits(int64_t max_len, int window, int64_t units, int64_t work, 
   return sp;
 }
 
+int decode_wave_capacity(const RpaParams* p);
+
 SplitPlan decode_plan(const RpaParams* p) {
   const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                      p->cu_kv_lens != nullptr);
@@ -165,7 +167,7 @@ SplitPlan decode_plan(const RpaParams* p) {
   int64_t work = p->sum_decode_kv_len > 0 ? p->sum_decode_kv_len * per_row : 0;
   if (p->sliding_window > 0) work = 0;  // visible lengths are not the raw lengths
   return plan_splits(bound, p->sliding_window, units, work, p->num_splits,
-                     env_int("RPA_DECODE_MIN_CHUNK", 64), env_int("RPA_DECODE_WAVE_CAPACITY", wave_capacity()));
+                     env_int("RPA_DECODE_MIN_CHUNK", 64), decode_wave_capacity(p));
 }
 
 // Balanced decode plan: a fixed number of waves (every wave slot of the GPU once) share the
@@ -178,8 +180,8 @@ bool decode_balanced() {
 // The balanced plan pays for itself on ragged batches that need splitting.  Rows of one known
 // length (the host's sum equals rows x bound) split evenly under the fixed plan already, and
 // batches the fixed plan does not split at all finish in one launch with no partial rows.
-int decode_waves_per_wg(int num_kv_heads);
-int decode_wgs(int num_kv_heads);
+int decode_waves_per_wg(const RpaParams* p);
+int decode_wgs(const RpaParams* p);
 
 bool use_balanced(const RpaParams* p, const SplitPlan& fixed) {
   if (!decode_balanced() || fixed.splits <= 1) return false;
@@ -187,10 +189,10 @@ bool use_balanced(const RpaParams* p, const SplitPlan& fixed) {
   // too little work to hand every workgroup its minimum piece: latency-bound, keep the launch count low
   const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                      p->cu_kv_lens != nullptr);
-  const int nw = decode_waves_per_wg(p->num_kv_heads);
+  const int nw = decode_waves_per_wg(p);
   const int64_t units = (int64_t)((p->num_kv_heads + nw - 1) / nw) * ((p->num_q_heads / p->num_kv_heads + 15) / 16);
   const int64_t min_blocks = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 64) / 32);
-  if ((int64_t)p->decode_end * ((bound + 31) / 32) * units <= (int64_t)decode_wgs(p->num_kv_heads) * min_blocks)
+  if ((int64_t)p->decode_end * ((bound + 31) / 32) * units <= (int64_t)decode_wgs(p) * min_blocks)
     return false;
   const bool equal_lengths = p->sum_decode_kv_len > 0 && p->max_kv_len > 0 &&
                              p->sum_decode_kv_len == (int64_t)p->decode_end * p->max_kv_len;
@@ -201,14 +203,45 @@ bool use_balanced(const RpaParams* p, const SplitPlan& fixed) {
   return true;
 }
 
-int decode_waves_per_wg(int num_kv_heads) {
-  const int nw = env_int("RPA_DECODE_WAVES_PER_WG", 2);
-  return std::max(1, std::min(std::min(nw, 4), num_kv_heads));
+// Bytes of KV the decode rows will read, as far as the host knows (its sum of lengths, or rows
+// times the length bound).
+int64_t decode_kv_bytes(const RpaParams* p) {
+  int64_t tokens = p->sum_decode_kv_len;
+  if (tokens <= 0)
+    tokens = (int64_t)p->decode_end * kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
+                                                   p->cu_kv_lens != nullptr);
+  if (p->sliding_window > 0) tokens = std::min(tokens, (int64_t)p->decode_end * (p->sliding_window + 31));
+  return tokens * 2 * p->num_kv_heads * p->head_dim * esize_of(p->kv_dtype);
 }
 
-int decode_wgs(int num_kv_heads) {
-  return std::max(1, env_int("RPA_DECODE_WAVE_CAPACITY", wave_capacity()) / decode_waves_per_wg(num_kv_heads));
+// Waves of a workgroup = neighbouring kv heads walked together (their rows are adjacent in the
+// cache).  Four on batches that stream tens of megabytes (C2 109 -> 105 us, C4 243 -> 238 us
+// against two); two on small, latency-bound batches, which want their few waves spread over
+// more CUs (C1 14.0 against 15.9 us).
+int decode_waves_per_wg(const RpaParams* p) {
+  const int dflt = decode_kv_bytes(p) >= (32ll << 20) ? 4 : 2;
+  const int nw = env_int("RPA_DECODE_WAVES_PER_WG", dflt);
+  return std::max(1, std::min(std::min(nw, 4), p->num_kv_heads));
 }
+
+// Decode waves resident at once.  A wave keeps one 32-token block of one head in flight: 16 KiB
+// of a 16-bit cache, 8 KiB of an fp8 one.  About 14 MB in flight saturate HBM; beyond that the
+// queues only get longer and DRAM locality worse (measured, C2 / C3 decode: 896 waves
+// 104.1 / 356 us, 1024: 105.2 / 362, 2048: 108.5 / 367; fp8 C4: 2048 best, 1536 equal, 1024
+// -25 %).  So four waves per CU for a 16-bit cache, less an eighth (the same 85 % the fixed plan
+// aims at on ragged rows), eight per CU for fp8 -- always a whole number of workgroups, and
+// never a workgroup count between one and two per CU, which the dispatcher spreads unevenly
+// (1152 waves in 4-wave workgroups: 133 us on C2).
+int decode_wave_capacity(const RpaParams* p) {
+  const int env = env_int("RPA_DECODE_WAVE_CAPACITY", 0);
+  if (env > 0) return env;
+  const int cus = wave_capacity() / 8;
+  if (esize_of(p->kv_dtype) == 1) return cus * 8;
+  const int nw = decode_waves_per_wg(p);
+  return std::max(nw, cus * 4 * 7 / 8 / nw * nw);
+}
+
+int decode_wgs(const RpaParams* p) { return std::max(1, decode_wave_capacity(p) / decode_waves_per_wg(p)); }
 
 int check_hip(hipError_t e, const char* what) {
   if (e == hipSuccess) return RPA_OK;
@@ -348,7 +381,7 @@ size_t rpa_workspace_bytes(const RpaParams* p) {
   if (p->head_dim == 256) return 0;  // the 256-dim kernel does not split sequences
   const SplitPlan sp = decode_plan(p);
   if (use_balanced(p, sp))
-    return (size_t)decode_wgs(p->num_kv_heads) * decode_waves_per_wg(p->num_kv_heads) * 2 * 16 * (p->head_dim + 2) *
+    return (size_t)decode_wgs(p) * decode_waves_per_wg(p) * 2 * 16 * (p->head_dim + 2) *
                sizeof(float) +
            ((size_t)p->decode_end + 1) * sizeof(int32_t);
   if (sp.splits <= 1) return 0;
@@ -402,8 +435,8 @@ int rpa_decode(const RpaParams* p, void* stream) {
   a.ws_ml = nullptr;
   a.cu_blocks = nullptr;
   a.balanced = use_balanced(p, sp) ? 1 : 0;
-  a.num_wgs = decode_wgs(p->num_kv_heads);
-  a.waves_per_wg = decode_waves_per_wg(p->num_kv_heads);
+  a.num_wgs = decode_wgs(p);
+  a.waves_per_wg = decode_waves_per_wg(p);
   a.min_blocks_per_wave = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 64) / 32);
   a.forced_blocks_per_wave = 0;
   if (p->num_splits > 0) {  // the caller pins the partition: about num_splits pieces for the longest row

@@ -1214,9 +1214,7 @@ hipError_t launch_decode_mt(const DecodeArgs& a, dim3 grid, dim3 block, bool uni
 
 hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream) {
   if (a.num_rows <= 0) return hipSuccess;
-  static const int nw_env = [] { const char* v = getenv("RPA_DECODE_WAVES_PER_WG"); return v ? atoi(v) : 0; }();
-  int nw = (nw_env >= 1 && nw_env <= 4) ? nw_env : 2;
-  if (nw > a.Hkv) nw = a.Hkv;
+  const int nw = min(max(a.waves_per_wg, 1), min(4, a.Hkv));  // kv heads walked together by one workgroup
   const int head_groups = (a.Hkv + nw - 1) / nw;
   // more than 16 query heads per kv head: further groups of 16 re-walk the KV (rare: MQA-like shapes)
   const int row_groups = (a.G + 15) / 16;
