@@ -50,10 +50,10 @@ DECODE_KERNEL = {
 }
 
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", "rpa_prefill_async_kernel"): 362.7e6 + 77.5e6,
-    ("c2", "rpa_decode_balanced_kernel"): 504.3e6 + 5.1e6,
-    ("c3", "rpa_decode_splitkv_kernel"): 2149.9e6 + 4.3e6,
-    ("c5", "rpa_mla_balanced_kernel"): 810.7e6 + 85.9e6,
+    ("c2", "rpa_prefill_async_kernel"): 364.1e6 + 77.5e6,
+    ("c2", "rpa_decode_balanced_kernel"): 501.0e6 + 2.7e6,
+    ("c3", "rpa_decode_splitkv_kernel"): 2148.6e6 + 1.9e6,
+    ("c5", "rpa_mla_balanced_kernel"): 820.4e6 + 85.9e6,
 }
 
 
