@@ -177,14 +177,21 @@ bool decode_balanced() {
   return on;
 }
 
-// The balanced plan pays for itself on ragged batches that need splitting.  Rows of one known
-// length (the host's sum equals rows x bound) split evenly under the fixed plan already, and
-// batches the fixed plan does not split at all finish in one launch with no partial rows.
+// The balanced plan pays for itself on ragged batches.  Rows of one known length (the host's
+// sum equals rows x bound) split evenly under the fixed plan already, and small batches the
+// fixed plan does not split at all finish in one launch with no partial rows.
 int decode_waves_per_wg(const RpaParams* p);
 int decode_wgs(const RpaParams* p);
+int64_t decode_kv_bytes(const RpaParams* p);
 
 bool use_balanced(const RpaParams* p, const SplitPlan& fixed) {
-  if (!decode_balanced() || fixed.splits <= 1) return false;
+  if (!decode_balanced()) return false;
+  if (p->num_splits == 1) return false;  // the caller asked for whole rows: one launch, no merge pass
+  // Rows the fixed plan leaves whole finish in one launch with no merge pass: right for small,
+  // latency-bound batches.  A large ragged batch is still better dealt out evenly -- one job per
+  // (row, kv head) of very different lengths, about one per wave slot, ends with the longest row
+  // (128 rows of 128..4096 tokens: 228 -> 205 us, 200 rows of 1000..3000: 351 -> 295 us).
+  if (fixed.splits <= 1 && decode_kv_bytes(p) < (64ll << 20)) return false;
   if (p->num_splits > 0) return true;
   // too little work to hand every workgroup its minimum piece: latency-bound, keep the launch count low
   const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,

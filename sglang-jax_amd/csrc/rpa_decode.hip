@@ -914,18 +914,20 @@ __device__ __forceinline__ void merge_rows(const DecodeArgs& a, int seq, int hea
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) lj += __shfl_xor(lj, off);
       den += lj;
+      // 32 partial rows requested at a time: a row with hundreds of partials (one long
+      // sequence cut over the whole GPU) is a chain of such round trips
       const int cnt = min(64, n - j0);
-      for (int jj = 0; jj < cnt; jj += 8) {
-        f32x2_t o[8];
-        float wv[8];
+      for (int jj = 0; jj < cnt; jj += 32) {
+        f32x2_t o[32];
+        float wv[32];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < 32; ++u) {
           const int js = min(jj + u, cnt - 1);
           wv[u] = (jj + u < cnt) ? __shfl(wj, js) : 0.f;
           o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + slot_of(j0 + js) * 128 + d);
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < 32; ++u) {
           o0 += o[u][0] * wv[u];
           o1 += o[u][1] * wv[u];
         }
