@@ -552,7 +552,13 @@ static int mla_wgs() { return std::max(1, env_int("RPA_MLA_WG_CAPACITY", wave_ca
 // same criteria as the MHA decode path: ragged sequence rows that need splitting
 static bool mla_use_balanced(const RpaMlaParams* p, const SplitPlan& fixed, bool token_rows) {
   static const bool on = env_int("RPA_MLA_BALANCED", 1) != 0;
-  if (!on || token_rows || fixed.splits <= 1) return false;
+  if (!on || token_rows || p->num_splits == 1) return false;
+  // Rows the fixed plan leaves whole: one workgroup job per row.  With many more jobs than
+  // workgroup slots the dispatcher evens them out by itself; with up to two per slot the kernel
+  // ends with the longest rows, and dealing the tiles out evenly pays (300 rows of 1000..8000
+  // tokens: 832 -> 673 us; 256 rows of 2048..16384: 1214 -> 1013 us; 1000 rows of 200..2000:
+  // 617 -> 659 us, so not there).
+  if (fixed.splits <= 1 && (int64_t)p->num_seqs * ((p->num_q_heads + 127) / 128) > 2 * (int64_t)mla_wgs()) return false;
   if (p->num_splits > 0) return true;
   const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                      p->cu_kv_lens != nullptr);
