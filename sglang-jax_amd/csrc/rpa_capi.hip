@@ -624,6 +624,7 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   a.num_wgs = mla_wgs();
   a.min_tiles_per_wg = std::max(1, env_int("RPA_MLA_MIN_CHUNK", 256) / 32);
   a.forced_tiles_per_wg = 0;
+  a.piece_pad = std::max(0, env_int("RPA_MLA_PIECE_PAD", 5));
   if (p->num_splits > 0) {
     const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                        p->cu_kv_lens != nullptr);

@@ -129,6 +129,7 @@ struct MlaDecodeArgs {
   int32_t num_wgs;
   int32_t min_tiles_per_wg;
   int32_t forced_tiles_per_wg;
+  int32_t piece_pad;  // balanced plan: what starting one more (row, head group) costs a workgroup, in tiles
   int32_t* cu_tiles;  // [num_rows + 1] prefix sum of tiles, written by the kernel
 };
 

@@ -385,10 +385,24 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
 // workgroup j takes tiles [j * pw, (j + 1) * pw).  Pieces that are whole rows are finished in
 // place, cut ones (at most the first and the last of a workgroup) leave partial rows in the
 // workspace slots 2j and 2j + 1 (128 heads each).
+//
+// Starting a piece is not free: 147 KB of queries and the first tiles have to arrive and the
+// piece before it has to be written out -- 17 us on the DeepSeek-V3 batch, five tiles' worth, and
+// a workgroup with three pieces finished 37 us after one with a single piece.  So the line the
+// workgroups share is padded: every (row, head group) is preceded by `piece_pad` tiles that hold
+// no work.  A workgroup that runs into a new row spends that much of its share on the way, which
+// is what the switch costs it; one that starts in the middle of a row, like most, pays nothing
+// extra -- every workgroup has one start of its own anyway.
 __device__ __forceinline__ int mla_tiles(int kv_len, int window) {
   if (kv_len <= 0) return 0;
   const int t_lo = (window > 0) ? max(0, kv_len - window) : 0;
   return (kv_len - (t_lo & ~(kTok - 1)) + kTok - 1) / kTok;
+}
+
+// extent of a (row, head group) on the padded line
+__device__ __forceinline__ int mla_extent(const MlaDecodeArgs& a, int kv_len) {
+  const int nt = mla_tiles(kv_len, a.sm.window);
+  return nt > 0 ? nt + a.piece_pad : 0;
 }
 
 __device__ __forceinline__ int mla_tiles_per_wg(const MlaDecodeArgs& a, int total) {
@@ -411,7 +425,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
     // first pass: total; second pass (below) locates this workgroup's first tile
     for (int s0 = 0; s0 < a.num_rows; s0 += 64) {
       const int s = s0 + lane;
-      int nt = (s < a.num_rows) ? mla_tiles(a.pt.kv_lens[s], a.sm.window) : 0;
+      int nt = (s < a.num_rows) ? mla_extent(a, a.pt.kv_lens[s]) : 0;
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) nt += __shfl_xor(nt, off);
       total += nt;
@@ -423,7 +437,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
     int base = 0;
     for (int s0 = 0; s0 < a.num_rows; s0 += 64) {
       const int s = s0 + lane;
-      const int nt = (s < a.num_rows) ? mla_tiles(a.pt.kv_lens[s], a.sm.window) : 0;
+      const int nt = (s < a.num_rows) ? mla_extent(a, a.pt.kv_lens[s]) : 0;
       int incl = nt;
 #pragma unroll
       for (int off = 1; off < 64; off <<= 1) {
@@ -438,12 +452,11 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
   if ((int64_t)wg * pw >= total) return;
   int x = wg * pw;
   const int x_end = min(total, x + pw);
-  const int x_first = x;
   {
     int base = 0;
     for (int s0 = 0; s0 < a.num_rows && seq < 0; s0 += 64) {
       const int s = s0 + lane;
-      const int nt = (s < a.num_rows) ? mla_tiles(a.pt.kv_lens[s], a.sm.window) : 0;
+      const int nt = (s < a.num_rows) ? mla_extent(a, a.pt.kv_lens[s]) : 0;
       int incl = nt;
 #pragma unroll
       for (int off = 1; off < 64; off <<= 1) {
@@ -463,10 +476,18 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
   }
   int kv_len = scalar_load_i32(a.pt.kv_lens + seq);
   int nt = mla_tiles(kv_len, a.sm.window);
+  const int pad = a.piece_pad;
+  bool first_piece = true;
   while (x < x_end) {
-    const int r = x - seq_first;
-    const int unit = r / nt;
-    const int tile = r - unit * nt;
+    const int r = x - seq_first;  // position inside the row's padded extents
+    const int unit = r / (nt + pad);
+    int off = r - unit * (nt + pad);
+    if (off < pad) {  // the padding in front of this (row, head group): no work there
+      x += pad - off;
+      off = pad;
+      if (x >= x_end) break;
+    }
+    const int tile = off - pad;
     const int take = min(nt - tile, x_end - x);
     const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
     const int t0 = t_lo & ~(kTok - 1);
@@ -477,12 +498,13 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
     mr.valid = true;
     MlaDest dest;
     dest.final_rows = (tile == 0) && (take == nt);
-    dest.base = ((int64_t)wg * 2 + (x == x_first ? 0 : 1)) * 128 - unit * 128;  // + head
+    dest.base = ((int64_t)wg * 2 + (first_piece ? 0 : 1)) * 128 - unit * 128;  // + head
+    first_piece = false;
     mla_segment<UNIFORM, CAP>(a, mr, unit * 128, t_lo, t0 + tile * kTok, min(kv_len, t0 + (tile + take) * kTok),
                               dest, slot0, slot1, slot2, slot3);
     x += take;
     if (x < x_end && tile + take == nt && unit == units - 1) {
-      seq_first += nt * units;
+      seq_first += (nt + pad) * units;
       do {
         ++seq;
         kv_len = scalar_load_i32(a.pt.kv_lens + seq);
@@ -501,11 +523,15 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const Mla
   const int total = a.cu_tiles[a.num_rows] * units;
   const int pw = mla_tiles_per_wg(a, total);
   const int unit = head >> 7;
-  const int first_tile = a.cu_tiles[seq] * units + unit * nt;
+  // the row's head group on the padded line: `piece_pad` empty tiles, then its nt tiles
+  const int extent_first = a.cu_tiles[seq] * units + unit * (nt + a.piece_pad);
+  const int first_tile = extent_first + a.piece_pad;
   const int w_first = first_tile / pw, w_last = (first_tile + nt - 1) / pw;
   if (w_first == w_last) return;  // one workgroup covered the row and wrote the finished output
   auto slot_of = [&](int wj) -> int64_t {
-    const int part = ((int64_t)wj * pw >= first_tile) ? 0 : 1;
+    // slot 0 holds a workgroup's first piece: this one iff its share starts inside this extent
+    // (padding included); a share that starts before it holds the last tile of the extent before
+    const int part = ((int64_t)wj * pw >= extent_first) ? 0 : 1;
     return ((int64_t)wj * 2 + part) * 128 + (head & 127);
   };
   float mstar = -INFINITY;
