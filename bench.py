@@ -7,7 +7,7 @@ A *step* is one pass of the hot path over one synthetic batch already resident
 in HBM: ``rpa_decode`` (split-KV kernel + combine) on the decode rows followed
 by ``rpa_prefill`` (flash kernel) on the prefill rows -- exactly what
 ``rpa_attention`` issues.  The default workload is the mixed Llama-3-8B batch
-(BASELINE.json configs[1]).
+(the configuration the headline metric is quoted on).
 
 One JSON line is printed:
   value       decode HBM GB/s of the workload's decode rows: algorithmic bytes /
