@@ -6,6 +6,7 @@ configuration."""
 
 import sys
 
+import numpy as np
 import pytest
 import torch
 
@@ -69,6 +70,24 @@ def test_mla_split_count_does_not_matter(pkg, wl, gpu):
         torch.testing.assert_close(got.float(), want.float(), **TOL)
         base = got if base is None else base
         torch.testing.assert_close(got.float(), base.float(), rtol=1e-2, atol=4e-3)
+
+
+def test_mla_many_ragged_rows_are_dealt_out_evenly(pkg, wl, gpu):
+    """More rows than workgroup slots, none long enough for the fixed plan to cut: the batch still
+    takes the balanced plan (at most two whole-row jobs per slot would end with the longest rows);
+    pieces are padded, so workgroups that cross into new rows get fewer tiles.  Against the
+    oracle and against whole rows (num_splits = 1)."""
+    rng = np.random.default_rng(79)
+    kv_lens = [int(x) for x in rng.integers(100, 900, size=300)]
+    say("mla 300 ragged rows")
+    b = wl.make_mla_batch("mla_many", [1] * len(kv_lens), kv_lens, num_q_heads=16, lkv_dim=512, rope_dim=64,
+                          page_size=64, seed=80, sm_scale=192 ** -0.5)
+    want = oracle(b)
+    auto = run_gpu(pkg, b, gpu)
+    whole = run_gpu(pkg, b, gpu, num_splits=1)
+    torch.testing.assert_close(auto.float(), want.float(), **TOL)
+    torch.testing.assert_close(auto.float(), whole.float(), rtol=1e-2, atol=4e-3)
+    assert not torch.equal(auto, whole)  # merged rows differ from whole ones in the last bits somewhere
 
 
 def test_mla_reference_padded_cache_layout(pkg, wl, gpu):

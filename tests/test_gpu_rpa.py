@@ -510,6 +510,24 @@ def test_balanced_plan_long_shares_and_tiny_rows(pkg, wl, gpu, monkeypatch):
         assert torch.equal(auto, again)
 
 
+def test_balanced_plan_when_rows_outnumber_wave_slots(pkg, wl, gpu):
+    """More (row, kv head) jobs than resident waves and far more than 64 MB of KV: the fixed plan
+    would leave every row whole (one job each, as different in length as the rows are), so the
+    batch is dealt out evenly instead -- most rows are then cut exactly once.  Against the
+    oracle and against whole rows (num_splits = 1, no merge pass)."""
+    rng = np.random.default_rng(77)
+    kv_lens = [int(x) for x in rng.integers(100, 3000, size=300)]
+    say("300 ragged rows, 4 kv heads")
+    b = wl.make_batch("many_rows", [1] * len(kv_lens), kv_lens, num_q_heads=8, num_kv_heads=4, head_dim=128,
+                      page_size=64, seed=78)
+    want = oracle_out(b)
+    auto = gpu_out(pkg, b, gpu)
+    whole = gpu_out(pkg, b, gpu, num_splits=1)
+    torch.testing.assert_close(auto.float(), want.float(), **BF16_TOL)
+    torch.testing.assert_close(auto.float(), whole.float(), rtol=1e-2, atol=4e-3)
+    assert not torch.equal(auto, whole)  # a merged row differs from a whole one in the last bits somewhere
+
+
 # ------------------------------------------------------------------ head_dim 256
 def batch256(wl, name, q_lens, kv_lens, seed, Hq=8, Hkv=2, P=16, **mk):
     return wl.make_batch(name, q_lens, kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=256, page_size=P,
