@@ -528,6 +528,30 @@ def test_balanced_plan_when_rows_outnumber_wave_slots(pkg, wl, gpu):
     assert not torch.equal(auto, whole)  # a merged row differs from a whole one in the last bits somewhere
 
 
+def test_balanced_plan_skips_rows_without_tokens(pkg, wl, gpu):
+    """Rows whose length is zero (padding inside a bucketed batch) hold no block: a wave that
+    reaches one moves on to the next row that has any -- also when that row lies beyond the 64
+    rows whose lengths it keeps in registers.  The other rows come out as if the empty rows
+    were not there."""
+    rng = np.random.default_rng(83)
+    kv_lens = [int(x) for x in rng.integers(300, 5000, size=150)]
+    b = wl.make_batch("empty_rows", [1] * len(kv_lens), kv_lens, num_q_heads=16, num_kv_heads=4, head_dim=128,
+                      page_size=64, seed=84)
+    want = oracle_out(b)
+    empty = [0, 5, 6, 63, 64, 70, 71, 72, 149]
+    keep = torch.tensor([i for i in range(len(kv_lens)) if i not in empty])
+    g = b.to(gpu)
+    lens = g.kv_lens.clone()
+    lens[torch.tensor(empty, device=gpu)] = 0
+    dist = b.distribution.cpu().numpy()
+    say("150 rows, 9 of them empty")
+    out, _ = pkg.ragged_paged_attention(
+        g.q, None, None, g.kv_cache, lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens, dist, None, sm_scale=b.sm_scale,
+        max_kv_len=int(max(kv_lens)), max_q_len=1)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu()[keep].float(), want[keep].float(), **BF16_TOL)
+
+
 # ------------------------------------------------------------------ head_dim 256
 def batch256(wl, name, q_lens, kv_lens, seed, Hq=8, Hkv=2, P=16, **mk):
     return wl.make_batch(name, q_lens, kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=256, page_size=P,
