@@ -472,8 +472,12 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   int rc = rpa_validate(p);
   if (rc != RPA_OK) return rc;
   if (p->num_seqs <= p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) return RPA_OK;
-  if (p->head_dim == 256) return rows256(p, p->decode_end, p->num_seqs, stream);
+  // 256-wide heads: bf16 caches take the flash kernel (two 128-dim halves per row, one workgroup
+  // per CU); fp8 caches and rows the caller masks itself stay on the row kernel
+  if (p->head_dim == 256 && (p->kv_dtype == RPA_KV_FP8_E4M3 || env_int("RPA_PREFILL_ROWS256", 0) != 0))
+    return rows256(p, p->decode_end, p->num_seqs, stream);
   rpa::PrefillArgs a;
+  a.head_dim = p->head_dim;
   a.q = static_cast<const uint16_t*>(p->q);
   a.out = static_cast<uint16_t*>(p->out);
   a.kv = kv_addr(p);

@@ -81,6 +81,7 @@ struct PrefillArgs {
   int32_t max_q_len;
   int32_t max_kv_len;  // host bound on kv_len of these sequences, 0 = unknown
   int32_t fp8;
+  int32_t head_dim;  // 128, or 256 (bf16 cache only)
 };
 
 struct GatherArgs {

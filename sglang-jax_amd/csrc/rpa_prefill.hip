@@ -213,8 +213,8 @@ __device__ __forceinline__ MaskCtx make_mask_ctx(const PrefillArgs& a, const Wor
   return mc;
 }
 
-template <bool CAP, bool EXT>
-__device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4], float& m, float& l,
+template <bool CAP, bool EXT, int ND = 4>
+__device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[ND], float& m, float& l,
                                              const Softmax<CAP>& sm, bool need_mask, int tb, int h, int qpos,
                                              int window, u32x4_t (&pB)[2][2], const MaskCtx& mc) {
   if constexpr (CAP) {
@@ -251,7 +251,7 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4],
     else mx = __builtin_fmaxf(mx, S[1][v]);
   }
   mx = swap_max(mx);
-  update_running_max<4>(mx, m, l, O, sm.sc2);
+  update_running_max<ND>(mx, m, l, O, sm.sc2);
   const float neg_m = -m * sm.sc2;
   // probabilities go straight into bf16 pairs (the B operands of the second product); the row
   // sum is taken over the rounded pairs, one dot instruction per pair
@@ -276,15 +276,16 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[4],
 }
 
 // lane (c, h) holds query row c, dims 32d + 8*(v/4) + 4h + v%4 in O[d][v]
+template <int ND = 4>
 __device__ __forceinline__ void write_rows(const PrefillArgs& a, const Work& w, const WaveRows& wr,
-                                           const f32x16_t (&O)[4], float l, int h, float m2) {
+                                           const f32x16_t (&O)[ND], float l, int h, float m2) {
   l += __shfl_xor(l, 32);
   if (!wr.active || wr.row >= w.q_len) return;
   const float vs = a.v_scale ? a.v_scale[w.hk] : 1.0f;
   const float inv = a.sm.sink ? vs * sink_inverse(m2, l, sink_logit(a.sm.sink, a.sm.round_logits, w.head)) : vs / l;
-  uint16_t* op = a.out + ((int64_t)(w.qg0 + wr.row) * a.Hq + w.head) * 128 + 4 * h;
+  uint16_t* op = a.out + ((int64_t)(w.qg0 + wr.row) * a.Hq + w.head) * (ND * 32) + 4 * h;
 #pragma unroll
-  for (int d = 0; d < 4; ++d)
+  for (int d = 0; d < ND; ++d)
 #pragma unroll
     for (int vq = 0; vq < 4; ++vq) {
       u32x2_t o = {pack_bf16x2(O[d][4 * vq + 0] * inv, O[d][4 * vq + 1] * inv),
@@ -294,56 +295,70 @@ __device__ __forceinline__ void write_rows(const PrefillArgs& a, const Work& w, 
 }
 
 // ==================================================================== async path (bf16 cache)
-constexpr int kRowB = 256;             // one K or V row of a head: 128 bf16, unpadded
-constexpr int kTileB = kBN * kRowB;    // 16 KiB
+// Geometry of a tile for head dim HD (128 or 256): rows stay row-major and unpadded in LDS.
+template <int HD>
+struct Tile {
+  static constexpr int kRowB = HD * 2;          // one K or V row of a head, bf16
+  static constexpr int kTileB = kBN * kRowB;    // 16 or 32 KiB
+  static constexpr int kChunks = HD / 8;        // 16-byte chunks per row
+  static constexpr int kSteps = HD / 16;        // k-steps of the first product
+  static constexpr int kDimTiles = HD / 32;     // 32-dim output tiles of the second product
+  static constexpr int kCopies = kChunks / 4;   // copy instructions per wave, for K and for V
+  static constexpr int kRowsPerCopy = 64 / kChunks;
+};
 
 // 16-byte chunk j of row t sits at chunk position j ^ swizzle(t):
 //   K: swizzle = t & 15      (ds_read_b128: 16 consecutive tokens -> 16 distinct chunk columns)
 //   V: swizzle = 4 * (t & 3) (transposing read: 4 consecutive tokens -> 4 distinct 64-byte windows)
-template <bool UNIFORM>
+template <bool UNIFORM, int HD>
 struct AsyncPages {
-  int32_t id[UNIFORM ? 1 : 4];
+  int32_t id[UNIFORM ? 1 : Tile<HD>::kCopies];
 };
 
-template <bool UNIFORM>
-__device__ __forceinline__ void async_fetch_pages(AsyncPages<UNIFORM>& pg, const TileSrc& s, int tb, int wave,
+template <bool UNIFORM, int HD>
+__device__ __forceinline__ void async_fetch_pages(AsyncPages<UNIFORM, HD>& pg, const TileSrc& s, int tb, int wave,
                                                   int lane) {
+  using T = Tile<HD>;
   tb = min(tb, s.last_tok & ~(kBN - 1));
   if constexpr (UNIFORM) {
     pg.id[0] = scalar_load_i32(s.pages + __builtin_amdgcn_readfirstlane(page_slot(s, tb)));
   } else {
 #pragma unroll
-    for (int n = 0; n < 4; ++n) {
-      const int t = (wave * 4 + n) * 4 + (lane >> 4);
+    for (int n = 0; n < T::kCopies; ++n) {
+      const int t = (wave * T::kCopies + n) * T::kRowsPerCopy + lane / T::kChunks;
       pg.id[n] = s.pages[page_slot(s, min(tb + t, s.last_tok))];
     }
   }
 }
 
-// Every wave copies 4 x 64 chunks of K and of V: chunk position p = 64*(4*wave + n) + lane of
-// the tile, i.e. row p / 16, chunk column p % 16.  For a full tile inside one page the byte
-// offset of a lane's chunk from the tile's first row never changes: it is computed once
-// (AsyncOffsets) and a copy costs no vector ALU work, only a scalar tile base.
+// Every wave copies kCopies x 64 chunks of K and of V: chunk position p = 64*(kCopies*wave + n) +
+// lane of the tile, i.e. row p / kChunks, chunk column p % kChunks.  For a full tile inside one
+// page the byte offset of a lane's chunk from the tile's first row never changes: it is computed
+// once (AsyncOffsets) and a copy costs no vector ALU work, only a scalar tile base.
+template <int HD>
 struct AsyncOffsets {
-  uint32_t k[4], v[4];
+  uint32_t k[Tile<HD>::kCopies], v[Tile<HD>::kCopies];
 };
 
-__device__ __forceinline__ AsyncOffsets make_async_offsets(const KvAddr& kv, int wave, int lane) {
-  AsyncOffsets o;
-  const int cp = lane & 15;
+template <int HD>
+__device__ __forceinline__ AsyncOffsets<HD> make_async_offsets(const KvAddr& kv, int wave, int lane) {
+  using T = Tile<HD>;
+  AsyncOffsets<HD> o;
+  const int cp = lane % T::kChunks;
 #pragma unroll
-  for (int n = 0; n < 4; ++n) {
-    const int t = (wave * 4 + n) * 4 + (lane >> 4);
+  for (int n = 0; n < T::kCopies; ++n) {
+    const int t = (wave * T::kCopies + n) * T::kRowsPerCopy + lane / T::kChunks;
     o.k[n] = (uint32_t)(t * kv.tok_stride + ((cp ^ (t & 15)) << 4));
     o.v[n] = (uint32_t)(t * kv.tok_stride + ((cp ^ ((t & 3) << 2)) << 4));
   }
   return o;
 }
 
-template <bool UNIFORM>
+template <bool UNIFORM, int HD>
 __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const TileSrc& s, const KvAddr& kv,
                                                 const char* kh, const char* vh, int tb, int wave, int lane,
-                                                const AsyncPages<UNIFORM>& pg, const AsyncOffsets& ofs) {
+                                                const AsyncPages<UNIFORM, HD>& pg, const AsyncOffsets<HD>& ofs) {
+  using T = Tile<HD>;
   typedef const __attribute__((address_space(1))) void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
   tb = min(tb, s.last_tok & ~(kBN - 1));  // past the end: re-copy the last tile
@@ -354,8 +369,8 @@ __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const 
       const char* kb = kh + base;
       const char* vb = vh + base;
 #pragma unroll
-      for (int n = 0; n < 4; ++n) {
-        const int blk = wave * 4 + n;
+      for (int n = 0; n < T::kCopies; ++n) {
+        const int blk = wave * T::kCopies + n;
         __builtin_amdgcn_global_load_lds((gptr_t)(kb + ofs.k[n]), (lptr_t)(lds_k + blk * 1024), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((gptr_t)(vb + ofs.v[n]), (lptr_t)(lds_v + blk * 1024), 16, 0, 0);
       }
@@ -363,11 +378,11 @@ __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const 
     }
   }
   // last, partial tile (rows clamped to the last valid token) or pages smaller than a tile
-  const int cp = lane & 15;
+  const int cp = lane % T::kChunks;
 #pragma unroll
-  for (int n = 0; n < 4; ++n) {
-    const int blk = wave * 4 + n;
-    const int t = blk * 4 + (lane >> 4);
+  for (int n = 0; n < T::kCopies; ++n) {
+    const int blk = wave * T::kCopies + n;
+    const int t = blk * T::kRowsPerCopy + lane / T::kChunks;
     const int64_t ro = row_offset<UNIFORM>(s, kv, tb, tb + t, pg.id[UNIFORM ? 0 : n]);
     const int jk = cp ^ (t & 15);
     const int jv = cp ^ ((t & 3) << 2);
@@ -378,8 +393,14 @@ __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const 
 
 // EXT compiles in the rarely used options (temperature factor, custom mask / no mask); the
 // plain causal instantiation keeps its scale in a scalar register and its mask test to one compare.
-template <bool UNIFORM, bool CAP, bool EXT>
-__global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const PrefillArgs a, int tiles, int nseq, bool by_level) {
+// HD = 256 doubles the rows in LDS (two 64 KiB slots), the Q^T operands and the accumulators: one
+// workgroup per CU, one wave per SIMD with up to 512 registers.
+template <bool UNIFORM, bool CAP, bool EXT, int HD = 128>
+__global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_kernel(const PrefillArgs a, int tiles, int nseq,
+                                                                                  bool by_level) {
+  using T = Tile<HD>;
+  constexpr int kRowB = T::kRowB;
+  constexpr int kTileB = T::kTileB;
   // Four separate arrays (not one indexed array): the compiler can then prove that the
   // asynchronous copy into one ring slot does not alias the LDS reads of the other slot and
   // does not drain the vector-memory queue in the middle of a tile.
@@ -406,15 +427,15 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
   wr.qpos = w.prefix + wr.row;
   const int W_ = a.sm.window;
 
-  u32x4_t qB[8];
+  u32x4_t qB[T::kSteps];
   {
     const int rr = min(wr.row, w.q_len - 1);
-    const uint16_t* qp = a.q + ((int64_t)(w.qg0 + rr) * a.Hq + w.head) * 128 + h * 8;
+    const uint16_t* qp = a.q + ((int64_t)(w.qg0 + rr) * a.Hq + w.head) * HD + h * 8;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qB[ks] = ld16(qp + ks * 16);
+    for (int ks = 0; ks < T::kSteps; ++ks) qB[ks] = ld16(qp + ks * 16);
     if (EXT && a.sm.q_scale > 0.f) {
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) qB[ks] = requantise_q(qB[ks], a.sm.q_scale, false);
+      for (int ks = 0; ks < T::kSteps; ++ks) qB[ks] = requantise_q(qB[ks], a.sm.q_scale, false);
     }
   }
   Softmax<CAP> sm;
@@ -429,9 +450,9 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
     sm.round_bf16 = a.sm.round_logits != 0;
   }
 
-  f32x16_t O[4];
+  f32x16_t O[T::kDimTiles];
 #pragma unroll
-  for (int d = 0; d < 4; ++d)
+  for (int d = 0; d < T::kDimTiles; ++d)
 #pragma unroll
     for (int v = 0; v < 16; ++v) O[d][v] = 0.f;
   float m = kMaxFloor, l = 0.f;
@@ -459,24 +480,24 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
   // The swizzled offsets are kept in registers for the whole loop (12 of them) instead of being
   // recomputed in front of each of the 48 LDS reads of a tile; slot bases and row steps fold
   // into the instructions' immediate offsets.
-  int koff[8], voff[4];
+  int koff[T::kSteps], voff[T::kDimTiles];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) {
+  for (int ks = 0; ks < T::kSteps; ++ks) {
     koff[ks] = k_row + ((ks * 32) ^ k_swz);
     asm volatile("" : "+v"(koff[ks]));
   }
 #pragma unroll
-  for (int d = 0; d < 4; ++d) {
+  for (int d = 0; d < T::kDimTiles; ++d) {
     voff[d] = v_row + v_in + ((d * 64) ^ v_swz);
     asm volatile("" : "+v"(voff[d]));
   }
 
   // ---- pipeline: page ids two tiles ahead, the asynchronous copy one tile ahead ----
-  const AsyncOffsets ofs = make_async_offsets(a.kv, wave, lane);
-  AsyncPages<UNIFORM> pg;
-  async_fetch_pages<UNIFORM>(pg, src, t_lo, wave, lane);
-  async_copy_tile<UNIFORM>(lds_k0, lds_v0, src, a.kv, kh, vh, t_lo, wave, lane, pg, ofs);
-  async_fetch_pages<UNIFORM>(pg, src, t_lo + kBN, wave, lane);
+  const AsyncOffsets<HD> ofs = make_async_offsets<HD>(a.kv, wave, lane);
+  AsyncPages<UNIFORM, HD> pg;
+  async_fetch_pages<UNIFORM, HD>(pg, src, t_lo, wave, lane);
+  async_copy_tile<UNIFORM, HD>(lds_k0, lds_v0, src, a.kv, kh, vh, t_lo, wave, lane, pg, ofs);
+  async_fetch_pages<UNIFORM, HD>(pg, src, t_lo + kBN, wave, lane);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the copies have landed in LDS
   __syncthreads();
 
@@ -484,8 +505,8 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
   auto tile_step = [&](const char* lds_k, const char* lds_v, char* nxt_k, char* nxt_v, int tb) {
     if (tb + kBN < t_hi) {
       // the other slot was last read before the barrier that ended the previous tile
-      async_copy_tile<UNIFORM>(nxt_k, nxt_v, src, a.kv, kh, vh, tb + kBN, wave, lane, pg, ofs);
-      async_fetch_pages<UNIFORM>(pg, src, tb + 2 * kBN, wave, lane);
+      async_copy_tile<UNIFORM, HD>(nxt_k, nxt_v, src, a.kv, kh, vh, tb + kBN, wave, lane, pg, ofs);
+      async_fetch_pages<UNIFORM, HD>(pg, src, tb + 2 * kBN, wave, lane);
     }
     // visible to this wave?  causal: some token <= last row's position; window: some token
     // newer than the first row's horizon
@@ -500,19 +521,19 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
         S[0] = mfma32(lds_ld16(lds_k + koff[0]), qB[0], kZero16);  // zero accumulator as an inline constant
         S[1] = mfma32(lds_ld16(lds_k + koff[0] + 32 * kRowB), qB[0], kZero16);
 #pragma unroll
-        for (int ks = 1; ks < 8; ++ks) {
+        for (int ks = 1; ks < T::kSteps; ++ks) {
           S[0] = mfma32(lds_ld16(lds_k + koff[ks]), qB[ks], S[0]);
           S[1] = mfma32(lds_ld16(lds_k + koff[ks] + 32 * kRowB), qB[ks], S[1]);
         }
         u32x4_t pB[2][2];
-        softmax_tile<CAP, EXT>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc);
-        // four independent accumulator chains (dim tiles), issued round-robin
+        softmax_tile<CAP, EXT, T::kDimTiles>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc);
+        // independent accumulator chains (dim tiles), issued round-robin
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
           for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
+            for (int d = 0; d < T::kDimTiles; ++d) {
               const char* vt = lds_v + voff[d] + (mt * 32 + kk * 16) * kRowB;
               const u32x2_t lo = lds_tr16(vt);
               const u32x2_t hi = lds_tr16(vt + 8 * kRowB);
@@ -528,7 +549,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_async_kernel(const Prefill
     if (tb + kBN >= t_hi) break;
     tile_step(lds_k1, lds_v1, lds_k0, lds_v0, tb + kBN);
   }
-  write_rows(a, w, wr, O, l, h, m * sm.sc2);
+  write_rows<T::kDimTiles>(a, w, wr, O, l, h, m * sm.sc2);
 }
 
 // ==================================================================== staged path (fp8 cache)
@@ -782,6 +803,8 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
 #define RPA_STAGED(F, U, C, E) \
   hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_ASYNC(U, C, E) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
+#define RPA_ASYNC256(U, C, E) \
+  hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E, 256>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_PICK(M, ...)                                            \
   switch ((uniform ? 4 : 0) | (cap ? 2 : 0) | (ext ? 1 : 0)) {        \
     case 0: M(__VA_ARGS__ false, false, false); break;              \
@@ -795,7 +818,10 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   }
 #define RPA_STAGED_FP8(U, C, E) RPA_STAGED(true, U, C, E)
 #define RPA_STAGED_BF16(U, C, E) RPA_STAGED(false, U, C, E)
-  if (!staged) {
+  if (a.head_dim == 256) {
+    if (a.fp8) return hipErrorInvalidValue;  // 256-wide fp8 rows go through the row kernel
+    RPA_PICK(RPA_ASYNC256, )
+  } else if (!staged) {
     RPA_PICK(RPA_ASYNC, )
   } else if (a.fp8) {
     RPA_PICK(RPA_STAGED_FP8, )
@@ -807,6 +833,7 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
 #undef RPA_PICK
 #undef RPA_STAGED
 #undef RPA_ASYNC
+#undef RPA_ASYNC256
   return hipGetLastError();
 }
 
