@@ -585,8 +585,20 @@ def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
         torch.testing.assert_close(gpu_out(pkg, b, gpu, **kw).float(), oracle_out(b, **kw).float(), **tol)
     # full attention (causal = 0 without a mask)
     torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=False).float(), oracle_out(b, causal=False).float(), **tol)
-    with pytest.raises(ValueError, match="custom masks"):
-        gpu_out(pkg, b, gpu, causal=False, custom_mask=torch.ones(1, dtype=torch.int32))
+    # custom masks: every row goes through the flash kernel, which is built for bf16 caches
+    rng = np.random.default_rng(11)
+    masks = []
+    for ql, kv in zip(q_lens, kv_lens):
+        mk = (rng.random((ql, kv)) < 0.6).astype(np.int32)
+        mk[:, 0] = 1
+        masks.append(mk)
+    cm = flat_mask(masks)
+    if kv_dtype == torch.bfloat16:
+        torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=False, custom_mask=cm.to(gpu)).float(),
+                                   oracle_out(b, causal=False, custom_mask=cm).float(), **tol)
+    else:
+        with pytest.raises(ValueError, match="custom masks"):
+            gpu_out(pkg, b, gpu, causal=False, custom_mask=cm.to(gpu))
 
 
 def test_head_dim_256_cache_write_and_gather(pkg, wl, gpu):
