@@ -255,6 +255,26 @@ int check_hip(hipError_t e, const char* what) {
   return fail(RPA_EHIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+// head_dim 256, decode rows: split like the fixed plan when there are too few rows to fill the GPU
+// (the row kernel keeps nothing in flight while it computes, so it wants every wave slot)
+SplitPlan rows256_plan(const RpaParams* p) {
+  const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
+                                     p->cu_kv_lens != nullptr);
+  const int G = p->num_q_heads / p->num_kv_heads;
+  const int64_t per_row = (int64_t)p->num_kv_heads * ((G + 15) / 16);
+  const int64_t units = (int64_t)p->decode_end * per_row;
+  int64_t work = p->sum_decode_kv_len > 0 ? p->sum_decode_kv_len * per_row : 0;
+  if (p->sliding_window > 0) work = 0;
+  return plan_splits(bound, p->sliding_window, units, work, p->num_splits, 256, wave_capacity());
+}
+
+size_t rows256_workspace(const RpaParams* p) {
+  if (p->decode_end <= 0) return 0;
+  const SplitPlan sp = rows256_plan(p);
+  if (sp.splits <= 1) return 0;
+  return (size_t)p->decode_end * sp.splits * p->num_q_heads * (p->head_dim + 2) * sizeof(float);
+}
+
 // head_dim 256: every query token of sequences [seq_begin, seq_end) is a row of the row kernel
 int rows256(const RpaParams* p, int seq_begin, int seq_end, void* stream) {
   if (seq_end <= seq_begin) return RPA_OK;
@@ -273,6 +293,18 @@ int rows256(const RpaParams* p, int seq_begin, int seq_end, void* stream) {
   a.fp8 = p->kv_dtype == RPA_KV_FP8_E4M3;
   // decode rows are one token each; other sequences are bounded by the tokens of the call
   const int rows = (seq_end <= p->decode_end) ? (seq_end - seq_begin) : p->num_tokens;
+  if (seq_begin == 0 && seq_end == p->decode_end) {
+    const SplitPlan sp = rows256_plan(p);
+    if (sp.splits > 1) {
+      const size_t need = rows256_workspace(p);
+      if (!p->workspace || p->workspace_bytes < need)
+        return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
+      a.chunk = sp.chunk;
+      a.max_splits = sp.splits;
+      a.ws_o = static_cast<float*>(p->workspace);
+      a.ws_ml = a.ws_o + (size_t)p->decode_end * sp.splits * p->num_q_heads * p->head_dim;
+    }
+  }
   return check_hip(rpa::launch_rows256(a, seq_begin, seq_end, rows, static_cast<hipStream_t>(stream)), "rpa rows256");
 }
 
@@ -387,7 +419,7 @@ int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t*
 
 size_t rpa_workspace_bytes(const RpaParams* p) {
   if (!p || p->decode_end <= 0) return 0;
-  if (p->head_dim == 256) return 0;  // the 256-dim kernel does not split sequences
+  if (p->head_dim == 256) return rows256_workspace(p);
   const SplitPlan sp = decode_plan(p);
   if (use_balanced(p, sp))
     return (size_t)decode_wgs(p) * decode_waves_per_wg(p) * 2 * 16 * (p->head_dim + 2) *

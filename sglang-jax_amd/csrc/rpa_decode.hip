@@ -854,19 +854,21 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
 // (nearly always) everything is requested at once -- the (max, sum) pairs by lanes 0..n-1, the
 // partial rows by all lanes, the row's query token before either -- so the merge costs one round
 // trip to memory instead of three dependent ones.
-template <int N, typename SlotOf>
+template <int N, int HD, typename SlotOf>
 __device__ __forceinline__ void merge_few(const DecodeArgs& a, int n, int lane, SlotOf slot_of, float& mstar,
-                                          float& den, float& o0, float& o1) {
-  const int d = lane * 2;
+                                          float& den, float (&acc)[HD / 64]) {
+  constexpr int kDpl = HD / 64;  // dims per lane
+  typedef float fvec_t __attribute__((ext_vector_type(kDpl)));
+  const int d = lane * kDpl;
   float mj = -INFINITY, lj = 0.f;
   if (lane < n) {
     const int64_t slot = slot_of(lane);
     mj = a.ws_ml[slot * 2];
     lj = a.ws_ml[slot * 2 + 1];
   }
-  f32x2_t o[N];
+  fvec_t o[N];
 #pragma unroll
-  for (int u = 0; u < N; ++u) o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + slot_of(min(u, n - 1)) * 128 + d);
+  for (int u = 0; u < N; ++u) o[u] = *reinterpret_cast<const fvec_t*>(a.ws_o + slot_of(min(u, n - 1)) * HD + d);
   mstar = mj;
 #pragma unroll
   for (int off = N / 2; off > 0; off >>= 1) mstar = fmaxf(mstar, __shfl_xor(mstar, off));
@@ -876,25 +878,30 @@ __device__ __forceinline__ void merge_few(const DecodeArgs& a, int n, int lane, 
 #pragma unroll
   for (int off = N / 2; off > 0; off >>= 1) den += __shfl_xor(den, off);
   den = __shfl(den, 0);
-  o0 = 0.f;
-  o1 = 0.f;
+#pragma unroll
+  for (int e = 0; e < kDpl; ++e) acc[e] = 0.f;
 #pragma unroll
   for (int u = 0; u < N; ++u) {
     const float wu = __shfl(wj, u);  // 0 beyond n: the repeated last row does not count
-    o0 += o[u][0] * wu;
-    o1 += o[u][1] * wu;
+#pragma unroll
+    for (int e = 0; e < kDpl; ++e) acc[e] += o[u][e] * wu;
   }
 }
 
-template <typename SlotOf>
+template <int HD = 128, typename SlotOf>
 __device__ __forceinline__ void merge_rows(const DecodeArgs& a, int seq, int head, int n, int lane, SlotOf slot_of) {
-  const int d = lane * 2;
+  constexpr int kDpl = HD / 64;  // dims per lane
+  typedef float fvec_t __attribute__((ext_vector_type(kDpl)));
+  const int d = lane * kDpl;
   const int tq = scalar_load_i32(a.pt.cu_q_lens + seq);
-  float mstar = -INFINITY, den = 0.f, o0 = 0.f, o1 = 0.f;
+  float mstar = -INFINITY, den = 0.f;
+  float acc[kDpl];
+#pragma unroll
+  for (int e = 0; e < kDpl; ++e) acc[e] = 0.f;
   if (n <= 8) {
-    merge_few<8>(a, n, lane, slot_of, mstar, den, o0, o1);
+    merge_few<8, HD>(a, n, lane, slot_of, mstar, den, acc);
   } else if (n <= 16) {
-    merge_few<16>(a, n, lane, slot_of, mstar, den, o0, o1);
+    merge_few<16, HD>(a, n, lane, slot_of, mstar, den, acc);
   } else {
     for (int j0 = 0; j0 < n; j0 += 64) {
       const int j = j0 + lane;
@@ -918,25 +925,25 @@ __device__ __forceinline__ void merge_rows(const DecodeArgs& a, int seq, int hea
       // sequence cut over the whole GPU) is a chain of such round trips
       const int cnt = min(64, n - j0);
       for (int jj = 0; jj < cnt; jj += 32) {
-        f32x2_t o[32];
+        fvec_t o[32];
         float wv[32];
 #pragma unroll
         for (int u = 0; u < 32; ++u) {
           const int js = min(jj + u, cnt - 1);
           wv[u] = (jj + u < cnt) ? __shfl(wj, js) : 0.f;
-          o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + slot_of(j0 + js) * 128 + d);
+          o[u] = *reinterpret_cast<const fvec_t*>(a.ws_o + slot_of(j0 + js) * HD + d);
         }
 #pragma unroll
-        for (int u = 0; u < 32; ++u) {
-          o0 += o[u][0] * wv[u];
-          o1 += o[u][1] * wv[u];
-        }
+        for (int u = 0; u < 32; ++u)
+#pragma unroll
+          for (int e = 0; e < kDpl; ++e) acc[e] += o[u][e] * wv[u];
       }
     }
   }
   const float inv = a.sm.sink ? sink_inverse(mstar, den, sink_logit(a.sm.sink, a.sm.round_logits, head)) : 1.0f / den;
-  uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * 128 + d);
-  *op = pack_bf16x2(o0 * inv, o1 * inv);
+  uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)tq * a.Hq + head) * HD + d);
+#pragma unroll
+  for (int e = 0; e < kDpl; e += 2) op[e / 2] = pack_bf16x2(acc[e] * inv, acc[e + 1] * inv);
 }
 
 // Merge the partial rows of the balanced plan.  grid = (Hq, decode rows); block = one wave.
@@ -992,7 +999,11 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
   const int lane = threadIdx.x;
   const int c = lane & 15, g = lane >> 4;
   const int rg = blockIdx.z, hk = blockIdx.y;
-  const int tok_row = blockIdx.x + a.pt.cu_q_lens[seq_begin];
+  // decode rows may be cut into max_splits pieces of `chunk` tokens (one token per row then, and
+  // row = sequence); partial rows go to the workspace in the fixed plan's layout
+  const int nsplit = max(a.max_splits, 1);
+  const int split = blockIdx.x % nsplit;
+  const int tok_row = blockIdx.x / nsplit + a.pt.cu_q_lens[seq_begin];
   if (tok_row >= a.pt.cu_q_lens[seq_end]) return;
   const int seq = owner_of_token(a.pt.cu_q_lens, seq_end, tok_row);
   const int q0 = a.pt.cu_q_lens[seq];
@@ -1041,7 +1052,13 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
     for (int j = 0; j < 8; ++j) acc[hf][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  for (int tb = t_lo & ~(kBlk - 1); tb < t_hi; tb += kBlk) {
+  int tb_begin = t_lo & ~(kBlk - 1), tb_end = t_hi;
+  if (nsplit > 1) {
+    tb_begin += split * a.chunk;
+    if (tb_begin >= t_hi) return;  // the merge pass knows how many pieces a row has
+    if (split < nsplit - 1) tb_end = min(t_hi, tb_begin + a.chunk);
+  }
+  for (int tb = tb_begin; tb < tb_end; tb += kBlk) {
     int page = 0;
     if constexpr (UNIFORM_PAGE) page = __builtin_amdgcn_readfirstlane(sv.pages[page_slot_of(sv, tb)]);
     KvRegs<FP8> r0, r1;
@@ -1072,7 +1089,7 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
       if (round_bf16) v = bf16_round(v);
       v = v * kLog2e;
       const int tok = tb + tok_slot(g, i);
-      x[i] = (tok >= t_hi || tok < t_lo) ? mask2 : v;
+      x[i] = (tok >= tb_end || tok < t_lo) ? mask2 : v;
     }
     float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
     mx = fmaxf(mx, __shfl_xor(mx, 16));
@@ -1106,6 +1123,24 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
   if (row >= a.G) return;
   const int head = hk * a.G + row;
   const float vs = a.v_scale ? a.v_scale[hk] : 1.0f;
+  if (nsplit > 1) {
+    const int64_t slot = ((int64_t)seq * nsplit + split) * a.Hq + head;
+    float* wo = a.ws_o + slot * 256 + g * 32;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        f32x4_t w0 = {acc[hf][0][r] * vs, acc[hf][1][r] * vs, acc[hf][2][r] * vs, acc[hf][3][r] * vs};
+        f32x4_t w1 = {acc[hf][4][r] * vs, acc[hf][5][r] * vs, acc[hf][6][r] * vs, acc[hf][7][r] * vs};
+        *reinterpret_cast<f32x4_t*>(wo + hf * 128 + r * 8) = w0;
+        *reinterpret_cast<f32x4_t*>(wo + hf * 128 + r * 8 + 4) = w1;
+      }
+    if (g == 0) {
+      a.ws_ml[slot * 2 + 0] = m;
+      a.ws_ml[slot * 2 + 1] = l;
+    }
+    return;
+  }
   const float inv = a.sm.sink ? vs * sink_inverse(m, l, sink_logit(a.sm.sink, a.sm.round_logits, head)) : vs / l;
   uint16_t* op = a.out + ((int64_t)tok_row * a.Hq + head) * 256 + g * 32;
 #pragma unroll
@@ -1124,6 +1159,7 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
 // first fetches (m_j, l_j) of split j, the wave reduces m* and the denominator
 // with shuffles, then the weights are broadcast lane by lane while the partial
 // rows stream in with independent loads.
+template <int HD>
 __global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a) {
   const int head = blockIdx.x;
   const int seq = blockIdx.y;
@@ -1133,7 +1169,7 @@ __global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a) {
   const int n = min(a.max_splits, (kv_len - t0 + a.chunk - 1) / a.chunk);
   if (n <= 0) return;
   const int64_t base = ((int64_t)seq * a.max_splits) * a.Hq + head;
-  merge_rows(a, seq, head, n, lane, [&](int j) -> int64_t { return base + (int64_t)j * a.Hq; });
+  merge_rows<HD>(a, seq, head, n, lane, [&](int j) -> int64_t { return base + (int64_t)j * a.Hq; });
 }
 
 // One thread copies one 16-byte piece of one gathered row.
@@ -1232,7 +1268,7 @@ hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream) {
   hipError_t e = launch_decode_mt(a, grid, block, uniform, stream);
   if (e != hipSuccess) return e;
   if (a.max_splits > 1) {
-    hipLaunchKernelGGL(rpa_combine_kernel, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
+    hipLaunchKernelGGL(rpa_combine_kernel<128>, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
     e = hipGetLastError();
   }
   return e;
@@ -1249,7 +1285,9 @@ hipError_t launch_gather(const GatherArgs& a, hipStream_t stream) {
 hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int max_token_rows, hipStream_t stream) {
   if (seq_end <= seq_begin || max_token_rows <= 0) return hipSuccess;
   if (a.Hkv > 65535) return hipErrorInvalidValue;  // grid.y
-  const dim3 grid(max_token_rows, a.Hkv, (a.G + 15) / 16), block(64);
+  const int nsplit = a.max_splits > 1 ? a.max_splits : 1;
+  if ((int64_t)max_token_rows * nsplit > 0x7fffffffLL) return hipErrorInvalidValue;
+  const dim3 grid(max_token_rows * nsplit, a.Hkv, (a.G + 15) / 16), block(64);
   const bool uniform = (a.pt.page_size % kBlk) == 0;
   if (a.fp8) {
     if (uniform) hipLaunchKernelGGL((rpa_rows256_kernel<true, true>), grid, block, 0, stream, a, seq_begin, seq_end);
@@ -1258,6 +1296,10 @@ hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int m
     if (uniform) hipLaunchKernelGGL((rpa_rows256_kernel<false, true>), grid, block, 0, stream, a, seq_begin, seq_end);
     else hipLaunchKernelGGL((rpa_rows256_kernel<false, false>), grid, block, 0, stream, a, seq_begin, seq_end);
   }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || nsplit == 1) return e;
+  if (a.num_rows > 65535) return hipErrorInvalidValue;  // rows sit on the second grid dimension
+  hipLaunchKernelGGL(rpa_combine_kernel<256>, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
   return hipGetLastError();
 }
 

@@ -601,6 +601,28 @@ def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
             gpu_out(pkg, b, gpu, causal=False, custom_mask=cm.to(gpu))
 
 
+@pytest.mark.parametrize("kv_dtype,window", [(torch.bfloat16, None), (torch.float8_e4m3fn, None), (torch.bfloat16, 3000)])
+def test_head_dim_256_long_decode_rows_are_split(pkg, wl, gpu, kv_dtype, window):
+    """A few long 256-wide decode rows: too few (row, kv head) jobs to fill the GPU, so the rows
+    are cut into pieces and merged; against the oracle, against whole rows (num_splits = 1) and
+    with an attention sink (the sink enters once, in the merge)."""
+    kv_lens = [9000, 1, 4097, 12000, 257]
+    b = batch256(wl, "d256long", [1] * len(kv_lens), kv_lens, 94, Hq=8, Hkv=2, P=64, kv_dtype=kv_dtype,
+                 sliding_window=window)
+    tol = BF16_TOL if kv_dtype == torch.bfloat16 else FP8_TOL
+    say(f"case d256 long decode rows {kv_dtype} window={window}")
+    want = oracle_out(b)
+    auto = gpu_out(pkg, b, gpu)
+    whole = gpu_out(pkg, b, gpu, num_splits=1)
+    torch.testing.assert_close(auto.float(), want.float(), **tol)
+    torch.testing.assert_close(auto.float(), whole.float(), rtol=1e-2, atol=4e-3)
+    assert not torch.equal(auto, whole)  # merged rows differ from whole ones in the last bits somewhere
+    torch.testing.assert_close(gpu_out(pkg, b, gpu, num_splits=7).float(), whole.float(), rtol=1e-2, atol=4e-3)
+    sink = torch.from_numpy(np.random.RandomState(101).randn(8).astype(np.float32))
+    torch.testing.assert_close(gpu_out(pkg, b, gpu, attention_sink=sink).float(),
+                               oracle_out(b, attention_sink=sink).float(), **tol)
+
+
 def test_head_dim_256_cache_write_and_gather(pkg, wl, gpu):
     """The new-token write and the page gather take any head width (bit-exact)."""
     q_lens, kv_lens = [1, 7], [33, 40]
