@@ -52,7 +52,8 @@ typedef enum RpaKvDtype {
 
 typedef enum RpaSoftmaxDtype {
   RPA_SOFTMAX_F32 = 0,
-  RPA_SOFTMAX_BF16 = 1
+  RPA_SOFTMAX_BF16 = 1,
+  RPA_SOFTMAX_F16 = 2
 } RpaSoftmaxDtype;
 
 enum RpaMaskMode {

@@ -98,7 +98,7 @@ class RpaParams(ctypes.Structure):
 
 
 MASK_CAUSAL, MASK_CUSTOM, MASK_NONE = 0, 1, 2
-SOFTMAX_F32, SOFTMAX_BF16 = 0, 1
+SOFTMAX_F32, SOFTMAX_BF16, SOFTMAX_F16 = 0, 1, 2
 
 
 class RpaMlaParams(ctypes.Structure):

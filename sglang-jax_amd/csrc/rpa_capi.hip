@@ -90,7 +90,7 @@ rpa::SoftmaxOpts softmax_opts(const RpaParams* p) {
   s.mask_rows_page_aligned = p->mask_rows_page_aligned;
   s.custom_mask = p->custom_mask;
   s.cu_mask_lens = p->cu_mask_lens;
-  s.round_logits = p->softmax_dtype == RPA_SOFTMAX_BF16 ? 1 : 0;
+  s.round_logits = p->softmax_dtype == RPA_SOFTMAX_BF16 ? 1 : (p->softmax_dtype == RPA_SOFTMAX_F16 ? 2 : 0);
   s.q_scale = p->q_scale;
   return s;
 }
@@ -356,7 +356,7 @@ int rpa_validate(const RpaParams* p) {
     return fail(RPA_EINVAL_NULL, "RPA_MASK_CUSTOM needs custom_mask and cu_mask_lens");
   if (p->mask_mode == RPA_MASK_CUSTOM && p->mask_rows_page_aligned && !p->cu_kv_lens)
     return fail(RPA_EINVAL_NULL, "page-aligned mask rows need cu_kv_lens");
-  if (p->softmax_dtype != RPA_SOFTMAX_F32 && p->softmax_dtype != RPA_SOFTMAX_BF16)
+  if (p->softmax_dtype != RPA_SOFTMAX_F32 && p->softmax_dtype != RPA_SOFTMAX_BF16 && p->softmax_dtype != RPA_SOFTMAX_F16)
     return fail(RPA_EINVAL_DTYPE, "softmax_dtype=%d is not an RpaSoftmaxDtype", p->softmax_dtype);
   if (p->q_scale < 0.0f || std::isnan(p->q_scale))
     return fail(RPA_EINVAL_SHAPE, "q_scale=%g must be positive (0 = off)", p->q_scale);

@@ -63,10 +63,15 @@ __device__ __forceinline__ float xai_factor(int qpos, float xai_len) {
 
 __device__ __forceinline__ float bf16_round(float x) { return bf16_lo_to_f32(pack_bf16x2(x, 0.f)); }
 
+__device__ __forceinline__ float f16_round(float x) { return (float)(_Float16)x; }
+
+// a logit rounded to the softmax dtype: 1 = bf16, 2 = f16 (0, no rounding, is handled by the callers)
+__device__ __forceinline__ float round_logit(float x, int mode) { return mode == 1 ? bf16_round(x) : f16_round(x); }
+
 // the sink logit of a query head, rounded like the other logits when rounding is on
 __device__ __forceinline__ float sink_logit(const float* sink, int round_logits, int head) {
   const float s = sink[head];
-  return round_logits ? bf16_round(s) : s;
+  return round_logits ? round_logit(s, round_logits) : s;
 }
 
 // Queries divided by q_scale and rounded to the cache's element type

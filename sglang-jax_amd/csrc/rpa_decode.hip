@@ -126,7 +126,7 @@ struct ScoreOpts {
   float scale2;     // sm_scale * k_scale * log2(e)  (plain path)
   float cap, inv_cap;
   float temp;       // temperature factor                (soft-cap path; the plain path folds it into scale2)
-  bool round_bf16;  // logits rounded to bf16 before the softmax (soft-cap path)
+  int round_mode;   // logits rounded to bf16 (1) or f16 (2) before the softmax (soft-cap path)
   float mask2;      // mask value in log2 units (finite)
   int t_lo;         // first visible token (sliding window), 0 otherwise
   int kv_len;
@@ -211,7 +211,7 @@ __device__ __forceinline__ void compute_block(const KvRegs<FP8>& r, const u32x4_
         v = v * so.scale;
         if (so.cap != 0.f) v = soft_cap_f(v, so.cap, so.inv_cap);
         v = v * so.temp;
-        if (so.round_bf16) v = bf16_round(v);
+        if (so.round_mode) v = round_logit(v, so.round_mode);
         v = v * kLog2e;
       } else {
         v = v * so.scale2;
@@ -381,7 +381,7 @@ __device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int
   so.scale = a.sm.sm_scale * ks * (a.sm.q_scale > 0.f ? a.sm.q_scale : 1.0f);
   so.scale2 = so.scale * kLog2e * temp;
   so.temp = temp;
-  so.round_bf16 = a.sm.round_logits != 0;
+  so.round_mode = a.sm.round_logits;
   so.cap = a.sm.soft_cap;
   so.inv_cap = (so.cap != 0.f) ? 1.0f / so.cap : 0.f;
   so.mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
@@ -733,7 +733,7 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
       so.scale = a.sm.sm_scale * ks * (a.sm.q_scale > 0.f ? a.sm.q_scale : 1.0f);
       so.scale2 = so.scale * kLog2e * temp;
       so.temp = temp;
-      so.round_bf16 = a.sm.round_logits != 0;
+      so.round_mode = a.sm.round_logits;
       so.cap = a.sm.soft_cap;
       so.inv_cap = (so.cap != 0.f) ? 1.0f / so.cap : 0.f;
       so.mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
@@ -1043,7 +1043,7 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
   const float cap = a.sm.soft_cap;
   const float inv_cap = (cap != 0.f) ? 1.0f / cap : 0.f;
   const float mask2 = fmaxf(a.sm.mask_value * kLog2e, -3.0e38f);
-  const bool round_bf16 = a.sm.round_logits != 0;
+  const int round_mode = a.sm.round_logits;
 
   f32x4_t acc[2][8];
 #pragma unroll
@@ -1086,7 +1086,7 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
       float v = s[i >> 2][i & 3] * scale;
       if (cap != 0.f) v = soft_cap_f(v, cap, inv_cap);
       v = v * temp;
-      if (round_bf16) v = bf16_round(v);
+      if (round_mode) v = round_logit(v, round_mode);
       v = v * kLog2e;
       const int tok = tb + tok_slot(g, i);
       x[i] = (tok >= tb_end || tok < t_lo) ? mask2 : v;

@@ -39,7 +39,7 @@ struct SoftmaxOpts {
   int32_t mask_rows_page_aligned;
   const int32_t* custom_mask;
   const int32_t* cu_mask_lens;
-  int32_t round_logits;  // 1: masked logits and the sink are rounded to bf16 before the softmax
+  int32_t round_logits;  // masked logits and the sink are rounded before the softmax: 1 to bf16, 2 to f16
   float q_scale;         // > 0: queries are divided by it and rounded to the cache's element type; 0 => off
 };
 

@@ -154,7 +154,7 @@ struct Softmax {
   float scale, cap, inv_cap;
   float sc2;   // raw score -> log2 units inside the exponent (per row: carries the temperature factor)
   float temp;  // soft-cap path: temperature factor
-  bool round_bf16;  // soft-cap path: logits rounded to bf16 before the softmax
+  int round_mode;   // soft-cap path: logits rounded to bf16 (1) or f16 (2) before the softmax
 };
 
 // Online-softmax update of one 64-token tile.  On entry S holds raw scores (MFMA units); on
@@ -226,7 +226,7 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[ND]
         float x = S[mt][v] * sm.scale;
         if (sm.cap != 0.f) x = soft_cap_f(x, sm.cap, sm.inv_cap);
         x = x * sm.temp;
-        if (sm.round_bf16) x = bf16_round(x);
+        if (sm.round_mode) x = round_logit(x, sm.round_mode);
         S[mt][v] = x * kLog2e;
       }
   }
@@ -447,7 +447,7 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
     const float temp = EXT ? xai_factor(wr.qpos, a.sm.xai_len) : 1.0f;  // per query row
     sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e * temp;
     sm.temp = temp;
-    sm.round_bf16 = a.sm.round_logits != 0;
+    sm.round_mode = a.sm.round_logits;
   }
 
   f32x16_t O[T::kDimTiles];
@@ -708,7 +708,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
     const float temp = EXT ? xai_factor(wr.qpos, a.sm.xai_len) : 1.0f;  // per query row
     sm.sc2 = CAP ? 1.0f : sm.scale * kLog2e * temp;
     sm.temp = temp;
-    sm.round_bf16 = a.sm.round_logits != 0;
+    sm.round_mode = a.sm.round_logits;
   }
 
   f32x16_t O[4];

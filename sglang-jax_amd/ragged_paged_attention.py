@@ -236,8 +236,10 @@ class RpaCall:
             p.softmax_dtype = _lib.SOFTMAX_F32
         elif softmax_dtype == torch.bfloat16:
             p.softmax_dtype = _lib.SOFTMAX_BF16
+        elif softmax_dtype == torch.float16:
+            p.softmax_dtype = _lib.SOFTMAX_F16
         elif isinstance(softmax_dtype, torch.dtype) and softmax_dtype.is_floating_point:
-            raise NotImplementedError(f"softmax_dtype={softmax_dtype}: only float32 and bfloat16 are built")
+            raise NotImplementedError(f"softmax_dtype={softmax_dtype}: float32, bfloat16 and float16 are built")
         else:
             raise ValueError(f"Expected softmax_dtype to be a floating point dtype, got {softmax_dtype}")
         # ---- q_scale (kernel rpa_v3:463-478): queries quantised to the cache's element type

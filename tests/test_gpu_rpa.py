@@ -395,8 +395,14 @@ def test_softmax_dtype_bfloat16(pkg, wl, gpu, cap, use_sink):
     got = gpu_out(pkg, b, gpu, softmax_dtype=torch.bfloat16, **kw)
     torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
     assert torch.equal(gpu_out(pkg, b, gpu, softmax_dtype=torch.float32, **kw), gpu_out(pkg, b, gpu, **kw))
+    # float16 logits: finer than bf16, so closer to the float32 result than the bf16 run is
+    want16 = oracle_out(b, softmax_dtype=torch.float16, **kw)
+    got16 = gpu_out(pkg, b, gpu, softmax_dtype=torch.float16, **kw)
+    torch.testing.assert_close(got16.float(), want16.float(), **BF16_TOL)
+    f32 = oracle_out(b, **kw).float()
+    assert (got16.float() - f32).abs().mean() <= (got.float() - f32).abs().mean()
     with pytest.raises(NotImplementedError):
-        gpu_out(pkg, b, gpu, softmax_dtype=torch.float16)
+        gpu_out(pkg, b, gpu, softmax_dtype=torch.float64)
     with pytest.raises(ValueError):
         gpu_out(pkg, b, gpu, softmax_dtype=torch.int32)
 
