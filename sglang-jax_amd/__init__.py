@@ -11,6 +11,8 @@ from .backend import (  # noqa: F401
     ForwardMode,
     MLAAttentionBackend,
     build_forward_metadata,
+    build_verify_metadata,
+    pad_page_indices,
 )
 from .dsa import compute_topk_pages, sparse_mla_page_level, sparse_mla_via_dense  # noqa: F401
 from .mla import mla_ragged_paged_attention  # noqa: F401
@@ -27,6 +29,8 @@ __all__ = [
     "ForwardMode",
     "MLAAttentionBackend",
     "build_forward_metadata",
+    "build_verify_metadata",
+    "pad_page_indices",
     "DEFAULT_MASK_VALUE",
     "gather_pages",
     "mla_ragged_paged_attention",

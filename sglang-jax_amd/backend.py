@@ -135,6 +135,98 @@ def build_forward_metadata(
     }
 
 
+def pad_page_indices(page_indices, max_num_seqs: int, fixed_capacity: int | None = None) -> np.ndarray:
+    """Length bucketing of the flat page table on the speculative-decoding paths
+    (flashattention_backend.py:42-69): zero-padded either to ``fixed_capacity`` entries (an error if
+    it holds more already) or to ``max_num_seqs`` times the pages per sequence rounded up to a power
+    of two, 16 at least -- so that the table's shape, which is part of a compiled call's signature,
+    takes few distinct values.  The padding entries are valid page ids (0) that no kernel reads."""
+    page_indices = np.asarray(page_indices, dtype=np.int32)
+    if fixed_capacity is not None:
+        target = int(fixed_capacity)
+        if target < len(page_indices):
+            raise ValueError(f"page_indices exceed fixed capacity: required={len(page_indices)}, capacity={target}")
+    elif max_num_seqs > 0 and len(page_indices) > 0:
+        per_seq = cdiv(len(page_indices), max_num_seqs)
+        target = max_num_seqs * max(16, 1 << max(0, per_seq - 1).bit_length())
+    else:
+        return page_indices
+    out = np.zeros(target, dtype=np.int32)
+    out[: len(page_indices)] = page_indices
+    return out
+
+
+def build_verify_metadata(
+    *,
+    seq_lens,
+    draft_token_num: int,
+    logits_indices_selector,
+    custom_mask=None,
+    page_size: int,
+    dp_size: int = 1,
+    per_dp_bs_size: int | None = None,
+) -> dict:
+    """Host arithmetic of the target-verify branch of ``get_eagle_forward_metadata``
+    (flashattention_backend.py:298-376, 430-437).
+
+    ``seq_lens`` are the verified lengths per batch slot (0 for padding slots); the slots named by
+    ``logits_indices_selector`` each get ``draft_token_num`` query tokens, which also count towards
+    their kv length.  ``custom_mask`` is the flat tree mask as the draft worker builds it: slot
+    after slot, ``draft_token_num`` rows of ``kv_len`` entries (a padding slot holds
+    ``draft_token_num * (draft_token_num - 1)`` entries that are dropped).  It is repacked so that
+    every row is as wide as the slot's page-aligned kv length -- the width the kernel reads with
+    ``mask_aligned_to_cu_kv`` -- and each DP rank's part is padded to one common length, at least
+    the original length per rank rounded up to a multiple of 8.
+    """
+    seq_lens = np.asarray(seq_lens, dtype=np.int32)
+    if per_dp_bs_size is None:
+        per_dp_bs_size = len(seq_lens) // max(dp_size, 1)
+    if per_dp_bs_size * dp_size != len(seq_lens):
+        raise ValueError(f"expected per_dp_bs_size * dp_size == len(seq_lens), got {per_dp_bs_size} * {dp_size} != {len(seq_lens)}")
+    q = int(draft_token_num)
+    extend = np.zeros(len(seq_lens), dtype=np.int32)
+    extend[np.asarray(logits_indices_selector, dtype=np.int64)] = q
+    kv = seq_lens + extend
+    aligned = ((kv + page_size - 1) // page_size) * page_size
+
+    def sectioned_cumsum(lens):
+        cu = np.zeros((dp_size, per_dp_bs_size + 1), dtype=np.int32)
+        cu[:, 1:] = np.cumsum(np.asarray(lens, dtype=np.int32).reshape(dp_size, per_dp_bs_size), axis=1)
+        return cu.ravel()
+
+    packed = None
+    if custom_mask is not None:
+        cm = np.asarray(custom_mask)
+        if cm.dtype == np.bool_:
+            raise ValueError("custom_mask bool dtype is not supported; use int32 instead.")
+        per_rank_target = ((len(cm) // dp_size + 7) // 8) * 8 or 8
+        held = np.where(kv > 0, kv, q - 1).astype(np.int64)  # entries per row as the draft worker wrote them
+        start = np.concatenate([[0], np.cumsum(q * held)])
+        ranks = []
+        for r in range(dp_size):
+            rows = []
+            for s in range(r * per_dp_bs_size, (r + 1) * per_dp_bs_size):
+                width = int(aligned[s])
+                if kv[s] > 0:
+                    m = cm[start[s] : start[s] + q * int(kv[s])].reshape(q, int(kv[s]))
+                    rows.append(np.pad(m, ((0, 0), (0, width - int(kv[s])))).reshape(-1))
+                elif width > 0:
+                    rows.append(np.zeros(q * width, dtype=cm.dtype))
+            ranks.append(np.concatenate(rows) if rows else np.zeros(0, dtype=cm.dtype))
+        common = max(max(len(x) for x in ranks), per_rank_target)
+        packed = np.concatenate([np.pad(x, (0, common - len(x))) for x in ranks]).astype(np.int32)
+
+    n = np.sum(seq_lens.reshape(dp_size, per_dp_bs_size) > 0, axis=1, dtype=np.int32)
+    return {
+        "extend_seq_lens": extend,
+        "seq_lens": kv,
+        "cu_q_lens": sectioned_cumsum(extend),
+        "cu_kv_lens": sectioned_cumsum(aligned),
+        "distribution": np.column_stack([np.zeros_like(n), n, n]).ravel().astype(np.int32),
+        "custom_mask": packed,
+    }
+
+
 @dataclass
 class FlashAttentionMetadata:
     """Built once per forward pass, reused by every layer (flashattention_backend.py:72-120)."""

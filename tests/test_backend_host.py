@@ -117,3 +117,86 @@ def test_mla_extend_distribution(pkg):
                                     cache_loc=np.arange(16, dtype=np.int32), page_size=4,
                                     extend_distribution_is_mixed=True)
     assert md["distribution"].tolist() == [2, 2, 2]
+
+
+def test_pad_page_indices_buckets(pkg):
+    """flashattention_backend.py:42-69, worked by hand: 4 slots, 70 pages -> 18 per slot -> 32 per
+    slot -> 128 entries; 3 pages -> the floor of 16 per slot; a fixed capacity wins over both."""
+    pad = pkg.backend.pad_page_indices
+    out = pad(np.arange(1, 71), 4)
+    assert out.dtype == np.int32 and len(out) == 128
+    assert np.array_equal(out[:70], np.arange(1, 71)) and not out[70:].any()
+    assert len(pad(np.arange(3), 4)) == 64
+    assert len(pad(np.arange(64), 4)) == 64  # exactly 16 per slot stays
+    assert len(pad(np.arange(65), 4)) == 128  # 17 -> 32
+    assert len(pad(np.arange(0), 4)) == 0
+    assert len(pad(np.arange(5), 4, fixed_capacity=24)) == 24
+    with pytest.raises(ValueError, match="exceed fixed capacity: required=5, capacity=4"):
+        pad(np.arange(5), 4, fixed_capacity=4)
+
+
+def test_verify_metadata_hand_case(pkg):
+    """Target-verify (flashattention_backend.py:298-376): 3 slots, the middle one padding, 2 draft
+    tokens, pages of 4.  Verified lengths 3 and 1 become kv lengths 5 and 3; mask rows widen to 8
+    and 4 entries; the padding slot's 2*(2-1) mask entries vanish."""
+    m0 = np.array([1, 1, 1, 1, 0, 1, 1, 1, 1, 1], dtype=np.int32)  # 2 rows of 5
+    pad_slot = np.array([7, 7], dtype=np.int32)  # dropped
+    m2 = np.array([1, 1, 0, 1, 1, 1], dtype=np.int32)  # 2 rows of 3
+    md = pkg.backend.build_verify_metadata(
+        seq_lens=[3, 0, 1], draft_token_num=2, logits_indices_selector=[0, 2],
+        custom_mask=np.concatenate([m0, pad_slot, m2]), page_size=4,
+    )
+    assert md["extend_seq_lens"].tolist() == [2, 0, 2]
+    assert md["seq_lens"].tolist() == [5, 0, 3]
+    assert md["cu_q_lens"].tolist() == [0, 2, 2, 4]
+    assert md["cu_kv_lens"].tolist() == [0, 8, 8, 12]
+    assert md["distribution"].tolist() == [0, 2, 2]
+    want = [1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1, 1, 0, 0, 0, 1, 1, 0, 0, 1, 1, 1, 0]
+    assert md["custom_mask"].tolist() == want  # 24 entries: 18 in, rounded to 24, equals the packed length
+    assert md["custom_mask"].dtype == np.int32
+
+
+def test_verify_metadata_two_ranks_share_one_length(pkg):
+    """dp_size 2: each rank's packed mask is padded to the longer one (or to the original length per
+    rank rounded up to 8 when that is more), and the cumulative lengths restart per rank."""
+    q, P = 2, 4
+    kv = [9, 2]  # after the draft tokens: verified 7 and 0 -> second slot is padding?  no: verified 0 means padding
+    mask = np.concatenate([np.ones(q * 9, np.int32), np.full(q * (q - 1), 5, np.int32)])
+    md = pkg.backend.build_verify_metadata(
+        seq_lens=[7, 0], draft_token_num=q, logits_indices_selector=[0], custom_mask=mask, page_size=P, dp_size=2,
+    )
+    assert md["seq_lens"].tolist() == [9, 0]
+    assert md["cu_q_lens"].tolist() == [0, 2, 0, 0]
+    assert md["cu_kv_lens"].tolist() == [0, 12, 0, 0]
+    assert md["distribution"].tolist() == [0, 1, 1, 0, 0, 0]
+    cm = md["custom_mask"].reshape(2, -1)
+    assert cm.shape == (2, 24)  # rank 0 packs 2 rows of 12; 20 // 2 -> 16 is less
+    assert cm[0].reshape(2, 12)[:, :9].all() and not cm[0].reshape(2, 12)[:, 9:].any()
+    assert not cm[1].any()
+    with pytest.raises(ValueError, match="bool dtype is not supported"):
+        pkg.backend.build_verify_metadata(
+            seq_lens=[7, 0], draft_token_num=q, logits_indices_selector=[0],
+            custom_mask=np.ones(22, dtype=bool), page_size=P, dp_size=2,
+        )
+
+
+def test_verify_mask_runs_through_the_oracle_shapes(pkg):
+    """The packed mask has exactly the layout the kernel's aligned mode indexes:
+    row t of slot s starts at q * cu_kv_aligned[s] + t * aligned_len[s]."""
+    rng = np.random.default_rng(3)
+    q, P = 4, 16
+    verified = np.array([33, 0, 7, 120], dtype=np.int32)
+    kv = np.where(verified > 0, verified + q, 0)
+    parts = [rng.integers(0, 2, q * (k if k > 0 else q - 1)).astype(np.int32) for k in kv]
+    md = pkg.backend.build_verify_metadata(
+        seq_lens=verified, draft_token_num=q, logits_indices_selector=np.flatnonzero(verified),
+        custom_mask=np.concatenate(parts), page_size=P,
+    )
+    cu = md["cu_kv_lens"]
+    for s, k in enumerate(kv):
+        if k == 0:
+            continue
+        width = cu[s + 1] - cu[s]
+        for t in range(q):
+            row = md["custom_mask"][q * cu[s] + t * width :][:width]
+            assert np.array_equal(row[:k], parts[s].reshape(q, k)[t]) and not row[k:].any()

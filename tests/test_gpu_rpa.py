@@ -468,6 +468,33 @@ def test_custom_mask_and_no_mask(pkg, wl, gpu, P):
     torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=0).float(), oracle_out(b, causal=False).float(), **BF16_TOL)
 
 
+def test_target_verify_metadata_feeds_the_kernel(pkg, wl, gpu):
+    """Speculative decoding's verify step end to end: the host helper widens the draft worker's tree
+    mask to page-aligned rows (flashattention_backend.py:298-376) and the kernel reads it in that
+    layout; a padding slot closes the batch."""
+    draft, P = 4, 16
+    verified = np.array([66, 130, 0], dtype=np.int32)
+    kv = [70, 134]
+    rng = np.random.default_rng(21)
+    masks = []
+    for k in kv:
+        m = np.ones((draft, k), dtype=np.int32)
+        m[:, k - draft:] = np.tril((rng.random((draft, draft)) < 0.5).astype(np.int32)) | np.eye(draft, dtype=np.int32)
+        masks.append(m)
+    flat = np.concatenate([masks[0].ravel(), masks[1].ravel(), np.zeros(draft * (draft - 1), np.int32)])
+    md = pkg.backend.build_verify_metadata(seq_lens=verified, draft_token_num=draft, logits_indices_selector=[0, 1],
+                                           custom_mask=flat, page_size=P)
+    b = wl.make_batch("verify", [draft, draft], kv, num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=P, seed=5)
+    assert md["cu_q_lens"][:3].tolist() == b.cu_q_lens.tolist()
+    assert md["cu_kv_lens"][:3].tolist() == b.cu_kv_lens.tolist()
+    assert md["distribution"].tolist() == [0, 2, 2]
+    b.distribution = torch.from_numpy(md["distribution"])
+    say("case target verify")
+    want = oracle_out(b, causal=False, custom_mask=flat_mask(masks))
+    got = gpu_out(pkg, b, gpu, causal=0, custom_mask=torch.from_numpy(md["custom_mask"]).to(gpu), mask_aligned_to_cu_kv=True)
+    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+
+
 # ------------------------------------------------------------------ balanced decode plan
 @pytest.mark.parametrize("Hq,Hkv,window,kv_dtype", [(32, 8, None, torch.bfloat16), (96, 3, None, torch.bfloat16),
                                                     (16, 4, 700, torch.bfloat16), (64, 8, None, torch.float8_e4m3fn)])
