@@ -50,8 +50,8 @@ DECODE_KERNEL = {
 }
 
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", "rpa_prefill_async_kernel"): 364.1e6 + 77.5e6,
-    ("c2", "rpa_decode_balanced_kernel"): 501.0e6 + 2.7e6,
+    ("c2", "rpa_prefill_async_kernel"): 365.6e6 + 77.5e6,
+    ("c2", "rpa_decode_balanced_kernel"): 500.9e6 + 2.7e6,
     ("c3", "rpa_decode_splitkv_kernel"): 2148.6e6 + 1.9e6,
     ("c5", "rpa_mla_balanced_kernel"): 817.4e6 + 83.1e6,
 }
