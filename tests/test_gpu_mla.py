@@ -255,3 +255,30 @@ def test_random_mla_batches_against_oracle(pkg, wl, gpu, seed):
     T = sum(q_lens)
     assert torch.isfinite(got[:T].float()).all()
     torch.testing.assert_close(got[:T].float(), want.float(), **TOL)
+
+
+@pytest.mark.parametrize("seed", list(range(8)))
+def test_random_large_mla_batches_against_oracle(pkg, wl, gpu, seed):
+    """Seeded random batches large enough for the balanced plan: up to 39 decode rows of up to 9000
+    tokens, sometimes one of 15000-40000, with chunks behind them on odd seeds."""
+    rng = np.random.default_rng(70000 + seed)
+    Hq = int(rng.choice([16, 32, 48, 64, 128, 160]))
+    P = int(rng.choice([8, 16, 32, 64, 128]))
+    n_dec, n_pre = int(rng.integers(6, 40)), (int(rng.integers(0, 3)) if seed % 2 else 0)
+    kv_dec = rng.integers(1, 9000, size=n_dec)
+    if rng.integers(0, 2):
+        kv_dec[rng.integers(0, n_dec)] = int(rng.integers(15000, 40000))
+    q_pre = rng.integers(2, 60, size=n_pre)
+    kv_pre = q_pre + rng.integers(0, 400, size=n_pre)
+    q_lens = [1] * n_dec + [int(x) for x in q_pre]
+    kv_lens = [int(x) for x in kv_dec] + [int(x) for x in kv_pre]
+    window = int(rng.integers(1, 3000)) if rng.integers(0, 3) == 0 else None
+    cap = 30.0 if rng.integers(0, 3) == 0 else None
+    say(f"mla random large seed={seed} Hq={Hq} P={P} n_dec={n_dec} max_kv={max(kv_lens)} q={q_lens[n_dec:]} window={window} cap={cap}")
+    b = wl.make_mla_batch("mla_rand_large", q_lens, kv_lens, num_q_heads=Hq, lkv_dim=512, rope_dim=64, page_size=P,
+                          seed=5000 + seed, sliding_window=window, soft_cap=cap)
+    want = oracle(b)
+    got = run_gpu(pkg, b, gpu)
+    T = sum(q_lens)
+    assert torch.isfinite(got[:T].float()).all()
+    torch.testing.assert_close(got[:T].float(), want.float(), **TOL)

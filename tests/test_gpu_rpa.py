@@ -798,3 +798,37 @@ def test_random_batches_against_oracle(pkg, wl, gpu, seed):
     got = gpu_out(pkg, b, gpu, **kw)
     assert torch.isfinite(got.float()).all()
     torch.testing.assert_close(got.float(), want.float(), **(FP8_TOL if fp8 else BF16_TOL))
+
+
+@pytest.mark.parametrize("seed", list(range(10)))
+def test_random_large_batches_against_oracle(pkg, wl, gpu, seed):
+    """Seeded random batches large enough for the balanced decode plan and the split 256-wide rows: up to
+    47 decode rows of up to 12000 tokens, sometimes one of 20000-60000, next to chunks with prefixes."""
+    rng = np.random.default_rng(50000 + seed)
+    D = 256 if seed % 5 == 4 else 128
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    G = int(rng.choice([1, 2, 4, 8] if D == 256 else [1, 2, 4, 8, 16]))
+    P = int(rng.choice([4, 16, 32, 64, 128, 256]))
+    n_dec, n_pre = int(rng.integers(8, 48)), int(rng.integers(0, 4))
+    kv_dec = rng.integers(1, 12000, size=n_dec)
+    if rng.integers(0, 2):
+        kv_dec[rng.integers(0, n_dec)] = int(rng.integers(20000, 60000))
+    q_pre = rng.integers(2, 600, size=n_pre)
+    kv_pre = q_pre + rng.integers(0, 2500, size=n_pre) * rng.integers(0, 2, size=n_pre)
+    q_lens = [1] * n_dec + [int(x) for x in q_pre]
+    kv_lens = [int(x) for x in kv_dec] + [int(x) for x in kv_pre]
+    fp8 = bool(rng.integers(0, 2))
+    window = int(rng.integers(1, 4000)) if rng.integers(0, 3) == 0 else None
+    cap = float(rng.choice([10.0, 30.0])) if rng.integers(0, 3) == 0 else None
+    kw = {}
+    if rng.integers(0, 3) == 0:
+        kw["attention_sink"] = torch.from_numpy(rng.standard_normal(Hkv * G).astype(np.float32))
+    say(f"case random large seed={seed} D={D} Hkv={Hkv} G={G} P={P} n_dec={n_dec} max_kv={max(kv_lens)} q={q_lens[n_dec:]} "
+        f"kv_pre={kv_lens[n_dec:]} fp8={fp8} window={window} cap={cap} {list(kw)}")
+    b = wl.make_batch("rand_large", q_lens, kv_lens, num_q_heads=Hkv * G, num_kv_heads=Hkv, head_dim=D, page_size=P,
+                      seed=3000 + seed, kv_dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16,
+                      sliding_window=window, soft_cap=cap)
+    want = oracle_out(b, **kw)
+    got = gpu_out(pkg, b, gpu, **kw)
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got.float(), want.float(), **(FP8_TOL if fp8 else BF16_TOL))
