@@ -328,8 +328,6 @@ int rpa_validate(const RpaParams* p) {
                 p->num_q_heads, p->num_kv_heads);
   if (p->head_dim != 128 && p->head_dim != 256)
     return fail(RPA_EUNSUPPORTED, "head_dim=%d: 128 and 256 are built", p->head_dim);
-  if (p->head_dim == 256 && p->q_scale > 0.0f)
-    return fail(RPA_EUNSUPPORTED, "head_dim=256: q_scale is not built");
   if (p->head_dim == 256 && p->mask_mode == RPA_MASK_CUSTOM && p->kv_dtype != RPA_KV_BF16)
     return fail(RPA_EUNSUPPORTED, "head_dim=256: custom masks are built for bf16 caches only");
   if (p->kv_dtype != RPA_KV_BF16 && p->kv_dtype != RPA_KV_FP8_E4M3)

@@ -1036,9 +1036,10 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
       for (int st = 0; st < 4; ++st) {
         const int d0 = hf * 128 + (FP8 ? (g * 32 + st * 8) : (st * 32 + g * 8));
         qB[hf][st] = ld16(qp + d0);
+        if (a.sm.q_scale > 0.f) qB[hf][st] = requantise_q(qB[hf][st], a.sm.q_scale, FP8);
       }
   }
-  const float scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[hk] : 1.0f);
+  const float scale = a.sm.sm_scale * (a.k_scale ? a.k_scale[hk] : 1.0f) * (a.sm.q_scale > 0.f ? a.sm.q_scale : 1.0f);
   const float temp = xai_factor(qpos, a.sm.xai_len);
   const float cap = a.sm.soft_cap;
   const float inv_cap = (cap != 0.f) ? 1.0f / cap : 0.f;

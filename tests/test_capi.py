@@ -64,13 +64,13 @@ def test_static_validation_codes(pkg):
     assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EINVAL_DISTRIBUTION"
     p = base_params(pkg); p.head_dim = 64
     assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EUNSUPPORTED"
-    # 256-wide heads: accepted, but not with q_scale, and no workspace is needed
+    # 256-wide heads: accepted (q_scale too), no workspace for short rows, custom masks with bf16 caches only
     p = base_params(pkg); p.head_dim = 256
     assert lib.rpa_validate(ctypes.byref(p)) == 0
     p.decode_end = p.num_seqs
     assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
     p.q_scale = 0.5
-    assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EUNSUPPORTED"
+    assert lib.rpa_validate(ctypes.byref(p)) == 0
     p = base_params(pkg); p.softmax_dtype = 7
     assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EINVAL_DTYPE"
     p = base_params(pkg); p.q_scale = -1.0

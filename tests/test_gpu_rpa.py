@@ -616,6 +616,14 @@ def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
     tol = BF16_TOL if kv_dtype == torch.bfloat16 else FP8_TOL
     for kw in ({}, {"attention_sink": sink}, {"xai_temperature_len": 64.0}, {"softmax_dtype": torch.bfloat16}):
         torch.testing.assert_close(gpu_out(pkg, b, gpu, **kw).float(), oracle_out(b, **kw).float(), **tol)
+    # queries quantised to the cache's element type (ragged_paged_attention_v3.py:463-478)
+    from oracle.ref_rpa import quantise_queries
+    got = gpu_out(pkg, b, gpu, q_scale=0.37)
+    q_orig, sm_orig = b.q, b.sm_scale
+    b.q, b.sm_scale = quantise_queries(q_orig, 0.37, kv_dtype), sm_orig * 0.37
+    want = oracle_out(b)
+    b.q, b.sm_scale = q_orig, sm_orig
+    torch.testing.assert_close(got.float(), want.float(), **tol)
     # full attention (causal = 0 without a mask)
     torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=False).float(), oracle_out(b, causal=False).float(), **tol)
     # custom masks: every row goes through the flash kernel, which is built for bf16 caches
