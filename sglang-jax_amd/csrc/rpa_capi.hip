@@ -293,7 +293,7 @@ int rows256(const RpaParams* p, int seq_begin, int seq_end, void* stream) {
   a.fp8 = p->kv_dtype == RPA_KV_FP8_E4M3;
   // decode rows are one token each; other sequences are bounded by the tokens of the call
   const int rows = (seq_end <= p->decode_end) ? (seq_end - seq_begin) : p->num_tokens;
-  if (seq_begin == 0 && seq_end == p->decode_end) {
+  if (seq_begin == 0 && seq_end == p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) {
     const SplitPlan sp = rows256_plan(p);
     if (sp.splits > 1) {
       const size_t need = rows256_workspace(p);
@@ -328,8 +328,6 @@ int rpa_validate(const RpaParams* p) {
                 p->num_q_heads, p->num_kv_heads);
   if (p->head_dim != 128 && p->head_dim != 256)
     return fail(RPA_EUNSUPPORTED, "head_dim=%d: 128 and 256 are built", p->head_dim);
-  if (p->head_dim == 256 && p->mask_mode == RPA_MASK_CUSTOM && p->kv_dtype != RPA_KV_BF16)
-    return fail(RPA_EUNSUPPORTED, "head_dim=256: custom masks are built for bf16 caches only");
   if (p->kv_dtype != RPA_KV_BF16 && p->kv_dtype != RPA_KV_FP8_E4M3)
     return fail(RPA_EINVAL_DTYPE, "kv_dtype=%d is not a floating point cache dtype", p->kv_dtype);
   if (p->layout != RPA_LAYOUT_FUSED && p->layout != RPA_LAYOUT_SPLIT)
@@ -507,7 +505,7 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   // 256-wide heads: bf16 caches take the flash kernel (two 128-dim halves per row, one workgroup
   // per CU); fp8 caches and rows the caller masks itself stay on the row kernel
   if (p->head_dim == 256 && (p->kv_dtype == RPA_KV_FP8_E4M3 || env_int("RPA_PREFILL_ROWS256", 0) != 0))
-    return rows256(p, p->decode_end, p->num_seqs, stream);
+    return rows256(p, (p->mask_mode == RPA_MASK_CUSTOM) ? 0 : p->decode_end, p->num_seqs, stream);
   rpa::PrefillArgs a;
   a.head_dim = p->head_dim;
   a.q = static_cast<const uint16_t*>(p->q);

@@ -1014,6 +1014,12 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
   const int t_hi = (a.sm.mask_mode == 0) ? qpos + 1 : kv_len;
   if (t_hi <= 0) return;
   const int t_lo = (a.sm.window > 0) ? max(0, qpos - a.sm.window + 1) : 0;
+  // the caller's own mask: one i32 per (query token, kv token), rows kv_len wide or padded to whole pages
+  const int32_t* mask_row = nullptr;
+  if (a.sm.mask_mode == 1) {
+    const int width = a.sm.mask_rows_page_aligned ? (a.pt.cu_kv_lens[seq + 1] - a.pt.cu_kv_lens[seq]) : kv_len;
+    mask_row = a.sm.custom_mask + a.sm.cu_mask_lens[seq] + (int64_t)(tok_row - q0) * width;
+  }
 
   SeqView sv;
   sv.page_size = a.pt.page_size;
@@ -1090,7 +1096,9 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
       if (round_mode) v = round_logit(v, round_mode);
       v = v * kLog2e;
       const int tok = tb + tok_slot(g, i);
-      x[i] = (tok >= tb_end || tok < t_lo) ? mask2 : v;
+      bool dead = tok >= tb_end || tok < t_lo;
+      if (mask_row && !dead) dead = mask_row[tok] < 1;
+      x[i] = dead ? mask2 : v;
     }
     float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
     mx = fmaxf(mx, __shfl_xor(mx, 16));

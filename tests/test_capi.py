@@ -64,7 +64,7 @@ def test_static_validation_codes(pkg):
     assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EINVAL_DISTRIBUTION"
     p = base_params(pkg); p.head_dim = 64
     assert status(pkg, lib.rpa_validate(ctypes.byref(p))) == "RPA_EUNSUPPORTED"
-    # 256-wide heads: accepted (q_scale too), no workspace for short rows, custom masks with bf16 caches only
+    # 256-wide heads: accepted (q_scale too), no workspace for short rows
     p = base_params(pkg); p.head_dim = 256
     assert lib.rpa_validate(ctypes.byref(p)) == 0
     p.decode_end = p.num_seqs

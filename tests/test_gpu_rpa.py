@@ -626,7 +626,7 @@ def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
     torch.testing.assert_close(got.float(), want.float(), **tol)
     # full attention (causal = 0 without a mask)
     torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=False).float(), oracle_out(b, causal=False).float(), **tol)
-    # custom masks: every row goes through the flash kernel, which is built for bf16 caches
+    # custom masks: every row goes through the flash kernel (bf16 caches) or the row kernel (fp8)
     rng = np.random.default_rng(11)
     masks = []
     for ql, kv in zip(q_lens, kv_lens):
@@ -634,12 +634,14 @@ def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
         mk[:, 0] = 1
         masks.append(mk)
     cm = flat_mask(masks)
-    if kv_dtype == torch.bfloat16:
-        torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=False, custom_mask=cm.to(gpu)).float(),
-                                   oracle_out(b, causal=False, custom_mask=cm).float(), **tol)
-    else:
-        with pytest.raises(ValueError, match="custom masks"):
-            gpu_out(pkg, b, gpu, causal=False, custom_mask=cm.to(gpu))
+    torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=False, custom_mask=cm.to(gpu)).float(),
+                               oracle_out(b, causal=False, custom_mask=cm).float(), **tol)
+    # the same masks in rows padded to whole pages
+    P = 32
+    padded = [np.pad(mk, ((0, 0), (0, -(-mk.shape[1] // P) * P - mk.shape[1]))) for mk in masks]
+    torch.testing.assert_close(
+        gpu_out(pkg, b, gpu, causal=False, custom_mask=flat_mask(padded).to(gpu), mask_aligned_to_cu_kv=True).float(),
+        oracle_out(b, causal=False, custom_mask=cm).float(), **tol)
 
 
 @pytest.mark.parametrize("kv_dtype,window", [(torch.bfloat16, None), (torch.float8_e4m3fn, None), (torch.bfloat16, 3000)])
