@@ -572,7 +572,6 @@ static int mla_validate(const RpaMlaParams* p) {
   if (p->row_stride < p->rope_offset + p->rope_dim || p->rope_offset < p->lkv_dim || (p->row_stride % 8) != 0 ||
       (p->rope_offset % 8) != 0)
     return fail(RPA_EINVAL_SHAPE, "row_stride=%d rope_offset=%d do not describe [kv_c | k_pe]", p->row_stride, p->rope_offset);
-  if (p->num_q_heads % 16 != 0) return fail(RPA_EUNSUPPORTED, "num_q_heads=%d must be a multiple of 16", p->num_q_heads);
   if (p->sliding_window < 0) return fail(RPA_EINVAL_WINDOW, "sliding_window=%d must be positive", p->sliding_window);
   if (p->num_seqs > 0 && (!p->ql_nope || !p->q_pe || !p->out || !p->cache_kv || !p->kv_lens || !p->page_indices || !p->cu_q_lens))
     return fail(RPA_EINVAL_NULL, "a required buffer is NULL");

@@ -282,3 +282,24 @@ def test_random_large_mla_batches_against_oracle(pkg, wl, gpu, seed):
     T = sum(q_lens)
     assert torch.isfinite(got[:T].float()).all()
     torch.testing.assert_close(got[:T].float(), want.float(), **TOL)
+
+
+@pytest.mark.parametrize("Hq", [8, 24, 40, 100, 136])
+def test_mla_head_counts_off_the_sixteen_head_tile(pkg, wl, gpu, Hq):
+    """Head counts that do not fill the last 16-head MFMA tile (a tensor-parallel share of 8 heads,
+    say): the spare columns read a clamped head and write nothing.  Decode rows (both plans) and
+    a mixed batch."""
+    say(f"mla heads Hq={Hq}")
+    b = wl.make_mla_batch("mla_heads", [1] * 5, [3, 700, 64, 2049, 130], num_q_heads=Hq, lkv_dim=512, rope_dim=64,
+                          page_size=32, seed=610 + Hq)
+    want = oracle(b)
+    for kw in ({}, {"num_splits": 1}, {"num_splits": 4}):
+        got = run_gpu(pkg, b, gpu, **kw)
+        torch.testing.assert_close(got[:5].float(), want.float(), **TOL)
+    q_lens, kv_lens = [1, 1, 9, 33], [40, 900, 9, 133]
+    b = wl.make_mla_batch("mla_heads_mixed", q_lens, kv_lens, num_q_heads=Hq, lkv_dim=512, rope_dim=64, page_size=16,
+                          seed=620 + Hq)
+    got = run_gpu(pkg, b, gpu)
+    T = sum(q_lens)
+    assert torch.isfinite(got[:T].float()).all()
+    torch.testing.assert_close(got[:T].float(), oracle(b).float(), **TOL)
