@@ -56,7 +56,7 @@ typedef enum RpaSoftmaxDtype {
   RPA_SOFTMAX_F16 = 2
 } RpaSoftmaxDtype;
 
-enum RpaMaskMode {
+typedef enum RpaMaskMode {
   RPA_MASK_CAUSAL = 0, /* query j of a sequence sees tokens <= kv_len - q_len + j */
   RPA_MASK_CUSTOM = 1, /* causal = 0 with custom_mask (speculative tree verification) */
   RPA_MASK_NONE = 2    /* causal = 0 without a mask: every query sees all kv_len tokens */

@@ -15,6 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(OUT_DIR, "librpa_mi355.so")
+HASH_PATH = os.path.join(OUT_DIR, "librpa_mi355.srchash")
 
 SOURCES = ["rpa_capi.hip", "rpa_decode.hip", "rpa_prefill.hip", "rpa_mla.hip"]
 
@@ -41,6 +42,20 @@ def _run(cmd):
     return out
 
 
+def source_hash() -> str:
+    """Hash of everything the library is compiled from (and of the flags)."""
+    import hashlib
+
+    h = hashlib.sha256(" ".join(FLAGS).encode())
+    files = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC))
+    files.append(os.path.join(os.path.dirname(HERE), "include", "rpa.h"))
+    for path in files:
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def build(verbose: bool = False, extra_flags=()) -> str:
     os.makedirs(OUT_DIR, exist_ok=True)
     objs = []
@@ -57,6 +72,11 @@ def build(verbose: bool = False, extra_flags=()) -> str:
     tmp = LIB_PATH + ".tmp"
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp])
     os.replace(tmp, LIB_PATH)
+    if not extra_flags:
+        with open(HASH_PATH, "w") as f:
+            f.write(source_hash() + "\n")
+    elif os.path.exists(HASH_PATH):
+        os.remove(HASH_PATH)  # an experimental build never passes for the committed sources
     for o in objs:
         os.remove(o)
     return LIB_PATH

@@ -28,6 +28,33 @@ def test_library_exports_every_declared_symbol(pkg):
     assert lib.rpa_version() == 100
 
 
+def test_header_links_from_two_translation_units(tmp_path):
+    """A consumer with several translation units (C or C++) must link: the header may define no
+    object, only types and declarations."""
+    import subprocess
+
+    inc = os.path.join(ROOT, "include")
+    for cc, ext in (("gcc", "c"), ("g++", "cc")):
+        a, b = tmp_path / f"a.{ext}", tmp_path / f"b.{ext}"
+        a.write_text('#include "rpa.h"\nint from_a(void) { RpaMaskMode m = RPA_MASK_CUSTOM; return (int)m + RPA_VERSION; }\n')
+        b.write_text('#include "rpa.h"\nint from_a(void);\nint main(void) { RpaLayout l = RPA_LAYOUT_SPLIT; '
+                     'return from_a() + (int)l + (int)sizeof(RpaParams) == 0; }\n')
+        out = tmp_path / f"two_units_{ext}"
+        r = subprocess.run([cc, "-Wall", "-Werror", "-I", inc, str(a), str(b), "-o", str(out)],
+                           capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr
+        assert subprocess.run([str(out)]).returncode == 0
+
+
+def test_library_exports_no_stray_data_symbol(pkg):
+    import subprocess
+
+    r = subprocess.run(["nm", "-D", "--defined-only", pkg._lib.LIB_PATH], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    data = [ln.split()[-1] for ln in r.stdout.splitlines() if len(ln.split()) == 3 and ln.split()[1] in "BDCbd"]
+    assert not [n for n in data if n.startswith("Rpa")], data
+
+
 def test_struct_layout_matches_header(pkg):
     # 11 pointers + size_t + 15 int32 + 3 float + int64
     assert ctypes.sizeof(pkg._lib.RpaParams) == 12 * 8 + 18 * 4 + 8 + 3 * 8 + 5 * 4 + 4  # + tail padding
