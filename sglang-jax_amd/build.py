@@ -17,7 +17,7 @@ OUT_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(OUT_DIR, "librpa_mi355.so")
 HASH_PATH = os.path.join(OUT_DIR, "librpa_mi355.srchash")
 
-SOURCES = ["rpa_capi.hip", "rpa_decode.hip", "rpa_prefill.hip", "rpa_mla.hip"]
+SOURCES = ["rpa_capi.hip", "rpa_decode.hip", "rpa_prefill.hip", "rpa_prefill_pipe.hip", "rpa_mla.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

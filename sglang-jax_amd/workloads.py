@@ -316,6 +316,134 @@ def config_c5(device="cpu", scale: float = 1.0, num_q_heads: int = 128) -> MlaBa
 
 
 # --------------------------------------------------------------------------
+# Peaked inputs: a few keys per (sequence, kv head) that every query of that head attends to
+# --------------------------------------------------------------------------
+def needle_positions(rng: np.random.Generator, kv_len: int, window: int | None, count: int = 4) -> list[int]:
+    """Token positions worth a needle: the first and last tiles of the row, tile / page / piece
+    borders inside it (multiples of 32 ... 4096 and their neighbours) and the edge of the sliding
+    window.  One position always comes from the first 64 tokens and one from the last 64."""
+    cand = {0, 1, 31, 32, 63, 64, kv_len - 1, kv_len - 2, kv_len - 32, kv_len - 33, kv_len - 64, kv_len - 65}
+    for step in (32, 64, 128, 256, 512, 1024, 4096):
+        for k in rng.integers(1, max(2, kv_len // step + 1), size=2):
+            cand.update({int(k) * step - 1, int(k) * step})
+    if window:
+        cand.update({kv_len - window - 1, kv_len - window, kv_len - window + 1})
+    cand = sorted(t for t in cand if 0 <= t < kv_len)
+    first = [t for t in cand if t < 64]
+    last = [t for t in cand if t >= kv_len - 64]
+    picks = {int(rng.choice(first)), int(rng.choice(last))}
+    picks.update(int(t) for t in rng.choice(cand, size=min(count, len(cand)), replace=False))
+    return sorted(picks)
+
+
+def plant_needles(b: Batch, *, logit: float = 14.0, seed: int = 0, count: int = 4) -> dict:
+    """Make the batch peaked, in place: for every (sequence, kv head) draw a
+    direction u of +-1/sqrt(D) entries, add a*u to the queries of that head group and overwrite the
+    K rows of a few tokens with a*u, a = sqrt(logit / sm_scale), so that those tokens score about
+    `logit` above the random ones and carry most of the softmax weight: output rows are O(1)
+    whatever the row length, and losing the tile, split or partial row that holds a needle
+    changes them by tens of per cent.  Returns {(seq, kv head): positions}."""
+    rng = np.random.Generator(np.random.PCG64(77000 + seed))
+    dev = b.q.device
+    P, Hkv = b.page_size, b.num_kv_heads
+    Hq, D = b.q.shape[1], b.q.shape[2]
+    G = Hq // Hkv
+    a = math.sqrt(logit / b.sm_scale)
+    kv = b.kv_lens.cpu().numpy()
+    cu_q = b.cu_q_lens.cpu().numpy()
+    cu_kv = b.cu_kv_lens.cpu().numpy()
+    pages = b.page_indices.cpu().numpy()
+    n = int(b.distribution[2])
+    k_scale = None if b.k_scale is None else b.k_scale.cpu()
+    fp8 = b.kv_cache.dtype != torch.bfloat16
+    placed = {}
+    q = b.q.float()
+    for i in range(n):
+        for h in range(Hkv):
+            u = torch.from_numpy(rng.choice([-1.0, 1.0], size=D).astype(np.float32)) / math.sqrt(D)
+            q[cu_q[i]:cu_q[i + 1], h * G:(h + 1) * G] += (a * u).to(dev)
+            pos = needle_positions(rng, int(kv[i]), b.sliding_window, count)
+            for t in pos:
+                page = int(pages[cu_kv[i] // P + t // P])
+                row = a * u
+                if fp8:
+                    row = row / k_scale[h]
+                b.kv_cache[page, t % P, 2 * h] = row.to(b.kv_cache.dtype).to(dev)
+            placed[(i, h)] = pos
+    b.q = q.to(torch.bfloat16)
+    return placed
+
+
+def plant_mla_needles(b: MlaBatch, *, logit: float = 14.0, seed: int = 0, count: int = 4) -> dict:
+    """`plant_needles` for the latent cache: one direction per sequence over the whole 576-wide
+    row, shared by every query head (they all read the same latent rows)."""
+    rng = np.random.Generator(np.random.PCG64(78000 + seed))
+    dev = b.ql_nope.device
+    P = b.page_size
+    lkv, rope = b.ql_nope.shape[2], b.q_pe.shape[2]
+    W = lkv + rope
+    a = math.sqrt(logit / b.sm_scale)
+    kv = b.kv_lens.cpu().numpy()
+    cu_q = b.cu_q_lens.cpu().numpy()
+    cu_kv = b.cu_kv_lens.cpu().numpy()
+    pages = b.page_indices.cpu().numpy()
+    placed = {}
+    qn, qp = b.ql_nope.float(), b.q_pe.float()
+    for i in range(int(b.distribution[2])):
+        u = (torch.from_numpy(rng.choice([-1.0, 1.0], size=W).astype(np.float32)) / math.sqrt(W)).to(dev)
+        qn[cu_q[i]:cu_q[i + 1]] += a * u[:lkv]
+        qp[cu_q[i]:cu_q[i + 1]] += a * u[lkv:]
+        pos = needle_positions(rng, int(kv[i]), b.sliding_window, count)
+        for t in pos:
+            page = int(pages[cu_kv[i] // P + t // P])
+            # the row is K and V at once: keep its random part (the value), add the needle
+            b.cache_kv[page, t % P, :W] = (b.cache_kv[page, t % P, :W].float() + a * u).to(torch.bfloat16)
+        placed[i] = pos
+    b.ql_nope, b.q_pe = qn.to(torch.bfloat16), qp.to(torch.bfloat16)
+    return placed
+
+
+def sub_batch(b: Batch, seqs, last_rows: int | None = None) -> Batch:
+    """The sequences `seqs` of `b` as a compact CPU batch of their own (pages renumbered 0..n-1,
+    same page contents).  With `last_rows`, a chunk keeps only its last `last_rows` query tokens
+    (their results do not depend on the tokens dropped: a causal row sees its own past only)."""
+    P = b.page_size
+    kv = b.kv_lens.cpu().numpy()
+    cu_q = b.cu_q_lens.cpu().numpy()
+    cu_kv = b.cu_kv_lens.cpu().numpy()
+    pages = b.page_indices.cpu().numpy()
+    q_rows, new_pages, q_lens, kv_lens = [], [], [], []
+    for i in seqs:
+        q0, q1 = int(cu_q[i]), int(cu_q[i + 1])
+        if last_rows is not None:
+            q0 = max(q0, q1 - last_rows)
+        q_rows.append(torch.arange(q0, q1))
+        cnt = -(-int(kv[i]) // P)
+        new_pages.append(pages[cu_kv[i] // P: cu_kv[i] // P + cnt])
+        q_lens.append(q1 - q0)
+        kv_lens.append(int(kv[i]))
+    q_rows = torch.cat(q_rows)
+    old = np.concatenate(new_pages).astype(np.int64)
+    counts = np.array([len(x) for x in new_pages])
+    cu_kv_new = np.zeros(len(seqs) + 1, dtype=np.int32)
+    cu_kv_new[1:] = np.cumsum(counts * P)
+    cu_q_new = np.zeros(len(seqs) + 1, dtype=np.int32)
+    cu_q_new[1:] = np.cumsum(q_lens)
+    dec = 0
+    while dec < len(seqs) and q_lens[dec] == 1:
+        dec += 1
+    dev = b.q.device
+    return Batch(
+        name=b.name + "_sample", q=b.q[q_rows.to(dev)].cpu(), kv_cache=b.kv_cache[torch.from_numpy(old).to(dev)].cpu(),
+        kv_lens=torch.tensor(kv_lens, dtype=torch.int32), page_indices=torch.arange(len(old), dtype=torch.int32),
+        cu_q_lens=torch.from_numpy(cu_q_new), cu_kv_lens=torch.from_numpy(cu_kv_new),
+        distribution=torch.tensor([dec, dec, len(seqs)], dtype=torch.int32), sm_scale=b.sm_scale, page_size=P,
+        num_kv_heads=b.num_kv_heads, sliding_window=b.sliding_window, soft_cap=b.soft_cap,
+        k_scale=None if b.k_scale is None else b.k_scale.cpu(), v_scale=None if b.v_scale is None else b.v_scale.cpu(),
+        meta={"q_lens": q_lens, "kv_lens": kv_lens, "rows": q_rows.tolist()})
+
+
+# --------------------------------------------------------------------------
 # Algorithmic bytes / FLOPs of a batch (the numerators of every roofline figure)
 # --------------------------------------------------------------------------
 def decode_bytes(b: Batch, lo: int = 0, hi: int | None = None) -> int:

@@ -15,6 +15,8 @@ import numpy as np
 import pytest
 import torch
 
+from parity import assert_parity, row_rel_error
+
 from oracle.ref_rpa import gather_pages as oracle_gather
 from oracle.ref_rpa import ref_ragged_paged_attention, ref_ragged_paged_attention_fused, split_fused_cache
 
@@ -57,7 +59,7 @@ def check(pkg, wl, dev, name, q_lens, kv_lens, *, Hq=32, Hkv=8, P=64, seed=0, to
     want = oracle_out(b)
     got = gpu_out(pkg, b, dev)
     assert torch.isfinite(got.float()).all()
-    torch.testing.assert_close(got.float(), want.float(), **tol)
+    assert_parity(got.float(), want.float(), **tol)
     return b, got
 
 
@@ -119,7 +121,7 @@ def test_decode_split_count_does_not_matter(pkg, wl, gpu):
     for ns in (1, 2, 3, 8, 33):
         say(f"num_splits {ns}")
         got = gpu_out(pkg, b, gpu, num_splits=ns)
-        torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+        assert_parity(got.float(), want.float(), **BF16_TOL)
         if base is None:
             base = got
         # different split counts agree to f32 rounding, far inside the oracle tolerance
@@ -192,7 +194,7 @@ def test_padded_batch_rows_are_ignored(pkg, wl, gpu):
                       seed=47, pad_tokens=22, pad_seqs=5)
     want = oracle_out(b)
     got = gpu_out(pkg, b, gpu)
-    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    assert_parity(got.float(), want.float(), **BF16_TOL)
 
 
 # ------------------------------------------------------------------ fp8 KV
@@ -234,7 +236,7 @@ def test_reference_surface_split_pages_and_2d_table(pkg, wl, gpu):
             b.q.to(gpu), kp.to(gpu), vp.to(gpu), b.kv_lens, table, b.cu_q_lens, [4], sm_scale=b.sm_scale,
             sliding_window=50, decode_end=decode_end, max_q_len=33)
         torch.cuda.synchronize()
-        torch.testing.assert_close(got.cpu().float(), want.float(), **BF16_TOL)
+        assert_parity(got.cpu().float(), want.float(), **BF16_TOL)
 
 
 def test_new_tokens_are_written_into_the_cache(pkg, wl, gpu):
@@ -264,7 +266,7 @@ def test_new_tokens_are_written_into_the_cache(pkg, wl, gpu):
         b.distribution.numpy(), None, sm_scale=b.sm_scale, max_kv_len=300, max_q_len=65)
     torch.cuda.synchronize()
     assert torch.equal(cache.cpu().view(torch.int16), b.kv_cache.view(torch.int16))
-    torch.testing.assert_close(out.cpu().float(), want.float(), **BF16_TOL)
+    assert_parity(out.cpu().float(), want.float(), **BF16_TOL)
 
 
 def test_dynamic_validation_through_the_wrapper(pkg, wl, gpu):
@@ -290,14 +292,14 @@ def test_benchmark_configs_against_oracle(pkg, wl, gpu, name, scale):
     tol = FP8_TOL if b.kv_cache.dtype != torch.bfloat16 else BF16_TOL
     want = oracle_out(b)
     got = gpu_out(pkg, b, gpu)
-    torch.testing.assert_close(got.float(), want.float(), **tol)
+    assert_parity(got.float(), want.float(), **tol)
 
 
 def test_c4_sliding_window_layer_against_oracle(pkg, wl, gpu):
     b = wl.config_c4(scale=0.1, window=True)
     want = oracle_out(b)
     got = gpu_out(pkg, b, gpu)
-    torch.testing.assert_close(got.float(), want.float(), **FP8_TOL)
+    assert_parity(got.float(), want.float(), **FP8_TOL)
 
 
 def _permute_pages(b, seed):
@@ -313,16 +315,20 @@ def _permute_pages(b, seed):
     return c
 
 
-@pytest.mark.parametrize("name", ["config_c3", "config_c2", "config_c4"])
+@pytest.mark.parametrize("name", ["config_c3", "config_c2", "config_c4", "config_c4_swa"])
 def test_full_size_page_permutation_invariance(pkg, wl, gpu, name):
-    """Full benchmark size, no oracle: the output must not depend, bit for bit, on
-    where pages physically live, and split-KV must agree with a single pass."""
-    scale = 0.25 if name == "config_c3" else 1.0  # C3 at 8192 tokens x 16 seqs = 0.5 GiB pool
-    b = getattr(wl, name)(device=gpu, scale=scale)
+    """Full benchmark size (C3: 16 rows of 32768 tokens, a 2 GiB pool) with peaked inputs.  The output
+    must not depend, bit for bit, on where pages physically live; split-KV must agree with a single
+    pass; and a sample of rows (first, longest and last decode rows, the last 128 rows of the last
+    chunk), re-run by the oracle on a compact copy of their pages, must match."""
+    b = wl.config_c4(device=gpu, window=True) if name == "config_c4_swa" else getattr(wl, name)(device=gpu)
+    wl.plant_needles(b, seed=17)
     q_lens = b.q_lens()
     n = int(b.distribution[2])
+    dec_end = int(b.distribution[0])
+    fp8 = b.kv_cache.dtype != torch.bfloat16
     kw = dict(sm_scale=b.sm_scale, max_kv_len=int(max(b.meta["kv_lens"])), max_q_len=int(q_lens[:n].max()),
-              k_scale=b.k_scale, v_scale=b.v_scale)
+              k_scale=b.k_scale, v_scale=b.v_scale, sliding_window=b.sliding_window)
     dist = b.distribution.cpu().numpy()
 
     def run(x, **extra):
@@ -333,10 +339,63 @@ def test_full_size_page_permutation_invariance(pkg, wl, gpu, name):
 
     a = run(b)
     assert torch.isfinite(a.float()).all()
+    kv = np.asarray(b.meta["kv_lens"])
+    seqs = sorted({0, int(np.argmax(kv[:dec_end])), dec_end - 1})
+    if n > dec_end:
+        seqs.append(n - 1)
+    sample = wl.sub_batch(b, seqs, last_rows=128)
+    say(f"{name}: oracle sample of sequences {seqs}, kv {sample.meta['kv_lens']}, q {sample.meta['q_lens']}")
+    assert_parity(a[torch.tensor(sample.meta["rows"], device=gpu)].cpu().float(), oracle_out(sample).float(),
+                  **(FP8_TOL if fp8 else BF16_TOL))
     c = _permute_pages(b, 5)
     assert torch.equal(a.view(torch.int16), run(c).view(torch.int16))
+    del c
     one = run(b, num_splits=1)
     torch.testing.assert_close(a.float(), one.float(), rtol=1e-2, atol=4e-3)
+    assert float(row_rel_error(a.float().cpu(), one.float().cpu()).max()) <= 1e-2
+
+
+NEEDLE_CASES = {
+    # name: (q_lens, kv_lens, Hq, Hkv, D, P, kv dtype, window)
+    "split_kv_few_long_rows": ([1] * 3, [32768, 32768, 32768], 32, 8, 128, 64, torch.bfloat16, None),
+    "one_row_60000": ([1], [60000], 32, 8, 128, 64, torch.bfloat16, None),
+    "balanced_ragged_rows": ([1] * 40, [4000 + 977 * i for i in range(40)], 32, 8, 128, 64, torch.bfloat16, None),
+    "balanced_fp8": ([1] * 40, [4100 + 1013 * i for i in range(40)], 64, 8, 128, 64, torch.float8_e4m3fn, None),
+    "window_4096_fp8": ([1] * 24, [3000 + 1501 * i for i in range(24)], 64, 8, 128, 64, torch.float8_e4m3fn, 4096),
+    "window_bf16": ([1] * 12, [5000 + 2503 * i for i in range(12)], 32, 8, 128, 16, torch.bfloat16, 3000),
+    "chunks_on_long_prefixes": ([300, 1000, 129], [8300, 5000, 20129], 32, 8, 128, 64, torch.bfloat16, None),
+    "chunks_fp8": ([257, 640], [9000, 4736], 16, 8, 128, 64, torch.float8_e4m3fn, None),
+    "chunks_window": ([700, 64], [6000, 12000], 32, 8, 128, 64, torch.bfloat16, 2048),
+    "mixed": ([1] * 20 + [500, 90], [4000 + 1300 * i for i in range(20)] + [4500, 16090], 32, 8, 128, 64, torch.bfloat16, None),
+    "wide_heads_rows": ([1] * 6, [9000, 4097, 12000, 30000, 5000, 7000], 8, 2, 256, 64, torch.bfloat16, None),
+    "wide_heads_rows_fp8": ([1] * 6, [9000, 4097, 12000, 30000, 5000, 7000], 8, 2, 256, 64, torch.float8_e4m3fn, None),
+    "wide_heads_chunks": ([200, 300], [4296, 8000], 16, 4, 256, 64, torch.bfloat16, None),
+}
+
+
+@pytest.mark.parametrize("case", list(NEEDLE_CASES))
+def test_peaked_long_rows_against_oracle(pkg, wl, gpu, case):
+    """Rows of 4000-60000 tokens whose softmax weight sits on a few planted keys (first and last
+    tiles, tile / page / piece borders, the window edge): outputs are O(1), so a lost tile, split or
+    partial row, or a wrong merge weight, shows up against the oracle.  Every plan is visited:
+    fixed split-KV, the balanced plan, fp8, windows, the flash kernel on long prefixes, 256-wide heads."""
+    q_lens, kv_lens, Hq, Hkv, D, P, dt, window = NEEDLE_CASES[case]
+    say(f"case needles {case}: q={q_lens} kv={kv_lens} Hq={Hq} Hkv={Hkv} D={D} P={P} {dt} window={window}")
+    # drawn and quantised on the GPU (the host takes minutes to cast a gigabyte to fp8)
+    b = wl.make_batch(case, q_lens, kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=D, page_size=P, seed=8100,
+                      kv_dtype=dt, sliding_window=window, device=gpu)
+    placed = wl.plant_needles(b, seed=len(case))
+    say(f"  needles of (seq 0, head 0): {placed[(0, 0)]}")
+    want = oracle_out(b.to("cpu"))
+    rms = float(want.float().pow(2).mean().sqrt())
+    assert rms > 0.1, rms  # the point of the exercise
+    tol = BF16_TOL if dt == torch.bfloat16 else FP8_TOL
+    got = gpu_out(pkg, b, gpu)
+    assert_parity(got.float(), want.float(), **tol)
+    if all(q == 1 for q in q_lens):
+        for ns in (1, 5):
+            say(f"  num_splits {ns}")
+            assert_parity(gpu_out(pkg, b, gpu, num_splits=ns).float(), want.float(), **tol)
 
 
 # ------------------------------------------------------------------ further options of the oracle
@@ -358,7 +417,7 @@ def test_attention_sink(pkg, wl, gpu, window, cap):
     say(f"case sink window={window} cap={cap}")
     want = oracle_out(b, attention_sink=sink)
     got = gpu_out(pkg, b, gpu, attention_sink=sink)
-    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    assert_parity(got.float(), want.float(), **BF16_TOL)
     # a sink far below every logit changes nothing; one far above takes all the weight
     none = gpu_out(pkg, b, gpu)
     low = gpu_out(pkg, b, gpu, attention_sink=torch.full((16,), -1.0e4))
@@ -377,7 +436,7 @@ def test_xai_temperature(pkg, wl, gpu, cap):
     for T in (64.0, 8192.0):  # rows on both sides of T / no row beyond T
         want = oracle_out(b, xai_temperature_len=T)
         got = gpu_out(pkg, b, gpu, xai_temperature_len=T)
-        torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+        assert_parity(got.float(), want.float(), **BF16_TOL)
     assert torch.equal(gpu_out(pkg, b, gpu, xai_temperature_len=8192.0), gpu_out(pkg, b, gpu))
 
 
@@ -393,12 +452,12 @@ def test_softmax_dtype_bfloat16(pkg, wl, gpu, cap, use_sink):
     say(f"case softmax_dtype cap={cap} sink={use_sink}")
     want = oracle_out(b, softmax_dtype=torch.bfloat16, **kw)
     got = gpu_out(pkg, b, gpu, softmax_dtype=torch.bfloat16, **kw)
-    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    assert_parity(got.float(), want.float(), **BF16_TOL)
     assert torch.equal(gpu_out(pkg, b, gpu, softmax_dtype=torch.float32, **kw), gpu_out(pkg, b, gpu, **kw))
     # float16 logits: finer than bf16, so closer to the float32 result than the bf16 run is
     want16 = oracle_out(b, softmax_dtype=torch.float16, **kw)
     got16 = gpu_out(pkg, b, gpu, softmax_dtype=torch.float16, **kw)
-    torch.testing.assert_close(got16.float(), want16.float(), **BF16_TOL)
+    assert_parity(got16.float(), want16.float(), **BF16_TOL)
     f32 = oracle_out(b, **kw).float()
     assert (got16.float() - f32).abs().mean() <= (got.float() - f32).abs().mean()
     with pytest.raises(NotImplementedError):
@@ -423,7 +482,7 @@ def test_q_scale_quantises_queries_to_the_cache_type(pkg, wl, gpu, kv_dtype):
     b.q, b.sm_scale = quantise_queries(b.q, q_scale, kv_dtype), sm_orig * q_scale
     want = oracle_out(b)
     b.q, b.sm_scale = q_orig, sm_orig
-    torch.testing.assert_close(got.float(), want.float(), **(FP8_TOL if kv_dtype != torch.bfloat16 else BF16_TOL))
+    assert_parity(got.float(), want.float(), **(FP8_TOL if kv_dtype != torch.bfloat16 else BF16_TOL))
     # and the kernels compute exactly what they compute on pre-quantised queries
     b.q, b.sm_scale = quantise_queries(q_orig, q_scale, kv_dtype), sm_orig * q_scale
     same = gpu_out(pkg, b, gpu)
@@ -449,7 +508,7 @@ def test_custom_mask_and_no_mask(pkg, wl, gpu, P):
     say(f"case custom mask P={P}")
     want = oracle_out(b, causal=False, custom_mask=cm)
     got = gpu_out(pkg, b, gpu, causal=0, custom_mask=cm.to(gpu))
-    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    assert_parity(got.float(), want.float(), **BF16_TOL)
     # rows padded to whole pages (mask_aligned_to_cu_kv, ragged_paged_attention_v3.py:1791-1806)
     padded = []
     for m in masks:
@@ -463,9 +522,9 @@ def test_custom_mask_and_no_mask(pkg, wl, gpu, P):
     causal = [(np.arange(kv)[None, :] <= (kv - ql) + np.arange(ql)[:, None]).astype(np.int32)
               for ql, kv in zip(q_lens, kv_lens)]
     got3 = gpu_out(pkg, b, gpu, causal=0, custom_mask=flat_mask(causal).to(gpu))
-    torch.testing.assert_close(got3.float(), oracle_out(b).float(), **BF16_TOL)
+    assert_parity(got3.float(), oracle_out(b).float(), **BF16_TOL)
     say("case no mask")
-    torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=0).float(), oracle_out(b, causal=False).float(), **BF16_TOL)
+    assert_parity(gpu_out(pkg, b, gpu, causal=0).float(), oracle_out(b, causal=False).float(), **BF16_TOL)
 
 
 def test_target_verify_metadata_feeds_the_kernel(pkg, wl, gpu):
@@ -492,7 +551,7 @@ def test_target_verify_metadata_feeds_the_kernel(pkg, wl, gpu):
     say("case target verify")
     want = oracle_out(b, causal=False, custom_mask=flat_mask(masks))
     got = gpu_out(pkg, b, gpu, causal=0, custom_mask=torch.from_numpy(md["custom_mask"]).to(gpu), mask_aligned_to_cu_kv=True)
-    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    assert_parity(got.float(), want.float(), **BF16_TOL)
 
 
 # ------------------------------------------------------------------ balanced decode plan
@@ -514,8 +573,8 @@ def test_balanced_decode_plan_on_ragged_batches(pkg, wl, gpu, Hq, Hkv, window, k
     tol = FP8_TOL if kv_dtype != torch.bfloat16 else BF16_TOL
     auto = gpu_out(pkg, b, gpu)  # large ragged batch: the balanced plan
     one = gpu_out(pkg, b, gpu, num_splits=1)  # every row in one piece, no merge pass
-    torch.testing.assert_close(auto.float(), want.float(), **tol)
-    torch.testing.assert_close(one.float(), want.float(), **tol)
+    assert_parity(auto.float(), want.float(), **tol)
+    assert_parity(one.float(), want.float(), **tol)
     torch.testing.assert_close(auto.float(), one.float(), rtol=1e-2, atol=4e-3)
     for ns in (3, 50):
         torch.testing.assert_close(gpu_out(pkg, b, gpu, num_splits=ns).float(), one.float(), rtol=1e-2, atol=4e-3)
@@ -537,7 +596,7 @@ def test_balanced_plan_long_shares_and_tiny_rows(pkg, wl, gpu, monkeypatch):
         tol = FP8_TOL if kv_dtype != torch.bfloat16 else BF16_TOL
         auto = gpu_out(pkg, b, gpu)
         one = gpu_out(pkg, b, gpu, num_splits=1)
-        torch.testing.assert_close(auto.float(), want.float(), **tol)
+        assert_parity(auto.float(), want.float(), **tol)
         torch.testing.assert_close(auto.float(), one.float(), rtol=1e-2, atol=4e-3)
         again = gpu_out(pkg, b, gpu)
         assert torch.equal(auto, again)
@@ -556,7 +615,7 @@ def test_balanced_plan_when_rows_outnumber_wave_slots(pkg, wl, gpu):
     want = oracle_out(b)
     auto = gpu_out(pkg, b, gpu)
     whole = gpu_out(pkg, b, gpu, num_splits=1)
-    torch.testing.assert_close(auto.float(), want.float(), **BF16_TOL)
+    assert_parity(auto.float(), want.float(), **BF16_TOL)
     torch.testing.assert_close(auto.float(), whole.float(), rtol=1e-2, atol=4e-3)
     assert not torch.equal(auto, whole)  # a merged row differs from a whole one in the last bits somewhere
 
@@ -582,7 +641,7 @@ def test_balanced_plan_skips_rows_without_tokens(pkg, wl, gpu):
         g.q, None, None, g.kv_cache, lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens, dist, None, sm_scale=b.sm_scale,
         max_kv_len=int(max(kv_lens)), max_q_len=1)
     torch.cuda.synchronize()
-    torch.testing.assert_close(out.cpu()[keep].float(), want[keep].float(), **BF16_TOL)
+    assert_parity(out.cpu()[keep].float(), want[keep].float(), **BF16_TOL)
 
 
 # ------------------------------------------------------------------ head_dim 256
@@ -602,7 +661,7 @@ def test_head_dim_256_decode_and_prefill(pkg, wl, gpu, Hq, Hkv, P):
     want = oracle_out(b)
     got = gpu_out(pkg, b, gpu)
     assert torch.isfinite(got.float()).all()
-    torch.testing.assert_close(got.float(), want.float(), **BF16_TOL)
+    assert_parity(got.float(), want.float(), **BF16_TOL)
 
 
 @pytest.mark.parametrize("window,cap,kv_dtype", [(40, None, torch.bfloat16), (None, 20.0, torch.bfloat16),
@@ -615,7 +674,7 @@ def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
     say(f"case d256 options window={window} cap={cap} {kv_dtype}")
     tol = BF16_TOL if kv_dtype == torch.bfloat16 else FP8_TOL
     for kw in ({}, {"attention_sink": sink}, {"xai_temperature_len": 64.0}, {"softmax_dtype": torch.bfloat16}):
-        torch.testing.assert_close(gpu_out(pkg, b, gpu, **kw).float(), oracle_out(b, **kw).float(), **tol)
+        assert_parity(gpu_out(pkg, b, gpu, **kw).float(), oracle_out(b, **kw).float(), **tol)
     # queries quantised to the cache's element type (ragged_paged_attention_v3.py:463-478)
     from oracle.ref_rpa import quantise_queries
     got = gpu_out(pkg, b, gpu, q_scale=0.37)
@@ -623,9 +682,9 @@ def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
     b.q, b.sm_scale = quantise_queries(q_orig, 0.37, kv_dtype), sm_orig * 0.37
     want = oracle_out(b)
     b.q, b.sm_scale = q_orig, sm_orig
-    torch.testing.assert_close(got.float(), want.float(), **tol)
+    assert_parity(got.float(), want.float(), **tol)
     # full attention (causal = 0 without a mask)
-    torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=False).float(), oracle_out(b, causal=False).float(), **tol)
+    assert_parity(gpu_out(pkg, b, gpu, causal=False).float(), oracle_out(b, causal=False).float(), **tol)
     # custom masks: every row goes through the flash kernel (bf16 caches) or the row kernel (fp8)
     rng = np.random.default_rng(11)
     masks = []
@@ -634,12 +693,12 @@ def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
         mk[:, 0] = 1
         masks.append(mk)
     cm = flat_mask(masks)
-    torch.testing.assert_close(gpu_out(pkg, b, gpu, causal=False, custom_mask=cm.to(gpu)).float(),
+    assert_parity(gpu_out(pkg, b, gpu, causal=False, custom_mask=cm.to(gpu)).float(),
                                oracle_out(b, causal=False, custom_mask=cm).float(), **tol)
     # the same masks in rows padded to whole pages
     P = 32
     padded = [np.pad(mk, ((0, 0), (0, -(-mk.shape[1] // P) * P - mk.shape[1]))) for mk in masks]
-    torch.testing.assert_close(
+    assert_parity(
         gpu_out(pkg, b, gpu, causal=False, custom_mask=flat_mask(padded).to(gpu), mask_aligned_to_cu_kv=True).float(),
         oracle_out(b, causal=False, custom_mask=cm).float(), **tol)
 
@@ -657,12 +716,12 @@ def test_head_dim_256_long_decode_rows_are_split(pkg, wl, gpu, kv_dtype, window)
     want = oracle_out(b)
     auto = gpu_out(pkg, b, gpu)
     whole = gpu_out(pkg, b, gpu, num_splits=1)
-    torch.testing.assert_close(auto.float(), want.float(), **tol)
+    assert_parity(auto.float(), want.float(), **tol)
     torch.testing.assert_close(auto.float(), whole.float(), rtol=1e-2, atol=4e-3)
     assert not torch.equal(auto, whole)  # merged rows differ from whole ones in the last bits somewhere
     torch.testing.assert_close(gpu_out(pkg, b, gpu, num_splits=7).float(), whole.float(), rtol=1e-2, atol=4e-3)
     sink = torch.from_numpy(np.random.RandomState(101).randn(8).astype(np.float32))
-    torch.testing.assert_close(gpu_out(pkg, b, gpu, attention_sink=sink).float(),
+    assert_parity(gpu_out(pkg, b, gpu, attention_sink=sink).float(),
                                oracle_out(b, attention_sink=sink).float(), **tol)
 
 
@@ -691,7 +750,7 @@ def test_head_dim_256_cache_write_and_gather(pkg, wl, gpu):
         o += -(-kv // 16)
     assert torch.equal(cache.cpu(), want_cache)
     b.kv_cache = want_cache
-    torch.testing.assert_close(out[:T].cpu().float(), oracle_out(b).float(), **BF16_TOL)
+    assert_parity(out[:T].cpu().float(), oracle_out(b).float(), **BF16_TOL)
 
 
 # ------------------------------------------------------------------ a captured step
@@ -770,11 +829,11 @@ def test_a_captured_step_replays_with_new_lengths_and_page_tables(pkg, wl, gpu):
         call.out.zero_()
         graph.replay()
         torch.cuda.synchronize()
-        torch.testing.assert_close(call.out[:T].cpu().float(), oracle_out(b).float(), **BF16_TOL)
+        assert_parity(call.out[:T].cpu().float(), oracle_out(b).float(), **BF16_TOL)
         assert torch.equal(st["cache"][: b.kv_cache.shape[0]].cpu(), b.kv_cache)  # the new rows are back in place
         # eager work between the replays
         other = batches[1 - which]
-        torch.testing.assert_close(gpu_out(pkg, other, gpu).float(), oracle_out(other).float(), **BF16_TOL)
+        assert_parity(gpu_out(pkg, other, gpu).float(), oracle_out(other).float(), **BF16_TOL)
 
 
 # ------------------------------------------------------------------ random shapes
@@ -807,7 +866,7 @@ def test_random_batches_against_oracle(pkg, wl, gpu, seed):
     want = oracle_out(b, **kw)
     got = gpu_out(pkg, b, gpu, **kw)
     assert torch.isfinite(got.float()).all()
-    torch.testing.assert_close(got.float(), want.float(), **(FP8_TOL if fp8 else BF16_TOL))
+    assert_parity(got.float(), want.float(), **(FP8_TOL if fp8 else BF16_TOL))
 
 
 @pytest.mark.parametrize("seed", list(range(10)))
@@ -838,7 +897,9 @@ def test_random_large_batches_against_oracle(pkg, wl, gpu, seed):
     b = wl.make_batch("rand_large", q_lens, kv_lens, num_q_heads=Hkv * G, num_kv_heads=Hkv, head_dim=D, page_size=P,
                       seed=3000 + seed, kv_dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16,
                       sliding_window=window, soft_cap=cap)
+    if seed % 2:
+        wl.plant_needles(b, seed=seed)  # peaked rows: O(1) outputs whatever the length
     want = oracle_out(b, **kw)
     got = gpu_out(pkg, b, gpu, **kw)
     assert torch.isfinite(got.float()).all()
-    torch.testing.assert_close(got.float(), want.float(), **(FP8_TOL if fp8 else BF16_TOL))
+    assert_parity(got.float(), want.float(), **(FP8_TOL if fp8 else BF16_TOL))
