@@ -12,17 +12,28 @@
 //     vector pipe   P(i)   = 2^(S(i) c - m c)      exponentials, packing, row sum, row maximum
 // so every vector instruction of the softmax has matrix instructions of the same wave to run
 // under, instead of relying on another wave being in the other phase.  Step t of a workgroup is
-// the pair of iterations (2t-1, 2t): it reads K tile t and V tile t-1, so the two-slot rings of
-// the unpipelined kernel suffice (V lags K by one tile) and there is still one barrier per tile.
+// the pair of iterations (2t-1, 2t): it reads K tile t and V tile t-1, so two ring slots per
+// matrix suffice (V lags K by one tile) and there is still one barrier per tile.
+//
+// The compiler does not keep such an interleave (it regroups the matrix instructions and spills),
+// and it will not keep two hundred registers in place around an assembly block that is only a loop
+// body, so the whole run of steady-state steps of a wave is one assembly block with fixed
+// registers, written by gen_prefill_pipe_loop.py into rpa_prefill_pipe_loop.inc; this file binds
+// the kernel's variables to those registers.  Steps that touch the causal diagonal or a window edge, the first and the
+// last steps run the same pipeline through a general iteration in C++ with masking and run-time
+// flags.
 //
 // The running maximum is checked after the fact: the exponentials of half i use the maximum known
 // before it; the half's own maximum is taken by the vector pipe next to them, and only if it
 // exceeds the stale one by more than 2^kMaxSlack is the half redone (its scores are still in
-// registers) and the accumulators rescaled.  Halves that touch the causal diagonal or a window
-// edge, the first and the last steps run the same pipeline through a general iteration with
-// masking and run-time flags.
+// registers) and the accumulators rescaled.
+//
+// The global -> LDS copies are issued as assembly too, so the compiler knows of no store into the
+// LDS ring and never waits for the copy queue on its own; the kernel waits (vmcnt(0)) in front of
+// the barrier that ends a step.
 
 #include "rpa_prefill_common.h"
+#include "rpa_prefill_pipe_loop.inc"
 
 namespace rpa {
 
@@ -33,38 +44,72 @@ namespace {
 constexpr int kRowB = 256;               // bytes of one K or V row of a head
 constexpr int kTileB = kBN * kRowB;      // 16 KiB
 constexpr int kHalfB = 32 * kRowB;       // byte distance between the halves of a tile
+constexpr int kKSlot = 0;                // ring slots inside the LDS array: K0 K1 V0 V1
+constexpr int kVSlot = 2 * kTileB;
 
-struct PipeState {
-  f32x16_t O[4];
-  float m, l;
-  float sc2;
+typedef uint32_t u32x16_t __attribute__((ext_vector_type(16)));
+typedef int32_t i32x8_t __attribute__((ext_vector_type(8)));
+typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x4v_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ u32x4_t lds_ld16_at(int addr) {
+  typedef const __attribute__((address_space(3))) u32x4_t* p_t;
+  return *(p_t)(uint32_t)addr;
+}
+__device__ __forceinline__ u32x2_t lds_tr16_at(int addr) {
+  typedef __attribute__((address_space(3))) s16x4v_t* p_t;
+  return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((p_t)(uint32_t)addr));
+}
+
+template <int KS>
+__device__ __forceinline__ u32x4_t q_frag(const u32x16_t& a, const u32x16_t& b) {
+  const u32x16_t& s = KS < 4 ? a : b;
+  constexpr int o = (KS & 3) * 4;
+  return u32x4_t{s[o], s[o + 1], s[o + 2], s[o + 3]};
+}
+
+// The registers of one wave's pipeline.  The assembly loop expects them in the registers the
+// RPA_PIPE_C_* constraints of rpa_prefill_pipe_loop.inc name.
+struct Pipe {
+  f32x16_t O[4];      // accumulators, lane (c, h): row c, dims 32d + 8*(v/4) + 4h + v%4
+  f32x16_t S0, S1;    // scores of the even / odd half in flight
+  u32x4_t P0[2], P1[2];  // probabilities of the even / odd half (B operands of the second product)
+  u32x16_t Qa, Qb;    // Q^T operands of the 8 k-steps
+  i32x8_t koff;       // LDS addresses of the K operand reads (slot 0, first half)
+  i32x4_t voff;       // LDS addresses of the V^T operand reads (slot 0, first half, first k-step)
+  float m, l;         // running maximum (raw score units), running sum
+  u32x4_t ofs_k, ofs_v;  // per-lane byte offsets of this wave's four K / V copy instructions
+  float sc2;          // raw score -> log2 units
 };
 
-// one matrix copy (K or V rows of a tile) global -> LDS: 4 instructions per wave
+// K or V rows of one tile, global -> LDS: 4 instructions per wave.  `lds_wave` is the LDS address
+// of this wave's first 1 KiB block of the slot.
 template <bool IS_V>
-__device__ __forceinline__ void copy_rows(char* lds, const TileSrc& s, const KvAddr& kv, const char* head, int tb,
+__device__ __forceinline__ void copy_rows(uint32_t lds_wave, const TileSrc& s, const KvAddr& kv, const char* head, int tb,
                                           int wave, int lane, int page, const AsyncOffsets<128>& ofs) {
-  typedef const __attribute__((address_space(1))) void* gptr_t;
-  typedef __attribute__((address_space(3))) void* lptr_t;
   tb = min(tb, s.last_tok & ~(kBN - 1));
   if (tb + kBN - 1 <= s.last_tok) {
     const int64_t base = (int64_t)page * kv.page_stride + (int64_t)(tb - page_slot(s, tb) * s.page_size) * kv.tok_stride;
-    const char* b = head + base;
+    const char* b = head + base;  // wave-uniform
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
-      const int blk = wave * 4 + n;
-      __builtin_amdgcn_global_load_lds((gptr_t)(b + (IS_V ? ofs.v[n] : ofs.k[n])), (lptr_t)(lds + blk * 1024), 16, 0, 0);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :: "s"(lds_wave + n * 1024), "v"(IS_V ? ofs.v[n] : ofs.k[n]), "s"(b)
+                   : "memory", "m0");
     }
     return;
   }
+  // last, partial tile: rows clamped to the last valid token
   const int cp = lane & 15;
 #pragma unroll
   for (int n = 0; n < 4; ++n) {
-    const int blk = wave * 4 + n;
-    const int t = blk * 4 + (lane >> 4);
+    const int t = (wave * 4 + n) * 4 + (lane >> 4);
     const int64_t ro = row_offset<true>(s, kv, tb, tb + t, page);
     const int j = IS_V ? (cp ^ ((t & 3) << 2)) : (cp ^ (t & 15));
-    __builtin_amdgcn_global_load_lds((gptr_t)(head + ro + j * 16), (lptr_t)(lds + blk * 1024), 16, 0, 0);
+    const char* g = head + ro + j * 16;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :: "s"(lds_wave + n * 1024), "v"(g)
+                 : "memory", "m0");
   }
 }
 
@@ -73,25 +118,29 @@ __device__ __forceinline__ int scalar_page(const TileSrc& s, int tb) {
   return scalar_load_i32(s.pages + __builtin_amdgcn_readfirstlane(page_slot(s, tb)));
 }
 
-// first product of one 32-token half: one chain of 8 MFMAs
-__device__ __forceinline__ f32x16_t qk_half(const char* lds_k_half, const int (&koff)[8], const u32x4_t (&qB)[8]) {
-  f32x16_t S = mfma32(lds_ld16(lds_k_half + koff[0]), qB[0], kZero16);
-#pragma unroll
-  for (int ks = 1; ks < 8; ++ks) S = mfma32(lds_ld16(lds_k_half + koff[ks]), qB[ks], S);
+// first product of one 32-token half: one chain of 8 MFMAs; `off` = slot and half offset
+__device__ __forceinline__ f32x16_t qk_half(const Pipe& p, int off) {
+  f32x16_t S = mfma32(lds_ld16_at(p.koff[0] + off), q_frag<0>(p.Qa, p.Qb), kZero16);
+  S = mfma32(lds_ld16_at(p.koff[1] + off), q_frag<1>(p.Qa, p.Qb), S);
+  S = mfma32(lds_ld16_at(p.koff[2] + off), q_frag<2>(p.Qa, p.Qb), S);
+  S = mfma32(lds_ld16_at(p.koff[3] + off), q_frag<3>(p.Qa, p.Qb), S);
+  S = mfma32(lds_ld16_at(p.koff[4] + off), q_frag<4>(p.Qa, p.Qb), S);
+  S = mfma32(lds_ld16_at(p.koff[5] + off), q_frag<5>(p.Qa, p.Qb), S);
+  S = mfma32(lds_ld16_at(p.koff[6] + off), q_frag<6>(p.Qa, p.Qb), S);
+  S = mfma32(lds_ld16_at(p.koff[7] + off), q_frag<7>(p.Qa, p.Qb), S);
   return S;
 }
 
 // second product of one 32-token half: four chains of 2 MFMAs
-__device__ __forceinline__ void pv_half(f32x16_t (&O)[4], const char* lds_v_half, const int (&voff)[4],
-                                        const u32x4_t (&P)[2]) {
+__device__ __forceinline__ void pv_half(Pipe& p, int off, const u32x4_t (&P)[2]) {
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      const char* vt = lds_v_half + voff[d] + kk * 16 * kRowB;
-      const u32x2_t lo = lds_tr16(vt);
-      const u32x2_t hi = lds_tr16(vt + 8 * kRowB);
-      O[d] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, P[kk], O[d]);
+      const int vt = p.voff[d] + off + kk * 16 * kRowB;
+      const u32x2_t lo = lds_tr16_at(vt);
+      const u32x2_t hi = lds_tr16_at(vt + 8 * kRowB);
+      p.O[d] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, P[kk], p.O[d]);
     }
 }
 
@@ -123,20 +172,8 @@ __device__ __forceinline__ float row_max16(const f32x16_t& S) {
   return swap_max(mx);
 }
 
-// raise the running maximum to cover mx and rescale what has been accumulated
-__device__ __forceinline__ void raise_max(PipeState& st, float mx) {
-  const float m_new = fmaxf(st.m, mx);
-  const float alpha = fast_exp2((st.m - m_new) * st.sc2);
-  st.m = m_new;
-  st.l *= alpha;
-#pragma unroll
-  for (int d = 0; d < 4; ++d)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) st.O[d][v] *= alpha;
-}
-
 // softmax of a half with the maximum taken first (first half of a row, masked halves)
-__device__ __forceinline__ void softmax_half_general(f32x16_t& S, PipeState& st, bool need_mask, int tb, int h, int qpos,
+__device__ __forceinline__ void softmax_half_general(f32x16_t& S, Pipe& p, bool need_mask, int tb, int h, int qpos,
                                                      int window, u32x4_t (&P)[2]) {
   if (need_mask) {
 #pragma unroll
@@ -147,16 +184,46 @@ __device__ __forceinline__ void softmax_half_general(f32x16_t& S, PipeState& st,
     }
   }
   const float mx = row_max16(S);
-  if (__builtin_amdgcn_ballot_w64((mx - st.m) * st.sc2 > kMaxSlack) != 0) raise_max(st, mx);
-  st.l += exp_pack(S, st.sc2, -st.m * st.sc2, P);
+  if (__builtin_amdgcn_ballot_w64((mx - p.m) * p.sc2 > kMaxSlack) != 0) {
+    const float m_new = fmaxf(p.m, mx);
+    const float alpha = fast_exp2((p.m - m_new) * p.sc2);
+    p.m = m_new;
+    p.l *= alpha;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) p.O[d][v] *= alpha;
+  }
+  p.l += exp_pack(S, p.sc2, -p.m * p.sc2, P);
 }
+
+// Steady-state steps [t, t_end) in assembly.  On entry K tile t is in K slot t & 1 and V tile t - 1
+// in V slot 1 - (t & 1), pg_a / pg_b are the pages of tiles t and t + 1; on exit the same holds for
+// t = t_end.  Every tile the loop copies (up to t_end) lies completely inside the sequence.
+struct LoopScalars {
+  int t_end, t_lo, pmask, pshift, tok_stride, last_tile_tok;
+  uint32_t pstr, kh_lo, kh_hi, vh_lo, vh_hi, lds_wave;
+  const int32_t* pages;
+};
+
+#define RPA_PIPE_LOOP(p, t, pg_a, pg_b, sc)                                                                       \
+  asm volatile(RPA_PIPE_LOOP_ASM                                                                                  \
+               : "+" RPA_PIPE_C_O0(p.O[0]), "+" RPA_PIPE_C_O1(p.O[1]), "+" RPA_PIPE_C_O2(p.O[2]),                 \
+                 "+" RPA_PIPE_C_O3(p.O[3]), "+" RPA_PIPE_C_S0(p.S0), "+" RPA_PIPE_C_S1(p.S1),                     \
+                 "+" RPA_PIPE_C_P00(p.P0[0]), "+" RPA_PIPE_C_P01(p.P0[1]), "+" RPA_PIPE_C_P10(p.P1[0]),           \
+                 "+" RPA_PIPE_C_P11(p.P1[1]), "+" RPA_PIPE_C_M(p.m), "+" RPA_PIPE_C_L(p.l),                       \
+                 [t] "+s"(t), [pg_a] "+s"(pg_a), [pg_b] "+s"(pg_b)                                                \
+               : RPA_PIPE_C_QA(p.Qa), RPA_PIPE_C_QB(p.Qb), RPA_PIPE_C_KOFF(p.koff), RPA_PIPE_C_VOFF(p.voff),      \
+                 RPA_PIPE_C_OFSK(p.ofs_k), RPA_PIPE_C_OFSV(p.ofs_v), [sc2] "s"(p.sc2), [nsc2] "s"(-p.sc2),        \
+                 [ones] "s"(0x3f803f80u), [t_end] "s"(sc.t_end), [t_lo] "s"(sc.t_lo), [pmask] "s"(sc.pmask),      \
+                 [pshift] "s"(sc.pshift), [tok_stride] "s"(sc.tok_stride), [last_tile_tok] "s"(sc.last_tile_tok), \
+                 [pstr] "s"(sc.pstr), [kh_lo] "s"(sc.kh_lo), [kh_hi] "s"(sc.kh_hi), [vh_lo] "s"(sc.vh_lo),        \
+                 [vh_hi] "s"(sc.vh_hi), [lds_wave] "s"(sc.lds_wave), [pages] "s"(sc.pages)                        \
+               : RPA_PIPE_LOOP_CLOBBERS)
 
 template <bool WIN>
 __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillArgs a, int tiles, int nseq, bool by_level) {
-  __shared__ __attribute__((aligned(1024))) char lds_k0[kTileB];
-  __shared__ __attribute__((aligned(1024))) char lds_k1[kTileB];
-  __shared__ __attribute__((aligned(1024))) char lds_v0[kTileB];
-  __shared__ __attribute__((aligned(1024))) char lds_v1[kTileB];
+  __shared__ __attribute__((aligned(1024))) char lds[4 * kTileB];
 
   const Work w = decompose(a, tiles, nseq, by_level);
   if (!w.valid) return;
@@ -167,6 +234,8 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillA
   const TileSrc src = make_src(a, w);
   const char* kh = a.kv.k_base + (int64_t)w.hk * a.kv.head_stride;
   const char* vh = a.kv.v_base + (int64_t)w.hk * a.kv.head_stride;
+  typedef __attribute__((address_space(3))) char* lds_ptr_t;
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)lds);
 
   WaveRows wr;
   wr.r_lo = w.q_start + wave * 32;
@@ -176,21 +245,28 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillA
   wr.qpos = w.prefix + wr.row;
   const int W_ = WIN ? a.sm.window : 0;
 
-  u32x4_t qB[8];
+  Pipe p;
   {
     const int rr = min(wr.row, w.q_len - 1);
     const uint16_t* qp = a.q + ((int64_t)(w.qg0 + rr) * a.Hq + w.head) * 128 + h * 8;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qB[ks] = ld16(qp + ks * 16);
+    for (int ks = 0; ks < 4; ++ks) {
+      const u32x4_t x = ld16(qp + ks * 16), y = ld16(qp + (ks + 4) * 16);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        p.Qa[4 * ks + e] = x[e];
+        p.Qb[4 * ks + e] = y[e];
+      }
+    }
   }
-  PipeState st;
-  st.sc2 = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f) * kLog2e;
+  p.sc2 = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f) * kLog2e;
 #pragma unroll
-  for (int d = 0; d < 4; ++d)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) st.O[d][v] = 0.f;
-  st.m = kMaxFloor;
-  st.l = 0.f;
+  for (int d = 0; d < 4; ++d) p.O[d] = kZero16;
+  p.S0 = kZero16;
+  p.S1 = kZero16;
+  p.P0[0] = p.P0[1] = p.P1[0] = p.P1[1] = u32x4_t{0, 0, 0, 0};
+  p.m = kMaxFloor;
+  p.l = 0.f;
 
   const int wg_r_hi = min(w.q_start + kBM, w.q_len) - 1;
   const int t_hi = min(w.kv_len, w.prefix + wg_r_hi + 1);  // exclusive
@@ -209,142 +285,102 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillA
     }
     i_f1 = min(i_f1, n_w);
   }
+  n_w = __builtin_amdgcn_readfirstlane(n_w);
+  i_f0 = __builtin_amdgcn_readfirstlane(i_f0);
+  i_f1 = __builtin_amdgcn_readfirstlane(i_f1);
 
-  // operand offsets inside a tile (see rpa_prefill_async_kernel)
-  const int k_row = c * kRowB;
-  const int k_swz = (h ^ (c & 15)) << 4;
-  const int r16 = lane & 15, b16 = lane >> 4;
-  const int v_row = (4 * h + (r16 >> 2)) * kRowB;
-  const int v_in = ((b16 & 1) << 5) + (((r16 & 3) >> 1) << 4) + ((r16 & 1) << 3);
-  const int v_swz = (r16 >> 2) << 6;
-  int koff[8], voff[4];
+  // operand addresses inside the LDS array (see rpa_prefill_async_kernel for the swizzles)
+  {
+    const int k_row = c * kRowB;
+    const int k_swz = (h ^ (c & 15)) << 4;
+    const int r16 = lane & 15, b16 = lane >> 4;
+    const int v_row = (4 * h + (r16 >> 2)) * kRowB;
+    const int v_in = ((b16 & 1) << 5) + (((r16 & 3) >> 1) << 4) + ((r16 & 1) << 3);
+    const int v_swz = (r16 >> 2) << 6;
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) {
-    koff[ks] = k_row + ((ks * 32) ^ k_swz);
-    asm volatile("" : "+v"(koff[ks]));
-  }
+    for (int ks = 0; ks < 8; ++ks) p.koff[ks] = (int)lds_base + kKSlot + k_row + ((ks * 32) ^ k_swz);
 #pragma unroll
-  for (int d = 0; d < 4; ++d) {
-    voff[d] = v_row + v_in + ((d * 64) ^ v_swz);
-    asm volatile("" : "+v"(voff[d]));
+    for (int d = 0; d < 4; ++d) p.voff[d] = (int)lds_base + kVSlot + v_row + v_in + ((d * 64) ^ v_swz);
   }
 
   const AsyncOffsets<128> ofs = make_async_offsets<128>(a.kv, wave, lane);
+#pragma unroll
+  for (int n = 0; n < 4; ++n) {
+    p.ofs_k[n] = ofs.k[n];
+    p.ofs_v[n] = ofs.v[n];
+  }
+  const uint32_t lds_wave = lds_base + wave * 4096;  // this wave's four 1 KiB blocks of slot K0
   int pg_a = scalar_page(src, t_lo);         // page of tile t
-  copy_rows<false>(lds_k0, src, a.kv, kh, t_lo, wave, lane, pg_a, ofs);
+  copy_rows<false>(lds_wave + kKSlot, src, a.kv, kh, t_lo, wave, lane, pg_a, ofs);
   int pg_b = scalar_page(src, t_lo + kBN);   // page of tile t + 1
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
 
-  // pipeline registers: scores of half i in S[i & 1], its probabilities in P[i & 1]
-  f32x16_t S0 = kZero16, S1 = kZero16;
-  u32x4_t P0[2] = {}, P1[2] = {};
-
   // iteration i of the general kind: Sn <- scores of half i + 1, Pc <- softmax of Sc (half i), O += P(i - 1) V
-  auto general_iter = [&](int i, f32x16_t& Sc, f32x16_t& Sn, u32x4_t (&Pc)[2], const u32x4_t (&Pp)[2],
-                          const char* lds_k_half, const char* lds_v_half) __attribute__((always_inline)) {
-    if (i + 1 < n_w) Sn = qk_half(lds_k_half, koff, qB);
-    if (i >= 1 && i - 1 < n_w) pv_half(st.O, lds_v_half, voff, Pp);
+  auto general_iter = [&](int i, f32x16_t& Sc, f32x16_t& Sn, u32x4_t (&Pc)[2], const u32x4_t (&Pp)[2], int k_off,
+                          int v_off) __attribute__((always_inline)) {
+    if (i + 1 < n_w) Sn = qk_half(p, k_off);
+    if (i >= 1 && i - 1 < n_w) pv_half(p, v_off, Pp);
     if (i >= 0 && i < n_w) {
       const bool need_mask = i < i_f0 || i >= i_f1;
-      softmax_half_general(Sc, st, need_mask, t_lo + 32 * i, h, wr.qpos, W_, Pc);
+      softmax_half_general(Sc, p, need_mask, t_lo + 32 * i, h, wr.qpos, W_, Pc);
     }
   };
 
-  // iteration i of the fast kind: no mask, every part present, maximum checked afterwards.  The
-  // source order is the intended issue order (one matrix instruction, then the vector work of one
-  // score pair); the group barriers at the end pin it.
-  auto fast_iter = [&](f32x16_t& Sc, f32x16_t& Sn, u32x4_t (&Pc)[2], const u32x4_t (&Pp)[2], const char* lds_k_half,
-                       const char* lds_v_half) __attribute__((always_inline)) {
-    const float neg_m = -st.m * st.sc2;
-    const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
-    float ps0 = 0.f, ps1 = 0.f;
-    float mx = Sc[0];
-    uint32_t w[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      // first product, k-step k
-      Sn = mfma32(lds_ld16(lds_k_half + koff[k]), qB[k], k == 0 ? kZero16 : Sn);
-      // second product: k-step k / 4 of dim tile k % 4
-      {
-        const char* vt = lds_v_half + voff[k & 3] + (k >> 2) * 16 * kRowB;
-        const u32x2_t lo = lds_tr16(vt);
-        const u32x2_t hi = lds_tr16(vt + 8 * kRowB);
-        st.O[k & 3] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, Pp[k >> 2], st.O[k & 3]);
-      }
-      // softmax of score pair k
-      const float p0 = fast_exp2(__builtin_fmaf(Sc[2 * k], st.sc2, neg_m));
-      const float p1 = fast_exp2(__builtin_fmaf(Sc[2 * k + 1], st.sc2, neg_m));
-      w[k] = pack_bf16x2(p0, p1);
-      if (k & 1) ps1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[k]), ones, ps1, false);
-      else ps0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[k]), ones, ps0, false);
-      mx = k == 0 ? __builtin_fmaxf(mx, Sc[1]) : __builtin_fmaxf(__builtin_fmaxf(mx, Sc[2 * k]), Sc[2 * k + 1]);
-    }
-    Pc[0] = u32x4_t{w[0], w[1], w[2], w[3]};
-    Pc[1] = u32x4_t{w[4], w[5], w[6], w[7]};
-    mx = swap_max(mx);
-    float ps = ps0 + ps1;
-    // the probabilities are final here in all but rare cases: keep them from being sunk behind the branch
-    asm volatile("" : "+v"(Pc[0]), "+v"(Pc[1]), "+v"(ps));
-    const bool raise = __builtin_amdgcn_ballot_w64((mx - st.m) * st.sc2 > kMaxSlack) != 0;
-#define RPA_PIPE_GROUP(LDS_A, LDS_B)                                                        \
-  __builtin_amdgcn_sched_group_barrier(0x100, LDS_A, 0); /* LDS reads run ahead */          \
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     /* MFMA of the first product */    \
-  __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                                        \
-  __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);                                        \
-  __builtin_amdgcn_sched_group_barrier(0x100, LDS_B, 0);                                    \
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     /* MFMA of the second product */   \
-  __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);                                        \
-  __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
-    RPA_PIPE_GROUP(6, 3)
-    RPA_PIPE_GROUP(3, 3)
-    RPA_PIPE_GROUP(3, 3)
-    RPA_PIPE_GROUP(3, 0)
-    RPA_PIPE_GROUP(0, 0)
-    RPA_PIPE_GROUP(0, 0)
-    RPA_PIPE_GROUP(0, 0)
-    RPA_PIPE_GROUP(0, 0)
-#undef RPA_PIPE_GROUP
-    if (raise) {
-      asm volatile("" ::: "memory");  // keep the rescale out of the common path
-      raise_max(st, mx);
-      st.l += exp_pack(Sc, st.sc2, -st.m * st.sc2, Pc);
-    } else {
-      st.l += ps;
-    }
-  };
-
-  // step t: iterations 2t - 1 and 2t; reads K tile t from (ck) and V tile t - 1 from (cv), fills the
-  // other K slot with tile t + 1 and the other V slot with tile t
-  auto step = [&](int t, const char* ck, const char* cv, char* fk, char* fv) __attribute__((always_inline)) {
-    if (t + 1 < nT) copy_rows<false>(fk, src, a.kv, kh, t_lo + (t + 1) * kBN, wave, lane, pg_b, ofs);
-    if (t < nT) copy_rows<true>(fv, src, a.kv, vh, t_lo + t * kBN, wave, lane, pg_a, ofs);
+  // step t: iterations 2t - 1 and 2t; with par = t & 1 it reads K tile t from K slot par and V tile
+  // t - 1 from V slot 1 - par, fills K slot 1 - par with tile t + 1 and V slot par with tile t
+  auto copies = [&](int t, int par) __attribute__((always_inline)) {
+    if (t + 1 < nT)
+      copy_rows<false>(lds_wave + kKSlot + (1 - par) * kTileB, src, a.kv, kh, t_lo + (t + 1) * kBN, wave, lane, pg_b, ofs);
+    if (t < nT) copy_rows<true>(lds_wave + kVSlot + par * kTileB, src, a.kv, vh, t_lo + t * kBN, wave, lane, pg_a, ofs);
     pg_a = pg_b;
     if (t + 2 < nT) pg_b = scalar_page(src, t_lo + (t + 2) * kBN);
-    const int i = 2 * t - 1;
-    if (i >= max(i_f0, 1) && i + 1 < i_f1) {
-      fast_iter(S1, S0, P1, P0, ck, cv);
-      fast_iter(S0, S1, P0, P1, ck + kHalfB, cv + kHalfB);
-    } else {
-      general_iter(i, S1, S0, P1, P0, ck, cv);
-      general_iter(i + 1, S0, S1, P0, P1, ck + kHalfB, cv + kHalfB);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
   };
-
-  for (int t = 0; t <= nT; t += 2) {
-    step(t, lds_k0, lds_v1, lds_k1, lds_v0);
-    if (t + 1 > nT) break;
-    step(t + 1, lds_k1, lds_v0, lds_k0, lds_v1);
+  // Steps [t_fb, t_fe) of this wave are steady-state steps (no mask, every part present, the tiles
+  // they copy lie completely inside the sequence); they run inside one assembly block.  All waves of
+  // the workgroup run nT + 1 steps with one barrier each, whichever kind each wave's step is.
+  const int t_fb = (max(i_f0, 1) + 2) >> 1;  // first t with 2t - 1 >= max(i_f0, 1)
+  const int n_full = (w.kv_len - t_lo) >> 6;  // tiles completely inside the sequence
+  const int t_fe = __builtin_amdgcn_readfirstlane(min((i_f1 + 1) >> 1, n_full - 1));  // 2t < i_f1, tile t + 1 is whole
+  LoopScalars sc;
+  sc.t_end = t_fe;
+  sc.t_lo = __builtin_amdgcn_readfirstlane(t_lo);
+  sc.pmask = src.page_size - 1;
+  sc.pshift = src.page_shift;
+  sc.tok_stride = a.kv.tok_stride;
+  sc.last_tile_tok = __builtin_amdgcn_readfirstlane(src.last_tok & ~(kBN - 1));
+  sc.pstr = (uint32_t)a.kv.page_stride;
+  sc.kh_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)kh);
+  sc.kh_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)kh >> 32));
+  sc.vh_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)vh);
+  sc.vh_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)vh >> 32));
+  sc.lds_wave = lds_wave;
+  sc.pages = src.pages;
+  int t = 0;
+  while (t <= nT) {
+    if (t >= t_fb && t < t_fe) {
+      RPA_PIPE_LOOP(p, t, pg_a, pg_b, sc);  // leaves t == t_fe
+    } else {
+      const int par = t & 1;
+      copies(t, par);
+      const int i = 2 * t - 1;
+      const int k_off = par * kTileB, v_off = (1 - par) * kTileB;
+      general_iter(i, p.S1, p.S0, p.P1, p.P0, k_off, v_off);
+      general_iter(i + 1, p.S0, p.S1, p.P0, p.P1, k_off + kHalfB, v_off + kHalfB);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+      ++t;
+    }
   }
-  write_rows<4>(a, w, wr, st.O, st.l, h, st.m * st.sc2);
+  write_rows<4>(a, w, wr, p.O, p.l, h, p.m * p.sc2);
 }
 
 }  // namespace
 
 bool prefill_pipe_applies(const PrefillArgs& a) {
-  return !a.fp8 && a.head_dim == 128 && (a.pt.page_size % kBN) == 0 && a.sm.mask_mode == 0 && a.sm.soft_cap == 0.f &&
+  const int P = a.pt.page_size;
+  return !a.fp8 && a.head_dim == 128 && P >= kBN && (P & (P - 1)) == 0 && a.kv.page_stride < (int64_t(1) << 32) &&
+         a.sm.mask_mode == 0 && a.sm.soft_cap == 0.f &&
          a.sm.round_logits == 0 && !(a.sm.xai_len > 0.f) && !(a.sm.q_scale > 0.f);
 }
 
