@@ -443,8 +443,8 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const bool cap = a.sm.soft_cap != 0.f || a.sm.round_logits != 0;
   static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
   const bool staged = a.fp8 || force_staged;
-  static const bool use_pipe = [] { const char* v = getenv("RPA_PREFILL_PIPE"); return v && *v == '1'; }();
-  if (use_pipe && !force_staged && prefill_pipe_applies(a)) return launch_prefill_pipe(a, tiles, nseq, by_level, (unsigned)grid, stream);
+  static const bool use_pipe = [] { const char* v = getenv("RPA_PREFILL_PIPE"); return !(v && *v == '0'); }();
+  if (use_pipe && !force_staged && prefill_pipe_applies(a)) return launch_prefill_pipe(a, nseq, level_order, stream);
   const dim3 g((unsigned)grid), blk(256);
   const bool ext = a.sm.xai_len > 0.f || a.sm.mask_mode != 0 || a.sm.q_scale > 0.f;
 #define RPA_STAGED(F, U, C, E) \

@@ -71,7 +71,7 @@ struct Work {
   bool valid;
 };
 
-__device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int nseq, bool by_level) {
+__device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int nseq, bool by_level, int bm = kBM) {
   Work w;
   w.valid = false;
   const int units = nseq * a.Hkv;
@@ -101,8 +101,8 @@ __device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int n
   w.kv_len = a.pt.kv_lens[w.seq];
   w.prefix = w.kv_len - w.q_len;
   int tile = tiles - 1 - tile_rev;
-  if (by_level) tile -= (max(w.prefix, 0) + kBM - 1) / kBM;
-  w.q_start = tile * kBM;
+  if (by_level) tile -= (max(w.prefix, 0) + bm - 1) / bm;
+  w.q_start = tile * bm;
   if (tile < 0 || w.q_start >= w.q_len) return w;
   w.valid = true;
   return w;
@@ -369,7 +369,6 @@ __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const 
 
 // rpa_prefill_pipe.hip: the software-pipelined kernel for the plain causal bf16 case
 bool prefill_pipe_applies(const PrefillArgs& a);
-hipError_t launch_prefill_pipe(const PrefillArgs& a, int tiles, int nseq, bool by_level, unsigned grid,
-                               hipStream_t stream);
+hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order, hipStream_t stream);
 
 }  // namespace rpa

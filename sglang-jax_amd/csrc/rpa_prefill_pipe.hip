@@ -1,36 +1,41 @@
 // Software-pipelined flash kernel for the common prefill case on gfx950: bf16 cache, 128-wide
-// heads, pages that hold whole 64-token tiles, causal mask (optionally with a sliding window),
+// heads, power-of-two pages of at least 64 tokens, causal mask (optionally with a sliding window),
 // no score options.
 //
-// Work split and LDS layout are those of rpa_prefill_async_kernel (a workgroup of 4 waves owns
-// 128 query rows of one query head, wave w owns 32 of them, K/V tiles of 64 tokens arrive through
-// global_load_lds_dwordx4 into XOR-swizzled row-major LDS tiles).  What differs is the order of
-// work inside a wave.  A 64-token tile is handled as two halves of 32 tokens, and iteration i
-// holds three independent instruction streams:
-//     matrix pipe   S(i+1) = K(i+1) . Q^T          8 MFMAs (one accumulator chain)
+// LDS layout and copies are those of rpa_prefill_async_kernel (K/V tiles of 64 tokens arrive through
+// global_load_lds_dwordx4 into XOR-swizzled row-major LDS tiles, two ring slots per matrix).  A
+// workgroup of 4 waves owns 128 * NQ query rows of one query head; wave w owns NQ blocks of 32 rows.
+// With NQ = 2 every K and V^T fragment read from LDS feeds two MFMAs and a tile copied into LDS
+// serves twice the rows; the wave then needs more than 256 registers, so one wave runs per SIMD and
+// the overlap between matrix, vector and LDS work has to come from inside the wave.  A 64-token tile
+// is handled as two halves of 32 tokens, and iteration i holds three independent instruction
+// streams per block of rows:
+//     matrix pipe   S(i+1) = K(i+1) . Q^T - m      8 MFMAs (one accumulator chain)
 //     matrix pipe   O     += V(i-1)^T . P(i-1)^T   8 MFMAs (four accumulator chains)
-//     vector pipe   P(i)   = 2^(S(i) c - m c)      exponentials, packing, row sum, row maximum
-// so every vector instruction of the softmax has matrix instructions of the same wave to run
-// under, instead of relying on another wave being in the other phase.  Step t of a workgroup is
-// the pair of iterations (2t-1, 2t): it reads K tile t and V tile t-1, so two ring slots per
-// matrix suffice (V lags K by one tile) and there is still one barrier per tile.
+//     vector pipe   P(i)   = 2^S(i)                exponentials, packing, row sum
+// Step t of a workgroup is the pair of iterations (2t-1, 2t): it reads K tile t and V tile t-1, so
+// two ring slots per matrix suffice (V lags K by one tile) and there is one barrier per tile.
+//
+// Scores leave the matrix pipe ready for v_exp_f32: the queries are multiplied by
+// sm_scale * log2(e) once (and rounded to bf16 again: a relative change of 2^-9 per element, the
+// size of the rounding they already carry), and the first MFMA of a score chain takes minus the
+// running maximum as its C operand.  The running maximum is checked after the fact: a half's
+// probabilities are taken against the maximum known before it; if a row sum of the half exceeds
+// 2^8 the half is redone against its true maximum and everything accumulated is rescaled.
 //
 // The compiler does not keep such an interleave (it regroups the matrix instructions and spills),
-// and it will not keep two hundred registers in place around an assembly block that is only a loop
+// and it will not keep hundreds of registers in place around an assembly block that is only a loop
 // body, so the whole run of steady-state steps of a wave is one assembly block with fixed
 // registers, written by gen_prefill_pipe_loop.py into rpa_prefill_pipe_loop.inc; this file binds
-// the kernel's variables to those registers.  Steps that touch the causal diagonal or a window edge, the first and the
-// last steps run the same pipeline through a general iteration in C++ with masking and run-time
-// flags.
-//
-// The running maximum is checked after the fact: the exponentials of half i use the maximum known
-// before it; the half's own maximum is taken by the vector pipe next to them, and only if it
-// exceeds the stale one by more than 2^kMaxSlack is the half redone (its scores are still in
-// registers) and the accumulators rescaled.
+// the kernel's variables to those registers.  Steps that touch the causal diagonal or a window
+// edge, the first and the last steps run the same pipeline through a general iteration in C++ with
+// masking and run-time flags.
 //
 // The global -> LDS copies are issued as assembly too, so the compiler knows of no store into the
 // LDS ring and never waits for the copy queue on its own; the kernel waits (vmcnt(0)) in front of
 // the barrier that ends a step.
+
+#include <type_traits>
 
 #include "rpa_prefill_common.h"
 #include "rpa_prefill_pipe_loop.inc"
@@ -46,8 +51,11 @@ constexpr int kTileB = kBN * kRowB;      // 16 KiB
 constexpr int kHalfB = 32 * kRowB;       // byte distance between the halves of a tile
 constexpr int kKSlot = 0;                // ring slots inside the LDS array: K0 K1 V0 V1
 constexpr int kVSlot = 2 * kTileB;
+constexpr float kRowSumLimit = 256.0f;   // a half's row sum above it: the stale maximum is too stale
+constexpr float kSeenFloor = -1.0e30f;   // a row maximum below it: every token so far was masked
 
-typedef uint32_t u32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x32_t __attribute__((ext_vector_type(32)));
+typedef uint32_t u32x8_t __attribute__((ext_vector_type(8)));
 typedef int32_t i32x8_t __attribute__((ext_vector_type(8)));
 typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x4v_t __attribute__((ext_vector_type(4)));
@@ -61,32 +69,35 @@ __device__ __forceinline__ u32x2_t lds_tr16_at(int addr) {
   return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((p_t)(uint32_t)addr));
 }
 
-template <int KS>
-__device__ __forceinline__ u32x4_t q_frag(const u32x16_t& a, const u32x16_t& b) {
-  const u32x16_t& s = KS < 4 ? a : b;
-  constexpr int o = (KS & 3) * 4;
-  return u32x4_t{s[o], s[o + 1], s[o + 2], s[o + 3]};
-}
-
-// The registers of one wave's pipeline.  The assembly loop expects them in the registers the
-// RPA_PIPE_C_* constraints of rpa_prefill_pipe_loop.inc name.
-struct Pipe {
-  f32x16_t O[4];      // accumulators, lane (c, h): row c, dims 32d + 8*(v/4) + 4h + v%4
-  f32x16_t S0, S1;    // scores of the even / odd half in flight
-  u32x4_t P0[2], P1[2];  // probabilities of the even / odd half (B operands of the second product)
-  u32x16_t Qa, Qb;    // Q^T operands of the 8 k-steps
-  i32x8_t koff;       // LDS addresses of the K operand reads (slot 0, first half)
-  i32x4_t voff;       // LDS addresses of the V^T operand reads (slot 0, first half, first k-step)
-  float m, l;         // running maximum (raw score units), running sum
-  u32x4_t ofs_k, ofs_v;  // per-lane byte offsets of this wave's four K / V copy instructions
-  float sc2;          // raw score -> log2 units
+// The registers of one block of 32 query rows.  The assembly loop expects them in the registers the
+// RPA_PIPE_NQn_C_* constraints of rpa_prefill_pipe_loop.inc name.
+struct RowBlock {
+  f32x16_t O[4];    // accumulators, lane (c, h): row c, dims 32d + 8*(v/4) + 4h + v%4
+  u32x32_t Q;       // Q^T operands of the 8 k-steps, scaled to log2 units
+  f32x16_t S[2];    // scores of the even / odd half in flight, minus the running maximum
+  u32x8_t P[2];     // probabilities of the even / odd half (two B operands of the second product each)
+  f32x16_t NM;      // minus the running maximum in all 16 registers (C operand of a score chain's first MFMA)
+  float m, l;       // running maximum (log2 units), running sum of this lane's tokens
+  float seen;       // 1 once the row has met a token it may see (same in both lanes of a row)
+  int qpos;         // position of this lane's row
 };
+
+struct Shared {   // what the row blocks of a wave share
+  i32x8_t koff;   // LDS addresses of the K operand reads (slot 0, first half)
+  i32x4_t voff;   // LDS addresses of the V^T operand reads (slot 0, first half, first k-step)
+  u32x4_t ofs_k, ofs_v;  // per-lane byte offsets of this wave's four K / V copy instructions
+};
+
+template <int KS>
+__device__ __forceinline__ u32x4_t q_frag(const u32x32_t& q) {
+  return u32x4_t{q[4 * KS], q[4 * KS + 1], q[4 * KS + 2], q[4 * KS + 3]};
+}
 
 // K or V rows of one tile, global -> LDS: 4 instructions per wave.  `lds_wave` is the LDS address
 // of this wave's first 1 KiB block of the slot.
 template <bool IS_V>
 __device__ __forceinline__ void copy_rows(uint32_t lds_wave, const TileSrc& s, const KvAddr& kv, const char* head, int tb,
-                                          int wave, int lane, int page, const AsyncOffsets<128>& ofs) {
+                                          int wave, int lane, int page, const Shared& sh) {
   tb = min(tb, s.last_tok & ~(kBN - 1));
   if (tb + kBN - 1 <= s.last_tok) {
     const int64_t base = (int64_t)page * kv.page_stride + (int64_t)(tb - page_slot(s, tb) * s.page_size) * kv.tok_stride;
@@ -94,7 +105,7 @@ __device__ __forceinline__ void copy_rows(uint32_t lds_wave, const TileSrc& s, c
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                   :: "s"(lds_wave + n * 1024), "v"(IS_V ? ofs.v[n] : ofs.k[n]), "s"(b)
+                   :: "s"(lds_wave + n * 1024), "v"(IS_V ? sh.ofs_v[n] : sh.ofs_k[n]), "s"(b)
                    : "memory", "m0");
     }
     return;
@@ -118,48 +129,44 @@ __device__ __forceinline__ int scalar_page(const TileSrc& s, int tb) {
   return scalar_load_i32(s.pages + __builtin_amdgcn_readfirstlane(page_slot(s, tb)));
 }
 
-// first product of one 32-token half: one chain of 8 MFMAs; `off` = slot and half offset
-__device__ __forceinline__ f32x16_t qk_half(const Pipe& p, int off) {
-  f32x16_t S = mfma32(lds_ld16_at(p.koff[0] + off), q_frag<0>(p.Qa, p.Qb), kZero16);
-  S = mfma32(lds_ld16_at(p.koff[1] + off), q_frag<1>(p.Qa, p.Qb), S);
-  S = mfma32(lds_ld16_at(p.koff[2] + off), q_frag<2>(p.Qa, p.Qb), S);
-  S = mfma32(lds_ld16_at(p.koff[3] + off), q_frag<3>(p.Qa, p.Qb), S);
-  S = mfma32(lds_ld16_at(p.koff[4] + off), q_frag<4>(p.Qa, p.Qb), S);
-  S = mfma32(lds_ld16_at(p.koff[5] + off), q_frag<5>(p.Qa, p.Qb), S);
-  S = mfma32(lds_ld16_at(p.koff[6] + off), q_frag<6>(p.Qa, p.Qb), S);
-  S = mfma32(lds_ld16_at(p.koff[7] + off), q_frag<7>(p.Qa, p.Qb), S);
+// first product of one 32-token half: one chain of 8 MFMAs starting from minus the running
+// maximum; `off` = slot and half offset
+__device__ __forceinline__ f32x16_t qk_half(const RowBlock& b, const Shared& sh, int off) {
+  f32x16_t S = mfma32(lds_ld16_at(sh.koff[0] + off), q_frag<0>(b.Q), b.NM);
+  S = mfma32(lds_ld16_at(sh.koff[1] + off), q_frag<1>(b.Q), S);
+  S = mfma32(lds_ld16_at(sh.koff[2] + off), q_frag<2>(b.Q), S);
+  S = mfma32(lds_ld16_at(sh.koff[3] + off), q_frag<3>(b.Q), S);
+  S = mfma32(lds_ld16_at(sh.koff[4] + off), q_frag<4>(b.Q), S);
+  S = mfma32(lds_ld16_at(sh.koff[5] + off), q_frag<5>(b.Q), S);
+  S = mfma32(lds_ld16_at(sh.koff[6] + off), q_frag<6>(b.Q), S);
+  S = mfma32(lds_ld16_at(sh.koff[7] + off), q_frag<7>(b.Q), S);
   return S;
 }
 
 // second product of one 32-token half: four chains of 2 MFMAs
-__device__ __forceinline__ void pv_half(Pipe& p, int off, const u32x4_t (&P)[2]) {
+__device__ __forceinline__ void pv_half(RowBlock& b, const Shared& sh, int off, const u32x8_t& P) {
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      const int vt = p.voff[d] + off + kk * 16 * kRowB;
+      const int vt = sh.voff[d] + off + kk * 16 * kRowB;
       const u32x2_t lo = lds_tr16_at(vt);
       const u32x2_t hi = lds_tr16_at(vt + 8 * kRowB);
-      p.O[d] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, P[kk], p.O[d]);
+      b.O[d] = mfma32(u32x4_t{lo[0], lo[1], hi[0], hi[1]}, u32x4_t{P[4 * kk], P[4 * kk + 1], P[4 * kk + 2], P[4 * kk + 3]},
+                      b.O[d]);
     }
 }
 
-// probabilities of 16 scores against a fixed reference: P = bf16(2^(S sc2 + neg_m)), their sum
-__device__ __forceinline__ float exp_pack(const f32x16_t& S, float sc2, float neg_m, u32x4_t (&P)[2]) {
+// probabilities of 16 scores that are already relative to the running maximum: P = bf16(2^S), their sum
+__device__ __forceinline__ float exp_pack(const f32x16_t& S, u32x8_t& P) {
   const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
   float ps0 = 0.f, ps1 = 0.f;
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk) {
-    uint32_t w[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float p0 = fast_exp2(__builtin_fmaf(S[8 * kk + 2 * j], sc2, neg_m));
-      const float p1 = fast_exp2(__builtin_fmaf(S[8 * kk + 2 * j + 1], sc2, neg_m));
-      w[j] = pack_bf16x2(p0, p1);
-      if (j & 1) ps1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[j]), ones, ps1, false);
-      else ps0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[j]), ones, ps0, false);
-    }
-    P[kk] = u32x4_t{w[0], w[1], w[2], w[3]};
+  for (int j = 0; j < 8; ++j) {
+    const uint32_t w = pack_bf16x2(fast_exp2(S[2 * j]), fast_exp2(S[2 * j + 1]));
+    P[j] = w;
+    if (j & 1) ps1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), ones, ps1, false);
+    else ps0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), ones, ps0, false);
   }
   return ps0 + ps1;
 }
@@ -172,60 +179,97 @@ __device__ __forceinline__ float row_max16(const f32x16_t& S) {
   return swap_max(mx);
 }
 
-// softmax of a half with the maximum taken first (first half of a row, masked halves)
-__device__ __forceinline__ void softmax_half_general(f32x16_t& S, Pipe& p, bool need_mask, int tb, int h, int qpos,
-                                                     int window, u32x4_t (&P)[2]) {
+// Softmax of a half with the maximum taken first (first halves of a row, masked halves).  Sc: the
+// half's scores relative to the running maximum; Sn: the scores of the next half, already computed
+// against the same maximum, which move with it.
+__device__ __forceinline__ void softmax_half_general(f32x16_t& Sc, f32x16_t& Sn, RowBlock& b, bool need_mask, int tb, int h,
+                                                     int window, u32x8_t& P) {
   if (need_mask) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int tok = tb + 8 * (v >> 2) + 4 * h + (v & 3);
-      const bool masked = tok > qpos || (window > 0 && tok <= qpos - window);
-      S[v] = masked ? kMaskRaw : S[v];
+      const bool masked = tok > b.qpos || (window > 0 && tok <= b.qpos - window);
+      Sc[v] = masked ? kMaskRaw : Sc[v];
     }
   }
-  const float mx = row_max16(S);
-  if (__builtin_amdgcn_ballot_w64((mx - p.m) * p.sc2 > kMaxSlack) != 0) {
-    const float m_new = fmaxf(p.m, mx);
-    const float alpha = fast_exp2((p.m - m_new) * p.sc2);
-    p.m = m_new;
-    p.l *= alpha;
+  const float mx = row_max16(Sc);
+  // a row that has seen nothing yet takes the half's maximum as it is (nothing to rescale); afterwards
+  // the maximum only rises, and only when it is off by more than the slack
+  const bool real = mx > kSeenFloor;
+  const float d = (b.seen == 0.f) ? (real ? mx : 0.f) : (mx > kMaxSlack ? mx : 0.f);
+  if (__builtin_amdgcn_ballot_w64(d != 0.f) != 0) {
+    const float alpha = (b.seen == 0.f) ? 1.0f : fast_exp2(-d);
+    b.m += d;
+    b.l *= alpha;
 #pragma unroll
-    for (int d = 0; d < 4; ++d)
+    for (int dd = 0; dd < 4; ++dd)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) p.O[d][v] *= alpha;
+      for (int v = 0; v < 16; ++v) b.O[dd][v] *= alpha;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      b.NM[v] = -b.m;
+      Sc[v] -= d;
+      Sn[v] -= d;
+    }
   }
-  p.l += exp_pack(S, p.sc2, -p.m * p.sc2, P);
+  if (real) b.seen = 1.0f;
+  b.l += exp_pack(Sc, P);
 }
 
-// Steady-state steps [t, t_end) in assembly.  On entry K tile t is in K slot t & 1 and V tile t - 1
-// in V slot 1 - (t & 1), pg_a / pg_b are the pages of tiles t and t + 1; on exit the same holds for
-// t = t_end.  Every tile the loop copies (up to t_end) lies completely inside the sequence.
 struct LoopScalars {
   int t_end, t_lo, pmask, pshift, tok_stride, last_tile_tok;
   uint32_t pstr, kh_lo, kh_hi, vh_lo, vh_hi, lds_wave;
   const int32_t* pages;
+  float limit;
 };
 
-#define RPA_PIPE_LOOP(p, t, pg_a, pg_b, sc)                                                                       \
-  asm volatile(RPA_PIPE_LOOP_ASM                                                                                  \
-               : "+" RPA_PIPE_C_O0(p.O[0]), "+" RPA_PIPE_C_O1(p.O[1]), "+" RPA_PIPE_C_O2(p.O[2]),                 \
-                 "+" RPA_PIPE_C_O3(p.O[3]), "+" RPA_PIPE_C_S0(p.S0), "+" RPA_PIPE_C_S1(p.S1),                     \
-                 "+" RPA_PIPE_C_P00(p.P0[0]), "+" RPA_PIPE_C_P01(p.P0[1]), "+" RPA_PIPE_C_P10(p.P1[0]),           \
-                 "+" RPA_PIPE_C_P11(p.P1[1]), "+" RPA_PIPE_C_M(p.m), "+" RPA_PIPE_C_L(p.l),                       \
-                 [t] "+s"(t), [pg_a] "+s"(pg_a), [pg_b] "+s"(pg_b)                                                \
-               : RPA_PIPE_C_QA(p.Qa), RPA_PIPE_C_QB(p.Qb), RPA_PIPE_C_KOFF(p.koff), RPA_PIPE_C_VOFF(p.voff),      \
-                 RPA_PIPE_C_OFSK(p.ofs_k), RPA_PIPE_C_OFSV(p.ofs_v), [sc2] "s"(p.sc2), [nsc2] "s"(-p.sc2),        \
-                 [ones] "s"(0x3f803f80u), [t_end] "s"(sc.t_end), [t_lo] "s"(sc.t_lo), [pmask] "s"(sc.pmask),      \
-                 [pshift] "s"(sc.pshift), [tok_stride] "s"(sc.tok_stride), [last_tile_tok] "s"(sc.last_tile_tok), \
-                 [pstr] "s"(sc.pstr), [kh_lo] "s"(sc.kh_lo), [kh_hi] "s"(sc.kh_hi), [vh_lo] "s"(sc.vh_lo),        \
-                 [vh_hi] "s"(sc.vh_hi), [lds_wave] "s"(sc.lds_wave), [pages] "s"(sc.pages)                        \
-               : RPA_PIPE_LOOP_CLOBBERS)
+// Steady-state steps [t, t_end) in assembly.  On entry K tile t is in K slot t & 1 and V tile t - 1
+// in V slot 1 - (t & 1), pg_a / pg_b are the pages of tiles t and t + 1; on exit the same holds for
+// t = t_end.  Every tile the loop copies (up to t_end) lies completely inside the sequence.
+#define RPA_PIPE_SCALARS(sc)                                                                                    \
+  [ones] "s"(0x3f803f80u), [limit] "s"(sc.limit), [t_end] "s"(sc.t_end), [t_lo] "s"(sc.t_lo), [pmask] "s"(sc.pmask), \
+      [pshift] "s"(sc.pshift), [tok_stride] "s"(sc.tok_stride), [last_tile_tok] "s"(sc.last_tile_tok),             \
+      [pstr] "s"(sc.pstr), [kh_lo] "s"(sc.kh_lo), [kh_hi] "s"(sc.kh_hi), [vh_lo] "s"(sc.vh_lo),                    \
+      [vh_hi] "s"(sc.vh_hi), [lds_wave] "s"(sc.lds_wave), [pages] "s"(sc.pages)
 
-template <bool WIN>
-__global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillArgs a, int tiles, int nseq, bool by_level) {
+__device__ __forceinline__ void pipe_loop(RowBlock (&b)[1], const Shared& sh, int& t, int& pg_a, int& pg_b,
+                                          const LoopScalars& sc) {
+#define C(n) RPA_PIPE_NQ1_C_##n
+  asm volatile(RPA_PIPE_NQ1_ASM
+               : "+" C(O00)(b[0].O[0]), "+" C(O01)(b[0].O[1]), "+" C(O02)(b[0].O[2]), "+" C(O03)(b[0].O[3]),
+                 "+" C(S00)(b[0].S[0]), "+" C(S01)(b[0].S[1]), "+" C(P00)(b[0].P[0]), "+" C(P01)(b[0].P[1]),
+                 "+" C(NM0)(b[0].NM), "+" C(M0)(b[0].m), "+" C(L0)(b[0].l),
+                 [t] "+s"(t), [pg_a] "+s"(pg_a), [pg_b] "+s"(pg_b)
+               : C(Q0)(b[0].Q), C(KOFF)(sh.koff), C(VOFF)(sh.voff), C(OFSK)(sh.ofs_k), C(OFSV)(sh.ofs_v),
+                 RPA_PIPE_SCALARS(sc)
+               : RPA_PIPE_NQ1_CLOBBERS);
+#undef C
+}
+
+__device__ __forceinline__ void pipe_loop(RowBlock (&b)[2], const Shared& sh, int& t, int& pg_a, int& pg_b,
+                                          const LoopScalars& sc) {
+#define C(n) RPA_PIPE_NQ2_C_##n
+  asm volatile(RPA_PIPE_NQ2_ASM
+               : "+" C(O00)(b[0].O[0]), "+" C(O01)(b[0].O[1]), "+" C(O02)(b[0].O[2]), "+" C(O03)(b[0].O[3]),
+                 "+" C(O10)(b[1].O[0]), "+" C(O11)(b[1].O[1]), "+" C(O12)(b[1].O[2]), "+" C(O13)(b[1].O[3]),
+                 "+" C(S00)(b[0].S[0]), "+" C(S01)(b[0].S[1]), "+" C(P00)(b[0].P[0]), "+" C(P01)(b[0].P[1]),
+                 "+" C(S10)(b[1].S[0]), "+" C(S11)(b[1].S[1]), "+" C(P10)(b[1].P[0]), "+" C(P11)(b[1].P[1]),
+                 "+" C(NM0)(b[0].NM), "+" C(M0)(b[0].m), "+" C(L0)(b[0].l),
+                 "+" C(NM1)(b[1].NM), "+" C(M1)(b[1].m), "+" C(L1)(b[1].l),
+                 [t] "+s"(t), [pg_a] "+s"(pg_a), [pg_b] "+s"(pg_b)
+               : C(Q0)(b[0].Q), C(Q1)(b[1].Q), C(KOFF)(sh.koff), C(VOFF)(sh.voff), C(OFSK)(sh.ofs_k), C(OFSV)(sh.ofs_v),
+                 RPA_PIPE_SCALARS(sc)
+               : RPA_PIPE_NQ2_CLOBBERS);
+#undef C
+}
+
+template <bool WIN, int NQ>
+__global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kernel(const PrefillArgs a, int tiles, int nseq,
+                                                                                 bool by_level, float row_sum_limit) {
+  constexpr int BM = 128 * NQ;  // query rows per workgroup
   __shared__ __attribute__((aligned(1024))) char lds[4 * kTileB];
 
-  const Work w = decompose(a, tiles, nseq, by_level);
+  const Work w = decompose(a, tiles, nseq, by_level, BM);
   if (!w.valid) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -237,50 +281,49 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillA
   typedef __attribute__((address_space(3))) char* lds_ptr_t;
   const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)lds);
 
-  WaveRows wr;
-  wr.r_lo = w.q_start + wave * 32;
-  wr.r_hi = min(wr.r_lo + 31, w.q_len - 1);
-  wr.active = wr.r_lo < w.q_len;
-  wr.row = wr.r_lo + c;
-  wr.qpos = w.prefix + wr.row;
+  // rows of the wave: NQ blocks of 32
+  const int r_lo = w.q_start + wave * 32 * NQ;
+  const int r_hi = min(r_lo + 32 * NQ - 1, w.q_len - 1);
+  const bool active = r_lo < w.q_len;
   const int W_ = WIN ? a.sm.window : 0;
+  const float sc2 = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f) * kLog2e;
 
-  Pipe p;
-  {
-    const int rr = min(wr.row, w.q_len - 1);
+  RowBlock b[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    const int row = r_lo + 32 * q + c;
+    b[q].qpos = w.prefix + row;
+    const int rr = min(row, w.q_len - 1);
     const uint16_t* qp = a.q + ((int64_t)(w.qg0 + rr) * a.Hq + w.head) * 128 + h * 8;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const u32x4_t x = ld16(qp + ks * 16), y = ld16(qp + (ks + 4) * 16);
+    for (int ks = 0; ks < 8; ++ks) {
+      const u32x4_t x = ld16(qp + ks * 16);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        p.Qa[4 * ks + e] = x[e];
-        p.Qb[4 * ks + e] = y[e];
-      }
+      for (int e = 0; e < 4; ++e)
+        b[q].Q[4 * ks + e] = pack_bf16x2(bf16_lo_to_f32(x[e]) * sc2, bf16_hi_to_f32(x[e]) * sc2);
     }
-  }
-  p.sc2 = a.sm.sm_scale * (a.k_scale ? a.k_scale[w.hk] : 1.0f) * kLog2e;
 #pragma unroll
-  for (int d = 0; d < 4; ++d) p.O[d] = kZero16;
-  p.S0 = kZero16;
-  p.S1 = kZero16;
-  p.P0[0] = p.P0[1] = p.P1[0] = p.P1[1] = u32x4_t{0, 0, 0, 0};
-  p.m = kMaxFloor;
-  p.l = 0.f;
+    for (int d = 0; d < 4; ++d) b[q].O[d] = kZero16;
+    b[q].S[0] = b[q].S[1] = b[q].NM = kZero16;
+    b[q].P[0] = b[q].P[1] = u32x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    b[q].m = 0.f;
+    b[q].l = 0.f;
+    b[q].seen = 0.f;
+  }
 
-  const int wg_r_hi = min(w.q_start + kBM, w.q_len) - 1;
+  const int wg_r_hi = min(w.q_start + BM, w.q_len) - 1;
   const int t_hi = min(w.kv_len, w.prefix + wg_r_hi + 1);  // exclusive
   int t_lo = 0;
   if (W_ > 0) t_lo = max(0, w.prefix + w.q_start - W_ + 1) & ~(kBN - 1);
   const int nT = (t_hi - t_lo + kBN - 1) / kBN;  // K/V tiles of the workgroup
 
-  // halves [0, n_w) of 32 tokens concern this wave; halves [i_f0, i_f1) need no mask
+  // halves [0, n_w) of 32 tokens concern this wave; halves [i_f0, i_f1) need no mask for any of its rows
   int n_w = 0, i_f0 = 0, i_f1 = 0;
-  if (wr.active) {
-    n_w = (min(w.kv_len, w.prefix + wr.r_hi + 1) - t_lo + 31) >> 5;
-    i_f1 = max(0, (w.prefix + wr.r_lo - t_lo + 1) >> 5);
+  if (active) {
+    n_w = (min(w.kv_len, w.prefix + r_hi + 1) - t_lo + 31) >> 5;
+    i_f1 = max(0, (w.prefix + r_lo - t_lo + 1) >> 5);
     if (W_ > 0) {
-      const int y = w.prefix + wr.r_hi - W_ - t_lo;
+      const int y = w.prefix + r_hi - W_ - t_lo;
       i_f0 = y >= 0 ? (y >> 5) + 1 : 0;
     }
     i_f1 = min(i_f1, n_w);
@@ -290,6 +333,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillA
   i_f1 = __builtin_amdgcn_readfirstlane(i_f1);
 
   // operand addresses inside the LDS array (see rpa_prefill_async_kernel for the swizzles)
+  Shared sh;
   {
     const int k_row = c * kRowB;
     const int k_swz = (h ^ (c & 15)) << 4;
@@ -298,32 +342,38 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillA
     const int v_in = ((b16 & 1) << 5) + (((r16 & 3) >> 1) << 4) + ((r16 & 1) << 3);
     const int v_swz = (r16 >> 2) << 6;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) p.koff[ks] = (int)lds_base + kKSlot + k_row + ((ks * 32) ^ k_swz);
+    for (int ks = 0; ks < 8; ++ks) sh.koff[ks] = (int)lds_base + kKSlot + k_row + ((ks * 32) ^ k_swz);
 #pragma unroll
-    for (int d = 0; d < 4; ++d) p.voff[d] = (int)lds_base + kVSlot + v_row + v_in + ((d * 64) ^ v_swz);
+    for (int d = 0; d < 4; ++d) sh.voff[d] = (int)lds_base + kVSlot + v_row + v_in + ((d * 64) ^ v_swz);
+    const AsyncOffsets<128> ofs = make_async_offsets<128>(a.kv, wave, lane);
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      sh.ofs_k[n] = ofs.k[n];
+      sh.ofs_v[n] = ofs.v[n];
+    }
   }
 
-  const AsyncOffsets<128> ofs = make_async_offsets<128>(a.kv, wave, lane);
-#pragma unroll
-  for (int n = 0; n < 4; ++n) {
-    p.ofs_k[n] = ofs.k[n];
-    p.ofs_v[n] = ofs.v[n];
-  }
   const uint32_t lds_wave = lds_base + wave * 4096;  // this wave's four 1 KiB blocks of slot K0
   int pg_a = scalar_page(src, t_lo);         // page of tile t
-  copy_rows<false>(lds_wave + kKSlot, src, a.kv, kh, t_lo, wave, lane, pg_a, ofs);
+  copy_rows<false>(lds_wave + kKSlot, src, a.kv, kh, t_lo, wave, lane, pg_a, sh);
   int pg_b = scalar_page(src, t_lo + kBN);   // page of tile t + 1
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
 
-  // iteration i of the general kind: Sn <- scores of half i + 1, Pc <- softmax of Sc (half i), O += P(i - 1) V
-  auto general_iter = [&](int i, f32x16_t& Sc, f32x16_t& Sn, u32x4_t (&Pc)[2], const u32x4_t (&Pp)[2], int k_off,
-                          int v_off) __attribute__((always_inline)) {
-    if (i + 1 < n_w) Sn = qk_half(p, k_off);
-    if (i >= 1 && i - 1 < n_w) pv_half(p, v_off, Pp);
+  // iteration i of the general kind, half i in buffer i & 1: scores of half i + 1, second product of
+  // half i - 1, softmax of half i
+  auto general_iter = [&](auto cur_tag, int i, int k_off, int v_off) __attribute__((always_inline)) {
+    constexpr int cur = decltype(cur_tag)::value, nxt = cur ^ 1;  // half i lives in buffer i & 1
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      if (i + 1 < n_w) b[q].S[nxt] = qk_half(b[q], sh, k_off);
+      if (i >= 1 && i - 1 < n_w) pv_half(b[q], sh, v_off, b[q].P[nxt]);
+    }
     if (i >= 0 && i < n_w) {
       const bool need_mask = i < i_f0 || i >= i_f1;
-      softmax_half_general(Sc, p, need_mask, t_lo + 32 * i, h, wr.qpos, W_, Pc);
+#pragma unroll
+      for (int q = 0; q < NQ; ++q)
+        softmax_half_general(b[q].S[cur], b[q].S[nxt], b[q], need_mask, t_lo + 32 * i, h, W_, b[q].P[cur]);
     }
   };
 
@@ -331,8 +381,8 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillA
   // t - 1 from V slot 1 - par, fills K slot 1 - par with tile t + 1 and V slot par with tile t
   auto copies = [&](int t, int par) __attribute__((always_inline)) {
     if (t + 1 < nT)
-      copy_rows<false>(lds_wave + kKSlot + (1 - par) * kTileB, src, a.kv, kh, t_lo + (t + 1) * kBN, wave, lane, pg_b, ofs);
-    if (t < nT) copy_rows<true>(lds_wave + kVSlot + par * kTileB, src, a.kv, vh, t_lo + t * kBN, wave, lane, pg_a, ofs);
+      copy_rows<false>(lds_wave + kKSlot + (1 - par) * kTileB, src, a.kv, kh, t_lo + (t + 1) * kBN, wave, lane, pg_b, sh);
+    if (t < nT) copy_rows<true>(lds_wave + kVSlot + par * kTileB, src, a.kv, vh, t_lo + t * kBN, wave, lane, pg_a, sh);
     pg_a = pg_b;
     if (t + 2 < nT) pg_b = scalar_page(src, t_lo + (t + 2) * kBN);
   };
@@ -356,23 +406,39 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillA
   sc.vh_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)vh >> 32));
   sc.lds_wave = lds_wave;
   sc.pages = src.pages;
+  sc.limit = row_sum_limit;
+  auto general_step = [&](int t) __attribute__((always_inline)) {
+    const int par = t & 1;
+    copies(t, par);
+    const int k_off = par * kTileB, v_off = (1 - par) * kTileB;
+    general_iter(std::integral_constant<int, 1>{}, 2 * t - 1, k_off, v_off);
+    general_iter(std::integral_constant<int, 0>{}, 2 * t, k_off + kHalfB, v_off + kHalfB);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+  };
+  // Three phases, each a loop of its own (one loop that switches between the assembly block and the
+  // general step would move the whole register state to a common place on every trip): general steps
+  // up to the first steady-state step, the assembly loop, general steps to the end.
+  const bool has_fast = t_fb < t_fe;
+  const int t_first = has_fast ? t_fb : nT + 1;
   int t = 0;
-  while (t <= nT) {
-    if (t >= t_fb && t < t_fe) {
-      RPA_PIPE_LOOP(p, t, pg_a, pg_b, sc);  // leaves t == t_fe
-    } else {
-      const int par = t & 1;
-      copies(t, par);
-      const int i = 2 * t - 1;
-      const int k_off = par * kTileB, v_off = (1 - par) * kTileB;
-      general_iter(i, p.S1, p.S0, p.P1, p.P0, k_off, v_off);
-      general_iter(i + 1, p.S0, p.S1, p.P0, p.P1, k_off + kHalfB, v_off + kHalfB);
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __syncthreads();
-      ++t;
-    }
+  for (; t < t_first; ++t) general_step(t);
+  if (has_fast) {
+    pipe_loop(b, sh, t, pg_a, pg_b, sc);  // leaves t == t_fe
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) b[q].seen = 1.0f;  // a steady-state half hides nothing from any row
+    for (; t <= nT; ++t) general_step(t);
   }
-  write_rows<4>(a, w, wr, p.O, p.l, h, p.m * p.sc2);
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    WaveRows wr;
+    wr.r_lo = r_lo + 32 * q;
+    wr.r_hi = min(wr.r_lo + 31, w.q_len - 1);
+    wr.active = wr.r_lo < w.q_len;
+    wr.row = wr.r_lo + c;
+    wr.qpos = b[q].qpos;
+    write_rows<4>(a, w, wr, b[q].O, b[q].l, h, b[q].m);
+  }
 }
 
 }  // namespace
@@ -380,14 +446,35 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_pipe_kernel(const PrefillA
 bool prefill_pipe_applies(const PrefillArgs& a) {
   const int P = a.pt.page_size;
   return !a.fp8 && a.head_dim == 128 && P >= kBN && (P & (P - 1)) == 0 && a.kv.page_stride < (int64_t(1) << 32) &&
-         a.sm.mask_mode == 0 && a.sm.soft_cap == 0.f &&
-         a.sm.round_logits == 0 && !(a.sm.xai_len > 0.f) && !(a.sm.q_scale > 0.f);
+         a.sm.mask_mode == 0 && a.sm.soft_cap == 0.f && a.sm.round_logits == 0 && !(a.sm.xai_len > 0.f) &&
+         !(a.sm.q_scale > 0.f);
 }
 
-hipError_t launch_prefill_pipe(const PrefillArgs& a, int tiles, int nseq, bool by_level, unsigned grid, hipStream_t stream) {
-  const dim3 g(grid), blk(256);
-  if (a.sm.window > 0) hipLaunchKernelGGL((rpa_prefill_pipe_kernel<true>), g, blk, 0, stream, a, tiles, nseq, by_level);
-  else hipLaunchKernelGGL((rpa_prefill_pipe_kernel<false>), g, blk, 0, stream, a, tiles, nseq, by_level);
+hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order, hipStream_t stream) {
+  static const int force_nq = [] { const char* v = getenv("RPA_PREFILL_PIPE_NQ"); return v ? atoi(v) : 0; }();
+  // a half's row sum above the limit sends a wave through the rescaling path (testing knob: -1 = always)
+  static const float limit = [] { const char* v = getenv("RPA_PREFILL_PIPE_LIMIT"); return v ? (float)atof(v) : kRowSumLimit; }();
+  const int nq = force_nq ? force_nq : 1;
+  const int bm = 128 * nq;
+  int tiles = (a.max_q_len + bm - 1) / bm;
+  const int levels = a.max_kv_len > 0 ? (a.max_kv_len + bm - 1) / bm + 1 : 0;
+  const bool by_level = level_order && levels > tiles && levels <= 2 * tiles + 2;
+  if (by_level) tiles = levels;
+  const int64_t units = (int64_t)nseq * a.Hkv;
+  const int64_t grid = (units >= 8 ? ((units + 7) / 8) * 8 : units) * a.G * tiles;
+  if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
+  const dim3 g((unsigned)grid), blk(256);
+  const bool win = a.sm.window > 0;
+#define RPA_LAUNCH(W, N) \
+  hipLaunchKernelGGL((rpa_prefill_pipe_kernel<W, N>), g, blk, 0, stream, a, tiles, nseq, by_level, limit)
+  if (nq == 1) {
+    if (win) RPA_LAUNCH(true, 1);
+    else RPA_LAUNCH(false, 1);
+  } else {
+    if (win) RPA_LAUNCH(true, 2);
+    else RPA_LAUNCH(false, 2);
+  }
+#undef RPA_LAUNCH
   return hipGetLastError();
 }
 

@@ -437,7 +437,13 @@ def test_xai_temperature(pkg, wl, gpu, cap):
         want = oracle_out(b, xai_temperature_len=T)
         got = gpu_out(pkg, b, gpu, xai_temperature_len=T)
         assert_parity(got.float(), want.float(), **BF16_TOL)
-    assert torch.equal(gpu_out(pkg, b, gpu, xai_temperature_len=8192.0), gpu_out(pkg, b, gpu))
+    # no row lies beyond T = 8192: the same result as without the option, bit for bit on the decode rows;
+    # the chunks take different kernels with and without the option (the plain case has its own), so
+    # they agree to rounding only
+    far, plain = gpu_out(pkg, b, gpu, xai_temperature_len=8192.0), gpu_out(pkg, b, gpu)
+    n_dec = sum(1 for x in q_lens if x == 1)
+    assert torch.equal(far[:n_dec], plain[:n_dec])
+    assert float(row_rel_error(far.float(), plain.float()).max()) <= 1e-2
 
 
 @pytest.mark.parametrize("cap,use_sink", [(None, False), (20.0, True)])
@@ -483,10 +489,11 @@ def test_q_scale_quantises_queries_to_the_cache_type(pkg, wl, gpu, kv_dtype):
     want = oracle_out(b)
     b.q, b.sm_scale = q_orig, sm_orig
     assert_parity(got.float(), want.float(), **(FP8_TOL if kv_dtype != torch.bfloat16 else BF16_TOL))
-    # and the kernels compute exactly what they compute on pre-quantised queries
+    # and the kernels compute what they compute on pre-quantised queries (to rounding: with the option
+    # off the chunks of a bf16 cache take the kernel of the plain case, which rounds elsewhere)
     b.q, b.sm_scale = quantise_queries(q_orig, q_scale, kv_dtype), sm_orig * q_scale
     same = gpu_out(pkg, b, gpu)
-    torch.testing.assert_close(got.float(), same.float(), rtol=8e-3, atol=1e-3)
+    assert float(row_rel_error(got.float(), same.float()).max()) <= 1e-2
 
 
 def flat_mask(masks):
