@@ -101,7 +101,7 @@ class Table:
         self.first_scratch = self._v
         self.PS = [[v(1), v(1)] for q in range(nq)]                # row-sum accumulators of the half
         self.MX, self.T0, self.T1 = v(1), v(1), v(1)
-        self.E = v(8)                                              # temporaries of the exponentials
+        self.E = [v(8) for q in range(nq)]                         # temporaries of the exponentials
         self.num_vgpr = self._v
         self.num_agpr = self._a - ACC
 
@@ -236,36 +236,54 @@ class Gen:
         ins.lds_need = None if "nolds" in X else [("vlo", f), ("vhi", f)]
         return ins
 
-    def softmax_block(self, q, sc):
-        """vector work of the 16 scores of S[q][sc]: exponentials, packed in pairs into P[q][sc], row sum in
-        PS[q][0].  The row-sum instruction of a pair is issued after the next pair's exponentials, so nothing
-        waits for the instruction in front of it."""
+    def softmax_ops(self, q, sc):
+        """The vector work of the 16 scores of S[q][sc] as three stages per score pair j: the two
+        exponentials, the packing into register j of P[q][sc], the row-sum update."""
         t = self.t
-        out = [valu(f"v_mov_b32 {vr(t.PS[q][0])}, 0", [], [t.PS[q][0]]), valu(f"v_mov_b32 {vr(t.PS[q][1])}, 0", [], [t.PS[q][1]])]
+
+        def exps(j):
+            s0, s1 = t.S[q][sc] + 2 * j, t.S[q][sc] + 2 * j + 1
+            e0, e1 = t.E[q] + 2 * (j % 4), t.E[q] + 2 * (j % 4) + 1
+            return [valu(f"v_exp_f32 {vr(e0)}, {vr(s0)}", [s0], [e0], "trans"),
+                    valu(f"v_exp_f32 {vr(e1)}, {vr(s1)}", [s1], [e1], "trans")]
+
+        def cvt(j):
+            e0, e1 = t.E[q] + 2 * (j % 4), t.E[q] + 2 * (j % 4) + 1
+            return [valu(f"v_cvt_pk_bf16_f32 {vr(t.P[q][sc] + j)}, {vr(e0)}, {vr(e1)}", [e0, e1], [t.P[q][sc] + j])]
 
         def dot(j):
             w, ps = t.P[q][sc] + j, t.PS[q][j & 1]
-            return valu(f"v_dot2c_f32_bf16 {vr(ps)}, %[ones], {vr(w)}", [w, ps], [ps], "dot")
+            return [valu(f"v_dot2c_f32_bf16 {vr(ps)}, %[ones], {vr(w)}", [w, ps], [ps], "dot")]
 
-        for j in range(8):
-            s0, s1 = t.S[q][sc] + 2 * j, t.S[q][sc] + 2 * j + 1
-            e0, e1 = t.E + 2 * (j % 4), t.E + 2 * (j % 4) + 1
-            out.append(valu(f"v_exp_f32 {vr(e0)}, {vr(s0)}", [s0], [e0], "trans"))
-            out.append(valu(f"v_exp_f32 {vr(e1)}, {vr(s1)}", [s1], [e1], "trans"))
-            if j > 0:
-                out.append(dot(j - 1))
-            out.append(valu(f"v_cvt_pk_bf16_f32 {vr(t.P[q][sc] + j)}, {vr(e0)}, {vr(e1)}", [e0, e1], [t.P[q][sc] + j]))
-        out.append(dot(7))
-        out.append(valu(f"v_add_f32 {vr(t.PS[q][0])}, {vr(t.PS[q][0])}, {vr(t.PS[q][1])}", t.PS[q], [t.PS[q][0]]))
-        return out
+        return exps, cvt, dot
 
-    def softmax_stream(self, sc):
-        t = self.t
+    def softmax_stream(self, sc, check=True):
+        """All row blocks' softmax work in issue order.  The stages of a pair are spread out (packing
+        `lag` pairs behind the exponentials, the row sum one pair behind the packing) and the row blocks
+        are interleaved, so no instruction needs the result of the few in front of it: a wave issues in
+        order, and a vector instruction that waits holds up the matrix instructions behind it."""
+        t, nq = self.t, self.nq
+        lag = 2 if nq == 1 else 1
         out = []
-        for q in range(self.nq):
-            out += self.softmax_block(q, sc)
+        ops = [self.softmax_ops(q, sc) for q in range(nq)]
+        for q in range(nq):
+            out += [valu(f"v_mov_b32 {vr(t.PS[q][0])}, 0", [], [t.PS[q][0]]), valu(f"v_mov_b32 {vr(t.PS[q][1])}, 0", [], [t.PS[q][1]])]
+        for step in range(8 + lag + 1):
+            for q in range(nq):
+                if step < 8:
+                    out += ops[q][0](step)
+            for q in range(nq):
+                if 0 <= step - lag < 8:
+                    out += ops[q][1](step - lag)
+            for q in range(nq):
+                if 0 <= step - lag - 1 < 8:
+                    out += ops[q][2](step - lag - 1)
+        for q in range(nq):
+            out.append(valu(f"v_add_f32 {vr(t.PS[q][0])}, {vr(t.PS[q][0])}, {vr(t.PS[q][1])}", t.PS[q], [t.PS[q][0]]))
+        if not check:
+            return out
         # any row sum of the half above the limit (or not a number)?
-        if self.nq == 2:
+        if nq == 2:
             out.append(valu(f"v_max_f32 {vr(t.T0)}, {vr(t.PS[0][0])}, {vr(t.PS[1][0])}", [t.PS[0][0], t.PS[1][0]], [t.T0]))
             out.append(valu(f"v_cmp_nle_f32 vcc, {vr(t.T0)}, %[limit]", [t.T0], []))
         else:
@@ -367,8 +385,8 @@ class Gen:
             for base in (t.NM[q], t.S[q][sc], t.S[q][sn]):
                 for v in range(16):
                     em.emit(valu(f"v_sub_f32 {vr(base + v)}, {vr(base + v)}, {vr(t.MX)}", [base + v, t.MX], [base + v]))
-            for x in self.softmax_block(q, sc):
-                em.emit(x)
+        for x in self.softmax_stream(sc, check=False):
+            em.emit(x)
         em.raw("s_nop 3", "nop")  # P, NM and O were written by the vector pipe; a matrix instruction may follow at once
         em.raw(f"s_branch {back}")
 
@@ -408,6 +426,11 @@ class Gen:
         copies = [self.copy_ins(n, False, 1 - ks) for n in range(4)] + [self.copy_ins(n, True, 1 - vs) for n in range(4)]
         if "nocopy" in X:
             copies = []
+        if "copyfirst" in X:
+            for grp in copies:
+                for x in grp:
+                    em.emit(x)
+            copies = []
         for it in (0, 1):
             self.iteration(em, it, ks, vs, copies)
             tag = uid + "ab"[it]
@@ -418,7 +441,7 @@ class Gen:
                 em.emit(valu(f"v_add_f32 {vr(t.L[q])}, {vr(t.L[q])}, {vr(t.PS[q][0])}", [t.L[q], t.PS[q][0]], [t.L[q]]))
         assert not copies and not em.lds_queue
         # ---- end of step: the copies have landed, everybody has finished reading the slots they overwrite next
-        em.raw("s_waitcnt vmcnt(0) lgkmcnt(0)", "wait")
+        em.raw("s_waitcnt lgkmcnt(0)" if "novmwait" in X else "s_waitcnt vmcnt(0) lgkmcnt(0)", "wait")
         em.raw("s_mov_b32 %[pg_a], %[pg_b]")
         em.raw(f"s_mov_b32 %[pg_b], s{PGC}")
         if "nobarrier" not in X:
