@@ -227,6 +227,19 @@ int rpa_prefill(const RpaParams* p, void* stream);
 int rpa_attention(const RpaParams* p, void* stream);
 
 /*
+ * rpa_attention for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it).  No counterpart in the reference, where XLA owns
+ * every buffer.  Same arguments and results as rpa_attention, except that p->workspace and
+ * p->workspace_bytes are ignored: the split-KV workspace is an array the library holds itself on
+ * every GPU, rpa_noalloc_max_workspace_bytes() (40 MiB) long.  A batch whose rpa_workspace_bytes()
+ * exceeds it is refused with RPA_EINVAL_WORKSPACE.  The call allocates and frees nothing.  All
+ * calls on one GPU share the array: calls that overlap on one GPU (two streams, a graph replay next
+ * to eager work) race on it; order them on one stream.
+ */
+size_t rpa_noalloc_max_workspace_bytes(void);
+int rpa_attention_noalloc(const RpaParams* p, void* stream);
+
+/*
  * Scatter the new K/V rows of every sequence into the paged cache: the fused
  * cache update of ragged_paged_attention_v3.py:670-719 / the standalone
  * kv_cache_update of kernels/update_kv_cache/update_kv_cache.py:120.  Token j of

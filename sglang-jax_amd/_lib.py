@@ -45,6 +45,8 @@ EXPORTED_SYMBOLS = (
     "rpa_decode",
     "rpa_prefill",
     "rpa_attention",
+    "rpa_noalloc_max_workspace_bytes",
+    "rpa_attention_noalloc",
     "rpa_kv_write",
     "rpa_mla_decode",
     "rpa_mla_attention_workspace_bytes",
@@ -168,7 +170,9 @@ def load() -> ctypes.CDLL:
     lib.rpa_gather_pages.restype = ctypes.c_int
     lib.rpa_gather_pages.argtypes = [P(RpaParams), ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p,
                                      ctypes.c_int32, ctypes.c_void_p]
-    for name in ("rpa_decode", "rpa_prefill", "rpa_attention"):
+    lib.rpa_noalloc_max_workspace_bytes.restype = ctypes.c_size_t
+    lib.rpa_noalloc_max_workspace_bytes.argtypes = []
+    for name in ("rpa_decode", "rpa_prefill", "rpa_attention", "rpa_attention_noalloc"):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [P(RpaParams), ctypes.c_void_p]

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -310,6 +311,29 @@ int rows256(const RpaParams* p, int seq_begin, int seq_end, void* stream) {
 
 }  // namespace
 
+// ---- rpa_attention_noalloc: the split-KV workspace as a static device array ----
+// Every GPU the library is loaded on holds one copy of the array until the process ends.
+constexpr size_t kNoAllocScratchBytes = (size_t)40 << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// The array's address on the current device (its name is only a host-side handle): looked up once
+// per device with that device current, then kept.
+int noalloc_scratch(void** out) {
+  int dev = -1;
+  if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+  if (dev < 0 || dev >= kMaxDevices) return fail(RPA_EUNSUPPORTED, "device ordinal %d: at most %d devices", dev, kMaxDevices);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    if (int rc = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+    if (!ptr) return fail(RPA_EHIP, "hipGetSymbolAddress(scratch) returned a null address");
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return RPA_OK;
+}
+
 extern "C" {
 
 int rpa_version(void) { return RPA_VERSION; }
@@ -530,6 +554,31 @@ int rpa_attention(const RpaParams* p, void* stream) {
   int rc = rpa_decode(p, stream);
   if (rc != RPA_OK) return rc;
   return rpa_prefill(p, stream);
+}
+
+size_t rpa_noalloc_max_workspace_bytes(void) { return kNoAllocScratchBytes; }
+
+int rpa_attention_noalloc(const RpaParams* p, void* stream) {
+  int rc = rpa_validate(p);
+  if (rc != RPA_OK) return rc;
+  const size_t need = rpa_workspace_bytes(p);
+  if (need > kNoAllocScratchBytes)
+    return fail(RPA_EINVAL_WORKSPACE,
+                "this batch needs a split-KV workspace of %zu bytes, the built-in one holds %zu: call rpa_attention "
+                "with a workspace of your own",
+                need, kNoAllocScratchBytes);
+  RpaParams q = *p;
+  q.workspace = nullptr;
+  q.workspace_bytes = 0;
+  if (need > 0) {
+    void* ptr = nullptr;
+    if ((rc = noalloc_scratch(&ptr)) != RPA_OK) return rc;
+    q.workspace = ptr;  // the device address, never the array's name
+    q.workspace_bytes = kNoAllocScratchBytes;
+  }
+  // Nothing in the workspace has to start at zero: partial rows, their (max, sum) pairs and the block
+  // prefix sums are all written by the decode kernel before the merge pass reads them.
+  return rpa_attention(&q, stream);
 }
 
 int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void* stream) {

@@ -62,11 +62,11 @@ typedef short s16x4v_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ u32x4_t lds_ld16_at(int addr) {
   typedef const __attribute__((address_space(3))) u32x4_t* p_t;
-  return *(p_t)(uint32_t)addr;
+  return *(p_t)(uintptr_t)(uint32_t)addr;
 }
 __device__ __forceinline__ u32x2_t lds_tr16_at(int addr) {
   typedef __attribute__((address_space(3))) s16x4v_t* p_t;
-  return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((p_t)(uint32_t)addr));
+  return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((p_t)(uintptr_t)(uint32_t)addr));
 }
 
 // The registers of one block of 32 query rows.  The assembly loop expects them in the registers the

@@ -289,6 +289,10 @@ class RpaCall:
     def attention(self):
         _lib.check(self.lib.rpa_attention(ctypes.byref(self.params), self._stream()))
 
+    def attention_noalloc(self):
+        """``rpa_attention_noalloc``: the library's own workspace instead of this call's."""
+        _lib.check(self.lib.rpa_attention_noalloc(ctypes.byref(self.params), self._stream()))
+
     def decode(self):
         _lib.check(self.lib.rpa_decode(ctypes.byref(self.params), self._stream()))
 
