@@ -15,8 +15,11 @@ One JSON line is printed:
   prefill_tflops, decode_frac_of_hbm_peak, prefill_frac_of_mfma_peak
   roofline    the workload's dominant kernel (largest average launch time),
               timed with events on the launch stream over the timed region
+  parity_sample  a few rows of the timed output against the CPU oracle (outside the timed region)
+  other_configs  the remaining configurations (C1, C3, C4, C4 windowed, C5), each with its kernel,
+              average / median / minimum launch time, algorithmic bytes or FLOPs and roofline fraction
+              (--main-only skips them)
   cpu_baseline  the CPU oracle timed on this box's host cores on a bounded sample
-  other_configs (with --all) decode GB/s of the remaining configurations
 """
 
 from __future__ import annotations
@@ -49,8 +52,10 @@ DECODE_KERNEL = {
     "c5": "rpa_mla_balanced_kernel",
 }
 
+PREFILL_KERNEL = "rpa_prefill_pipe_kernel"
+
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", "rpa_prefill_async_kernel"): 365.6e6 + 77.5e6,
+    ("c2", PREFILL_KERNEL): 365.6e6 + 77.5e6,
     ("c2", "rpa_decode_balanced_kernel"): 500.9e6 + 2.7e6,
     ("c3", "rpa_decode_splitkv_kernel"): 2148.6e6 + 1.9e6,
     ("c5", "rpa_mla_balanced_kernel"): 817.4e6 + 83.1e6,
@@ -63,9 +68,15 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
+def _stats(ms):
+    ms = sorted(ms)
+    n = len(ms)
+    return {"mean": sum(ms) / n, "median": ms[n // 2] if n % 2 else 0.5 * (ms[n // 2 - 1] + ms[n // 2]), "min": ms[0]}
+
+
 def time_partitions(call, steps, warmup, has_decode, has_prefill):
     """W warm-up steps, then exactly `steps` timed steps; returns wall ms per step and
-    the average event-timed duration of each partition inside the timed region."""
+    mean / median / min of the event-timed duration of each partition inside the timed region."""
     import torch
 
     def one(ev=None):
@@ -89,8 +100,8 @@ def time_partitions(call, steps, warmup, has_decode, has_prefill):
         one(evs[i])
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    dec = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
-    pre = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    dec = _stats([e[0].elapsed_time(e[1]) for e in evs])
+    pre = _stats([e[1].elapsed_time(e[2]) for e in evs])
     return (t1 - t0) * 1e3 / steps, dec, pre
 
 
@@ -108,23 +119,49 @@ def make_call(pkg, b):
                      sum_decode_kv_len=int(sum(b.meta["kv_lens"][:dec_end])))
 
 
-def run_rpa_config(pkg, wl, b, steps, warmup):
+def run_rpa_config(pkg, wl, b, steps, warmup, keep_call=False):
     dec_end, n = int(b.distribution[0]), int(b.distribution[2])
     call = make_call(pkg, b)
-    ms, dec_ms, pre_ms = time_partitions(call, steps, warmup, dec_end > 0, n > dec_end)
+    ms, dec, pre = time_partitions(call, steps, warmup, dec_end > 0, n > dec_end)
     res = {"workload": b.name, "ms_per_step": ms}
     if dec_end > 0:
         nbytes = wl.decode_bytes(b, 0, dec_end)
-        res.update(decode_ms=dec_ms, decode_bytes=nbytes, decode_gbps=nbytes / (dec_ms * 1e-3) / 1e9)
+        res.update(decode_ms=dec["mean"], decode_ms_median=dec["median"], decode_ms_min=dec["min"], decode_bytes=nbytes,
+                   decode_gbps=nbytes / (dec["mean"] * 1e-3) / 1e9)
     if n > dec_end:
         flops = wl.prefill_flops(b, dec_end, n)
-        res.update(prefill_ms=pre_ms, prefill_flops=flops, prefill_tflops=flops / (pre_ms * 1e-3) / 1e12)
-    return res
+        res.update(prefill_ms=pre["mean"], prefill_ms_median=pre["median"], prefill_ms_min=pre["min"],
+                   prefill_flops=flops, prefill_tflops=flops / (pre["mean"] * 1e-3) / 1e12)
+    return (res, call) if keep_call else res
+
+
+def parity_sample(wl, b, call):
+    """A few rows of the output the timed steps left behind against the CPU oracle: the first, the
+    longest and the last decode row and the last 128 rows of the last chunk, re-run by the oracle on
+    a compact copy of their pages.  Outside the timed region."""
+    import numpy as np
+    import torch
+
+    from oracle.ref_rpa import ref_ragged_paged_attention_fused
+
+    dec_end, n = int(b.distribution[0]), int(b.distribution[2])
+    kv = np.asarray(b.meta["kv_lens"])
+    seqs = sorted({0, int(np.argmax(kv[:dec_end])), dec_end - 1}) if dec_end > 0 else []
+    if n > dec_end:
+        seqs.append(n - 1)
+    sample = wl.sub_batch(b, seqs, last_rows=128)
+    want = ref_ragged_paged_attention_fused(sample.q, sample.kv_cache, sample.kv_lens, sample.padded_page_table(),
+                                            sample.cu_q_lens, [len(seqs)], sm_scale=sample.sm_scale,
+                                            sliding_window=sample.sliding_window, soft_cap=sample.soft_cap,
+                                            k_scale=sample.k_scale, v_scale=sample.v_scale).float()
+    torch.cuda.synchronize()
+    got = call.out[torch.tensor(sample.meta["rows"], device=call.out.device)].float().cpu()
+    rel = ((got - want).norm(dim=-1) / want.norm(dim=-1).clamp_min(1e-30)).max()
+    return {"sequences": seqs, "rows": int(got.shape[0]), "max_abs_err": float((got - want).abs().max()),
+            "max_row_rel_err": float(rel), "tolerance": "rtol = atol = 2e-2 (5e-2 fp8 KV), row-relative 1e-2 (3e-2)"}
 
 
 def run_mla_config(pkg, wl, b, steps, warmup):
-    import ctypes
-
     import torch
 
     n = int(b.distribution[2])
@@ -146,10 +183,12 @@ def run_mla_config(pkg, wl, b, steps, warmup):
         e[1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    st = _stats([e[0].elapsed_time(e[1]) for e in evs])
+    ms = st["mean"]
     nbytes, flops = wl.mla_decode_bytes(b), wl.mla_decode_flops(b)
-    return {"workload": b.name, "ms_per_step": (t1 - t0) * 1e3 / steps, "decode_ms": ms, "decode_bytes": nbytes,
-            "decode_gbps": nbytes / (ms * 1e-3) / 1e9, "tflops": flops / (ms * 1e-3) / 1e12}
+    return {"workload": b.name, "ms_per_step": (t1 - t0) * 1e3 / steps, "decode_ms": ms, "decode_ms_median": st["median"],
+            "decode_ms_min": st["min"], "decode_bytes": nbytes, "decode_gbps": nbytes / (ms * 1e-3) / 1e9,
+            "tflops": flops / (ms * 1e-3) / 1e12}
 
 
 def cpu_baseline(wl, budget_s=15.0):
@@ -187,10 +226,11 @@ def cpu_baseline(wl, budget_s=15.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5"])
-    ap.add_argument("--all", action="store_true", help="also time the other configurations")
+    ap.add_argument("--all", action="store_true", help="(default) also time the other configurations")
+    ap.add_argument("--main-only", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy (10 launches): the known-size kernel "
@@ -225,30 +265,42 @@ def main():
                 "c4": lambda: wl.config_c4(dev), "c4swa": lambda: wl.config_c4(dev, window=True),
                 "c5": lambda: wl.config_c5(dev)}[name]()
 
-    def run(name):
+    def run(name, keep=False):
         b = build(name)
-        r = run_mla_config(pkg, wl, b, args.steps, args.warmup) if name == "c5" else \
-            run_rpa_config(pkg, wl, b, args.steps, args.warmup)
+        if name == "c5":
+            r = run_mla_config(pkg, wl, b, args.steps, args.warmup)
+        elif keep:
+            r, call = run_rpa_config(pkg, wl, b, args.steps, args.warmup, keep_call=True)
+            r = (r, parity_sample(wl, b, call))
+            del call
+        else:
+            r = run_rpa_config(pkg, wl, b, args.steps, args.warmup)
         del b
         torch.cuda.empty_cache()
         return r
 
-    main_res = run(args.config)
+    def decode_roofline(name, res):
+        kernel = DECODE_KERNEL[name]
+        return {"kernel": kernel + (" + combine" if name != "c1" else ""), "bound": "hbm",
+                "achieved": res["decode_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": res["decode_gbps"] / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get((name, kernel)),
+                "avg_launch_ms": res["decode_ms"], "median_launch_ms": res["decode_ms_median"],
+                "min_launch_ms": res["decode_ms_min"], "bytes_per_launch": res["decode_bytes"]}
+
+    if args.config == "c5":
+        main_res, sample = run(args.config), None
+    else:
+        main_res, sample = run(args.config, keep=True)
     dec_gbps = main_res.get("decode_gbps")
     pre_tflops = main_res.get("prefill_tflops")
     # dominant kernel of the workload (largest average launch time inside the timed region)
-    dec_kernel = DECODE_KERNEL[args.config]
-    roofline_decode = None
-    if dec_gbps is not None:
-        roofline_decode = {"kernel": dec_kernel + (" + combine" if args.config != "c1" else ""), "bound": "hbm",
-                           "achieved": dec_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": dec_gbps / HBM_PEAK_GBPS,
-                           "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dec_kernel)),
-                           "avg_launch_ms": main_res["decode_ms"], "bytes_per_launch": main_res["decode_bytes"]}
+    roofline_decode = decode_roofline(args.config, main_res) if dec_gbps is not None else None
     if pre_tflops is not None and main_res.get("prefill_ms", 0) >= main_res.get("decode_ms", 0):
-        roofline = {"kernel": "rpa_prefill_async_kernel", "bound": "mfma", "achieved": pre_tflops,
+        roofline = {"kernel": PREFILL_KERNEL, "bound": "mfma", "achieved": pre_tflops,
                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": pre_tflops / MFMA_BF16_PEAK_TFLOPS,
-                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, "rpa_prefill_async_kernel")),
-                    "avg_launch_ms": main_res["prefill_ms"], "flops_per_launch": main_res["prefill_flops"]}
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, PREFILL_KERNEL)),
+                    "avg_launch_ms": main_res["prefill_ms"], "median_launch_ms": main_res["prefill_ms_median"],
+                    "min_launch_ms": main_res["prefill_ms_min"], "flops_per_launch": main_res["prefill_flops"]}
     else:
         roofline = roofline_decode
     line = {
@@ -265,9 +317,24 @@ def main():
         "partitions": main_res,
         "roofline": roofline,
         "roofline_decode": roofline_decode,
+        "parity_sample": sample,
     }
-    if args.all:
-        line["other_configs"] = {n: run(n) for n in ("c1", "c2", "c3", "c4", "c4swa", "c5") if n != args.config}
+    if not args.main_only:
+        others = {}
+        for name in ("c1", "c2", "c3", "c4", "c4swa", "c5"):
+            if name == args.config:
+                continue
+            r = run(name)
+            r["roofline"] = decode_roofline(name, r)
+            if name == "c5":
+                r["roofline"]["mfma_frac"] = r["tflops"] / MFMA_BF16_PEAK_TFLOPS
+            if "prefill_tflops" in r:
+                r["roofline_prefill"] = {"kernel": PREFILL_KERNEL, "bound": "mfma", "achieved": r["prefill_tflops"],
+                                         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                         "frac": r["prefill_tflops"] / MFMA_BF16_PEAK_TFLOPS,
+                                         "avg_launch_ms": r["prefill_ms"], "flops_per_launch": r["prefill_flops"]}
+            others[name] = r
+        line["other_configs"] = others
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(line))
