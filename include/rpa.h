@@ -171,6 +171,12 @@ typedef struct RpaMlaParams {
   float soft_cap;             /* 0 => off */
   float mask_value;           /* 0 => default */
   int64_t sum_kv_len;         /* sum of kv_lens (host-side, balances the split plan); 0 => unknown */
+  /* Scalar scales of kernels/mla/v2/kernel.py:1354-1356 (used at :372-375, :408-409; oracle
+   * kernels/mla/v1/ref.py:223-226, 241-242): logits are multiplied by k_scale and q_scale next to
+   * sm_scale, the output by v_scale.  0 => off. */
+  float q_scale;
+  float k_scale;
+  float v_scale;
 } RpaMlaParams;
 
 /* Library version (RPA_VERSION of the build). */

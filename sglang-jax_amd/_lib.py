@@ -132,6 +132,9 @@ class RpaMlaParams(ctypes.Structure):
         ("soft_cap", ctypes.c_float),
         ("mask_value", ctypes.c_float),
         ("sum_kv_len", ctypes.c_int64),
+        ("q_scale", ctypes.c_float),
+        ("k_scale", ctypes.c_float),
+        ("v_scale", ctypes.c_float),
     ]
 
 

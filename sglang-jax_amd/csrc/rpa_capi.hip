@@ -690,7 +690,10 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   a.pt.cu_kv_lens = p->cu_kv_lens;
   a.pt.pages_per_seq = p->pages_per_seq;
   a.pt.page_size = p->page_size;
-  a.sm = softmax_opts(p->sm_scale, p->soft_cap, p->mask_value, p->sliding_window);
+  // the scalar scales of the logits fold into sm_scale (they multiply the dot product before the soft cap)
+  const float logit_scale = p->sm_scale * (p->k_scale > 0.f ? p->k_scale : 1.0f) * (p->q_scale > 0.f ? p->q_scale : 1.0f);
+  a.sm = softmax_opts(logit_scale, p->soft_cap, p->mask_value, p->sliding_window);
+  a.out_scale = p->v_scale > 0.f ? p->v_scale : 1.0f;
   a.num_rows = (int32_t)rows;
   a.num_seqs = p->num_seqs;
   a.rows_are_tokens = token_rows ? 1 : 0;

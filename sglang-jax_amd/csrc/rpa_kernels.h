@@ -132,6 +132,7 @@ struct MlaDecodeArgs {
   int32_t forced_tiles_per_wg;
   int32_t piece_pad;  // balanced plan: what starting one more (row, head group) costs a workgroup, in tiles
   int32_t* cu_tiles;  // [num_rows + 1] prefix sum of tiles, written by the kernel
+  float out_scale;    // finished rows are multiplied by it (v_scale; 1 when off)
 };
 
 struct MlaWriteArgs {

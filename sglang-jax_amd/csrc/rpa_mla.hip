@@ -336,7 +336,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   const int head = head0 + c;
   if (!wave_on || head >= a.Hq) return;
   if (dest.final_rows) {
-    const float inv = 1.0f / l;
+    const float inv = a.out_scale / l;
     uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 512 + g * 4;
 #pragma unroll
     for (int j = 0; j < 32; ++j) {
@@ -545,7 +545,7 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const Mla
     den += a.ws_ml[slot * 2 + 1] * w;
     o += *reinterpret_cast<const f32x4_t*>(a.ws_o + slot * 512 + d) * w;
   }
-  const float inv = 1.0f / den;
+  const float inv = a.out_scale / den;
   const int tq = a.pt.cu_q_lens[seq];
   u32x2_t w = {pack_bf16x2(o[0] * inv, o[1] * inv), pack_bf16x2(o[2] * inv, o[3] * inv)};
   *reinterpret_cast<u32x2_t*>(a.out + ((int64_t)tq * a.Hq + head) * 512 + d) = w;
@@ -573,7 +573,7 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_kernel(const MlaDecodeArg
     den += a.ws_ml[slot * 2 + 1] * w;
     o += *reinterpret_cast<const f32x4_t*>(a.ws_o + slot * 512 + d) * w;
   }
-  const float inv = 1.0f / den;
+  const float inv = a.out_scale / den;
   const int tq = mr.tq;
   u32x2_t w = {pack_bf16x2(o[0] * inv, o[1] * inv), pack_bf16x2(o[2] * inv, o[3] * inv)};
   *reinterpret_cast<u32x2_t*>(a.out + ((int64_t)tq * a.Hq + head) * 512 + d) = w;

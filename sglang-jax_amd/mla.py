@@ -69,8 +69,9 @@ def mla_ragged_paged_attention(
         raise ValueError(f"soft_cap={soft_cap} must not be 0.0.")
     if (new_kv_c is None) != (new_k_pe is None):
         raise ValueError("new_kv_c and new_k_pe must be given together")
-    if q_scale is not None or k_scale is not None or v_scale is not None:
-        raise NotImplementedError("q_scale/k_scale/v_scale are not built for MLA")
+    for name, val in (("q_scale", q_scale), ("k_scale", k_scale), ("v_scale", v_scale)):
+        if val is not None and not val > 0:
+            raise ValueError(f"{name}={val} must be positive.")
     dist = np.asarray(distribution.cpu() if isinstance(distribution, torch.Tensor) else distribution)
     i, j, k = (int(x) for x in dist)
     if not (0 <= i <= j <= k):
@@ -122,6 +123,10 @@ def mla_ragged_paged_attention(
     p.sm_scale = float(sm_scale)
     p.soft_cap = float(soft_cap) if soft_cap else 0.0
     p.mask_value = float(mask_value) if mask_value is not None else DEFAULT_MASK_VALUE
+    # scalar scales (mla_v2:372-375, 408-409): 0 in the C struct means "off"
+    p.q_scale = float(q_scale) if q_scale is not None else 0.0
+    p.k_scale = float(k_scale) if k_scale is not None else 0.0
+    p.v_scale = float(v_scale) if v_scale is not None else 0.0
     lib = _lib.load()
     stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     if new_kv_c is not None:

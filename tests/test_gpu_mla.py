@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from parity import assert_parity
+from parity import assert_parity, row_rel_error
 
 from oracle.ref_mla import ref_mla_ragged_paged_attention
 
@@ -23,11 +23,11 @@ def say(*a):
     sys.stdout.flush()
 
 
-def oracle(b):
+def oracle(b, **kw):
     n = int(b.distribution[2])
     out, _ = ref_mla_ragged_paged_attention(
         b.ql_nope, b.q_pe, None, None, b.cache_kv, b.kv_lens, b.padded_page_indices(), b.cu_q_lens, [n, n, n],
-        sm_scale=b.sm_scale, sliding_window=b.sliding_window, soft_cap=b.soft_cap)
+        sm_scale=b.sm_scale, sliding_window=b.sliding_window, soft_cap=b.soft_cap, **kw)
     return out
 
 
@@ -339,3 +339,35 @@ def test_mla_peaked_long_rows_against_oracle(pkg, wl, gpu, case):
         for ns in (1, 3):
             say(f"  num_splits {ns}")
             assert_parity(run_gpu(pkg, b, gpu, num_splits=ns)[:T].float(), want.float(), **TOL)
+
+
+@pytest.mark.parametrize("cap", [None, 30.0])
+def test_mla_scalar_scales(pkg, wl, gpu, cap):
+    """q_scale, k_scale and v_scale of kernels/mla/v2/kernel.py:1354-1356: the logits are multiplied by
+    k_scale and q_scale (before the soft cap), the output by v_scale; decode rows whole and split, and
+    chunks (token rows)."""
+    q_lens = [1, 1, 1, 9, 40]
+    kv_lens = [700, 33, 5000, 300, 40]
+    b = wl.make_mla_batch("mla_scales", q_lens, kv_lens, num_q_heads=32, lkv_dim=512, rope_dim=64, page_size=32,
+                          seed=8301, soft_cap=cap)
+    wl.plant_mla_needles(b, seed=2, logit=9.0)
+    T = sum(q_lens)
+    scales = dict(q_scale=0.61, k_scale=1.7, v_scale=0.37)
+    say(f"mla scales cap={cap} {scales}")
+    want = oracle(b, **scales)
+    got = run_gpu(pkg, b, gpu, **scales)
+    assert_parity(got[:T].float(), want.float(), **TOL)
+    # each scale alone does what the formula says: v_scale scales the rows, q_scale * k_scale acts like sm_scale
+    plain = run_gpu(pkg, b, gpu)
+    half = run_gpu(pkg, b, gpu, v_scale=0.5)
+    assert float(row_rel_error(half[:T].float(), 0.5 * plain[:T].float()).max()) <= 1e-2
+    folded = run_gpu(pkg, b, gpu, q_scale=0.61 * 1.7)
+    both = run_gpu(pkg, b, gpu, q_scale=0.61, k_scale=1.7)
+    assert float(row_rel_error(folded[:T].float(), both[:T].float()).max()) <= 1e-2
+    # decode rows only, split
+    d = wl.make_mla_batch("mla_scales_dec", [1, 1], [6000, 900], num_q_heads=128, lkv_dim=512, rope_dim=64, page_size=64,
+                          seed=8302)
+    wl.plant_mla_needles(d, seed=3)
+    want = oracle(d, **scales)
+    for ns in (0, 1, 4):
+        assert_parity(run_gpu(pkg, d, gpu, num_splits=ns, **scales)[:2].float(), want.float(), **TOL)
