@@ -105,13 +105,20 @@ def time_partitions(call, steps, warmup, has_decode, has_prefill):
     return (t1 - t0) * 1e3 / steps, dec, pre
 
 
-def make_call(pkg, b):
+def make_call(pkg, b, static_shapes=False):
     import numpy as np
 
     m = importlib.import_module("sglang_jax_amd.ragged_paged_attention")
     n = int(b.distribution[2])
     q_lens = b.q_lens()[:n]
     dec_end = int(b.distribution[0])
+    if static_shapes:
+        # nothing but static shapes on the host: the kernels read the composition from the device
+        return m.RpaCall(b.q, b.kv_cache, None, b.kv_lens, b.page_indices, b.cu_q_lens, b.cu_kv_lens,
+                         num_seqs=int(b.kv_lens.shape[0]), decode_end=0, sm_scale=b.sm_scale,
+                         sliding_window=b.sliding_window, soft_cap=b.soft_cap, k_scale=b.k_scale, v_scale=b.v_scale,
+                         max_q_len=2048 if n > dec_end else 0,  # the workload's chunk size: a static bound, like chunk_prefill_size
+                         distribution_d=b.distribution)
     return m.RpaCall(b.q, b.kv_cache, None, b.kv_lens, b.page_indices, b.cu_q_lens, b.cu_kv_lens, num_seqs=n,
                      decode_end=dec_end, sm_scale=b.sm_scale, sliding_window=b.sliding_window, soft_cap=b.soft_cap,
                      k_scale=b.k_scale, v_scale=b.v_scale, max_kv_len=int(max(b.meta["kv_lens"])),
@@ -119,9 +126,9 @@ def make_call(pkg, b):
                      sum_decode_kv_len=int(sum(b.meta["kv_lens"][:dec_end])))
 
 
-def run_rpa_config(pkg, wl, b, steps, warmup, keep_call=False):
+def run_rpa_config(pkg, wl, b, steps, warmup, keep_call=False, static_shapes=False):
     dec_end, n = int(b.distribution[0]), int(b.distribution[2])
-    call = make_call(pkg, b)
+    call = make_call(pkg, b, static_shapes)
     ms, dec, pre = time_partitions(call, steps, warmup, dec_end > 0, n > dec_end)
     res = {"workload": b.name, "ms_per_step": ms}
     if dec_end > 0:
@@ -231,6 +238,9 @@ def main():
     ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5"])
     ap.add_argument("--all", action="store_true", help="(default) also time the other configurations")
     ap.add_argument("--main-only", action="store_true", help="skip the other configurations")
+    ap.add_argument("--static-shapes", action="store_true",
+                    help="run the main configuration with the batch composition read on the device (grids sized "
+                         "from static shapes only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy (10 launches): the known-size kernel "
@@ -270,7 +280,8 @@ def main():
         if name == "c5":
             r = run_mla_config(pkg, wl, b, args.steps, args.warmup)
         elif keep:
-            r, call = run_rpa_config(pkg, wl, b, args.steps, args.warmup, keep_call=True)
+            r, call = run_rpa_config(pkg, wl, b, args.steps, args.warmup, keep_call=True,
+                                     static_shapes=args.static_shapes)
             r = (r, parity_sample(wl, b, call))
             del call
         else:
@@ -310,7 +321,8 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.config not in ("c4", "c4swa") else "bf16 (fp8-e4m3 KV)", "data": "synthetic",
-        "config": {"workload": main_res["workload"], "value_is": "decode partition (split-KV + combine) algorithmic bytes / time"},
+        "config": {"workload": main_res["workload"], "value_is": "decode partition (split-KV + combine) algorithmic bytes / time",
+                   "call_mode": "static shapes, composition read on the device" if args.static_shapes else "host integers"},
         "decode_frac_of_hbm_peak": None if dec_gbps is None else dec_gbps / HBM_PEAK_GBPS,
         "prefill_tflops": pre_tflops,
         "prefill_frac_of_mfma_peak": None if pre_tflops is None else pre_tflops / MFMA_BF16_PEAK_TFLOPS,

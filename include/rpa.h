@@ -134,6 +134,14 @@ typedef struct RpaParams {
   float q_scale;                /* > 0: queries are divided by it and rounded to the cache's element type
                                    (fp8 saturating at +-448) before the first product, the logits multiplied
                                    by it (kernel :463-478); 0 => off */
+  /* ---- static-shape mode: the batch composition read on the device ----
+   * Device i32[3] (decode_end, prefill_end, num_seqs) as ragged_paged_attention takes it
+   * (ragged_paged_attention_v3.py:1676, dispatch :2060-2090), or NULL.  When given, the host fields
+   * decode_end and sum_decode_kv_len are ignored and num_seqs is only the static bound S (the length of
+   * kv_lens): grids are sized from T, S and the page-table bound, every workgroup reads the
+   * composition itself and the ones with nothing to do leave at once, so one compiled call serves
+   * every batch of a bucket and nothing is read back to the host.  head_dim 128 only. */
+  const int32_t* distribution;
 } RpaParams;
 
 /*
@@ -177,6 +185,10 @@ typedef struct RpaMlaParams {
   float q_scale;
   float k_scale;
   float v_scale;
+  /* Static-shape mode (see RpaParams.distribution): device i32[3] or NULL.  When given, num_seqs is
+   * the static bound and rpa_mla_attention / rpa_mla_kv_write read distribution[2] on the device;
+   * rpa_mla_decode (decode rows known on the host) does not take it. */
+  const int32_t* distribution;
 } RpaMlaParams;
 
 /* Library version (RPA_VERSION of the build). */

@@ -96,6 +96,7 @@ class RpaParams(ctypes.Structure):
         ("mask_rows_page_aligned", ctypes.c_int32),
         ("softmax_dtype", ctypes.c_int32),
         ("q_scale", ctypes.c_float),
+        ("distribution", ctypes.c_void_p),
     ]
 
 
@@ -135,6 +136,7 @@ class RpaMlaParams(ctypes.Structure):
         ("q_scale", ctypes.c_float),
         ("k_scale", ctypes.c_float),
         ("v_scale", ctypes.c_float),
+        ("distribution", ctypes.c_void_p),
     ]
 
 

@@ -360,7 +360,9 @@ int rpa_validate(const RpaParams* p) {
     return fail(RPA_EINVAL_NULL, "split layout needs v_pages");
   if (p->sliding_window < 0) return fail(RPA_EINVAL_WINDOW, "sliding_window=%d must be positive", p->sliding_window);
   if (std::isnan(p->soft_cap)) return fail(RPA_EINVAL_SOFTCAP, "soft_cap must not be NaN");
-  if (p->decode_end < 0 || p->decode_end > p->num_seqs)
+  if (p->distribution && p->head_dim != 128)
+    return fail(RPA_EUNSUPPORTED, "a device-side distribution is built for head_dim 128 only, got %d", p->head_dim);
+  if (!p->distribution && (p->decode_end < 0 || p->decode_end > p->num_seqs))
     return fail(RPA_EINVAL_DISTRIBUTION, "distribution must satisfy 0 <= decode_end=%d <= num_seqs=%d",
                 p->decode_end, p->num_seqs);
   if (p->num_seqs > 0) {
@@ -437,8 +439,22 @@ int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t*
   return RPA_OK;
 }
 
-size_t rpa_workspace_bytes(const RpaParams* p) {
-  if (!p || p->decode_end <= 0) return 0;
+// Static-shape mode: every sequence may be a decode row, nothing is known about their lengths
+// beyond the page-table bound.
+static RpaParams planning_view(const RpaParams* p) {
+  RpaParams q = *p;
+  if (p->distribution) {
+    q.decode_end = p->num_seqs;
+    q.sum_decode_kv_len = 0;
+  }
+  return q;
+}
+
+size_t rpa_workspace_bytes(const RpaParams* p_in) {
+  if (!p_in) return 0;
+  const RpaParams pv = planning_view(p_in);
+  const RpaParams* p = &pv;
+  if (p->decode_end <= 0) return 0;
   if (p->head_dim == 256) return rows256_workspace(p);
   const SplitPlan sp = decode_plan(p);
   if (use_balanced(p, sp))
@@ -468,9 +484,11 @@ int rpa_gather_pages(const RpaParams* p, int32_t seq, void* k_out, void* v_out, 
   return check_hip(rpa::launch_gather(a, static_cast<hipStream_t>(stream)), "rpa_gather_pages");
 }
 
-int rpa_decode(const RpaParams* p, void* stream) {
-  int rc = rpa_validate(p);
+int rpa_decode(const RpaParams* p_in, void* stream) {
+  int rc = rpa_validate(p_in);
   if (rc != RPA_OK) return rc;
+  const RpaParams pv = planning_view(p_in);
+  const RpaParams* p = &pv;
   if (p->decode_end <= 0) return RPA_OK;
   if (p->mask_mode == RPA_MASK_CUSTOM) return RPA_OK;  // masked rows all go through the prefill kernel
   if (p->head_dim == 256) return rows256(p, 0, p->decode_end, stream);
@@ -495,6 +513,7 @@ int rpa_decode(const RpaParams* p, void* stream) {
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
   a.cu_blocks = nullptr;
+  a.dist = p->distribution;
   a.balanced = use_balanced(p, sp) ? 1 : 0;
   a.num_wgs = decode_wgs(p);
   a.waves_per_wg = decode_waves_per_wg(p);
@@ -525,7 +544,9 @@ int rpa_decode(const RpaParams* p, void* stream) {
 int rpa_prefill(const RpaParams* p, void* stream) {
   int rc = rpa_validate(p);
   if (rc != RPA_OK) return rc;
-  if (p->num_seqs <= p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) return RPA_OK;
+  const bool dyn = p->distribution != nullptr;
+  if (!dyn && p->num_seqs <= p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) return RPA_OK;
+  if (dyn && p->num_seqs <= 0) return RPA_OK;
   // 256-wide heads: bf16 caches take the flash kernel (two 128-dim halves per row, one workgroup
   // per CU); fp8 caches and rows the caller masks itself stay on the row kernel
   if (p->head_dim == 256 && (p->kv_dtype == RPA_KV_FP8_E4M3 || env_int("RPA_PREFILL_ROWS256", 0) != 0))
@@ -539,8 +560,9 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   a.sm = softmax_opts(p);
   a.k_scale = p->k_scale;
   a.v_scale = p->v_scale;
-  a.seq_begin = (p->mask_mode == RPA_MASK_CUSTOM) ? 0 : p->decode_end;
+  a.seq_begin = (p->mask_mode == RPA_MASK_CUSTOM || dyn) ? 0 : p->decode_end;  // dyn: the kernels read it
   a.seq_end = p->num_seqs;
+  a.dist = p->distribution;
   a.Hq = p->num_q_heads;
   a.Hkv = p->num_kv_heads;
   a.G = p->num_q_heads / p->num_kv_heads;
@@ -591,6 +613,7 @@ int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void*
   a.keys = static_cast<const char*>(keys);
   a.values = static_cast<const char*>(values);
   a.num_seqs = p->num_seqs;
+  a.dist = p->distribution;
   a.Hkv = p->num_kv_heads;
   a.head_bytes = p->head_dim * esize_of(p->kv_dtype);
   a.num_tokens = p->num_tokens;
@@ -694,6 +717,9 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   const float logit_scale = p->sm_scale * (p->k_scale > 0.f ? p->k_scale : 1.0f) * (p->q_scale > 0.f ? p->q_scale : 1.0f);
   a.sm = softmax_opts(logit_scale, p->soft_cap, p->mask_value, p->sliding_window);
   a.out_scale = p->v_scale > 0.f ? p->v_scale : 1.0f;
+  a.dist = p->distribution;
+  if (p->distribution && !token_rows)
+    return fail(RPA_EUNSUPPORTED, "rpa_mla_decode takes the batch composition from the host: use rpa_mla_attention");
   a.num_rows = (int32_t)rows;
   a.num_seqs = p->num_seqs;
   a.rows_are_tokens = token_rows ? 1 : 0;
@@ -754,6 +780,7 @@ int rpa_mla_kv_write(const RpaMlaParams* p, const void* new_kv_c, const void* ne
   a.new_k_pe = static_cast<const uint16_t*>(new_k_pe);
   a.num_tokens = p->num_tokens;
   a.num_seqs = p->num_seqs;
+  a.dist = p->distribution;
   a.row_stride = p->row_stride;
   a.rope_offset = p->rope_offset;
   return check_hip(rpa::launch_mla_kv_write(a, static_cast<hipStream_t>(stream)), "rpa_mla_kv_write");

@@ -426,7 +426,10 @@ __device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int
 
 // ---- fixed split plan: grid = (max_splits, decode rows, head groups * row groups); block = NW waves
 template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
-__global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const DecodeArgs a_in) {
+  DecodeArgs a = a_in;  // static-shape mode: the number of decode rows comes from the device
+  if (a.dist) a.num_rows = min(a.num_rows, scalar_load_i32(a.dist));
+  if ((int)blockIdx.y >= a.num_rows) return;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
@@ -593,7 +596,10 @@ struct Piece {
 // and neither does a block: under load a small dependent load waits behind megabytes of queued
 // KV traffic (10 us and more), so there are none after the first block.
 template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
-__global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const DecodeArgs a_in) {
+  DecodeArgs a = a_in;  // static-shape mode: the number of decode rows comes from the device
+  if (a.dist) a.num_rows = min(a.num_rows, scalar_load_i32(a.dist));
+  if (a.num_rows <= 0) return;
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
@@ -947,7 +953,10 @@ __device__ __forceinline__ void merge_rows(const DecodeArgs& a, int seq, int hea
 }
 
 // Merge the partial rows of the balanced plan.  grid = (Hq, decode rows); block = one wave.
-__global__ __launch_bounds__(64) void rpa_combine_balanced_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(64) void rpa_combine_balanced_kernel(const DecodeArgs a_in) {
+  DecodeArgs a = a_in;  // static-shape mode: the number of decode rows comes from the device
+  if (a.dist) a.num_rows = min(a.num_rows, scalar_load_i32(a.dist));
+  if ((int)blockIdx.y >= a.num_rows) return;
   const int head = blockIdx.x;
   const int seq = blockIdx.y;
   const int lane = threadIdx.x;
@@ -1169,7 +1178,10 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
 // with shuffles, then the weights are broadcast lane by lane while the partial
 // rows stream in with independent loads.
 template <int HD>
-__global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a_in) {
+  DecodeArgs a = a_in;  // static-shape mode: the number of decode rows comes from the device
+  if (a.dist) a.num_rows = min(a.num_rows, scalar_load_i32(a.dist));
+  if ((int)blockIdx.y >= a.num_rows) return;
   const int head = blockIdx.x;
   const int seq = blockIdx.y;
   const int lane = threadIdx.x;
@@ -1205,7 +1217,9 @@ __global__ __launch_bounds__(256) void rpa_gather_kernel(const GatherArgs a) {
 // New-token cache write: token j of sequence i lands at position kv_len-q_len+j.
 // grid.x covers (token, 16-byte piece); the sequence of a token is found by
 // binary search in cu_q_lens.
-__global__ __launch_bounds__(256) void rpa_kv_write_kernel(const KvWriteArgs a) {
+__global__ __launch_bounds__(256) void rpa_kv_write_kernel(const KvWriteArgs a_in) {
+  KvWriteArgs a = a_in;
+  if (a.dist) a.num_seqs = min(a.num_seqs, a.dist[2]);
   const int pieces = a.Hkv * a.head_bytes / 16;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int total_tokens = min(a.num_tokens, a.pt.cu_q_lens[a.num_seqs]);

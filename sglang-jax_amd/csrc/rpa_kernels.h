@@ -66,6 +66,9 @@ struct DecodeArgs {
   int32_t min_blocks_per_wave;
   int32_t forced_blocks_per_wave;  // > 0: tests pin the partition
   int32_t* cu_blocks;              // [num_rows + 1] prefix sum of 32-token blocks, written by the kernel
+  // device i32[3] (decode_end, prefill_end, num_seqs) or nullptr: when given, num_rows is only a bound
+  // and the rows to process are [0, min(num_rows, dist[0]))
+  const int32_t* dist;
 };
 
 struct PrefillArgs {
@@ -82,6 +85,9 @@ struct PrefillArgs {
   int32_t max_kv_len;  // host bound on kv_len of these sequences, 0 = unknown
   int32_t fp8;
   int32_t head_dim;  // 128, or 256 (bf16 cache only)
+  // device i32[3] or nullptr: when given, seq_end is only a bound and the sequences to process are
+  // [dist[0], min(seq_end, dist[2])) (custom-mask calls: [0, ...))
+  const int32_t* dist;
 };
 
 struct GatherArgs {
@@ -105,6 +111,7 @@ struct KvWriteArgs {
   int32_t Hkv;
   int32_t head_bytes;
   int32_t num_tokens;
+  const int32_t* dist;  // device i32[3] or nullptr: when given, num_seqs is only a bound on dist[2]
 };
 
 struct MlaDecodeArgs {
@@ -133,6 +140,7 @@ struct MlaDecodeArgs {
   int32_t piece_pad;  // balanced plan: what starting one more (row, head group) costs a workgroup, in tiles
   int32_t* cu_tiles;  // [num_rows + 1] prefix sum of tiles, written by the kernel
   float out_scale;    // finished rows are multiplied by it (v_scale; 1 when off)
+  const int32_t* dist;  // device i32[3] or nullptr: when given, num_seqs is only a bound on dist[2]
 };
 
 struct MlaWriteArgs {
@@ -144,6 +152,7 @@ struct MlaWriteArgs {
   int32_t num_seqs;
   int32_t row_stride;
   int32_t rope_offset;
+  const int32_t* dist;  // device i32[3] or nullptr: when given, num_seqs is only a bound on dist[2]
 };
 
 hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream);

@@ -141,21 +141,24 @@ struct MlaRow {
 __device__ __forceinline__ MlaRow mla_row(const MlaDecodeArgs& a, int row) {
   MlaRow r;
   r.valid = true;
+  // static-shape mode: num_seqs is a bound, the number of sequences comes from the device
+  const int num_seqs = a.dist ? min(a.num_seqs, scalar_load_i32(a.dist + 2)) : a.num_seqs;
   if (a.rows_are_tokens) {
-    if (row >= scalar_load_i32(a.pt.cu_q_lens + a.num_seqs)) {
+    if (row >= scalar_load_i32(a.pt.cu_q_lens + num_seqs)) {
       r.valid = false;
       r.seq = r.kv_len = r.tq = 0;
       return r;
     }
-    r.seq = owner_of_token(a.pt.cu_q_lens, a.num_seqs, row);
+    r.seq = owner_of_token(a.pt.cu_q_lens, num_seqs, row);
     const int q0 = scalar_load_i32(a.pt.cu_q_lens + r.seq);
     const int q_len = scalar_load_i32(a.pt.cu_q_lens + r.seq + 1) - q0;
     r.kv_len = scalar_load_i32(a.pt.kv_lens + r.seq) - q_len + (row - q0) + 1;
     r.tq = row;
   } else {
     r.seq = row;
-    r.kv_len = a.pt.kv_lens[row];
+    r.kv_len = (row < num_seqs) ? a.pt.kv_lens[row] : 0;
     r.tq = a.pt.cu_q_lens[row];
+    r.valid = row < num_seqs;
   }
   return r;
 }
@@ -584,8 +587,9 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_kernel(const MlaDecodeArg
 // grid = tokens; block = 128 threads of which 72 move 16 bytes each.
 __global__ __launch_bounds__(128) void rpa_mla_kv_write_kernel(const MlaWriteArgs a) {
   const int tok = blockIdx.x;
-  if (tok >= scalar_load_i32(a.pt.cu_q_lens + a.num_seqs)) return;
-  const int seq = owner_of_token(a.pt.cu_q_lens, a.num_seqs, tok);
+  const int num_seqs = a.dist ? min(a.num_seqs, scalar_load_i32(a.dist + 2)) : a.num_seqs;
+  if (tok >= scalar_load_i32(a.pt.cu_q_lens + num_seqs)) return;
+  const int seq = owner_of_token(a.pt.cu_q_lens, num_seqs, tok);
   const int q0 = scalar_load_i32(a.pt.cu_q_lens + seq);
   const int q_len = scalar_load_i32(a.pt.cu_q_lens + seq + 1) - q0;
   const int pos = scalar_load_i32(a.pt.kv_lens + seq) - q_len + (tok - q0);

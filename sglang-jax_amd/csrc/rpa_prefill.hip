@@ -41,8 +41,13 @@ namespace {
 // HD = 256 doubles the rows in LDS (two 64 KiB slots), the Q^T operands and the accumulators: one
 // workgroup per CU, one wave per SIMD with up to 512 registers.
 template <bool UNIFORM, bool CAP, bool EXT, int HD = 128>
-__global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_kernel(const PrefillArgs a, int tiles, int nseq,
+__global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_kernel(const PrefillArgs a_in, int tiles, int nseq,
                                                                                   bool by_level) {
+  PrefillArgs a = a_in;  // static-shape mode: the sequences to process come from the device
+  if (a.dist) {
+    a.seq_begin = (a.sm.mask_mode == 1) ? 0 : scalar_load_i32(a.dist);
+    a.seq_end = min(a.seq_end, scalar_load_i32(a.dist + 2));
+  }
   using T = Tile<HD>;
   constexpr int kRowB = T::kRowB;
   constexpr int kTileB = T::kTileB;
@@ -312,7 +317,12 @@ __device__ __forceinline__ void tile_lstore(const Stage<FP8>& st, char* lds_k, c
 }
 
 template <bool FP8, bool UNIFORM, bool CAP, bool EXT>
-__global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const PrefillArgs a, int tiles, int nseq, bool by_level) {
+__global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const PrefillArgs a_in, int tiles, int nseq, bool by_level) {
+  PrefillArgs a = a_in;  // static-shape mode: the sequences to process come from the device
+  if (a.dist) {
+    a.seq_begin = (a.sm.mask_mode == 1) ? 0 : scalar_load_i32(a.dist);
+    a.seq_end = min(a.seq_end, scalar_load_i32(a.dist + 2));
+  }
   __shared__ __attribute__((aligned(16))) char lds_k_buf[2][kBN * kKPitch];
   __shared__ __attribute__((aligned(16))) char lds_v_buf[2][128 * kVPitch];
 

@@ -96,6 +96,7 @@ __device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int n
   w.hk = u - si * a.Hkv;
   w.head = w.hk * a.G + gi;
   w.seq = a.seq_begin + si;
+  if (w.seq >= a.seq_end) return w;  // the grid was sized for a bound on the number of sequences
   w.qg0 = a.pt.cu_q_lens[w.seq];
   w.q_len = a.pt.cu_q_lens[w.seq + 1] - w.qg0;
   w.kv_len = a.pt.kv_lens[w.seq];

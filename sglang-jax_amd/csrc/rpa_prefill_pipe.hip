@@ -264,8 +264,13 @@ __device__ __forceinline__ void pipe_loop(RowBlock (&b)[2], const Shared& sh, in
 }
 
 template <bool WIN, int NQ>
-__global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kernel(const PrefillArgs a, int tiles, int nseq,
+__global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kernel(const PrefillArgs a_in, int tiles, int nseq,
                                                                                  bool by_level, float row_sum_limit) {
+  PrefillArgs a = a_in;  // static-shape mode: the sequences to process come from the device
+  if (a.dist) {
+    a.seq_begin = (a.sm.mask_mode == 1) ? 0 : scalar_load_i32(a.dist);
+    a.seq_end = min(a.seq_end, scalar_load_i32(a.dist + 2));
+  }
   constexpr int BM = 128 * NQ;  // query rows per workgroup
   __shared__ __attribute__((aligned(1024))) char lds[4 * kTileB];
 

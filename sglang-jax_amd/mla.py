@@ -72,11 +72,21 @@ def mla_ragged_paged_attention(
     for name, val in (("q_scale", q_scale), ("k_scale", k_scale), ("v_scale", v_scale)):
         if val is not None and not val > 0:
             raise ValueError(f"{name}={val} must be positive.")
-    dist = np.asarray(distribution.cpu() if isinstance(distribution, torch.Tensor) else distribution)
-    i, j, k = (int(x) for x in dist)
-    if not (0 <= i <= j <= k):
-        raise ValueError(f"distribution must satisfy 0 <= i <= j <= k, got ({i}, {j}, {k})")
-    decode_only = i == j == k
+    # Static-shape mode: a distribution on the GPU is never read back; the kernels take the number of
+    # sequences from it and every query token runs as a row of its own (any batch composition).
+    static_shapes = isinstance(distribution, torch.Tensor) and distribution.is_cuda
+    if static_shapes:
+        if distribution.dtype != torch.int32 or tuple(distribution.shape) != (3,):
+            raise ValueError(f"Expected int32 distribution of shape (3,), got {distribution.dtype} {tuple(distribution.shape)}")
+        i = j = 0
+        k = int(kv_lens.shape[0])
+        decode_only = False
+    else:
+        dist = np.asarray(distribution.cpu() if isinstance(distribution, torch.Tensor) else distribution)
+        i, j, k = (int(x) for x in dist)
+        if not (0 <= i <= j <= k):
+            raise ValueError(f"distribution must satisfy 0 <= i <= j <= k, got ({i}, {j}, {k})")
+        decode_only = i == j == k
     device = ql_nope.device
     if cache_kv.dim() == 4:
         s = cache_kv.shape
@@ -127,6 +137,10 @@ def mla_ragged_paged_attention(
     p.q_scale = float(q_scale) if q_scale is not None else 0.0
     p.k_scale = float(k_scale) if k_scale is not None else 0.0
     p.v_scale = float(v_scale) if v_scale is not None else 0.0
+    dist_d = None
+    if static_shapes:
+        dist_d = distribution.contiguous()
+        p.distribution = dist_d.data_ptr()
     lib = _lib.load()
     stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     if new_kv_c is not None:

@@ -189,7 +189,7 @@ class RpaCall:
                  sm_scale, sliding_window=None, soft_cap=None, mask_value=DEFAULT_MASK_VALUE, k_scale=None,
                  v_scale=None, max_kv_len=0, max_q_len=0, num_splits=0, out=None, sum_decode_kv_len=0,
                  attention_sink=None, xai_temperature_len=None, causal=True, custom_mask=None,
-                 mask_aligned_to_cu_kv=False, softmax_dtype=None, q_scale=None):
+                 mask_aligned_to_cu_kv=False, softmax_dtype=None, q_scale=None, distribution_d=None):
         self.lib = _lib.load()
         self.device = queries.device
         fused = v_pages is None
@@ -217,6 +217,14 @@ class RpaCall:
         p.pages_per_seq = page_d.shape[1] if page_d.dim() == 2 else 0
         p.k_scale = self.ks.data_ptr() if self.ks is not None else None
         p.v_scale = self.vs.data_ptr() if self.vs is not None else None
+        # ---- static-shape mode: (decode_end, prefill_end, num_seqs) stays on the device (rpa_v3:1676);
+        # num_seqs is then the static bound and decode_end is not read
+        self.distribution_d = None
+        if distribution_d is not None:
+            if distribution_d.dtype != torch.int32 or tuple(distribution_d.shape) != (3,):
+                raise ValueError(f"Expected int32 distribution of shape (3,), got {distribution_d.dtype} {tuple(distribution_d.shape)}")
+            self.distribution_d = distribution_d.to(self.device).contiguous()
+            p.distribution = self.distribution_d.data_ptr()
         # ---- attention sink: scalar or one logit per query head (rpa_v3:185-193)
         self.sink = None
         if attention_sink is not None:
@@ -351,11 +359,19 @@ def ragged_paged_attention(
     ``max_kv_len``/``max_q_len`` are host values used only to size launch grids;
     ``host_kv_lens`` is an optional host copy of ``kv_lens`` (the split plan balances on its
     sum) for callers that pass ``kv_lens`` as a device tensor.
+
+    Static-shape mode: a ``distribution`` that lives on the GPU is never read back.  Grids are then
+    sized from the static shapes alone (tokens, ``kv_lens.shape[0]`` sequences, the page-table
+    bound) and the kernels read the batch composition themselves, as the jitted reference does
+    (rpa_v3:1676): one prepared call serves every batch of a bucket.
     """
     _require_gpu(queries, "queries")
     _require_gpu(kv_cache_fused, "kv_cache_fused")
     device = queries.device
-    if isinstance(distribution, torch.Tensor):
+    static_shapes = isinstance(distribution, torch.Tensor) and distribution.is_cuda
+    if static_shapes:
+        dist = np.array([0, 0, kv_lens.shape[0]], dtype=np.int32)  # bounds only; the device holds the values
+    elif isinstance(distribution, torch.Tensor):
         dist = distribution.cpu().numpy()
     elif isinstance(distribution, np.ndarray):
         dist = distribution
@@ -390,12 +406,16 @@ def ragged_paged_attention(
                    k_scale=k_scale, v_scale=v_scale,
                    max_kv_len=max_kv_len if max_kv_len is not None else _host_max(
                        host_kv_lens if host_kv_lens is not None else kv_lens),
-                   max_q_len=max_q_len if max_q_len is not None else 0, num_splits=num_splits,
+                   # the static chunk size bounds a chunk's length (rpa_v3:1691): it sizes the prefill grid
+                   max_q_len=max_q_len if max_q_len is not None else (chunk_prefill_size or 0), num_splits=num_splits,
                    sum_decode_kv_len=_host_decode_sum(host_kv_lens if host_kv_lens is not None else kv_lens, i),
                    attention_sink=attention_sink, xai_temperature_len=xai_temperature_len, causal=bool(causal),
                    custom_mask=custom_mask, mask_aligned_to_cu_kv=mask_aligned_to_cu_kv,
-                   softmax_dtype=softmax_dtype, q_scale=q_scale)
+                   softmax_dtype=softmax_dtype, q_scale=q_scale,
+                   distribution_d=distribution if static_shapes else None)
     if validate_values:
+        if static_shapes:
+            raise ValueError("validate_values reads the metadata back to the host: not available with a device-side distribution")
         dynamic_validate_inputs(call.params, kv_lens_d.cpu().numpy(), page_d.cpu().numpy(), cu_q_d.cpu().numpy(),
                                 cu_kv_d.cpu().numpy(), dist.astype(np.int32))
     if keys is not None:

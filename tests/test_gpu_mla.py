@@ -371,3 +371,33 @@ def test_mla_scalar_scales(pkg, wl, gpu, cap):
     want = oracle(d, **scales)
     for ns in (0, 1, 4):
         assert_parity(run_gpu(pkg, d, gpu, num_splits=ns, **scales)[:2].float(), want.float(), **TOL)
+
+
+def test_mla_device_side_distribution(pkg, wl, gpu):
+    """Static-shape mode: the number of sequences read on the device (a bucket padded with empty
+    sequences and spare tokens); same results as with host integers, new rows written first."""
+    q_lens = [1, 1, 1, 9, 40]
+    kv_lens = [700, 33, 2100, 300, 40]
+    b = wl.make_mla_batch("mla_static", q_lens, kv_lens, num_q_heads=32, lkv_dim=512, rope_dim=64, page_size=32, seed=8303)
+    wl.plant_mla_needles(b, seed=6, logit=9.0)
+    T, S = sum(q_lens), len(q_lens)
+    pad_s, pad_t = 11, 12
+    g = b.to(gpu)
+    kv_pad = torch.cat([g.kv_lens, torch.zeros(pad_s, dtype=torch.int32, device=gpu)])
+    cu_q_pad = torch.cat([g.cu_q_lens, torch.full((pad_s,), T, dtype=torch.int32, device=gpu)])
+    cu_kv_pad = torch.cat([g.cu_kv_lens, g.cu_kv_lens[-1:].expand(pad_s)])
+    qn = torch.cat([g.ql_nope, torch.zeros(pad_t, 32, 512, dtype=torch.bfloat16, device=gpu)])
+    qp = torch.cat([g.q_pe, torch.zeros(pad_t, 32, 64, dtype=torch.bfloat16, device=gpu)])
+    want = oracle(b)
+    host, _ = pkg.mla_ragged_paged_attention(qn, qp, None, None, g.cache_kv, kv_pad, g.page_indices, cu_q_pad, cu_kv_pad,
+                                             b.distribution.cpu().numpy(), sm_scale=b.sm_scale, max_kv_len=max(kv_lens),
+                                             num_splits=1)
+    dev, _ = pkg.mla_ragged_paged_attention(qn, qp, None, None, g.cache_kv, kv_pad, g.page_indices, cu_q_pad, cu_kv_pad,
+                                            g.distribution, sm_scale=b.sm_scale, num_splits=1)
+    auto, _ = pkg.mla_ragged_paged_attention(qn, qp, None, None, g.cache_kv, kv_pad, g.page_indices, cu_q_pad, cu_kv_pad,
+                                             g.distribution, sm_scale=b.sm_scale)
+    torch.cuda.synchronize()
+    assert_parity(dev[:T].cpu().float(), want.float(), **TOL)
+    assert_parity(auto[:T].cpu().float(), want.float(), **TOL)
+    # whole rows in both modes: the same arithmetic, bit for bit
+    assert torch.equal(dev[:T].view(torch.int16), host[:T].view(torch.int16))

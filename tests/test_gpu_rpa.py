@@ -910,3 +910,49 @@ def test_random_large_batches_against_oracle(pkg, wl, gpu, seed):
     got = gpu_out(pkg, b, gpu, **kw)
     assert torch.isfinite(got.float()).all()
     assert_parity(got.float(), want.float(), **(FP8_TOL if fp8 else BF16_TOL))
+
+
+# ------------------------------------------------------------------ static-shape mode
+@pytest.mark.parametrize("kv_dtype", [torch.bfloat16, torch.float8_e4m3fn])
+def test_device_side_distribution_matches_host_integers(pkg, wl, gpu, kv_dtype):
+    """The composition (decode_end, prefill_end, num_seqs) read on the device (rpa_v3:1676): the same
+    results as with host integers -- bit for bit when both modes cut the decode rows alike (here: not
+    at all), to rounding otherwise -- on a bucket padded with empty sequences and spare tokens, and one
+    prepared call serves different batches of the bucket."""
+    tol = BF16_TOL if kv_dtype == torch.bfloat16 else FP8_TOL
+    q_lens = [1] * 5 + [70, 300, 129]
+    kv_lens = [900, 33, 2500, 64, 1] + [70, 1324, 640]
+    b = wl.make_batch("static", q_lens, kv_lens, num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=64, seed=8401,
+                      kv_dtype=kv_dtype, pad_tokens=37, pad_seqs=8)
+    wl.plant_needles(b, seed=4, logit=10.0)
+    want = oracle_out(b)
+    g = b.to(gpu)
+    T = sum(q_lens)
+    kw = dict(sm_scale=b.sm_scale, k_scale=g.k_scale, v_scale=g.v_scale)
+    dist_host = b.distribution.cpu().numpy()
+
+    def run(dist, **extra):
+        out, _ = pkg.ragged_paged_attention(g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens,
+                                            g.cu_kv_lens, dist, None, **kw, **extra)
+        torch.cuda.synchronize()
+        return out[:T].cpu()
+
+    say(f"static-shape mode {kv_dtype}: distribution {dist_host.tolist()} of {g.kv_lens.shape[0]} sequences")
+    host_whole = run(dist_host, num_splits=1, max_kv_len=max(kv_lens), max_q_len=max(q_lens))
+    dev_whole = run(g.distribution, num_splits=1)
+    assert_parity(dev_whole.float(), want.float(), **tol)
+    assert torch.equal(dev_whole.view(torch.int16), host_whole.view(torch.int16))
+    dev_auto = run(g.distribution)  # the plan for the bound: every sequence a possible decode row
+    assert_parity(dev_auto.float(), want.float(), **tol)
+    # the same prepared parameters, another composition of the bucket: all decode / all chunks
+    for dist in ([5, 5, 5], [0, 0, 3]):
+        sub_q = [1] * 5 if dist[2] == 5 else [70, 300, 129]
+        sub_kv = kv_lens[:5] if dist[2] == 5 else [70, 1324, 640]
+        c = wl.make_batch("static2", sub_q, sub_kv, num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=64,
+                          seed=8402, kv_dtype=kv_dtype, pad_seqs=13 - len(sub_q), pad_tokens=5)
+        gc = c.to(gpu)
+        out, _ = pkg.ragged_paged_attention(gc.q, None, None, gc.kv_cache, gc.kv_lens, gc.page_indices, gc.cu_q_lens,
+                                            gc.cu_kv_lens, torch.tensor(dist, dtype=torch.int32, device=gpu), None,
+                                            sm_scale=c.sm_scale, k_scale=gc.k_scale, v_scale=gc.v_scale)
+        torch.cuda.synchronize()
+        assert_parity(out[: sum(sub_q)].cpu().float(), oracle_out(c).float(), **tol)
