@@ -44,6 +44,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # kernel that streams the KV bytes of each workload's decode rows: ragged batches that need
 # splitting take the balanced plan, equal-length and tiny ones the fixed split plan
 DECODE_KERNEL = {
+    "c5p": "rpa_mla_decode_kernel",
     "c1": "rpa_decode_splitkv_kernel",
     "c2": "rpa_decode_balanced_kernel",
     "c3": "rpa_decode_splitkv_kernel",
@@ -192,6 +193,10 @@ def run_mla_config(pkg, wl, b, steps, warmup):
     t1 = time.perf_counter()
     st = _stats([e[0].elapsed_time(e[1]) for e in evs])
     ms = st["mean"]
+    if any(q != 1 for q in b.meta["q_lens"]):  # prefill chunks: a FLOP figure, no decode bytes
+        flops = wl.mla_attention_flops(b)
+        return {"workload": b.name, "ms_per_step": (t1 - t0) * 1e3 / steps, "prefill_ms": ms, "prefill_ms_median": st["median"],
+                "prefill_ms_min": st["min"], "prefill_flops": flops, "prefill_tflops": flops / (ms * 1e-3) / 1e12}
     nbytes, flops = wl.mla_decode_bytes(b), wl.mla_decode_flops(b)
     return {"workload": b.name, "ms_per_step": (t1 - t0) * 1e3 / steps, "decode_ms": ms, "decode_ms_median": st["median"],
             "decode_ms_min": st["min"], "decode_bytes": nbytes, "decode_gbps": nbytes / (ms * 1e-3) / 1e9,
@@ -235,7 +240,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5"])
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5", "c5p"],
+                    help="c5p: absorbed-MLA prefill chunks (512 tokens on 4096-token prefixes), DeepSeek-V3 shape")
     ap.add_argument("--all", action="store_true", help="(default) also time the other configurations")
     ap.add_argument("--main-only", action="store_true", help="skip the other configurations")
     ap.add_argument("--static-shapes", action="store_true",
@@ -273,11 +279,11 @@ def main():
     def build(name):
         return {"c1": lambda: wl.config_c1(dev), "c2": lambda: wl.config_c2(dev), "c3": lambda: wl.config_c3(dev),
                 "c4": lambda: wl.config_c4(dev), "c4swa": lambda: wl.config_c4(dev, window=True),
-                "c5": lambda: wl.config_c5(dev)}[name]()
+                "c5": lambda: wl.config_c5(dev), "c5p": lambda: wl.config_c5_prefill(dev)}[name]()
 
     def run(name, keep=False):
         b = build(name)
-        if name == "c5":
+        if name in ("c5", "c5p"):
             r = run_mla_config(pkg, wl, b, args.steps, args.warmup)
         elif keep:
             r, call = run_rpa_config(pkg, wl, b, args.steps, args.warmup, keep_call=True,
@@ -298,7 +304,7 @@ def main():
                 "avg_launch_ms": res["decode_ms"], "median_launch_ms": res["decode_ms_median"],
                 "min_launch_ms": res["decode_ms_min"], "bytes_per_launch": res["decode_bytes"]}
 
-    if args.config == "c5":
+    if args.config in ("c5", "c5p"):
         main_res, sample = run(args.config), None
     else:
         main_res, sample = run(args.config, keep=True)
@@ -306,10 +312,11 @@ def main():
     pre_tflops = main_res.get("prefill_tflops")
     # dominant kernel of the workload (largest average launch time inside the timed region)
     roofline_decode = decode_roofline(args.config, main_res) if dec_gbps is not None else None
+    prefill_kernel = "rpa_mla_decode_kernel (one row per query token)" if args.config == "c5p" else PREFILL_KERNEL
     if pre_tflops is not None and main_res.get("prefill_ms", 0) >= main_res.get("decode_ms", 0):
-        roofline = {"kernel": PREFILL_KERNEL, "bound": "mfma", "achieved": pre_tflops,
+        roofline = {"kernel": prefill_kernel, "bound": "mfma", "achieved": pre_tflops,
                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": pre_tflops / MFMA_BF16_PEAK_TFLOPS,
-                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, PREFILL_KERNEL)),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, prefill_kernel)),
                     "avg_launch_ms": main_res["prefill_ms"], "median_launch_ms": main_res["prefill_ms_median"],
                     "min_launch_ms": main_res["prefill_ms_min"], "flops_per_launch": main_res["prefill_flops"]}
     else:
@@ -333,10 +340,17 @@ def main():
     }
     if not args.main_only:
         others = {}
-        for name in ("c1", "c2", "c3", "c4", "c4swa", "c5"):
+        for name in ("c1", "c2", "c3", "c4", "c4swa", "c5", "c5p"):
             if name == args.config:
                 continue
             r = run(name)
+            if name == "c5p":
+                r["roofline"] = {"kernel": "rpa_mla_decode_kernel (one row per query token)", "bound": "mfma",
+                                 "achieved": r["prefill_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                 "frac": r["prefill_tflops"] / MFMA_BF16_PEAK_TFLOPS, "avg_launch_ms": r["prefill_ms"],
+                                 "flops_per_launch": r["prefill_flops"]}
+                others[name] = r
+                continue
             r["roofline"] = decode_roofline(name, r)
             if name == "c5":
                 r["roofline"]["mfma_frac"] = r["tflops"] / MFMA_BF16_PEAK_TFLOPS

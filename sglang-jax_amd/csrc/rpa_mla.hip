@@ -367,7 +367,8 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot3[kSlotB];
-  const int row_id = blockIdx.y, split = blockIdx.x;
+  const int row_id = blockIdx.y;
+  const int split = blockIdx.x;
   const MlaRow mr = mla_row(a, row_id);
   if (!mr.valid) return;
   const int kv_len = mr.kv_len;

@@ -315,6 +315,17 @@ def config_c5(device="cpu", scale: float = 1.0, num_q_heads: int = 128) -> MlaBa
                           sm_scale=1.0 / math.sqrt(192.0))
 
 
+def config_c5_prefill(device="cpu", scale: float = 1.0, num_q_heads: int = 128, num_seqs: int = 4) -> MlaBatch:
+    """Absorbed-MLA prefill chunks, DeepSeek-V3 shape: `num_seqs` sequences, each a 512-token chunk
+    on a 4096-token prefix (kv_len 4608); 128 q heads, latent 512 + rope 64, P=64."""
+    seed = 1006
+    q = _scaled(512, scale)
+    kv = _scaled(4096, scale) + q
+    return make_mla_batch("c5p_deepseek_v3_mla_prefill", np.full(num_seqs, q), np.full(num_seqs, kv),
+                          num_q_heads=num_q_heads, lkv_dim=512, rope_dim=64, page_size=64, seed=seed, device=device,
+                          sm_scale=1.0 / math.sqrt(192.0))
+
+
 # --------------------------------------------------------------------------
 # Peaked inputs: a few keys per (sequence, kv head) that every query of that head attends to
 # --------------------------------------------------------------------------
@@ -486,6 +497,16 @@ def mla_decode_bytes(b: MlaBatch) -> int:
     total += T * Hq * width * 2 + T * Hq * lkv * 2
     total += int((-(-kv // b.page_size)).sum()) * 4 + (2 * len(kv) + 1) * 4
     return total
+
+
+def mla_attention_flops(b: MlaBatch) -> int:
+    """Any batch composition: Hq * (2 * 576 + 2 * 512) FLOP per visible (query token, cached token) pair."""
+    ql = np.asarray(b.meta["q_lens"], dtype=np.int64)
+    kv = np.asarray(b.meta["kv_lens"], dtype=np.int64)
+    _, Hq, lkv = b.ql_nope.shape
+    width = b.cache_kv.shape[-1]
+    pairs = int((ql * (kv - ql) + ql * (ql + 1) // 2).sum())
+    return pairs * Hq * (2 * width + 2 * lkv)
 
 
 def mla_decode_flops(b: MlaBatch) -> int:
