@@ -336,11 +336,16 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   // ---- epilogue: lane (c, g) holds head head0+c, dims 16j + 4g + r in acc[j][r] ----
   l += __shfl_xor(l, 16);
   l += __shfl_xor(l, 32);
-  const int head = head0 + c;
+  // The lane parts of the output addresses are worked out here, from values the compiler cannot
+  // trace back across the tile loop: hoisted out of it they would sit in registers the loop has
+  // none to spare for (they were spilled to scratch memory).
+  int c_out = c, g_out = g;
+  asm volatile("" : "+v"(c_out), "+v"(g_out));
+  const int head = head0 + c_out;
   if (!wave_on || head >= a.Hq) return;
   if (dest.final_rows) {
     const float inv = a.out_scale / l;
-    uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 512 + g * 4;
+    uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 512 + g_out * 4;
 #pragma unroll
     for (int j = 0; j < 32; ++j) {
       u32x2_t w = {pack_bf16x2(acc[j][0] * inv, acc[j][1] * inv), pack_bf16x2(acc[j][2] * inv, acc[j][3] * inv)};
@@ -348,10 +353,10 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     }
   } else {
     const int64_t slot = dest.base + head;
-    float* wo = a.ws_o + slot * 512 + g * 4;
+    float* wo = a.ws_o + slot * 512 + g_out * 4;
 #pragma unroll
     for (int j = 0; j < 32; ++j) *reinterpret_cast<f32x4_t*>(wo + j * 16) = acc[j];
-    if (g == 0) {
+    if (g_out == 0) {
       a.ws_ml[slot * 2 + 0] = m;
       a.ws_ml[slot * 2 + 1] = l;
     }
