@@ -450,6 +450,26 @@ static RpaParams planning_view(const RpaParams* p) {
   return q;
 }
 
+namespace {
+// Workspace of the balanced decode plan: partial rows, their (max, sum) pairs, the prefix sum of
+// the rows' blocks, and one 8-byte arrival word per (row, unit, wave of the workgroup).
+struct BalancedLayout {
+  size_t ml, cu_blocks, counters, total;  // byte offsets
+};
+BalancedLayout balanced_layout(const RpaParams* p) {
+  const size_t groups = (size_t)decode_wgs(p) * decode_waves_per_wg(p) * 2 * 16;
+  const int nw = decode_waves_per_wg(p);
+  const size_t units = (size_t)((p->num_kv_heads + nw - 1) / nw) * ((p->num_q_heads / p->num_kv_heads + 15) / 16);
+  BalancedLayout l;
+  l.ml = groups * p->head_dim * sizeof(float);
+  l.cu_blocks = l.ml + groups * 2 * sizeof(float);
+  l.counters = (l.cu_blocks + ((size_t)p->decode_end + 1) * sizeof(int32_t) + 7) & ~(size_t)7;
+  l.total = l.counters + (size_t)p->decode_end * units * nw * sizeof(unsigned long long);
+  return l;
+}
+std::atomic<unsigned long long> g_decode_generation{1};
+}  // namespace
+
 size_t rpa_workspace_bytes(const RpaParams* p_in) {
   if (!p_in) return 0;
   const RpaParams pv = planning_view(p_in);
@@ -458,9 +478,7 @@ size_t rpa_workspace_bytes(const RpaParams* p_in) {
   if (p->head_dim == 256) return rows256_workspace(p);
   const SplitPlan sp = decode_plan(p);
   if (use_balanced(p, sp))
-    return (size_t)decode_wgs(p) * decode_waves_per_wg(p) * 2 * 16 * (p->head_dim + 2) *
-               sizeof(float) +
-           ((size_t)p->decode_end + 1) * sizeof(int32_t);
+    return balanced_layout(p).total;
   if (sp.splits <= 1) return 0;
   return (size_t)p->decode_end * sp.splits * p->num_q_heads * (p->head_dim + 2) * sizeof(float);
 }
@@ -513,6 +531,8 @@ int rpa_decode(const RpaParams* p_in, void* stream) {
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
   a.cu_blocks = nullptr;
+  a.merge_counters = nullptr;
+  a.generation = 0;
   a.dist = p->distribution;
   a.balanced = use_balanced(p, sp) ? 1 : 0;
   a.num_wgs = decode_wgs(p);
@@ -528,9 +548,21 @@ int rpa_decode(const RpaParams* p_in, void* stream) {
     const size_t need = rpa_workspace_bytes(p);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
-    a.ws_o = static_cast<float*>(p->workspace);
-    a.ws_ml = a.ws_o + (size_t)a.num_wgs * a.waves_per_wg * 2 * 16 * p->head_dim;
-    a.cu_blocks = reinterpret_cast<int32_t*>(a.ws_ml + (size_t)a.num_wgs * a.waves_per_wg * 2 * 16 * 2);
+    const BalancedLayout lay = balanced_layout(p);
+    char* ws = static_cast<char*>(p->workspace);
+    a.ws_o = reinterpret_cast<float*>(ws);
+    a.ws_ml = reinterpret_cast<float*>(ws + lay.ml);
+    a.cu_blocks = reinterpret_cast<int32_t*>(ws + lay.cu_blocks);
+    // Opt-in: the wave that arrives last at a cut row merges it, and the second launch goes.
+    // Every workgroup of the balanced grid is resident from the start and ends with its cut
+    // piece, so all merges fall at the very end of the kernel, where they cost what the second
+    // launch costs, and the written-through partial rows cost more: it measures slower.
+    if (env_int("RPA_DECODE_MERGE_IN_KERNEL", 0) != 0 && (reinterpret_cast<uintptr_t>(ws) & 7) == 0) {
+      a.merge_counters = reinterpret_cast<unsigned long long*>(ws + lay.counters);
+      // 48 bits, never zero: the arrival words are never cleared, and a word of zeros must not
+      // look like this call's
+      a.generation = (g_decode_generation.fetch_add(1, std::memory_order_relaxed) % ((1ull << 48) - 1)) + 1;
+    }
   } else if (sp.splits > 1) {
     const size_t need = rpa_workspace_bytes(p);
     if (!p->workspace || p->workspace_bytes < need)

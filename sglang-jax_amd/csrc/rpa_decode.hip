@@ -331,16 +331,30 @@ __device__ __forceinline__ void write_rows(const DecodeArgs& a, const f32x4_t (&
     } else {
       const int64_t slot = dest.base + (dest.by_head ? head : row - row0);
       float* wo = a.ws_o + slot * 128 + g * 32;
+      // merged inside the same launch: the rows are written through to device scope, so that the
+      // merging wave (on another part of the GPU, behind another L2) reads them without any
+      // cache-wide write-back or invalidate
+      const bool through = a.merge_counters != nullptr;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         f32x4_t w0 = {acc[mt][0][r] * vs, acc[mt][1][r] * vs, acc[mt][2][r] * vs, acc[mt][3][r] * vs};
         f32x4_t w1 = {acc[mt][4][r] * vs, acc[mt][5][r] * vs, acc[mt][6][r] * vs, acc[mt][7][r] * vs};
-        *reinterpret_cast<f32x4_t*>(wo + r * 8) = w0;
-        *reinterpret_cast<f32x4_t*>(wo + r * 8 + 4) = w1;
+        if (through) {
+          asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(wo + r * 8), "v"(w0) : "memory");
+          asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(wo + r * 8 + 4), "v"(w1) : "memory");
+        } else {
+          *reinterpret_cast<f32x4_t*>(wo + r * 8) = w0;
+          *reinterpret_cast<f32x4_t*>(wo + r * 8 + 4) = w1;
+        }
       }
       if (g == 0) {
-        a.ws_ml[slot * 2 + 0] = m[mt];
-        a.ws_ml[slot * 2 + 1] = lt;
+        if (through) {
+          __hip_atomic_store(a.ws_ml + slot * 2 + 0, m[mt], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(a.ws_ml + slot * 2 + 1, lt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+          a.ws_ml[slot * 2 + 0] = m[mt];
+          a.ws_ml[slot * 2 + 1] = lt;
+        }
       }
     }
   }
@@ -587,6 +601,89 @@ struct Piece {
   bool final_rows;
 };
 
+// The wave that arrives last at a cut unit merges it.  A unit (row, kv head, group of 16 query
+// heads) whose blocks n workgroups share leaves n groups of 16 partial rows; each wave, once its
+// rows are written and fenced, adds one to the unit's arrival word, and the wave that brings it
+// to n reads all n groups back and writes the 16 finished rows.  The word carries the call's
+// generation in its upper 48 bits: a word left by another call (or by nothing: the memory is
+// never cleared) counts as zero, and the merging wave sets the count back to zero so that a
+// replay of the same launch with the same generation starts clean.
+//
+// A wave has at most two cut units, the first and the last piece of its share, and merges what
+// falls to it after its last block: the registers of the block pipeline are free by then, so
+// four groups of partial rows are in flight at a time, and no other wave waits for the rows.
+struct PendingMerge {
+  int n;  // 0: nothing to merge
+  int w_first;
+  int64_t first_block;
+  int tq, head0, rows;
+  unsigned long long* ctr;
+};
+
+// Every access is a device-scope atomic (relaxed): it reads what the other waves wrote through,
+// whatever this part of the GPU still caches of an earlier call.  Lanes: dims 2 lane, 2 lane + 1
+// of each of the 16 rows; lane r < 16 also owns the (max, sum) of row r.
+__device__ __forceinline__ float load_agent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void load2_agent(const float* p, float& x, float& y) {
+  const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+  x = __uint_as_float((uint32_t)v);
+  y = __uint_as_float((uint32_t)(v >> 32));
+}
+
+__device__ __forceinline__ void merge_unit(const DecodeArgs& a, const PendingMerge& pm, int pw, int wave, int nw,
+                                           unsigned long long generation, int lane) {
+  const int n = pm.n;
+  const int r = lane & 15;
+  auto slot16 = [&](int j) -> int64_t {
+    const int wj = pm.w_first + min(j, n - 1);
+    const int part = ((int64_t)wj * pw >= pm.first_block) ? 0 : 1;
+    return (((int64_t)wj * nw + wave) * 2 + part) * 16;
+  };
+  float mstar = -INFINITY;
+  for (int j = 0; j < n; ++j) mstar = fmaxf(mstar, load_agent(a.ws_ml + (slot16(j) + r) * 2));
+  float den = 0.f;
+  float acc[16][2];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i][0] = acc[i][1] = 0.f;
+  for (int j0 = 0; j0 < n; j0 += 4) {  // four groups of partial rows in flight
+    float o[4][16][2];
+    float wgt[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t s = slot16(j0 + u);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) load2_agent(a.ws_o + (s + i) * 128 + 2 * lane, o[u][i][0], o[u][i][1]);
+      float mj, lj;
+      load2_agent(a.ws_ml + (s + r) * 2, mj, lj);
+      wgt[u] = (j0 + u < n) ? fast_exp2(mj - mstar) : 0.f;  // a repeated group counts nothing
+      den += lj * wgt[u];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float wu = __shfl(wgt[u], i);
+        acc[i][0] += o[u][i][0] * wu;
+        acc[i][1] += o[u][i][1] * wu;
+      }
+  }
+  const float inv_r =
+      a.sm.sink ? sink_inverse(mstar, den, sink_logit(a.sm.sink, a.sm.round_logits, pm.head0 + min(r, pm.rows - 1)))
+                : 1.0f / den;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const float inv = __shfl(inv_r, i);
+    if (i < pm.rows) {
+      uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)pm.tq * a.Hq + pm.head0 + i) * 128 + 2 * lane);
+      *op = pack_bf16x2(acc[i][0] * inv, acc[i][1] * inv);
+    }
+  }
+  if (lane == 0) __hip_atomic_store(pm.ctr, generation << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // grid = num_wgs workgroups of NW = waves_per_wg waves.
 //
 // A wave treats its share as one stream of blocks: the block prefetched behind the last block of
@@ -725,6 +822,7 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
                                   page_in(win, cur.t_first), c, g);
   }
 
+  PendingMerge pm_first = {}, pm_last = {};
   for (;;) {
     // ---- this piece
     const int hk = min(cur.hk, a.Hkv - 1);
@@ -840,6 +938,39 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
       dest.by_head = false;
       dest.base = ((int64_t)w * 2 + (x == x_first ? 0 : 1)) * 16;
       write_rows<MT>(a, acc, m, l, cur.row.tq, hk, cur.rg * 16 * MT, dest, c, g);
+      if (a.merge_counters && !cur.final_rows) {
+        // the unit's first block in the linear order, and the workgroups that share the unit
+        const int64_t first_block = (int64_t)x - (cur.t_first - (cur.t_lo & ~(kBlk - 1))) / kBlk;
+        const int w_first = (int)(first_block / pw), w_last = (int)((first_block + cur.row.nb - 1) / pw);
+        const unsigned long long n = (unsigned long long)(w_last - w_first + 1);
+        unsigned long long* ctr = a.merge_counters + ((int64_t)cur.row.seq * units + cur_unit) * nw + wave;
+        // this wave's rows, written through, have reached device scope before it arrives
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        int is_last = 0;
+        if (lane == 0) {
+          unsigned long long old = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (;;) {
+            const unsigned long long cnt = ((old >> 16) == a.generation) ? (old & 0xffffull) : 0ull;
+            const unsigned long long neu = (a.generation << 16) | (cnt + 1);
+            if (__hip_atomic_compare_exchange_strong(ctr, &old, neu, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT)) {
+              is_last = (cnt + 1 == n) ? 1 : 0;
+              break;
+            }
+          }
+        }
+        is_last = __builtin_amdgcn_readfirstlane(is_last);
+        if (is_last) {
+          PendingMerge& pm = (x == x_first) ? pm_first : pm_last;
+          pm.n = (int)n;
+          pm.w_first = w_first;
+          pm.first_block = first_block;
+          pm.tq = cur.row.tq;
+          pm.head0 = hk * a.G + cur.rg * 16;
+          pm.rows = min(16, a.G - cur.rg * 16);
+          pm.ctr = ctr;
+        }
+      }
     }
     if (!has_next) break;
     x += cur.nblk;
@@ -852,6 +983,10 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
     }
     // the queries queue up right behind the piece's first block, which is already on its way
     load_queries<MT, FP8>(a, cur.row.tq, min(cur.hk, a.Hkv - 1), cur.rg * 16 * MT, c, g, qB);
+  }
+  if (pm_first.n | pm_last.n) {
+    if (pm_first.n) merge_unit(a, pm_first, pw, wave, nw, a.generation, lane);
+    if (pm_last.n) merge_unit(a, pm_last, pw, wave, nw, a.generation, lane);
   }
 }
 
@@ -1283,7 +1418,8 @@ hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream) {
   if (a.balanced) {
     hipError_t e = launch_decode_mt(a, dim3(a.num_wgs), dim3(a.waves_per_wg * 64), uniform, stream);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(rpa_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
+    if (!a.merge_counters)
+      hipLaunchKernelGGL(rpa_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
     return hipGetLastError();
   }
   dim3 grid(a.max_splits, a.num_rows, head_groups * row_groups);

@@ -66,6 +66,10 @@ struct DecodeArgs {
   int32_t min_blocks_per_wave;
   int32_t forced_blocks_per_wave;  // > 0: tests pin the partition
   int32_t* cu_blocks;              // [num_rows + 1] prefix sum of 32-token blocks, written by the kernel
+  // balanced plan, merge inside the kernel: one arrival word per (row, unit, wave of the
+  // workgroup), [generation : 48 | arrivals : 16]; nullptr => a second launch merges
+  unsigned long long* merge_counters;
+  unsigned long long generation;  // of this call; a word of another generation counts as zero
   // device i32[3] (decode_end, prefill_end, num_seqs) or nullptr: when given, num_rows is only a bound
   // and the rows to process are [0, min(num_rows, dist[0]))
   const int32_t* dist;

@@ -609,6 +609,40 @@ def test_balanced_plan_long_shares_and_tiny_rows(pkg, wl, gpu, monkeypatch):
         assert torch.equal(auto, again)
 
 
+def test_balanced_plan_merge_inside_the_kernel(pkg, wl, gpu, monkeypatch):
+    """The opt-in single-launch form of the balanced plan (RPA_DECODE_MERGE_IN_KERNEL=1): the wave
+    that arrives last at a cut row merges it, counted by one arrival word per (row, unit, wave)
+    that carries the call's generation and is never cleared.  Against the two-launch form and
+    the oracle: rows cut once, rows cut into dozens of pieces (eight workgroups for the whole
+    batch, and a pinned partition), and call after call on one workspace -- the arrival words
+    of the call before are still there."""
+    rng = np.random.default_rng(191)
+    kv_lens = [int(x) for x in rng.integers(1, 6000, size=90)]
+    for Hq, Hkv, kv_dtype in ((32, 8, torch.bfloat16), (96, 3, torch.bfloat16), (64, 8, torch.float8_e4m3fn)):
+        say(f"merge in kernel Hq={Hq} Hkv={Hkv} {kv_dtype}")
+        b = wl.make_batch("merge_in_kernel", [1] * len(kv_lens), kv_lens, num_q_heads=Hq, num_kv_heads=Hkv,
+                          head_dim=128, page_size=64, seed=192, kv_dtype=kv_dtype)
+        want = oracle_out(b)
+        tol = FP8_TOL if kv_dtype != torch.bfloat16 else BF16_TOL
+        two = {ns: gpu_out(pkg, b, gpu, num_splits=ns) for ns in (0, 3, 50)}
+        monkeypatch.setenv("RPA_DECODE_MERGE_IN_KERNEL", "1")
+        for rep in range(2):
+            for ns in (0, 3, 50):
+                got = gpu_out(pkg, b, gpu, num_splits=ns)
+                assert_parity(got.float(), want.float(), **tol)
+                assert float(row_rel_error(got.float(), two[ns].float()).max()) < 4e-3
+        monkeypatch.delenv("RPA_DECODE_MERGE_IN_KERNEL")
+    monkeypatch.setenv("RPA_DECODE_WAVE_CAPACITY", "16")
+    kv_lens = [9000, 5000, 70, 1, 12000, 64, 33, 7000]
+    b = wl.make_batch("merge_in_kernel_long", [1] * len(kv_lens), kv_lens, num_q_heads=8, num_kv_heads=2,
+                      head_dim=128, page_size=64, seed=195)
+    want = oracle_out(b)
+    monkeypatch.setenv("RPA_DECODE_MERGE_IN_KERNEL", "1")
+    got = gpu_out(pkg, b, gpu)
+    assert_parity(got.float(), want.float(), **BF16_TOL)
+    assert torch.equal(got, gpu_out(pkg, b, gpu))
+
+
 def test_balanced_plan_when_rows_outnumber_wave_slots(pkg, wl, gpu):
     """More (row, kv head) jobs than resident waves and far more than 64 MB of KV: the fixed plan
     would leave every row whole (one job each, as different in length as the rows are), so the
