@@ -156,10 +156,11 @@ def test_workspace_size_is_deterministic(pkg):
     p.num_q_heads, p.num_kv_heads, p.page_size, p.total_pages = 32, 8, 64, 8192
     p.max_kv_len = 32768
     # lengths unknown to the host: the balanced plan, two groups of 16 partial rows per wave slot
-    # plus the prefix sum of blocks; its size does not depend on the batch
+    # plus the prefix sum of blocks (17 words, padded to 8 bytes) and one 8-byte arrival word per
+    # (row, unit, wave): 16 rows x 2 units x 4 waves; its size does not depend on the batch
     a = lib.rpa_workspace_bytes(ctypes.byref(p))
     assert a > 0 and a == lib.rpa_workspace_bytes(ctypes.byref(p))
-    assert (a - 17 * 4) % (2 * 16 * 130 * 4) == 0
+    assert (a - 18 * 4 - 16 * 2 * 4 * 8) % (2 * 16 * 130 * 4) == 0
     p.max_kv_len = 8192
     assert lib.rpa_workspace_bytes(ctypes.byref(p)) == a
     # all rows of one known length: the fixed plan, one partial row per (row, split, head)
