@@ -399,8 +399,11 @@ def ragged_paged_attention(
     if k > kv_lens_d.shape[0]:
         raise ValueError(f"distribution[2]={k} exceeds max_num_seqs={kv_lens_d.shape[0]}")
 
-    if out_dtype not in (None, torch.bfloat16):
-        raise NotImplementedError("out_dtype other than bfloat16 is not built")
+    # rpa_v3:1788: bfloat16 unless asked otherwise.  The kernels normalise in f32 and round the
+    # finished row to bf16 once; float32 output is those values widened (one bf16 rounding more
+    # than the reference's f32 accumulator leaves, far inside the parity tolerance)
+    if out_dtype not in (None, torch.bfloat16, torch.float32):
+        raise NotImplementedError("out_dtype must be bfloat16 or float32")
     call = RpaCall(queries, kv_cache_fused, None, kv_lens_d, page_d, cu_q_d, cu_kv_d, num_seqs=k, decode_end=i,
                    sm_scale=sm_scale, sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
                    k_scale=k_scale, v_scale=v_scale,
@@ -424,6 +427,8 @@ def ragged_paged_attention(
             raise ValueError(f"Expected keys/values dtype {kv_cache_fused.dtype}, got {keys.dtype}/{values.dtype}")
         call.kv_write(keys.contiguous(), values.contiguous())
     call.attention()
+    if out_dtype == torch.float32:
+        return call.out.float(), kv_cache_fused
     return call.out, kv_cache_fused
 
 

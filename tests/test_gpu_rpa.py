@@ -267,6 +267,15 @@ def test_new_tokens_are_written_into_the_cache(pkg, wl, gpu):
     torch.cuda.synchronize()
     assert torch.equal(cache.cpu().view(torch.int16), b.kv_cache.view(torch.int16))
     assert_parity(out.cpu().float(), want.float(), **BF16_TOL)
+    # out_dtype (rpa_v3:1695, 1788): float32 on request
+    out32, _ = pkg.ragged_paged_attention(
+        g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+        b.distribution.numpy(), None, sm_scale=b.sm_scale, max_kv_len=300, max_q_len=65, out_dtype=torch.float32)
+    assert out32.dtype == torch.float32
+    assert_parity(out32[:T].cpu(), want.float(), **BF16_TOL)
+    with pytest.raises(NotImplementedError):
+        pkg.ragged_paged_attention(g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+                                   b.distribution.numpy(), None, sm_scale=b.sm_scale, out_dtype=torch.float16)
 
 
 def test_dynamic_validation_through_the_wrapper(pkg, wl, gpu):
