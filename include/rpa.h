@@ -124,7 +124,11 @@ typedef struct RpaParams {
                                    Read only when mask_mode == RPA_MASK_CUSTOM */
   const int32_t* cu_mask_lens;  /* device i32[S+1]: cumulative q_len_i * row_width_i (:123-129, 1801-1806) */
   float xai_temperature_len;    /* > 0: logits of a query at position p > len are multiplied by
-                                   log2(p) / log2(len) (:171-177); 0 => off */
+                                   log2(p) / log2(len) (:171-177); 0 => off.  With soft_cap set as well
+                                   the factor multiplies the capped logit, the order of
+                                   ref_ragged_paged_attention (:166-177); the reference's TPU kernel
+                                   multiplies first and caps after (:481-486), so the reference's two
+                                   paths differ from each other when both options are on */
   int32_t mask_mode;            /* RpaMaskMode */
   int32_t mask_rows_page_aligned; /* custom mask row_width_i: 0 => kv_len_i, 1 => kv_len_i rounded up to
                                    pages (cu_kv_lens delta; mask_aligned_to_cu_kv, :1791-1806) */

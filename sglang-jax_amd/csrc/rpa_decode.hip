@@ -304,7 +304,7 @@ __device__ __forceinline__ void requantise_queries(const DecodeArgs& a, u32x4_t 
 
 // Leave the result of one piece of work: lane (c, g) holds q row c, dims 32g + 8r + j in
 // acc[mt][j][r].
-template <int MT>
+template <int MT, bool THROUGH = false>
 __device__ __forceinline__ void write_rows(const DecodeArgs& a, const f32x4_t (&acc)[MT][8], const float (&m)[MT],
                                            const float (&l)[MT], int tq, int hk, int row0, const PartDest dest,
                                            int c, int g) {
@@ -334,7 +334,7 @@ __device__ __forceinline__ void write_rows(const DecodeArgs& a, const f32x4_t (&
       // merged inside the same launch: the rows are written through to device scope, so that the
       // merging wave (on another part of the GPU, behind another L2) reads them without any
       // cache-wide write-back or invalidate
-      const bool through = a.merge_counters != nullptr;
+      constexpr bool through = THROUGH;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         f32x4_t w0 = {acc[mt][0][r] * vs, acc[mt][1][r] * vs, acc[mt][2][r] * vs, acc[mt][3][r] * vs};
@@ -692,7 +692,7 @@ __device__ __forceinline__ void merge_unit(const DecodeArgs& a, const PendingMer
 // are requested right behind that first block.  A piece border costs no round trip to memory,
 // and neither does a block: under load a small dependent load waits behind megabytes of queued
 // KV traffic (10 us and more), so there are none after the first block.
-template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
+template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP, bool MERGE>
 __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const DecodeArgs a_in) {
   DecodeArgs a = a_in;  // static-shape mode: the number of decode rows comes from the device
   if (a.dist) a.num_rows = min(a.num_rows, scalar_load_i32(a.dist));
@@ -937,8 +937,8 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
       dest.final_rows = cur.final_rows;
       dest.by_head = false;
       dest.base = ((int64_t)w * 2 + (x == x_first ? 0 : 1)) * 16;
-      write_rows<MT>(a, acc, m, l, cur.row.tq, hk, cur.rg * 16 * MT, dest, c, g);
-      if (a.merge_counters && !cur.final_rows) {
+      write_rows<MT, MERGE>(a, acc, m, l, cur.row.tq, hk, cur.rg * 16 * MT, dest, c, g);
+      if (MERGE && !cur.final_rows) {
         // the unit's first block in the linear order, and the workgroups that share the unit
         const int64_t first_block = (int64_t)x - (cur.t_first - (cur.t_lo & ~(kBlk - 1))) / kBlk;
         const int w_first = (int)(first_block / pw), w_last = (int)((first_block + cur.row.nb - 1) / pw);
@@ -984,7 +984,7 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
     // the queries queue up right behind the piece's first block, which is already on its way
     load_queries<MT, FP8>(a, cur.row.tq, min(cur.hk, a.Hkv - 1), cur.rg * 16 * MT, c, g, qB);
   }
-  if (pm_first.n | pm_last.n) {
+  if (MERGE && (pm_first.n | pm_last.n)) {
     if (pm_first.n) merge_unit(a, pm_first, pw, wave, nw, a.generation, lane);
     if (pm_last.n) merge_unit(a, pm_last, pw, wave, nw, a.generation, lane);
   }
@@ -1385,7 +1385,10 @@ __global__ __launch_bounds__(256) void rpa_kv_write_kernel(const KvWriteArgs a_i
 
 template <bool FP8, bool UNIFORM, bool CAP>
 void launch_decode_variant(const DecodeArgs& a, dim3 grid, dim3 block, hipStream_t st) {
-  if (a.balanced) hipLaunchKernelGGL((rpa_decode_balanced_kernel<1, FP8, UNIFORM, CAP>), grid, block, 0, st, a);
+  if (a.balanced && a.merge_counters)
+    hipLaunchKernelGGL((rpa_decode_balanced_kernel<1, FP8, UNIFORM, CAP, true>), grid, block, 0, st, a);
+  else if (a.balanced)
+    hipLaunchKernelGGL((rpa_decode_balanced_kernel<1, FP8, UNIFORM, CAP, false>), grid, block, 0, st, a);
   else hipLaunchKernelGGL((rpa_decode_splitkv_kernel<1, FP8, UNIFORM, CAP>), grid, block, 0, st, a);
 }
 

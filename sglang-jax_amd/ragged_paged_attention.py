@@ -183,13 +183,20 @@ class RpaCall:
     ``attention()`` = ``rpa_attention`` (decode rows, then prefill/mixed rows);
     ``decode()`` / ``prefill()`` run the two partitions on their own, which is how
     the benchmark times them separately.  Launches go to torch's current stream.
+
+    The split-KV workspace is by default the one grow-only buffer of (device, stream current at
+    construction), shared by every call prepared on that stream: calls that share it must be
+    ordered on one stream.  A call that is kept and launched from elsewhere -- captured into a
+    graph, replayed while eager calls run, issued on another stream -- takes
+    ``own_workspace=True`` and holds a buffer of its own for as long as it lives.
     """
 
     def __init__(self, queries, kv_cache, v_pages, kv_lens_d, page_d, cu_q_d, cu_kv_d, *, num_seqs, decode_end,
                  sm_scale, sliding_window=None, soft_cap=None, mask_value=DEFAULT_MASK_VALUE, k_scale=None,
                  v_scale=None, max_kv_len=0, max_q_len=0, num_splits=0, out=None, sum_decode_kv_len=0,
                  attention_sink=None, xai_temperature_len=None, causal=True, custom_mask=None,
-                 mask_aligned_to_cu_kv=False, softmax_dtype=None, q_scale=None, distribution_d=None):
+                 mask_aligned_to_cu_kv=False, softmax_dtype=None, q_scale=None, distribution_d=None,
+                 own_workspace=False):
         self.lib = _lib.load()
         self.device = queries.device
         fused = v_pages is None
@@ -286,7 +293,8 @@ class RpaCall:
         need = self.lib.rpa_workspace_bytes(ctypes.byref(p))
         self.workspace = None
         if need:
-            self.workspace = _workspace(self.device, need)
+            self.workspace = (torch.empty(need, dtype=torch.uint8, device=self.device) if own_workspace
+                              else _workspace(self.device, need))
             p.workspace = self.workspace.data_ptr()
             p.workspace_bytes = self.workspace.numel()
         self.params = p

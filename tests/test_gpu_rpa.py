@@ -435,10 +435,12 @@ def test_attention_sink(pkg, wl, gpu, window, cap):
     assert float(high.float().abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("cap", [None, 20.0])
+@pytest.mark.parametrize("cap", [None, 20.0, 1.0])
 def test_xai_temperature(pkg, wl, gpu, cap):
     """Logits of queries beyond position T are multiplied by log2(pos)/log2(T)
-    (ragged_paged_attention_v3.py:171-177)."""
+    (ragged_paged_attention_v3.py:171-177).  With a soft cap the factor multiplies the capped
+    logit (:166-177); a cap of 1 saturates on these inputs, so multiplying before the cap
+    instead (as the reference's TPU kernel does, :481-486) would fail the comparison."""
     q_lens, kv_lens, b = options_batch(wl, "xai", 72)
     b.soft_cap = cap
     say(f"case xai cap={cap}")
@@ -856,7 +858,8 @@ def test_a_captured_step_replays_with_new_lengths_and_page_tables(pkg, wl, gpu):
         st["vals"].copy_(vals)
 
     call = RpaCall(st["q"], st["cache"], None, st["kv_lens"], st["pages"], st["cu_q"], st["cu_kv"], num_seqs=S,
-                   decode_end=3, sm_scale=batches[0].sm_scale, max_kv_len=1024, max_q_len=max(q_lens))
+                   decode_end=3, sm_scale=batches[0].sm_scale, max_kv_len=1024, max_q_len=max(q_lens),
+                   own_workspace=True)  # replayed next to eager calls: not the buffer those share
 
     def step():
         call.kv_write(st["keys"], st["vals"])
