@@ -47,7 +47,7 @@ def source_hash() -> str:
     import hashlib
 
     h = hashlib.sha256(" ".join(FLAGS).encode())
-    files = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC))
+    files = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if os.path.isfile(os.path.join(CSRC, f)))
     files.append(os.path.join(os.path.dirname(HERE), "include", "rpa.h"))
     for path in files:
         h.update(os.path.basename(path).encode())

@@ -26,6 +26,7 @@
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
+#include "rpa_mla_pipe_loop.inc"
 
 namespace rpa {
 
@@ -40,6 +41,8 @@ constexpr int kCopiesPerWave = 5;        // every wave issues 5 copy instruction
 
 __device__ __forceinline__ u32x4_t lds_ld16(const char* p) { return *reinterpret_cast<const u32x4_t*>(p); }
 
+typedef uint32_t u32x32_t __attribute__((ext_vector_type(32)));
+typedef uint32_t u32x8_t __attribute__((ext_vector_type(8)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ u32x2_t lds_tr16(const char* p) {
   typedef __attribute__((address_space(3))) s16x4_t* lds_ptr_t;
@@ -173,7 +176,11 @@ struct MlaDest {
 // One workgroup, one row, one group of 128 heads, tokens [t_begin, t_end).  Every wave of the
 // workgroup calls it with the same arguments; all LDS reads of an earlier call are behind a
 // barrier when it returns.
-template <bool UNIFORM, bool CAP>
+// PIPE: the tiles of the segment that are whole and unmasked, all but the first, run inside the
+// assembly loop of rpa_mla_pipe_loop.inc (same LDS ring, same copy protocol, same registers as the
+// compiled step, which still does the first tile, masked tiles and the last three before a
+// partial one).  Needs UNIFORM pages of a power-of-two size, no soft cap, every wave at work.
+template <bool UNIFORM, bool CAP, bool PIPE = false>
 __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
                                             int t_begin, int t_end, const MlaDest dest, char* slot0, char* slot1,
                                             char* slot2, char* slot3) {
@@ -322,14 +329,87 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
-  for (int tb = t_begin; tb < t_end; tb += 4 * kTok) {
-    tile_step(slot0, slot3, tb);
-    if (tb + kTok >= t_end) break;
-    tile_step(slot1, slot0, tb + kTok);
-    if (tb + 2 * kTok >= t_end) break;
-    tile_step(slot2, slot1, tb + 2 * kTok);
-    if (tb + 3 * kTok >= t_end) break;
-    tile_step(slot3, slot2, tb + 3 * kTok);
+  if constexpr (!PIPE) {
+    for (int tb = t_begin; tb < t_end; tb += 4 * kTok) {
+      tile_step(slot0, slot3, tb);
+      if (tb + kTok >= t_end) break;
+      tile_step(slot1, slot0, tb + kTok);
+      if (tb + 2 * kTok >= t_end) break;
+      tile_step(slot2, slot1, tb + 2 * kTok);
+      if (tb + 3 * kTok >= t_end) break;
+      tile_step(slot3, slot2, tb + 3 * kTok);
+    }
+  } else {
+    const int nT = (t_end - t_begin + kTok - 1) / kTok;  // tiles of the segment
+    // tiles [k0, k1) go through the assembly loop: past the first tile (which fixes the reference the
+    // probabilities are taken against) and past the window's edge; the loop copies tile k + 3 without
+    // clamping rows, so that one has to be a whole tile of the row
+    int k0 = 1;
+    if (t_begin < t_lo) k0 = max(k0, (t_lo - t_begin + kTok - 1) / kTok);
+    const int k1 = min(nT, (kv_len - t_begin) / kTok - 3);
+    auto slot_of = [&](int k) -> char* {
+      k &= 3;
+      return k == 0 ? slot0 : (k == 1 ? slot1 : (k == 2 ? slot2 : slot3));
+    };
+    typedef __attribute__((address_space(3))) char* lds_ptr_t;
+    int k = 0;
+    for (int phase = 0; phase < 2; ++phase) {
+      const int stop = (phase == 0 && k0 < k1) ? k0 : nT;
+      for (; k < stop; ++k) tile_step(slot_of(k), slot_of(k + 3), t_begin + k * kTok);
+      if (k >= nT) break;
+      // ---- tiles k .. k1 - 1 in assembly
+      f32x16_t o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[i][e] = acc[4 * i + (e >> 2)][e & 3];
+      u32x32_t q0, q1;
+      u32x8_t q2;
+#pragma unroll
+      for (int e = 0; e < 32; ++e) {
+        q0[e] = qB[e >> 2][e & 3];
+        q1[e] = qB[8 + (e >> 2)][e & 3];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) q2[e] = qB[16 + (e >> 2)][e & 3];
+      int ln = lane;
+      asm volatile("" : "+v"(ln));  // the lane parts below are worked out here, not carried from the top
+      const int cc = ln & 15, gg = ln >> 4;
+      u32x4_t ml = {__float_as_uint(m), __float_as_uint(l), (uint32_t)(cc * kRowB + gg * 16),
+                    (uint32_t)((4 * gg + (cc >> 2)) * kRowB + (cc & 3) * 8)};
+      u32x8_t ofs = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int n = 0; n < kCopiesPerWave; ++n) {
+        int row, inner;
+        chunk_of(src, wave, ln, n, row, inner);
+        ofs[n] = (uint32_t)(row * src.row_bytes + inner);
+      }
+      const uint32_t s0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)slot0);
+      const uint32_t s1 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)slot1);
+      const uint32_t s2 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)slot2);
+      const uint32_t s3 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)slot3);
+      const uint32_t cache_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)a.cache);
+      const uint32_t cache_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)a.cache >> 32));
+      const int last_tile_tok = __builtin_amdgcn_readfirstlane(src.last_tok & ~(kTok - 1));
+      const int wave_blk = wave * kCopiesPerWave * 1024;
+#define C(n) RPA_MLA_PIPE_C_##n
+      asm volatile(RPA_MLA_PIPE_ASM
+                   : "+" C(O0)(o[0]), "+" C(O1)(o[1]), "+" C(O2)(o[2]), "+" C(O3)(o[3]), "+" C(O4)(o[4]),
+                     "+" C(O5)(o[5]), "+" C(O6)(o[6]), "+" C(O7)(o[7]), "+" C(ML)(ml), "+" C(OFS)(ofs),
+                     [t] "+s"(k), [pg] "+s"(pg_next)
+                   : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), [t_end] "s"(k1), [t_begin] "s"(t_begin),
+                     [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),
+                     [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2),
+                     [wave_blk] "s"(wave_blk), [slot0] "s"(s0), [slot1] "s"(s1), [slot2] "s"(s2), [slot3] "s"(s3)
+                   : RPA_MLA_PIPE_CLOBBERS);
+#undef C
+      m = __uint_as_float(ml[0]);
+      l = __uint_as_float(ml[1]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[4 * i + (e >> 2)][e & 3] = o[i][e];
+    }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the copies issued past the end
 
@@ -364,7 +444,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
 }
 
 // ---- fixed split plan: grid = (max_splits, rows, head groups of 128); block = 512 threads
-template <bool UNIFORM, bool CAP>
+template <bool UNIFORM, bool CAP, bool PIPE = false>
 __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeArgs a) {
   // three separate arrays: lets the compiler see that a copy into one slot does not alias the
   // reads of another, so it does not drain the vector-memory queue before LDS reads
@@ -386,7 +466,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   MlaDest dest;
   dest.final_rows = a.max_splits == 1;
   dest.base = ((int64_t)row_id * a.max_splits + split) * a.Hq;
-  mla_segment<UNIFORM, CAP>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
+  mla_segment<UNIFORM, CAP, PIPE>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
 }
 
 // ---- balanced plan (one row per sequence): the 32-token tiles of the whole batch, sequence by
@@ -419,7 +499,7 @@ __device__ __forceinline__ int mla_tiles_per_wg(const MlaDecodeArgs& a, int tota
   return max(a.forced_tiles_per_wg > 0 ? a.forced_tiles_per_wg : a.min_tiles_per_wg, even);
 }
 
-template <bool UNIFORM, bool CAP>
+template <bool UNIFORM, bool CAP, bool PIPE = false>
 __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecodeArgs a) {
   __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
@@ -509,8 +589,8 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
     dest.final_rows = (tile == 0) && (take == nt);
     dest.base = ((int64_t)wg * 2 + (first_piece ? 0 : 1)) * 128 - unit * 128;  // + head
     first_piece = false;
-    mla_segment<UNIFORM, CAP>(a, mr, unit * 128, t_lo, t0 + tile * kTok, min(kv_len, t0 + (tile + take) * kTok),
-                              dest, slot0, slot1, slot2, slot3);
+    mla_segment<UNIFORM, CAP, PIPE>(a, mr, unit * 128, t_lo, t0 + tile * kTok,
+                                    min(kv_len, t0 + (tile + take) * kTok), dest, slot0, slot1, slot2, slot3);
     x += take;
     if (x < x_end && tile + take == nt && unit == units - 1) {
       seq_first += (nt + pad) * units;
@@ -624,9 +704,16 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   const dim3 grid(a.max_splits, a.num_rows, head_groups), block(512);
   const bool uniform = (a.pt.page_size % kTok) == 0;
   const bool cap = a.sm.soft_cap != 0.f;
+  // the assembly tile loop: whole tiles inside one page, every wave of a workgroup at work
+  static const bool use_pipe = [] { const char* v = getenv("RPA_MLA_PIPE"); return !(v && *v == '0'); }();
+  const int P = a.pt.page_size;
+  const bool pipe = use_pipe && uniform && !cap && (P & (P - 1)) == 0 && (a.Hq % 128) == 0 &&
+                    (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);
   if (a.balanced) {
     const dim3 bgrid(a.num_wgs);
-    if (uniform) {
+    if (pipe) {
+      hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, false, true>), bgrid, block, 0, stream, a);
+    } else if (uniform) {
       if (cap) hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, true>), bgrid, block, 0, stream, a);
       else hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, false>), bgrid, block, 0, stream, a);
     } else {
@@ -638,7 +725,9 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
     return hipGetLastError();
   }
-  if (uniform) {
+  if (pipe) {
+    hipLaunchKernelGGL((rpa_mla_decode_kernel<true, false, true>), grid, block, 0, stream, a);
+  } else if (uniform) {
     if (cap) hipLaunchKernelGGL((rpa_mla_decode_kernel<true, true>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((rpa_mla_decode_kernel<true, false>), grid, block, 0, stream, a);
   } else {
