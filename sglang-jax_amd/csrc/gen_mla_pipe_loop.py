@@ -170,6 +170,15 @@ def step(em, k):
             em.emit(x)
     copies = [] if "nocopy" in X else [copy_group(n, fill) for n in range(COPIES)]
     copy_at = {4 + 6 * n: n for n in range(COPIES)}            # behind these matrix instructions of the first product
+    if "copypv" in X:
+        copy_at = {38 + 6 * n: n for n in range(COPIES)}
+    if "copyend" in X:
+        copy_at = {67: -1}
+    if "copyfirst" in X:
+        copy_at = {}
+        for grp in copies:
+            for x in grp:
+                em.emit(x)
     sm = softmax()
     for f in range(36):
         em.emit(frag_mfma(f))
@@ -192,6 +201,10 @@ def step(em, k):
         if f + AHEAD < 68:
             for x in frag_read(f + AHEAD):
                 em.emit(x)
+        if f in copy_at and copies:
+            for grp in (copies if copy_at[f] < 0 else [copies[copy_at[f]]]):
+                for x in grp:
+                    em.emit(x)
     assert not em.lds_queue
     # end of step: tile t + 1 has landed once only the ten newest copies (tiles t + 2, t + 3) are outstanding;
     # every LDS read of tile t has returned, so its slot may be refilled after the barrier

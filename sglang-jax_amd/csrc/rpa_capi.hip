@@ -777,15 +777,16 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
     const size_t need = mla_workspace(p, rows, token_rows);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
-    a.ws_o = static_cast<float*>(p->workspace);
-    a.ws_ml = a.ws_o + (size_t)a.num_wgs * 2 * 128 * p->lkv_dim;
+    // partial rows are bf16 (the workspace is sized for f32 rows: room to spare)
+    a.ws_o = static_cast<uint16_t*>(p->workspace);
+    a.ws_ml = reinterpret_cast<float*>(a.ws_o + (size_t)a.num_wgs * 2 * 128 * p->lkv_dim);
     a.cu_tiles = reinterpret_cast<int32_t*>(a.ws_ml + (size_t)a.num_wgs * 2 * 128 * 2);
   } else if (sp.splits > 1) {
     const size_t need = mla_workspace(p, rows, token_rows);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
-    a.ws_o = static_cast<float*>(p->workspace);
-    a.ws_ml = a.ws_o + (size_t)rows * sp.splits * p->num_q_heads * p->lkv_dim;
+    a.ws_o = static_cast<uint16_t*>(p->workspace);
+    a.ws_ml = reinterpret_cast<float*>(a.ws_o + (size_t)rows * sp.splits * p->num_q_heads * p->lkv_dim);
   }
   return check_hip(rpa::launch_mla_decode(a, static_cast<hipStream_t>(stream)),
                    token_rows ? "rpa_mla_attention" : "rpa_mla_decode");

@@ -125,8 +125,8 @@ struct MlaDecodeArgs {
   const char* cache;        // [pages, P, row_stride] bf16
   PageTable pt;
   SoftmaxOpts sm;
-  float* ws_o;   // [T, max_splits, Hq, lkv]
-  float* ws_ml;  // [T, max_splits, Hq, 2]
+  uint16_t* ws_o;  // [T, max_splits, Hq, lkv] unnormalised partial outputs, bf16
+  float* ws_ml;    // [T, max_splits, Hq, 2] (reference in log2 units, sum)
   int32_t num_rows;     // grid rows: sequences (rows_are_tokens == 0) or query tokens
   int32_t num_seqs;
   int32_t rows_are_tokens;  // 1: row r is query token r of whatever sequence owns it (any q_len)

@@ -433,9 +433,14 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     }
   } else {
     const int64_t slot = dest.base + head;
-    float* wo = a.ws_o + slot * 512 + g_out * 4;
+    // partial rows are left as bf16: the merge reads half the bytes, and the result is rounded to
+    // bf16 anyway
+    uint16_t* wo = a.ws_o + slot * 512 + g_out * 4;
 #pragma unroll
-    for (int j = 0; j < 32; ++j) *reinterpret_cast<f32x4_t*>(wo + j * 16) = acc[j];
+    for (int j = 0; j < 32; ++j) {
+      u32x2_t w = {pack_bf16x2(acc[j][0], acc[j][1]), pack_bf16x2(acc[j][2], acc[j][3])};
+      *reinterpret_cast<u32x2_t*>(wo + j * 16) = w;
+    }
     if (g_out == 0) {
       a.ws_ml[slot * 2 + 0] = m;
       a.ws_ml[slot * 2 + 1] = l;
@@ -632,7 +637,8 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const Mla
     const int64_t slot = slot_of(wj);
     const float w = fast_exp2(a.ws_ml[slot * 2] - mstar);
     den += a.ws_ml[slot * 2 + 1] * w;
-    o += *reinterpret_cast<const f32x4_t*>(a.ws_o + slot * 512 + d) * w;
+    const u32x2_t pr = *reinterpret_cast<const u32x2_t*>(a.ws_o + slot * 512 + d);
+    o += f32x4_t{bf16_lo_to_f32(pr[0]), bf16_hi_to_f32(pr[0]), bf16_lo_to_f32(pr[1]), bf16_hi_to_f32(pr[1])} * w;
   }
   const float inv = a.out_scale / den;
   const int tq = a.pt.cu_q_lens[seq];
@@ -660,7 +666,8 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_kernel(const MlaDecodeArg
     const int64_t slot = base + (int64_t)j * a.Hq;
     const float w = fast_exp2(a.ws_ml[slot * 2] - mstar);
     den += a.ws_ml[slot * 2 + 1] * w;
-    o += *reinterpret_cast<const f32x4_t*>(a.ws_o + slot * 512 + d) * w;
+    const u32x2_t pr = *reinterpret_cast<const u32x2_t*>(a.ws_o + slot * 512 + d);
+    o += f32x4_t{bf16_lo_to_f32(pr[0]), bf16_hi_to_f32(pr[0]), bf16_lo_to_f32(pr[1]), bf16_hi_to_f32(pr[1])} * w;
   }
   const float inv = a.out_scale / den;
   const int tq = mr.tq;
