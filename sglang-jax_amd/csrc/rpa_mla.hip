@@ -608,6 +608,45 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
   }
 }
 
+// Merge the n partial rows of one (row, head): 128 threads, 4 dims each.  Partials are taken eight at
+// a time with every load of a group (references, sums, rows) requested before any is used -- one
+// round trip to memory per group instead of one per partial -- and groups are chained like tiles of
+// an online softmax.
+template <typename SlotOf>
+__device__ __forceinline__ void mla_merge(const MlaDecodeArgs& a, int n, SlotOf slot_of, int head, int tq) {
+  const int d = threadIdx.x * 4;
+  float mstar = -INFINITY, den = 0.f;
+  f32x4_t o = {0.f, 0.f, 0.f, 0.f};
+  for (int j0 = 0; j0 < n; j0 += 8) {
+    float mj[8], lj[8];
+    u32x2_t pr[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t slot = slot_of(min(j0 + u, n - 1));
+      mj[u] = a.ws_ml[slot * 2];
+      lj[u] = a.ws_ml[slot * 2 + 1];
+      pr[u] = *reinterpret_cast<const u32x2_t*>(a.ws_o + slot * 512 + d);
+    }
+    float mnew = mstar;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) mnew = fmaxf(mnew, mj[u]);  // a repeated last partial changes nothing
+    const float keep = fast_exp2(mstar - mnew);  // 0 for the first group
+    den *= keep;
+    o *= keep;
+    mstar = mnew;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float w = (j0 + u < n) ? fast_exp2(mj[u] - mstar) : 0.f;
+      den += lj[u] * w;
+      o += f32x4_t{bf16_lo_to_f32(pr[u][0]), bf16_hi_to_f32(pr[u][0]), bf16_lo_to_f32(pr[u][1]),
+                   bf16_hi_to_f32(pr[u][1])} * w;
+    }
+  }
+  const float inv = a.out_scale / den;
+  u32x2_t w = {pack_bf16x2(o[0] * inv, o[1] * inv), pack_bf16x2(o[2] * inv, o[3] * inv)};
+  *reinterpret_cast<u32x2_t*>(a.out + ((int64_t)tq * a.Hq + head) * 512 + d) = w;
+}
+
 // Merge of the balanced plan.  grid = (Hq, rows); block = 128 threads, 4 dims each.
 __global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const MlaDecodeArgs a) {
   const int head = blockIdx.x, seq = blockIdx.y;
@@ -628,22 +667,8 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const Mla
     const int part = ((int64_t)wj * pw >= extent_first) ? 0 : 1;
     return ((int64_t)wj * 2 + part) * 128 + (head & 127);
   };
-  float mstar = -INFINITY;
-  for (int wj = w_first; wj <= w_last; ++wj) mstar = fmaxf(mstar, a.ws_ml[slot_of(wj) * 2]);
-  float den = 0.f;
-  f32x4_t o = {0.f, 0.f, 0.f, 0.f};
-  const int d = threadIdx.x * 4;
-  for (int wj = w_first; wj <= w_last; ++wj) {
-    const int64_t slot = slot_of(wj);
-    const float w = fast_exp2(a.ws_ml[slot * 2] - mstar);
-    den += a.ws_ml[slot * 2 + 1] * w;
-    const u32x2_t pr = *reinterpret_cast<const u32x2_t*>(a.ws_o + slot * 512 + d);
-    o += f32x4_t{bf16_lo_to_f32(pr[0]), bf16_hi_to_f32(pr[0]), bf16_lo_to_f32(pr[1]), bf16_hi_to_f32(pr[1])} * w;
-  }
-  const float inv = a.out_scale / den;
-  const int tq = a.pt.cu_q_lens[seq];
-  u32x2_t w = {pack_bf16x2(o[0] * inv, o[1] * inv), pack_bf16x2(o[2] * inv, o[3] * inv)};
-  *reinterpret_cast<u32x2_t*>(a.out + ((int64_t)tq * a.Hq + head) * 512 + d) = w;
+  const int tq = scalar_load_i32(a.pt.cu_q_lens + seq);
+  mla_merge(a, w_last - w_first + 1, [&](int j) { return slot_of(w_first + j); }, head, tq);
 }
 
 // grid = (Hq, rows); block = 128 threads, 4 dims each.
@@ -657,22 +682,7 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_kernel(const MlaDecodeArg
   const int n = min(a.max_splits, (kv_len - t0 + a.chunk - 1) / a.chunk);
   if (n <= 0) return;
   const int64_t base = ((int64_t)row_id * a.max_splits) * a.Hq + head;
-  float mstar = -INFINITY;
-  for (int j = 0; j < n; ++j) mstar = fmaxf(mstar, a.ws_ml[(base + (int64_t)j * a.Hq) * 2]);
-  float den = 0.f;
-  f32x4_t o = {0.f, 0.f, 0.f, 0.f};
-  const int d = threadIdx.x * 4;
-  for (int j = 0; j < n; ++j) {
-    const int64_t slot = base + (int64_t)j * a.Hq;
-    const float w = fast_exp2(a.ws_ml[slot * 2] - mstar);
-    den += a.ws_ml[slot * 2 + 1] * w;
-    const u32x2_t pr = *reinterpret_cast<const u32x2_t*>(a.ws_o + slot * 512 + d);
-    o += f32x4_t{bf16_lo_to_f32(pr[0]), bf16_hi_to_f32(pr[0]), bf16_lo_to_f32(pr[1]), bf16_hi_to_f32(pr[1])} * w;
-  }
-  const float inv = a.out_scale / den;
-  const int tq = mr.tq;
-  u32x2_t w = {pack_bf16x2(o[0] * inv, o[1] * inv), pack_bf16x2(o[2] * inv, o[3] * inv)};
-  *reinterpret_cast<u32x2_t*>(a.out + ((int64_t)tq * a.Hq + head) * 512 + d) = w;
+  mla_merge(a, n, [&](int jj) { return base + (int64_t)jj * a.Hq; }, head, mr.tq);
 }
 
 // New latent rows into the paged cache (mla/v1/ref.py:56-105): token j of sequence i goes to
@@ -712,7 +722,8 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   const bool uniform = (a.pt.page_size % kTok) == 0;
   const bool cap = a.sm.soft_cap != 0.f;
   // the assembly tile loop: whole tiles inside one page, every wave of a workgroup at work
-  static const bool use_pipe = [] { const char* v = getenv("RPA_MLA_PIPE"); return !(v && *v == '0'); }();
+  const char* pipe_env = getenv("RPA_MLA_PIPE");  // read per call: tests switch it
+  const bool use_pipe = !(pipe_env && *pipe_env == '0');
   const int P = a.pt.page_size;
   const bool pipe = use_pipe && uniform && !cap && (P & (P - 1)) == 0 && (a.Hq % 128) == 0 &&
                     (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);

@@ -341,6 +341,37 @@ def test_mla_peaked_long_rows_against_oracle(pkg, wl, gpu, case):
             assert_parity(run_gpu(pkg, b, gpu, num_splits=ns)[:T].float(), want.float(), **TOL)
 
 
+@pytest.mark.parametrize("window", [None, 3000])
+def test_mla_assembly_loop_against_compiled_loop(pkg, wl, gpu, window, monkeypatch):
+    """128 heads and 64-token pages: whole unmasked tiles run inside the assembly loop
+    (rpa_mla_pipe_loop.inc), the first tile, window-edge tiles and the last tiles of a row in the
+    compiled step.  Rows from one tile to 400, ends on and off tile borders, with and without planted
+    keys (which send the loop through its reference-raising path), every plan: against the oracle
+    and against the same call with the loop switched off (RPA_MLA_PIPE=0)."""
+    kv_lens = [1, 31, 32, 33, 96, 127, 128, 129, 160, 161, 1000, 2048, 4097, 6001, 12800, 9999]
+    for needles in (False, True):
+        b = wl.make_mla_batch("mla_pipe", [1] * len(kv_lens), kv_lens, num_q_heads=128, lkv_dim=512, rope_dim=64,
+                              page_size=64, seed=8600 + needles, sliding_window=window)
+        if needles:
+            wl.plant_mla_needles(b, seed=5)
+        want = oracle(b)
+        for kw in ({}, {"num_splits": 1}, {"num_splits": 3}, {"num_splits": 40}):
+            say(f"mla assembly loop window={window} needles={needles} {kw}")
+            monkeypatch.setenv("RPA_MLA_PIPE", "1")
+            on = run_gpu(pkg, b, gpu, **kw)[:len(kv_lens)]
+            monkeypatch.setenv("RPA_MLA_PIPE", "0")
+            off = run_gpu(pkg, b, gpu, **kw)[:len(kv_lens)]
+            assert_parity(on.float(), want.float(), **TOL)
+            assert_parity(off.float(), want.float(), **TOL)
+            assert float(row_rel_error(on.float(), off.float()).max()) < 1e-2
+    # chunks on long prefixes: one row per query token
+    monkeypatch.setenv("RPA_MLA_PIPE", "1")
+    q_lens, kv_lens = [1, 70, 33], [5000, 4170, 1033]
+    b = wl.make_mla_batch("mla_pipe_chunks", q_lens, kv_lens, num_q_heads=128, lkv_dim=512, rope_dim=64, page_size=64,
+                          seed=8610, sliding_window=window)
+    assert_parity(run_gpu(pkg, b, gpu)[:sum(q_lens)].float(), oracle(b).float(), **TOL)
+
+
 @pytest.mark.parametrize("cap", [None, 30.0])
 def test_mla_scalar_scales(pkg, wl, gpu, cap):
     """q_scale, k_scale and v_scale of kernels/mla/v2/kernel.py:1354-1356: the logits are multiplied by
