@@ -424,7 +424,7 @@ __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kerne
   // Three phases, each a loop of its own (one loop that switches between the assembly block and the
   // general step would move the whole register state to a common place on every trip): general steps
   // up to the first steady-state step, the assembly loop, general steps to the end.
-  const bool has_fast = t_fb < t_fe;
+  const bool has_fast = t_fb < t_fe && row_sum_limit > -1.5f;  // (limit -2: a probe that keeps every step general)
   const int t_first = has_fast ? t_fb : nT + 1;
   int t = 0;
   for (; t < t_first; ++t) general_step(t);
