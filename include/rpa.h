@@ -159,7 +159,7 @@ typedef struct RpaMlaParams {
   const void* ql_nope;        /* bf16 [T, Hq, lkv_dim] */
   const void* q_pe;           /* bf16 [T, Hq, rope_dim] */
   void* out;                  /* bf16 [T, Hq, lkv_dim] */
-  const void* cache_kv;       /* bf16 [pages, P, row_stride] */
+  const void* cache_kv;       /* bf16 (or fp8-e4m3, see cache_dtype) [pages, P, row_stride] */
   const int32_t* kv_lens;
   const int32_t* page_indices;
   const int32_t* cu_q_lens;
@@ -193,6 +193,12 @@ typedef struct RpaMlaParams {
    * the static bound and rpa_mla_attention / rpa_mla_kv_write read distribution[2] on the device;
    * rpa_mla_decode (decode rows known on the host) does not take it. */
   const int32_t* distribution;
+  /* Element type of cache_kv (and of the rows rpa_mla_kv_write takes): RPA_KV_BF16 (0, the default) or
+   * RPA_KV_FP8_E4M3 -- latent rows of one byte per element, expanded to bf16 on their way through
+   * LDS; k_scale / v_scale above are their dequantisation scales (kernels/mla/v1/ref.py:223-226,
+   * 241-242).  row_stride and rope_offset stay in elements (multiples of 16 for fp8). */
+  int32_t cache_dtype;
+  int32_t reserved0;
 } RpaMlaParams;
 
 /* Library version (RPA_VERSION of the build). */

@@ -137,6 +137,8 @@ class RpaMlaParams(ctypes.Structure):
         ("k_scale", ctypes.c_float),
         ("v_scale", ctypes.c_float),
         ("distribution", ctypes.c_void_p),
+        ("cache_dtype", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
     ]
 
 

@@ -676,6 +676,11 @@ static int mla_validate(const RpaMlaParams* p) {
   if (p->row_stride < p->rope_offset + p->rope_dim || p->rope_offset < p->lkv_dim || (p->row_stride % 8) != 0 ||
       (p->rope_offset % 8) != 0)
     return fail(RPA_EINVAL_SHAPE, "row_stride=%d rope_offset=%d do not describe [kv_c | k_pe]", p->row_stride, p->rope_offset);
+  if (p->cache_dtype != RPA_KV_BF16 && p->cache_dtype != RPA_KV_FP8_E4M3)
+    return fail(RPA_EINVAL_SHAPE, "cache_dtype=%d is neither RPA_KV_BF16 nor RPA_KV_FP8_E4M3", p->cache_dtype);
+  if (p->cache_dtype == RPA_KV_FP8_E4M3 && ((p->row_stride % 16) != 0 || (p->rope_offset % 16) != 0))
+    return fail(RPA_EINVAL_SHAPE, "fp8 latent rows: row_stride=%d and rope_offset=%d must be multiples of 16", p->row_stride,
+                p->rope_offset);
   if (p->sliding_window < 0) return fail(RPA_EINVAL_WINDOW, "sliding_window=%d must be positive", p->sliding_window);
   if (p->num_seqs > 0 && (!p->ql_nope || !p->q_pe || !p->out || !p->cache_kv || !p->kv_lens || !p->page_indices || !p->cu_q_lens))
     return fail(RPA_EINVAL_NULL, "a required buffer is NULL");
@@ -750,6 +755,7 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   a.sm = softmax_opts(logit_scale, p->soft_cap, p->mask_value, p->sliding_window);
   a.out_scale = p->v_scale > 0.f ? p->v_scale : 1.0f;
   a.dist = p->distribution;
+  a.fp8 = p->cache_dtype == RPA_KV_FP8_E4M3 ? 1 : 0;
   if (p->distribution && !token_rows)
     return fail(RPA_EUNSUPPORTED, "rpa_mla_decode takes the batch composition from the host: use rpa_mla_attention");
   a.num_rows = (int32_t)rows;
@@ -809,8 +815,9 @@ int rpa_mla_kv_write(const RpaMlaParams* p, const void* new_kv_c, const void* ne
   a.pt.cu_kv_lens = p->cu_kv_lens;
   a.pt.pages_per_seq = p->pages_per_seq;
   a.pt.page_size = p->page_size;
-  a.new_kv_c = static_cast<const uint16_t*>(new_kv_c);
-  a.new_k_pe = static_cast<const uint16_t*>(new_k_pe);
+  a.new_kv_c = static_cast<const char*>(new_kv_c);
+  a.new_k_pe = static_cast<const char*>(new_k_pe);
+  a.fp8 = p->cache_dtype == RPA_KV_FP8_E4M3 ? 1 : 0;
   a.num_tokens = p->num_tokens;
   a.num_seqs = p->num_seqs;
   a.dist = p->distribution;

@@ -122,7 +122,7 @@ struct MlaDecodeArgs {
   const uint16_t* ql_nope;  // [T, Hq, lkv]
   const uint16_t* q_pe;     // [T, Hq, rope]
   uint16_t* out;            // [T, Hq, lkv]
-  const char* cache;        // [pages, P, row_stride] bf16
+  const char* cache;        // [pages, P, row_stride] bf16 or e4m3
   PageTable pt;
   SoftmaxOpts sm;
   uint16_t* ws_o;  // [T, max_splits, Hq, lkv] unnormalised partial outputs, bf16
@@ -145,13 +145,15 @@ struct MlaDecodeArgs {
   int32_t* cu_tiles;  // [num_rows + 1] prefix sum of tiles, written by the kernel
   float out_scale;    // finished rows are multiplied by it (v_scale; 1 when off)
   const int32_t* dist;  // device i32[3] or nullptr: when given, num_seqs is only a bound on dist[2]
+  int32_t fp8;          // cache rows are e4m3 bytes (row_stride / rope_offset stay in elements)
 };
 
 struct MlaWriteArgs {
   char* cache;              // [pages, P, row_stride] bf16
   PageTable pt;
-  const uint16_t* new_kv_c;  // [T, 512]
-  const uint16_t* new_k_pe;  // [T, 64]
+  const char* new_kv_c;  // [T, 512] in the cache's element type
+  const char* new_k_pe;  // [T, 64]
+  int32_t fp8;
   int32_t num_tokens;
   int32_t num_seqs;
   int32_t row_stride;

@@ -38,6 +38,12 @@ constexpr int kChunks = 74;              // 16-byte chunks per row (72 data + 2 
 constexpr int kUsedBlocks = 37;          // copy blocks of 64 chunks that hold a tile (32 rows x 74 chunks)
 constexpr int kSlotB = kUsedBlocks * 1024;  // one ring slot
 constexpr int kCopiesPerWave = 5;        // every wave issues 5 copy instructions per tile
+// fp8 caches: a tile arrives as bytes in a staging area (rows of 576 bytes, no padding: 18 copy
+// blocks) and is expanded to the bf16 layout above by all waves together
+constexpr int kF8Chunks = 36;            // 16-byte chunks per staged row
+constexpr int kF8Blocks = 18;            // copy blocks per staged tile (32 rows x 36 chunks)
+constexpr int kF8StageB = kF8Blocks * 1024;
+constexpr int kF8CopiesPerWave = 3;      // 8 x 3 = 24 copy instructions cover 18 blocks (the rest repeat block 0)
 
 __device__ __forceinline__ u32x4_t lds_ld16(const char* p) { return *reinterpret_cast<const u32x4_t*>(p); }
 
@@ -120,6 +126,61 @@ __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* 
   }
 }
 
+// fp8 caches: the same copy, of a tile of bytes into a staging area.  Position p = 64 * block + lane
+// is chunk p % 36 of row p / 36; chunks 0..31 are kv_c, 32..35 k_pe.
+template <bool UNIFORM>
+__device__ __forceinline__ void copy_tile_f8(char* stage, const Src& s, const char* cache, int tb, int wave, int lane,
+                                             int page) {
+  tb = min(tb, s.last_tok & ~(kTok - 1));
+  const bool whole = UNIFORM && (tb + kTok - 1 <= s.last_tok);
+  const char* base = cache + (int64_t)page * s.page_stride + (int64_t)(tb - page_slot(s, tb) * s.page_size) * s.row_bytes;
+  int ln = lane;
+  asm volatile("" : "+v"(ln));
+#pragma unroll
+  for (int n = 0; n < kF8CopiesPerWave; ++n) {
+    int blk = wave * kF8CopiesPerWave + n;
+    if (blk >= kF8Blocks) blk = 0;
+    const int p = blk * 64 + ln;
+    const int row = p / kF8Chunks;
+    const int j = p - row * kF8Chunks;
+    const int inner = j < 32 ? j * 16 : s.rope_byte + (j - 32) * 16;
+    if (whole) {
+      async_copy16(base + (uint32_t)(row * s.row_bytes + inner), stage + blk * 1024);
+    } else {  // last, partial tile (rows clamped to the last valid token) or pages smaller than a tile
+      const int tok = min(tb + row, s.last_tok);
+      const int ps = page_slot(s, tok);
+      const int pg = UNIFORM ? page : s.pages[ps];
+      async_copy16(cache + (int64_t)pg * s.page_stride + (int64_t)(tok - ps * s.page_size) * s.row_bytes + inner,
+                   stage + blk * 1024);
+    }
+  }
+}
+
+// e4m3 bytes of a staged tile -> bf16 rows of a ring slot (exact).  512 threads, 1152 chunks of 16
+// elements: three rounds, the last one a quarter full.
+__device__ __forceinline__ void expand_f8_tile(const char* stage, char* slot, int tid) {
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    const int p = tid + 512 * i;
+    if (p < kTok * kF8Chunks) {
+      const int row = p / kF8Chunks;
+      const int j = p - row * kF8Chunks;
+      const u32x4_t w = lds_ld16(stage + p * 16);
+      u32x4_t lo, hi;
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        lo[2 * d] = fp8x2_to_bf16x2(w[d], false);
+        lo[2 * d + 1] = fp8x2_to_bf16x2(w[d], true);
+        hi[2 * d] = fp8x2_to_bf16x2(w[2 + d], false);
+        hi[2 * d + 1] = fp8x2_to_bf16x2(w[2 + d], true);
+      }
+      char* dst = slot + row * kRowB + j * 32;
+      *reinterpret_cast<u32x4_t*>(dst) = lo;
+      *reinterpret_cast<u32x4_t*>(dst + 16) = hi;
+    }
+  }
+}
+
 // Sequence that owns query token `row`: the last one whose first token is <= row
 // (zero-length sequences are skipped).  cu_q_lens[0 .. num_seqs] is non-decreasing.
 __device__ __forceinline__ int owner_of_token(const int32_t* cu_q_lens, int num_seqs, int row) {
@@ -180,7 +241,10 @@ struct MlaDest {
 // assembly loop of rpa_mla_pipe_loop.inc (same LDS ring, same copy protocol, same registers as the
 // compiled step, which still does the first tile, masked tiles and the last three before a
 // partial one).  Needs UNIFORM pages of a power-of-two size, no soft cap, every wave at work.
-template <bool UNIFORM, bool CAP, bool PIPE = false>
+// FP8: the cache holds e4m3 bytes.  Slots 0 and 1 are the bf16 ring, slot 2 (two halves) and slot 3 three
+// staging areas; a step copies the bytes of tile k + 3, multiplies tile k, and ends by expanding tile
+// k + 1 between two barriers.
+template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false>
 __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
                                             int t_begin, int t_end, const MlaDest dest, char* slot0, char* slot1,
                                             char* slot2, char* slot3) {
@@ -199,9 +263,9 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   src.last_tok = kv_len - 1;
   src.pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[seq] / a.pt.page_size)
                                                   : (int64_t)seq * a.pt.pages_per_seq);
-  src.row_bytes = a.row_stride * 2;
+  src.row_bytes = a.row_stride * (FP8 ? 1 : 2);
   src.page_stride = (int64_t)src.row_bytes * a.pt.page_size;
-  src.rope_byte = a.rope_offset * 2;
+  src.rope_byte = a.rope_offset * (FP8 ? 1 : 2);
   auto page_of = [&](int tb) -> int {
     if constexpr (UNIFORM) {
       tb = min(tb, src.last_tok & ~(kTok - 1));
@@ -245,21 +309,43 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   // ---- pipeline: copies run three tiles ahead of the MFMAs (4-slot ring, 148 of the CU's 160 KiB:
   // 111 KiB per CU in flight, which is what HBM latency under load asks for) ----
   int pg_next = page_of(t_begin + 3 * kTok);
-  copy_tile<UNIFORM>(slot0, src, a.cache, t_begin, wave, lane, page_of(t_begin));
-  copy_tile<UNIFORM>(slot1, src, a.cache, t_begin + kTok, wave, lane, page_of(t_begin + kTok));
-  copy_tile<UNIFORM>(slot2, src, a.cache, t_begin + 2 * kTok, wave, lane, page_of(t_begin + 2 * kTok));
+  auto stage_of = [&](int i) -> char* { return i == 0 ? slot2 : (i == 1 ? slot2 + kF8StageB : slot3); };
+  if constexpr (FP8) {
+    copy_tile_f8<UNIFORM>(stage_of(0), src, a.cache, t_begin, wave, lane, page_of(t_begin));
+    copy_tile_f8<UNIFORM>(stage_of(1), src, a.cache, t_begin + kTok, wave, lane, page_of(t_begin + kTok));
+    copy_tile_f8<UNIFORM>(stage_of(2), src, a.cache, t_begin + 2 * kTok, wave, lane, page_of(t_begin + 2 * kTok));
+  } else {
+    copy_tile<UNIFORM>(slot0, src, a.cache, t_begin, wave, lane, page_of(t_begin));
+    copy_tile<UNIFORM>(slot1, src, a.cache, t_begin + kTok, wave, lane, page_of(t_begin + kTok));
+    copy_tile<UNIFORM>(slot2, src, a.cache, t_begin + 2 * kTok, wave, lane, page_of(t_begin + 2 * kTok));
+  }
   // Touch every Q^T register here: the compiler then waits for the Q loads now, instead of
   // re-checking them with s_waitcnt vmcnt(0..4) inside the loop, where such a wait would also
   // drain the copy queue.
 #pragma unroll
   for (int ks = 0; ks < 18; ++ks) asm volatile("" ::"v"(qB[ks]));
   // wait for the first tile (all but the 10 newest copies), then meet
-  __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kCopiesPerWave));
+  constexpr int kAhead = 2 * (FP8 ? kF8CopiesPerWave : kCopiesPerWave);  // copies of the two tiles behind the next one
+  __builtin_amdgcn_s_waitcnt(0x0F70 | kAhead);
   __syncthreads();
+  auto bare_barrier = [&]() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  // expand the staged tile `from` into ring slot `to`: every wave's bytes have landed (wait + barrier
+  // before), every wave's LDS writes are done before the barrier behind it
+  auto expand = [&](const char* from, char* to) {
+    expand_f8_tile(from, to, tid);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0) only: the copies in flight stay in flight
+    bare_barrier();
+  };
+  if constexpr (FP8) expand(stage_of(0), slot0);
 
-  auto tile_step = [&](const char* cur, char* fill, int tb) {
+  auto tile_step = [&](const char* cur, char* fill, int tb, const char* next_stage = nullptr, char* next_slot = nullptr) {
     // `fill` held tile tb - 32, which every wave finished before the last barrier
-    copy_tile<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane, pg_next);
+    if constexpr (FP8) copy_tile_f8<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane, pg_next);
+    else copy_tile<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane, pg_next);
     pg_next = page_of(tb + 4 * kTok);
     if (wave_on) {
       // two independent accumulator chains (token halves), issued alternately
@@ -324,12 +410,18 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     // wait for ALL outstanding copies, which would shorten the prefetch distance to one tile.
     // Every LDS read of this tile has returned (its MFMA consumed it) before the barrier, and
     // each wave has waited for its own share of the next tile, so no fence is needed.
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kCopiesPerWave));
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | kAhead);
+    bare_barrier();
+    if constexpr (FP8) expand(next_stage, next_slot);  // tile tb + 32 becomes bf16 rows
   };
-  if constexpr (!PIPE) {
+  if constexpr (FP8) {
+    int k3 = 0;  // k mod 3
+    for (int k = 0, tb = t_begin; tb < t_end; ++k, tb += kTok) {
+      const int n3 = k3 == 2 ? 0 : k3 + 1;
+      tile_step((k & 1) ? slot1 : slot0, stage_of(k3), tb, stage_of(n3), (k & 1) ? slot0 : slot1);
+      k3 = n3;
+    }
+  } else if constexpr (!PIPE) {
     for (int tb = t_begin; tb < t_end; tb += 4 * kTok) {
       tile_step(slot0, slot3, tb);
       if (tb + kTok >= t_end) break;
@@ -449,7 +541,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
 }
 
 // ---- fixed split plan: grid = (max_splits, rows, head groups of 128); block = 512 threads
-template <bool UNIFORM, bool CAP, bool PIPE = false>
+template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false>
 __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeArgs a) {
   // three separate arrays: lets the compiler see that a copy into one slot does not alias the
   // reads of another, so it does not drain the vector-memory queue before LDS reads
@@ -471,7 +563,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   MlaDest dest;
   dest.final_rows = a.max_splits == 1;
   dest.base = ((int64_t)row_id * a.max_splits + split) * a.Hq;
-  mla_segment<UNIFORM, CAP, PIPE>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
+  mla_segment<UNIFORM, CAP, PIPE, FP8>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
 }
 
 // ---- balanced plan (one row per sequence): the 32-token tiles of the whole batch, sequence by
@@ -504,7 +596,7 @@ __device__ __forceinline__ int mla_tiles_per_wg(const MlaDecodeArgs& a, int tota
   return max(a.forced_tiles_per_wg > 0 ? a.forced_tiles_per_wg : a.min_tiles_per_wg, even);
 }
 
-template <bool UNIFORM, bool CAP, bool PIPE = false>
+template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false>
 __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecodeArgs a) {
   __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
@@ -594,7 +686,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
     dest.final_rows = (tile == 0) && (take == nt);
     dest.base = ((int64_t)wg * 2 + (first_piece ? 0 : 1)) * 128 - unit * 128;  // + head
     first_piece = false;
-    mla_segment<UNIFORM, CAP, PIPE>(a, mr, unit * 128, t_lo, t0 + tile * kTok,
+    mla_segment<UNIFORM, CAP, PIPE, FP8>(a, mr, unit * 128, t_lo, t0 + tile * kTok,
                                     min(kv_len, t0 + (tile + take) * kTok), dest, slot0, slot1, slot2, slot3);
     x += take;
     if (x < x_end && tile + take == nt && unit == units - 1) {
@@ -701,10 +793,13 @@ __global__ __launch_bounds__(128) void rpa_mla_kv_write_kernel(const MlaWriteArg
   const int32_t* pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[seq] / P)
                                                               : (int64_t)seq * a.pt.pages_per_seq);
   const int page = pages[pos / P];
-  char* row = a.cache + ((int64_t)page * P + (pos % P)) * a.row_stride * 2;
+  const int es = a.fp8 ? 1 : 2;  // bytes per element
+  char* row = a.cache + ((int64_t)page * P + (pos % P)) * a.row_stride * es;
   const int t = threadIdx.x;
-  if (t < 64) st16(row + t * 16, ld16(a.new_kv_c + (int64_t)tok * 512 + t * 8));
-  else if (t < 72) st16(row + a.rope_offset * 2 + (t - 64) * 16, ld16(a.new_k_pe + (int64_t)tok * 64 + (t - 64) * 8));
+  const int nc = 32 * es;  // 16-byte chunks of kv_c; k_pe has an eighth of that
+  if (t < nc) st16(row + t * 16, ld16(a.new_kv_c + ((int64_t)tok * 512 * es + t * 16)));
+  else if (t < nc + 4 * es)
+    st16(row + a.rope_offset * es + (t - nc) * 16, ld16(a.new_k_pe + ((int64_t)tok * 64 * es + (t - nc) * 16)));
 }
 
 }  // namespace
@@ -727,6 +822,36 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   const int P = a.pt.page_size;
   const bool pipe = use_pipe && uniform && !cap && (P & (P - 1)) == 0 && (a.Hq % 128) == 0 &&
                     (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);
+  if (a.fp8) {  // e4m3 caches: the compiled loop with the staged expansion
+    if (a.balanced) {
+      const dim3 bgrid(a.num_wgs);
+      if (uniform) {
+        if (cap) hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, true, false, true>), bgrid, block, 0, stream, a);
+        else hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, false, false, true>), bgrid, block, 0, stream, a);
+      } else {
+        if (cap) hipLaunchKernelGGL((rpa_mla_balanced_kernel<false, true, false, true>), bgrid, block, 0, stream, a);
+        else hipLaunchKernelGGL((rpa_mla_balanced_kernel<false, false, false, true>), bgrid, block, 0, stream, a);
+      }
+      hipError_t eb = hipGetLastError();
+      if (eb != hipSuccess) return eb;
+      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      return hipGetLastError();
+    }
+    if (uniform) {
+      if (cap) hipLaunchKernelGGL((rpa_mla_decode_kernel<true, true, false, true>), grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((rpa_mla_decode_kernel<true, false, false, true>), grid, block, 0, stream, a);
+    } else {
+      if (cap) hipLaunchKernelGGL((rpa_mla_decode_kernel<false, true, false, true>), grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((rpa_mla_decode_kernel<false, false, false, true>), grid, block, 0, stream, a);
+    }
+    hipError_t ef = hipGetLastError();
+    if (ef != hipSuccess) return ef;
+    if (a.max_splits > 1) {
+      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      ef = hipGetLastError();
+    }
+    return ef;
+  }
   if (a.balanced) {
     const dim3 bgrid(a.num_wgs);
     if (pipe) {

@@ -93,8 +93,10 @@ def mla_ragged_paged_attention(
         cache_kv = cache_kv.view(s[0], s[1] * s[2], s[3])
     if not (ql_nope.is_contiguous() and q_pe.is_contiguous() and cache_kv.is_contiguous()):
         raise ValueError("ql_nope, q_pe and cache_kv must be contiguous")
-    if not (ql_nope.dtype == q_pe.dtype == cache_kv.dtype == torch.bfloat16):
-        raise ValueError("Expected bfloat16 ql_nope, q_pe and cache_kv")
+    if not (ql_nope.dtype == q_pe.dtype == torch.bfloat16):
+        raise ValueError("Expected bfloat16 ql_nope and q_pe")
+    if cache_kv.dtype not in (torch.bfloat16, torch.float8_e4m3fn):
+        raise ValueError(f"Expected a bfloat16 or float8_e4m3fn latent cache, got {cache_kv.dtype}")
     T, Hq, lkv = ql_nope.shape
     rope = q_pe.shape[2]
     total_pages, page_size, width = cache_kv.shape
@@ -122,6 +124,7 @@ def mla_ragged_paged_attention(
     p.lkv_dim = lkv
     p.rope_dim = rope
     p.row_stride = width
+    p.cache_dtype = _lib.RPA_KV_FP8_E4M3 if cache_kv.dtype == torch.float8_e4m3fn else _lib.RPA_KV_BF16
     p.rope_offset = rope_offset
     p.page_size = page_size
     p.total_pages = total_pages

@@ -272,7 +272,8 @@ def config_c4(device="cpu", scale: float = 1.0, window: bool = False) -> Batch:
 
 
 def make_mla_batch(name, q_lens, kv_lens, *, num_q_heads, lkv_dim, rope_dim, page_size, seed,
-                   device="cpu", sm_scale=None, std=0.5, sliding_window=None, soft_cap=None) -> MlaBatch:
+                   device="cpu", sm_scale=None, std=0.5, sliding_window=None, soft_cap=None,
+                   kv_dtype=torch.bfloat16) -> MlaBatch:
     rng = np.random.Generator(np.random.PCG64(seed))
     q_lens = np.asarray(q_lens, dtype=np.int64)
     kv_lens = np.asarray(kv_lens, dtype=np.int64)
@@ -288,7 +289,7 @@ def make_mla_batch(name, q_lens, kv_lens, *, num_q_heads, lkv_dim, rope_dim, pag
         name=name,
         ql_nope=_normal((T, num_q_heads, lkv_dim), std, torch.bfloat16, device, seed * 7 + 1),
         q_pe=_normal((T, num_q_heads, rope_dim), std, torch.bfloat16, device, seed * 7 + 3),
-        cache_kv=_normal((pool_pages, page_size, lkv_dim + rope_dim), std, torch.bfloat16, device, seed * 7 + 2),
+        cache_kv=_normal((pool_pages, page_size, lkv_dim + rope_dim), std, kv_dtype, device, seed * 7 + 2),
         kv_lens=torch.from_numpy(kv_lens.astype(np.int32)).to(device),
         page_indices=torch.from_numpy(perm).to(device),
         cu_q_lens=torch.from_numpy(cu_q).to(device),
@@ -302,7 +303,7 @@ def make_mla_batch(name, q_lens, kv_lens, *, num_q_heads, lkv_dim, rope_dim, pag
     )
 
 
-def config_c5(device="cpu", scale: float = 1.0, num_q_heads: int = 128) -> MlaBatch:
+def config_c5(device="cpu", scale: float = 1.0, num_q_heads: int = 128, kv_dtype=torch.bfloat16) -> MlaBatch:
     """Absorbed-MLA decode, DeepSeek-V3 shape: 64 seqs x 1 token, 128 q heads,
     latent 512 + rope 64 (one shared 576-wide row per token), kv ~ U[2048,16384],
     P=64, values ~ N(0, 0.5), sm_scale 1/sqrt(192)."""
@@ -310,9 +311,10 @@ def config_c5(device="cpu", scale: float = 1.0, num_q_heads: int = 128) -> MlaBa
     rng = np.random.Generator(np.random.PCG64(seed))
     S = 64
     kv = rng.integers(_scaled(2048, scale), _scaled(16384, scale), size=S, endpoint=True)
-    return make_mla_batch("c5_deepseek_v3_mla_decode", np.ones(S, int), kv, num_q_heads=num_q_heads,
+    name = "c5_deepseek_v3_mla_decode" + ("" if kv_dtype == torch.bfloat16 else "_fp8")
+    return make_mla_batch(name, np.ones(S, int), kv, num_q_heads=num_q_heads,
                           lkv_dim=512, rope_dim=64, page_size=64, seed=seed, device=device,
-                          sm_scale=1.0 / math.sqrt(192.0))
+                          sm_scale=1.0 / math.sqrt(192.0), kv_dtype=kv_dtype)
 
 
 def config_c5_prefill(device="cpu", scale: float = 1.0, num_q_heads: int = 128, num_seqs: int = 4) -> MlaBatch:
@@ -408,7 +410,7 @@ def plant_mla_needles(b: MlaBatch, *, logit: float = 14.0, seed: int = 0, count:
         for t in pos:
             page = int(pages[cu_kv[i] // P + t // P])
             # the row is K and V at once: keep its random part (the value), add the needle
-            b.cache_kv[page, t % P, :W] = (b.cache_kv[page, t % P, :W].float() + a * u).to(torch.bfloat16)
+            b.cache_kv[page, t % P, :W] = (b.cache_kv[page, t % P, :W].float() + a * u).to(b.cache_kv.dtype)
         placed[i] = pos
     b.ql_nope, b.q_pe = qn.to(torch.bfloat16), qp.to(torch.bfloat16)
     return placed
@@ -493,7 +495,7 @@ def mla_decode_bytes(b: MlaBatch) -> int:
     kv = np.asarray(b.meta["kv_lens"], dtype=np.int64)
     T, Hq, lkv = b.ql_nope.shape
     width = b.cache_kv.shape[-1]
-    total = int(kv.sum()) * width * 2
+    total = int(kv.sum()) * width * b.cache_kv.element_size()
     total += T * Hq * width * 2 + T * Hq * lkv * 2
     total += int((-(-kv // b.page_size)).sum()) * 4 + (2 * len(kv) + 1) * 4
     return total

@@ -60,7 +60,7 @@ def test_struct_layout_matches_header(pkg):
     # ... and the device-side distribution pointer at the end
     assert ctypes.sizeof(pkg._lib.RpaParams) == 12 * 8 + 18 * 4 + 8 + 3 * 8 + 5 * 4 + 4 + 8  # incl. padding
     # 10 pointers / size_t + 13 int32 + 3 float + int64 + 3 float (+ tail padding)
-    assert ctypes.sizeof(pkg._lib.RpaMlaParams) == 10 * 8 + 13 * 4 + 3 * 4 + 8 + 3 * 4 + 4 + 8
+    assert ctypes.sizeof(pkg._lib.RpaMlaParams) == 10 * 8 + 13 * 4 + 3 * 4 + 8 + 3 * 4 + 4 + 8 + 2 * 4
 
 
 def base_params(pkg):

@@ -372,6 +372,84 @@ def test_mla_assembly_loop_against_compiled_loop(pkg, wl, gpu, window, monkeypat
     assert_parity(run_gpu(pkg, b, gpu)[:sum(q_lens)].float(), oracle(b).float(), **TOL)
 
 
+FP8 = torch.float8_e4m3fn
+FP8_TOL = dict(rtol=5e-2, atol=5e-2)
+
+
+def fp8_oracle(b, **kw):
+    """The oracle on the cache's values widened to bf16 (exact): what the kernels compute.  The
+    reference's jnp oracle itself rounds the NORMALISED probabilities to the cache's element type
+    (mla/v1/ref.py:237), which in e4m3 flushes every row of more than a few hundred tokens to zero;
+    its kernel keeps them in f32 (mla/v2/kernel.py:401-404), and so does this one."""
+    wide = b.to("cpu")
+    wide.cache_kv = wide.cache_kv.to(torch.bfloat16)
+    return oracle(wide, **kw)
+
+
+@pytest.mark.parametrize("P", [16, 32, 64])
+@pytest.mark.parametrize("Hq", [16, 128])
+def test_mla_fp8_latent_cache_decode(pkg, wl, gpu, P, Hq):
+    """e4m3 latent rows with k_scale / v_scale (mla/v2/kernel.py:1354-1356): decode rows of one to
+    sixty tiles, fixed and balanced plans."""
+    kv_lens = [1, 31, 32, 33, 129, 500, 1025, 1900]
+    say(f"mla fp8 decode P={P} Hq={Hq}")
+    b = wl.make_mla_batch("mla_fp8", [1] * len(kv_lens), kv_lens, num_q_heads=Hq, lkv_dim=512, rope_dim=64,
+                          page_size=P, seed=8700 + P, kv_dtype=FP8)
+    scales = dict(k_scale=0.75, v_scale=1.5)
+    want = fp8_oracle(b, **scales)
+    for kw in ({}, {"num_splits": 1}, {"num_splits": 3}):
+        got = run_gpu(pkg, b, gpu, **scales, **kw)[:len(kv_lens)]
+        assert torch.isfinite(got.float()).all()
+        assert_parity(got.float(), want.float(), **FP8_TOL, rel=1e-2)  # exact widening: the bf16 bar holds
+
+
+def test_mla_fp8_latent_cache_long_rows_and_chunks(pkg, wl, gpu):
+    """Balanced plan over ragged long rows with planted keys, then chunks on prefixes (one row per
+    query token) with a sliding window, all on an e4m3 cache."""
+    kv_lens = [3000 + 911 * i for i in range(24)]
+    b = wl.make_mla_batch("mla_fp8_long", [1] * len(kv_lens), kv_lens, num_q_heads=128, lkv_dim=512, rope_dim=64,
+                          page_size=64, seed=8710, kv_dtype=FP8)
+    wl.plant_mla_needles(b, seed=3)
+    want = fp8_oracle(b, k_scale=0.5)
+    assert float(want.float().pow(2).mean().sqrt()) > 0.1
+    say("mla fp8 long rows")
+    assert_parity(run_gpu(pkg, b, gpu, k_scale=0.5)[:len(kv_lens)].float(), want.float(), **FP8_TOL, rel=1e-2)
+    q_lens, kv_lens = [1, 1, 37, 64], [700, 90, 1200, 64]
+    for window in (None, 500):
+        say(f"mla fp8 chunks window={window}")
+        b = wl.make_mla_batch("mla_fp8_mixed", q_lens, kv_lens, num_q_heads=32, lkv_dim=512, rope_dim=64, page_size=32,
+                              seed=8711, kv_dtype=FP8, sliding_window=window)
+        assert_parity(run_gpu(pkg, b, gpu)[:sum(q_lens)].float(), fp8_oracle(b).float(), **FP8_TOL, rel=1e-2)
+
+
+def test_mla_fp8_new_rows_are_written_into_the_cache(pkg, wl, gpu):
+    """rpa_mla_kv_write on an e4m3 cache: the new rows (bytes) land in their slots, bit for bit."""
+    q_lens, kv_lens, P = [1, 5, 33], [40, 5, 100], 16
+    b = wl.make_mla_batch("mla_fp8_write", q_lens, kv_lens, num_q_heads=16, lkv_dim=512, rope_dim=64, page_size=P,
+                          seed=8720, kv_dtype=FP8)
+    cache = b.cache_kv
+    table = b.padded_page_indices().view(len(q_lens), -1)
+    T = sum(q_lens)
+    new_c = torch.empty(T, 512, dtype=FP8)
+    new_r = torch.empty(T, 64, dtype=FP8)
+    holed = cache.clone()
+    t = 0
+    for i, (ql, kv) in enumerate(zip(q_lens, kv_lens)):
+        for j in range(ql):
+            pos = kv - ql + j
+            page, row = int(table[i, pos // P]), pos % P
+            new_c[t], new_r[t] = cache[page, row, :512], cache[page, row, 512:576]
+            holed.view(torch.uint8)[page, row] = 0x7F  # NaN in e4m3fn
+            t += 1
+    g = b.to(gpu)
+    out, got_cache = pkg.mla_ragged_paged_attention(
+        g.ql_nope, g.q_pe, new_c.to(gpu), new_r.to(gpu), holed.to(gpu), g.kv_lens, g.page_indices, g.cu_q_lens,
+        g.cu_kv_lens, b.distribution.numpy(), sm_scale=b.sm_scale, max_kv_len=100)
+    torch.cuda.synchronize()
+    assert torch.equal(got_cache.cpu().view(torch.uint8), cache.view(torch.uint8))
+    assert_parity(out.cpu()[:T].float(), fp8_oracle(b).float(), **FP8_TOL, rel=1e-2)
+
+
 @pytest.mark.parametrize("cap", [None, 30.0])
 def test_mla_scalar_scales(pkg, wl, gpu, cap):
     """q_scale, k_scale and v_scale of kernels/mla/v2/kernel.py:1354-1356: the logits are multiplied by
