@@ -24,6 +24,13 @@ matching power of two) until the sum fits or eight rounds have passed.  No maxim
 across lanes.  Results do not depend on the reference: the normalisation divides it out, and the
 merge of partial rows takes whatever (reference, sum) pair a piece leaves.
 
+The loop is generated twice.  For bf16 caches as described.  For e4m3 caches (macros with F8 in their
+names) a tile arrives as bytes in one of three staging areas (18 copy blocks, three copy instructions
+per wave) and the ring has two bf16 slots: a step ends with a barrier (the bytes of tile t + 1 have
+landed), the expansion of that tile -- every thread reads up to three 16-byte chunks, converts them with
+v_cvt_scalef32_pk_bf16_fp8 and writes 32 bytes each into the ring slot the next step reads -- and a
+second barrier; six unrolled steps cover the two-slot ring and the three staging areas.
+
 Register use follows one table shared with the C++ side through the emitted constraint macros;
 waits for LDS data and the issue distances the hardware does not interlock come from the
 emitter of gen_prefill_pipe_loop.py.
@@ -43,9 +50,9 @@ AHEAD = int(os.environ.get("RPA_MLA_PIPE_AHEAD", 3))
 NBUF = 4
 
 ROW_B = 1184                 # bytes of a latent row in LDS
-SLOT_B = 37 * 1024           # one ring slot
-BLOCKS = 37                  # 1 KiB copy blocks per slot
-COPIES = 5                   # copy instructions per wave and tile
+F8 = False                   # which of the two loops is being generated (set by emit_text)
+BLOCKS = 37                  # 1 KiB copy blocks per tile (18 for a tile of bytes)
+COPIES = 5                   # copy instructions per wave and tile (3)
 
 # ---- vector registers
 O = 0                        # 32 accumulators of 4
@@ -56,10 +63,15 @@ E = 212                      # 8 exponent temporaries
 RING = 220                   # NBUF operand buffers of 4
 ML = 236                     # M, L, KBASE, VBASE (one operand of 4)
 M, L, KBASE, VBASE = 236, 237, 238, 239
-OFS = 240                    # per-lane byte offsets of the wave's 5 copies; lanes 5..7 of the operand are scratch
+OFS = 240                    # one operand of 8: per-lane byte offsets of the wave's copies first, scratch behind
 NEGM, PS, KADDR = 245, 246, 247
 VADDR, D, A = 248, 249, 250
 NUM_VGPR = 251
+# e4m3 caches: three copy offsets, then what the expansion needs of every thread
+F8_SRC = 243                 # byte offset of the thread's first chunk inside a staging area (16 * thread)
+F8_DST = [244, 245, 246]     # byte offsets of its three chunks inside a ring slot
+F8_TABLE = dict(NEGM=247, PS=248, KADDR=249, VADDR=250, D=251, A=252, NUM_VGPR=253)
+BF_TABLE = dict(NEGM=245, PS=246, KADDR=247, VADDR=248, D=249, A=250, NUM_VGPR=251)
 
 # ---- scalar registers used inside the block (all listed as clobbers)
 SB = 60                      # s[60:61] global base of the tile being copied
@@ -129,10 +141,11 @@ def softmax(check=True):
 def copy_group(n, fill_slot):
     """copy n of this wave: block 5 * wave + n of the slot (blocks past the 37th repeat block 0)"""
     a = f"s{ST[0]}"
+    dst = f"%[stage{fill_slot}]" if F8 else f"%[slot{fill_slot}]"
     return [Ins(f"s_add_u32 {a}, %[wave_blk], {n * 1024}", "salu"),
             Ins(f"s_cmp_lt_u32 {a}, {BLOCKS * 1024}", "salu"),
             Ins(f"s_cselect_b32 {a}, {a}, 0", "salu"),
-            Ins(f"s_add_u32 m0, {a}, %[slot{fill_slot}]", "salu"),
+            Ins(f"s_add_u32 m0, {a}, {dst}", "salu"),
             Ins("s_nop 0", "nop"),
             Ins(f"global_load_lds_dwordx4 {vr(OFS + n)}, s[{SB}:{SB + 1}]", "vmem", [OFS + n], [])]
 
@@ -159,17 +172,58 @@ def tile_scalars(em):
     em.raw(f"s_load_dword s{PGN}, %[pages], {t1}")
 
 
+def expansion(em, stage, slot):
+    """e4m3 caches: the staged bytes of the next tile become bf16 rows of ring slot `slot`.  Thread i owns chunks
+    i, i + 512 and (waves 0 and 1 only) i + 1024 of the tile's 1152 chunks of 16 elements."""
+    # registers that are idle between two steps: (bytes read, bf16 out) twice over, used alternately so that no
+    # conversion writes what an LDS write issued just before still reads
+    sets = [(RING, RING + 4), (RING + 12, E)]
+    em.emit(valu(f"v_add_u32 {vr(KADDR)}, %[stage{stage}], {vr(F8_SRC)}", [F8_SRC], [KADDR]))
+
+    def read(i):
+        src = sets[i & 1][0]
+        em.emit(Ins(f"ds_read_b128 {vr(src, 4)}, {vr(KADDR)} offset:{8192 * i}", "lds", [KADDR], rng(src, 4), lds_tag=("x", i)))
+
+    def convert_and_write(i):
+        src, tmp = sets[i & 1]
+        em.emit(valu(f"v_add_u32 {vr(VADDR)}, %[slot{slot}], {vr(F8_DST[i])}", [F8_DST[i]], [VADDR]))
+        for d in range(4):
+            lo = valu(f"v_cvt_scalef32_pk_bf16_fp8 {vr(tmp + 2 * d)}, {vr(src + d)}, 1.0", [src + d], [tmp + 2 * d])
+            lo.lds_need = [("x", i)]
+            em.emit(lo)
+            em.emit(valu(f"v_cvt_scalef32_pk_bf16_fp8 {vr(tmp + 2 * d + 1)}, {vr(src + d)}, 1.0 op_sel:[1,0,0]", [src + d],
+                         [tmp + 2 * d + 1]))
+        em.emit(Ins(f"ds_write_b128 {vr(VADDR)}, {vr(tmp, 4)}", "lds", [VADDR] + list(rng(tmp, 4)), []))
+        em.emit(Ins(f"ds_write_b128 {vr(VADDR)}, {vr(tmp + 4, 4)} offset:16", "lds", [VADDR] + list(rng(tmp + 4, 4)), []))
+        em.raw("s_nop 1", "nop")       # the address register is rewritten next: let the writes pick it up
+
+    read(0)
+    read(1)
+    convert_and_write(0)
+    convert_and_write(1)
+    em.raw(f"s_cmp_lt_u32 %[wave_blk], {2 * COPIES * 1024}")   # waves 0 and 1
+    em.raw(f"s_cbranch_scc0 L_expanded_{stage}_{slot}_%=")
+    read(2)
+    convert_and_write(2)
+    em.label(f"L_expanded_{stage}_{slot}_%=")
+    em.raw("s_waitcnt lgkmcnt(0)", "wait")
+    em.lds_queue = []
+    em.raw("s_barrier")
+
+
 def step(em, k):
-    """tile t in slot k; tile t + 3 goes to slot (k + 3) & 3"""
-    fill = (k + 3) & 3
+    """bf16: tile t in slot k, tile t + 3 goes to slot (k + 3) & 3.  e4m3: tile t in ring slot k & 1, the bytes of
+    tile t + 3 go to staging area k % 3, tile t + 1 (staging area (k + 1) % 3) is expanded into the other slot."""
+    fill = (k % 3) if F8 else ((k + 3) & 3)
+    cur = (k & 1) if F8 else k
     tile_scalars(em)
-    em.emit(valu(f"v_add_u32 {vr(KADDR)}, %[slot{k}], {vr(KBASE)}", [KBASE], [KADDR]))
-    em.emit(valu(f"v_add_u32 {vr(VADDR)}, %[slot{k}], {vr(VBASE)}", [VBASE], [VADDR]))
+    em.emit(valu(f"v_add_u32 {vr(KADDR)}, %[slot{cur}], {vr(KBASE)}", [KBASE], [KADDR]))
+    em.emit(valu(f"v_add_u32 {vr(VADDR)}, %[slot{cur}], {vr(VBASE)}", [VBASE], [VADDR]))
     for f in range(AHEAD):
         for x in frag_read(f):
             em.emit(x)
     copies = [] if "nocopy" in X else [copy_group(n, fill) for n in range(COPIES)]
-    copy_at = {4 + 6 * n: n for n in range(COPIES)}            # behind these matrix instructions of the first product
+    copy_at = {4 + (30 // COPIES) * n: n for n in range(COPIES)}   # behind these matrix instructions of the first product
     if "copypv" in X:
         copy_at = {38 + 6 * n: n for n in range(COPIES)}
     if "copyend" in X:
@@ -212,6 +266,8 @@ def step(em, k):
     em.raw(f"s_mov_b32 %[pg], s{PGN}")
     if "nobarrier" not in X:
         em.raw("s_barrier")
+    if F8:
+        expansion(em, (k + 1) % 3, (k + 1) & 1)
     em.raw("s_add_u32 %[t], %[t], 1")
     em.raw("s_cmp_lt_i32 %[t], %[t_end]")
 
@@ -264,43 +320,59 @@ def generate():
     em.raw(f"s_sub_u32 s{PMASK}, s{PMASK}, 1")
     em.raw(f"s_lshl_b32 s{PSTR}, %[row_bytes], %[pshift]")
     em.emit(valu(f"v_mul_f32 {vr(NEGM)}, -1.0, {vr(M)}", [M], [NEGM]))
-    # slot of tile t: (t & 3); the four copies of the step differ in their LDS constants only
-    a = f"s{ST[0]}"
-    em.raw(f"s_and_b32 {a}, %[t], 3")
-    for k in (1, 2, 3):
+    # the unrolled copies of the step differ in their LDS constants only: tile t takes copy t & 3 (bf16: four
+    # ring slots) or t % 6 (e4m3: two ring slots, three staging areas)
+    a, b = f"s{ST[0]}", f"s{ST[1]}"
+    n_steps = 6 if F8 else 4
+    if F8:
+        em.raw(f"s_mul_hi_u32 {a}, %[t], 0xaaaaaaab")
+        em.raw(f"s_lshr_b32 {a}, {a}, 2")                       # t / 6
+        em.raw(f"s_mul_i32 {a}, {a}, 6")
+        em.raw(f"s_sub_u32 {a}, %[t], {a}")
+    else:
+        em.raw(f"s_and_b32 {a}, %[t], 3")
+    for k in range(1, n_steps):
         em.raw(f"s_cmp_eq_u32 {a}, {k}")
         em.raw(f"s_cbranch_scc1 L_step_{k}_%=")
-    for k in range(4):
+    for k in range(n_steps):
         em.label(f"L_step_{k}_%=")
         step(em, k)
-        if k < 3:
+        if k < n_steps - 1:
             em.raw("s_cbranch_scc0 L_exit_%=")
         else:
             em.raw("s_cbranch_scc1 L_step_0_%=")
             em.raw("s_branch L_exit_%=")
-    for k in range(4):
+    for k in range(n_steps):
         rare_block(em, k)
     em.label("L_exit_%=")
     em.raw("s_nop 11", "nop")
     return em
 
 
-def emit_text():
+def emit_text(f8):
+    global F8, BLOCKS, COPIES, NEGM, PS, KADDR, VADDR, D, A, NUM_VGPR
+    F8 = f8
+    BLOCKS, COPIES = (18, 3) if f8 else (37, 5)
+    tab = F8_TABLE if f8 else BF_TABLE
+    NEGM, PS, KADDR, VADDR, D, A, NUM_VGPR = (tab[k] for k in ("NEGM", "PS", "KADDR", "VADDR", "D", "A", "NUM_VGPR"))
     em = generate()
     n_mfma = sum(1 for i in em.out if i.kind == "mfma")
     n_valu = sum(1 for i in em.out if i.kind in ("valu", "trans", "swap", "dot"))
-    text = (f"// {len(em.out)} lines, {n_mfma} matrix and {n_valu} vector instructions (four unrolled steps and their rare "
-            f"paths), {em.nops} padding wait states; {NUM_VGPR} vector registers\n")
-    binds = {f"O{i}": (O + 16 * i, 16) for i in range(8)}
-    binds.update({"Q0": (Q, 32), "Q1": (Q + 32, 32), "Q2": (Q + 64, 8), "ML": (ML, 4), "OFS": (OFS, 8)})
-    for name, (lo, n) in binds.items():
-        text += f'#define RPA_MLA_PIPE_C_{name} "{{{vr(lo, n)}}}"\n'
+    pre = "RPA_MLA_PIPE_F8" if f8 else "RPA_MLA_PIPE"
+    text = (f"// {'e4m3' if f8 else 'bf16'} caches: {len(em.out)} lines, {n_mfma} matrix and {n_valu} vector instructions "
+            f"({6 if f8 else 4} unrolled steps and their rare paths), {em.nops} padding wait states; {NUM_VGPR} vector registers\n")
+    if not f8:
+        binds = {f"O{i}": (O + 16 * i, 16) for i in range(8)}
+        binds.update({"Q0": (Q, 32), "Q1": (Q + 32, 32), "Q2": (Q + 64, 8), "ML": (ML, 4), "OFS": (OFS, 8)})
+        for name, (lo, n) in binds.items():
+            text += f'#define RPA_MLA_PIPE_C_{name} "{{{vr(lo, n)}}}"\n'
     lines = ['    "%s\\n"' % ins.text for ins in em.out]
-    text += "#define RPA_MLA_PIPE_ASM \\\n" + " \\\n".join(lines) + "\n"
-    clob = ['"v%d"' % r for r in list(range(S[0], ML)) + list(range(VADDR, NUM_VGPR))]
+    text += f"#define {pre}_ASM \\\n" + " \\\n".join(lines) + "\n"
+    clob = ['"v%d"' % r for r in list(range(S[0], ML)) + list(range(OFS + 8, NUM_VGPR))]
     clob += ['"s%d"' % r for r in SGPR_CLOBBERS]
-    text += "#define RPA_MLA_PIPE_CLOBBERS " + ", ".join(clob) + ', "vcc", "scc", "m0", "memory"\n'
-    print(f"MLA: {len(em.out)} lines, {n_mfma} MFMAs, {n_valu} vector, {em.nops} padding wait states, {NUM_VGPR} VGPRs")
+    text += f"#define {pre}_CLOBBERS " + ", ".join(clob) + ', "vcc", "scc", "m0", "memory"\n'
+    print(f"MLA {'e4m3' if f8 else 'bf16'}: {len(em.out)} lines, {n_mfma} MFMAs, {n_valu} vector, {em.nops} padding wait states, "
+          f"{NUM_VGPR} VGPRs")
     return text
 
 
@@ -310,7 +382,8 @@ def main():
             "// Steady-state tile loop of the absorbed-MLA kernels: tiles t .. t_end-1 of one wave (16 heads).  The\n"
             "// RPA_MLA_PIPE_C_* macros are the register constraints that bind the kernel's variables to the\n"
             "// registers the assembly uses.\n")
-    text += emit_text()
+    text += emit_text(False)
+    text += emit_text(True)
     with open(os.path.join(here, "rpa_mla_pipe_loop.inc"), "w") as f:
         f.write(text)
 

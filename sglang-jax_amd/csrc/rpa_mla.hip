@@ -128,6 +128,19 @@ __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* 
 
 // fp8 caches: the same copy, of a tile of bytes into a staging area.  Position p = 64 * block + lane
 // is chunk p % 36 of row p / 36; chunks 0..31 are kv_c, 32..35 k_pe.
+__device__ __forceinline__ int f8_copy_block(int wave, int n) {
+  const int blk = wave * kF8CopiesPerWave + n;
+  return blk < kF8Blocks ? blk : 0;
+}
+
+// row and byte offset inside a cached row of the chunk that lane `lane` moves with copy n of wave `wave`
+__device__ __forceinline__ void f8_chunk_of(const Src& s, int wave, int lane, int n, int& row, int& inner) {
+  const int p = f8_copy_block(wave, n) * 64 + lane;
+  row = p / kF8Chunks;
+  const int j = p - row * kF8Chunks;
+  inner = j < 32 ? j * 16 : s.rope_byte + (j - 32) * 16;
+}
+
 template <bool UNIFORM>
 __device__ __forceinline__ void copy_tile_f8(char* stage, const Src& s, const char* cache, int tb, int wave, int lane,
                                              int page) {
@@ -138,12 +151,9 @@ __device__ __forceinline__ void copy_tile_f8(char* stage, const Src& s, const ch
   asm volatile("" : "+v"(ln));
 #pragma unroll
   for (int n = 0; n < kF8CopiesPerWave; ++n) {
-    int blk = wave * kF8CopiesPerWave + n;
-    if (blk >= kF8Blocks) blk = 0;
-    const int p = blk * 64 + ln;
-    const int row = p / kF8Chunks;
-    const int j = p - row * kF8Chunks;
-    const int inner = j < 32 ? j * 16 : s.rope_byte + (j - 32) * 16;
+    const int blk = f8_copy_block(wave, n);
+    int row, inner;
+    f8_chunk_of(s, wave, ln, n, row, inner);
     if (whole) {
       async_copy16(base + (uint32_t)(row * s.row_bytes + inner), stage + blk * 1024);
     } else {  // last, partial tile (rows clamped to the last valid token) or pages smaller than a tile
@@ -414,13 +424,21 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     bare_barrier();
     if constexpr (FP8) expand(next_stage, next_slot);  // tile tb + 32 becomes bf16 rows
   };
-  if constexpr (FP8) {
-    int k3 = 0;  // k mod 3
-    for (int k = 0, tb = t_begin; tb < t_end; ++k, tb += kTok) {
-      const int n3 = k3 == 2 ? 0 : k3 + 1;
-      tile_step((k & 1) ? slot1 : slot0, stage_of(k3), tb, stage_of(n3), (k & 1) ? slot0 : slot1);
-      k3 = n3;
+  // compiled step for tile k of the segment, whichever ring it uses
+  auto step_at = [&](int k) {
+    const int tb = t_begin + k * kTok;
+    if constexpr (FP8) {
+      const int k3 = k % 3;
+      tile_step((k & 1) ? slot1 : slot0, stage_of(k3), tb, stage_of(k3 == 2 ? 0 : k3 + 1), (k & 1) ? slot0 : slot1);
+    } else {
+      const int c4 = k & 3, f4 = (k + 3) & 3;
+      tile_step(c4 == 0 ? slot0 : (c4 == 1 ? slot1 : (c4 == 2 ? slot2 : slot3)),
+                f4 == 0 ? slot0 : (f4 == 1 ? slot1 : (f4 == 2 ? slot2 : slot3)), tb);
     }
+  };
+  if constexpr (FP8 && !PIPE) {
+    const int nT = (t_end - t_begin + kTok - 1) / kTok;
+    for (int k = 0; k < nT; ++k) step_at(k);
   } else if constexpr (!PIPE) {
     for (int tb = t_begin; tb < t_end; tb += 4 * kTok) {
       tile_step(slot0, slot3, tb);
@@ -439,15 +457,11 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     int k0 = 1;
     if (t_begin < t_lo) k0 = max(k0, (t_lo - t_begin + kTok - 1) / kTok);
     const int k1 = min(nT, (kv_len - t_begin) / kTok - 3);
-    auto slot_of = [&](int k) -> char* {
-      k &= 3;
-      return k == 0 ? slot0 : (k == 1 ? slot1 : (k == 2 ? slot2 : slot3));
-    };
     typedef __attribute__((address_space(3))) char* lds_ptr_t;
     int k = 0;
     for (int phase = 0; phase < 2; ++phase) {
       const int stop = (phase == 0 && k0 < k1) ? k0 : nT;
-      for (; k < stop; ++k) tile_step(slot_of(k), slot_of(k + 3), t_begin + k * kTok);
+      for (; k < stop; ++k) step_at(k);
       if (k >= nT) break;
       // ---- tiles k .. k1 - 1 in assembly
       f32x16_t o[8];
@@ -470,11 +484,30 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
       u32x4_t ml = {__float_as_uint(m), __float_as_uint(l), (uint32_t)(cc * kRowB + gg * 16),
                     (uint32_t)((4 * gg + (cc >> 2)) * kRowB + (cc & 3) * 8)};
       u32x8_t ofs = {0, 0, 0, 0, 0, 0, 0, 0};
+      if constexpr (FP8) {
 #pragma unroll
-      for (int n = 0; n < kCopiesPerWave; ++n) {
-        int row, inner;
-        chunk_of(src, wave, ln, n, row, inner);
-        ofs[n] = (uint32_t)(row * src.row_bytes + inner);
+        for (int n = 0; n < kF8CopiesPerWave; ++n) {
+          int row, inner;
+          f8_chunk_of(src, wave, ln, n, row, inner);
+          ofs[n] = (uint32_t)(row * src.row_bytes + inner);
+        }
+        // what the expansion needs of this thread: where its chunks start in a staging area, where they go
+        int td = tid;
+        asm volatile("" : "+v"(td));
+        ofs[3] = (uint32_t)(td * 16);
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+          const int p = td + 512 * i;
+          const int row = p / kF8Chunks;
+          ofs[4 + i] = (uint32_t)(row * kRowB + (p - row * kF8Chunks) * 32);
+        }
+      } else {
+#pragma unroll
+        for (int n = 0; n < kCopiesPerWave; ++n) {
+          int row, inner;
+          chunk_of(src, wave, ln, n, row, inner);
+          ofs[n] = (uint32_t)(row * src.row_bytes + inner);
+        }
       }
       const uint32_t s0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)slot0);
       const uint32_t s1 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)slot1);
@@ -483,17 +516,31 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
       const uint32_t cache_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)a.cache);
       const uint32_t cache_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)a.cache >> 32));
       const int last_tile_tok = __builtin_amdgcn_readfirstlane(src.last_tok & ~(kTok - 1));
-      const int wave_blk = wave * kCopiesPerWave * 1024;
 #define C(n) RPA_MLA_PIPE_C_##n
-      asm volatile(RPA_MLA_PIPE_ASM
-                   : "+" C(O0)(o[0]), "+" C(O1)(o[1]), "+" C(O2)(o[2]), "+" C(O3)(o[3]), "+" C(O4)(o[4]),
-                     "+" C(O5)(o[5]), "+" C(O6)(o[6]), "+" C(O7)(o[7]), "+" C(ML)(ml), "+" C(OFS)(ofs),
-                     [t] "+s"(k), [pg] "+s"(pg_next)
-                   : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), [t_end] "s"(k1), [t_begin] "s"(t_begin),
-                     [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),
-                     [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2),
-                     [wave_blk] "s"(wave_blk), [slot0] "s"(s0), [slot1] "s"(s1), [slot2] "s"(s2), [slot3] "s"(s3)
-                   : RPA_MLA_PIPE_CLOBBERS);
+      if constexpr (FP8) {
+        const int wave_blk = wave * kF8CopiesPerWave * 1024;
+        asm volatile(RPA_MLA_PIPE_F8_ASM
+                     : "+" C(O0)(o[0]), "+" C(O1)(o[1]), "+" C(O2)(o[2]), "+" C(O3)(o[3]), "+" C(O4)(o[4]),
+                       "+" C(O5)(o[5]), "+" C(O6)(o[6]), "+" C(O7)(o[7]), "+" C(ML)(ml), "+" C(OFS)(ofs),
+                       [t] "+s"(k), [pg] "+s"(pg_next)
+                     : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), [t_end] "s"(k1), [t_begin] "s"(t_begin),
+                       [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),
+                       [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2),
+                       [wave_blk] "s"(wave_blk), [slot0] "s"(s0), [slot1] "s"(s1), [stage0] "s"(s2),
+                       [stage1] "s"(s2 + (uint32_t)kF8StageB), [stage2] "s"(s3)
+                     : RPA_MLA_PIPE_F8_CLOBBERS);
+      } else {
+        const int wave_blk = wave * kCopiesPerWave * 1024;
+        asm volatile(RPA_MLA_PIPE_ASM
+                     : "+" C(O0)(o[0]), "+" C(O1)(o[1]), "+" C(O2)(o[2]), "+" C(O3)(o[3]), "+" C(O4)(o[4]),
+                       "+" C(O5)(o[5]), "+" C(O6)(o[6]), "+" C(O7)(o[7]), "+" C(ML)(ml), "+" C(OFS)(ofs),
+                       [t] "+s"(k), [pg] "+s"(pg_next)
+                     : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), [t_end] "s"(k1), [t_begin] "s"(t_begin),
+                       [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),
+                       [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2),
+                       [wave_blk] "s"(wave_blk), [slot0] "s"(s0), [slot1] "s"(s1), [slot2] "s"(s2), [slot3] "s"(s3)
+                     : RPA_MLA_PIPE_CLOBBERS);
+      }
 #undef C
       m = __uint_as_float(ml[0]);
       l = __uint_as_float(ml[1]);
@@ -822,10 +869,12 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   const int P = a.pt.page_size;
   const bool pipe = use_pipe && uniform && !cap && (P & (P - 1)) == 0 && (a.Hq % 128) == 0 &&
                     (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);
-  if (a.fp8) {  // e4m3 caches: the compiled loop with the staged expansion
+  if (a.fp8) {  // e4m3 caches
     if (a.balanced) {
       const dim3 bgrid(a.num_wgs);
-      if (uniform) {
+      if (pipe) {
+        hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, false, true, true>), bgrid, block, 0, stream, a);
+      } else if (uniform) {
         if (cap) hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, true, false, true>), bgrid, block, 0, stream, a);
         else hipLaunchKernelGGL((rpa_mla_balanced_kernel<true, false, false, true>), bgrid, block, 0, stream, a);
       } else {
@@ -837,7 +886,9 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
       hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
       return hipGetLastError();
     }
-    if (uniform) {
+    if (pipe) {
+      hipLaunchKernelGGL((rpa_mla_decode_kernel<true, false, true, true>), grid, block, 0, stream, a);
+    } else if (uniform) {
       if (cap) hipLaunchKernelGGL((rpa_mla_decode_kernel<true, true, false, true>), grid, block, 0, stream, a);
       else hipLaunchKernelGGL((rpa_mla_decode_kernel<true, false, false, true>), grid, block, 0, stream, a);
     } else {
