@@ -6,6 +6,7 @@ static/dynamic_validate_inputs
 import ctypes
 import os
 import re
+import sys
 
 import numpy as np
 import pytest
@@ -196,3 +197,22 @@ def test_python_wrapper_raises_like_the_reference(pkg):
         m.static_validate_inputs(q, None, None, cache, torch.zeros(2, dtype=torch.int64), i32(2), i32(3), i32(3), i32(3))
     with pytest.raises(ValueError, match="Expected 3D"):
         m.static_validate_inputs(q, torch.zeros(4, 2), torch.zeros(4, 2), cache, i32(2), i32(2), i32(3), i32(3), i32(3))
+
+
+def test_generated_assembly_is_up_to_date(tmp_path):
+    """The two generated include files (the assembly loops of the prefill and MLA kernels) are what
+    their generators write today, with no experiment switch set."""
+    import shutil
+    import subprocess
+
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "sglang-jax_amd", "csrc")
+    work = tmp_path / "csrc"
+    work.mkdir()
+    for name in ("gen_prefill_pipe_loop.py", "gen_mla_pipe_loop.py"):
+        shutil.copy(os.path.join(csrc, name), work / name)
+    env = {k: v for k, v in os.environ.items() if not k.startswith(("RPA_PIPE_", "RPA_MLA_PIPE_"))}
+    env["PYTHONDONTWRITEBYTECODE"] = "1"
+    for gen, inc in (("gen_prefill_pipe_loop.py", "rpa_prefill_pipe_loop.inc"), ("gen_mla_pipe_loop.py", "rpa_mla_pipe_loop.inc")):
+        subprocess.run([sys.executable, str(work / gen)], check=True, env=env, stdout=subprocess.DEVNULL)
+        with open(work / inc) as f, open(os.path.join(csrc, inc)) as g:
+            assert f.read() == g.read(), f"{inc} is stale: run {gen}"
