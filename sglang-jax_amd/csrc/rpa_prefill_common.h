@@ -71,25 +71,29 @@ struct Work {
   bool valid;
 };
 
-__device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int nseq, bool by_level, int bm = kBM) {
+// `heads` query heads of a kv head per workgroup (1, or 4 when the waves of a workgroup take a head each):
+// Work.head is then the first of them.
+__device__ __forceinline__ Work decompose(const PrefillArgs& a, int tiles, int nseq, bool by_level, int bm = kBM,
+                                          int heads = 1) {
   Work w;
   w.valid = false;
   const int units = nseq * a.Hkv;
+  const int groups = a.G / heads;  // workgroups per (sequence, kv head, tile)
   int tile_rev, u, gi;
   if (units >= 8) {
     const int xcd = blockIdx.x & 7, r = blockIdx.x >> 3;
     const int units_per_xcd = (units + 7) >> 3;
-    const int per_tile = units_per_xcd * a.G;
+    const int per_tile = units_per_xcd * groups;
     tile_rev = r / per_tile;
     const int rest = r - tile_rev * per_tile;
-    u = xcd + 8 * (rest / a.G);
-    gi = rest % a.G;
+    u = xcd + 8 * (rest / groups);
+    gi = (rest % groups) * heads;
   } else {
-    const int per_tile = units * a.G;
+    const int per_tile = units * groups;
     tile_rev = blockIdx.x / per_tile;
     const int rest = blockIdx.x - tile_rev * per_tile;
-    u = rest / a.G;
-    gi = rest % a.G;
+    u = rest / groups;
+    gi = (rest % groups) * heads;
   }
   if (u >= units || tile_rev >= tiles) return w;
   const int si = u / a.Hkv;

@@ -263,7 +263,10 @@ __device__ __forceinline__ void pipe_loop(RowBlock (&b)[2], const Shared& sh, in
 #undef C
 }
 
-template <bool WIN, int NQ>
+// HEADS4: the short-chunk tile.  A workgroup owns 32 query positions of FOUR query heads of a kv head, one
+// head per wave, instead of 128 positions of one head: chunks of a few dozen tokens (a verify step, a short
+// prompt, the tail of a long one) then fill their tiles, and the four waves still share every K/V tile.
+template <bool WIN, int NQ, bool HEADS4 = false>
 __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kernel(const PrefillArgs a_in, int tiles, int nseq,
                                                                                  bool by_level, float row_sum_limit) {
   PrefillArgs a = a_in;  // static-shape mode: the sequences to process come from the device
@@ -271,14 +274,16 @@ __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kerne
     a.seq_begin = (a.sm.mask_mode == 1) ? 0 : scalar_load_i32(a.dist);
     a.seq_end = min(a.seq_end, scalar_load_i32(a.dist + 2));
   }
-  constexpr int BM = 128 * NQ;  // query rows per workgroup
+  static_assert(!HEADS4 || NQ == 1, "the short-chunk tile has one block of rows per wave");
+  constexpr int BM = HEADS4 ? 32 : 128 * NQ;  // query positions per workgroup
   __shared__ __attribute__((aligned(1024))) char lds[4 * kTileB];
 
-  const Work w = decompose(a, tiles, nseq, by_level, BM);
+  Work w = decompose(a, tiles, nseq, by_level, BM, HEADS4 ? 4 : 1);
   if (!w.valid) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if constexpr (HEADS4) w.head += wave;  // this wave's head
   const int c = lane & 31, h = lane >> 5;
   const TileSrc src = make_src(a, w);
   const char* kh = a.kv.k_base + (int64_t)w.hk * a.kv.head_stride;
@@ -287,7 +292,7 @@ __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kerne
   const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)lds);
 
   // rows of the wave: NQ blocks of 32
-  const int r_lo = w.q_start + wave * 32 * NQ;
+  const int r_lo = w.q_start + (HEADS4 ? 0 : wave * 32 * NQ);
   const int r_hi = min(r_lo + 32 * NQ - 1, w.q_len - 1);
   const bool active = r_lo < w.q_len;
   const int W_ = WIN ? a.sm.window : 0;
@@ -460,19 +465,27 @@ hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order,
   // a half's row sum above the limit sends a wave through the rescaling path (testing knob: -1 = always)
   static const float limit = [] { const char* v = getenv("RPA_PREFILL_PIPE_LIMIT"); return v ? (float)atof(v) : kRowSumLimit; }();
   const int nq = force_nq ? force_nq : 1;
-  const int bm = 128 * nq;
+  // Tile by shape (the reference's per-shape block sizes, tuned_block_sizes.py, have this one counterpart
+  // here): chunks of at most 64 tokens take 32 positions x 4 heads per workgroup when the heads come in fours
+  const char* tile_env = getenv("RPA_PREFILL_PIPE_TILE");  // 32 / 128 force a tile (read per call: tests switch it)
+  const int force_tile = tile_env ? atoi(tile_env) : 0;
+  const bool heads4 = nq == 1 && (a.G % 4) == 0 && (force_tile ? force_tile == 32 : a.max_q_len <= 64);
+  const int bm = heads4 ? 32 : 128 * nq;
   int tiles = (a.max_q_len + bm - 1) / bm;
   const int levels = a.max_kv_len > 0 ? (a.max_kv_len + bm - 1) / bm + 1 : 0;
   const bool by_level = level_order && levels > tiles && levels <= 2 * tiles + 2;
   if (by_level) tiles = levels;
   const int64_t units = (int64_t)nseq * a.Hkv;
-  const int64_t grid = (units >= 8 ? ((units + 7) / 8) * 8 : units) * a.G * tiles;
+  const int64_t grid = (units >= 8 ? ((units + 7) / 8) * 8 : units) * (heads4 ? a.G / 4 : a.G) * tiles;
   if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
   const dim3 g((unsigned)grid), blk(256);
   const bool win = a.sm.window > 0;
 #define RPA_LAUNCH(W, N) \
   hipLaunchKernelGGL((rpa_prefill_pipe_kernel<W, N>), g, blk, 0, stream, a, tiles, nseq, by_level, limit)
-  if (nq == 1) {
+  if (heads4) {
+    if (win) hipLaunchKernelGGL((rpa_prefill_pipe_kernel<true, 1, true>), g, blk, 0, stream, a, tiles, nseq, by_level, limit);
+    else hipLaunchKernelGGL((rpa_prefill_pipe_kernel<false, 1, true>), g, blk, 0, stream, a, tiles, nseq, by_level, limit);
+  } else if (nq == 1) {
     if (win) RPA_LAUNCH(true, 1);
     else RPA_LAUNCH(false, 1);
   } else {

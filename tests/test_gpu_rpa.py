@@ -620,6 +620,33 @@ def test_balanced_plan_long_shares_and_tiny_rows(pkg, wl, gpu, monkeypatch):
         assert torch.equal(auto, again)
 
 
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (16, 2), (8, 2)])
+def test_short_chunks_take_the_four_head_tile(pkg, wl, gpu, Hq, Hkv, monkeypatch):
+    """Chunks of at most 64 tokens run on workgroups of 32 positions x 4 query heads (one head per
+    wave) instead of 128 positions of one head.  Chunks of 2..64 tokens on prefixes of 0..5000 tokens,
+    with and without a window, plain and with planted keys: against the oracle and against the same
+    call forced onto the 128-position tile (RPA_PREFILL_PIPE_TILE)."""
+    q_lens = [1, 1, 2, 5, 16, 31, 32, 33, 64, 47]
+    kv_lens = [300, 5000, 2, 5, 4016, 31, 1056, 97, 64, 5047]
+    for window, needles in ((None, False), (None, True), (700, True)):
+        say(f"short chunks Hq={Hq} Hkv={Hkv} window={window} needles={needles}")
+        b = wl.make_batch("short_chunks", q_lens, kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=128, page_size=64,
+                          seed=4100 + Hq, sliding_window=window)
+        if needles:
+            wl.plant_needles(b, seed=7)
+        want = oracle_out(b)
+        monkeypatch.setenv("RPA_PREFILL_PIPE_TILE", "32")
+        small = gpu_out(pkg, b, gpu)
+        monkeypatch.setenv("RPA_PREFILL_PIPE_TILE", "128")
+        big = gpu_out(pkg, b, gpu)
+        monkeypatch.delenv("RPA_PREFILL_PIPE_TILE")
+        auto = gpu_out(pkg, b, gpu)
+        assert_parity(small.float(), want.float(), **BF16_TOL)
+        assert_parity(big.float(), want.float(), **BF16_TOL)
+        assert torch.equal(auto, small)  # every chunk here is at most 64 tokens long
+        assert float(row_rel_error(small.float(), big.float()).max()) < 1e-2
+
+
 def test_balanced_plan_merge_inside_the_kernel(pkg, wl, gpu, monkeypatch):
     """The opt-in single-launch form of the balanced plan (RPA_DECODE_MERGE_IN_KERNEL=1): the wave
     that arrives last at a cut row merges it, counted by one arrival word per (row, unit, wave)
