@@ -56,6 +56,17 @@ __device__ __forceinline__ u32x2_t lds_tr16(const char* p) {
   return __builtin_bit_cast(u32x2_t, v);
 }
 
+// The lane id behind a fence the compiler cannot see through: values derived from it are not common
+// subexpressions of anything earlier, so they are worked out again where they are used instead of being
+// kept in registers across code that has none to spare (the assembly loop pins 251 of a wave's 256; with
+// them carried over it, 23-37 registers went to scratch memory per segment, 100 MB a launch on a
+// prefill batch).  Taken from threadIdx: the same helper on v_mbcnt made the allocator spill 140.
+__device__ __forceinline__ int fresh_lane() {
+  int ln = (int)(threadIdx.x & 63);
+  asm volatile("" : "+v"(ln));
+  return ln;
+}
+
 // token (inside a tile) behind slot i = 4b + r of lane group g in the S^T result registers
 __device__ __forceinline__ int tok_of(int g, int i) {
   return 16 * (i >> 2) + 4 * g + (i & 3);
@@ -346,23 +357,29 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   // expand the staged tile `from` into ring slot `to`: every wave's bytes have landed (wait + barrier
   // before), every wave's LDS writes are done before the barrier behind it
   auto expand = [&](const char* from, char* to) {
-    expand_f8_tile(from, to, tid);
+    expand_f8_tile(from, to, PIPE ? wave * 64 + fresh_lane() : tid);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0) only: the copies in flight stay in flight
     bare_barrier();
   };
   if constexpr (FP8) expand(stage_of(0), slot0);
 
   auto tile_step = [&](const char* cur, char* fill, int tb, const char* next_stage = nullptr, char* next_slot = nullptr) {
+    // with the assembly loop in the same function every lane-dependent value is worked out here, per
+    // step, rather than carried over that loop
+    const int lane_t = PIPE ? fresh_lane() : lane;
+    const int c_t = PIPE ? (lane_t & 15) : c, g_t = PIPE ? (lane_t >> 4) : g;
+    const int k_off_t = PIPE ? (c_t * kRowB + g_t * 16) : k_off;
+    const int v_off_t = PIPE ? ((4 * g_t + (c_t >> 2)) * kRowB + (c_t & 3) * 8) : v_off;
     // `fill` held tile tb - 32, which every wave finished before the last barrier
-    if constexpr (FP8) copy_tile_f8<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane, pg_next);
-    else copy_tile<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane, pg_next);
+    if constexpr (FP8) copy_tile_f8<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane_t, pg_next);
+    else copy_tile<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane_t, pg_next);
     pg_next = page_of(tb + 4 * kTok);
     if (wave_on) {
       // two independent accumulator chains (token halves), issued alternately
       f32x4_t s[2];
       s[0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       s[1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      const char* kp = cur + k_off;
+      const char* kp = cur + k_off_t;
 #pragma unroll
       for (int ks = 0; ks < 18; ++ks) {
         s[0] = mfma16(lds_ld16(kp + ks * 64), qB[ks], s[0]);
@@ -382,7 +399,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
       if ((tb + kTok > kv_len) || (tb < t_lo)) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          const int tok = tb + tok_of(g, i);
+          const int tok = tb + tok_of(g_t, i);
           if (tok >= kv_len || tok < t_lo) x[i] = mask2;
         }
       }
@@ -405,7 +422,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
 #pragma unroll
         for (int j = 0; j < 32; ++j) acc[j] = acc[j] * alpha;
       }
-      const char* vp = cur + v_off;
+      const char* vp = cur + v_off_t;
 #pragma unroll
       for (int j = 0; j < 32; ++j) {
         const char* vt = vp + j * 32;
@@ -478,8 +495,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) q2[e] = qB[16 + (e >> 2)][e & 3];
-      int ln = lane;
-      asm volatile("" : "+v"(ln));  // the lane parts below are worked out here, not carried from the top
+      const int ln = fresh_lane();  // the lane parts below are worked out here, not carried from the top
       const int cc = ln & 15, gg = ln >> 4;
       u32x4_t ml = {__float_as_uint(m), __float_as_uint(l), (uint32_t)(cc * kRowB + gg * 16),
                     (uint32_t)((4 * gg + (cc >> 2)) * kRowB + (cc & 3) * 8)};
@@ -492,8 +508,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
           ofs[n] = (uint32_t)(row * src.row_bytes + inner);
         }
         // what the expansion needs of this thread: where its chunks start in a staging area, where they go
-        int td = tid;
-        asm volatile("" : "+v"(td));
+        const int td = wave * 64 + ln;
         ofs[3] = (uint32_t)(td * 16);
 #pragma unroll
         for (int i = 0; i < 3; ++i) {
@@ -516,6 +531,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
       const uint32_t cache_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)a.cache);
       const uint32_t cache_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)a.cache >> 32));
       const int last_tile_tok = __builtin_amdgcn_readfirstlane(src.last_tok & ~(kTok - 1));
+      const uint32_t scale2_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(scale2));
 #define C(n) RPA_MLA_PIPE_C_##n
       if constexpr (FP8) {
         const int wave_blk = wave * kF8CopiesPerWave * 1024;
@@ -525,7 +541,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
                        [t] "+s"(k), [pg] "+s"(pg_next)
                      : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), [t_end] "s"(k1), [t_begin] "s"(t_begin),
                        [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),
-                       [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2),
+                       [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2_bits),
                        [wave_blk] "s"(wave_blk), [slot0] "s"(s0), [slot1] "s"(s1), [stage0] "s"(s2),
                        [stage1] "s"(s2 + (uint32_t)kF8StageB), [stage2] "s"(s3)
                      : RPA_MLA_PIPE_F8_CLOBBERS);
@@ -537,7 +553,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
                        [t] "+s"(k), [pg] "+s"(pg_next)
                      : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), [t_end] "s"(k1), [t_begin] "s"(t_begin),
                        [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),
-                       [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2),
+                       [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2_bits),
                        [wave_blk] "s"(wave_blk), [slot0] "s"(s0), [slot1] "s"(s1), [slot2] "s"(s2), [slot3] "s"(s3)
                      : RPA_MLA_PIPE_CLOBBERS);
       }
@@ -559,6 +575,11 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   // trace back across the tile loop: hoisted out of it they would sit in registers the loop has
   // none to spare for (they were spilled to scratch memory).
   int c_out = c, g_out = g;
+  if constexpr (PIPE) {
+    const int ln = fresh_lane();
+    c_out = ln & 15;
+    g_out = ln >> 4;
+  }
   asm volatile("" : "+v"(c_out), "+v"(g_out));
   const int head = head0 + c_out;
   if (!wave_on || head >= a.Hq) return;
