@@ -225,6 +225,89 @@ def run_mla_config(pkg, wl, b, steps, warmup):
             "tflops": flops / (ms * 1e-3) / 1e12}
 
 
+# The reference's own published figures for this path: the perf-guard baselines of its TPU kernel
+# (benchmark/kernels/flash_attention/bench_flashattention.py:264-328; device time of the op in ms,
+# bf16, head_dim 128, 600 000-token pool; heads are per device).  key: (mode, page_size, tokens or
+# batch, q heads, kv heads) -> (TPU v6e, TPU v7).
+REFERENCE_PUBLISHED_MS = {
+    ("prefill", 128, 1024, 4, 1): (0.0334175, 0.014767107), ("prefill", 128, 1024, 4, 2): (0.05767375, 0.015102041),
+    ("prefill", 128, 1024, 8, 1): (0.04415, 0.022470588), ("prefill", 128, 1024, 8, 4): (0.0835275, 0.023110444),
+    ("prefill", 128, 4096, 4, 1): (0.19460875, 0.0794994), ("prefill", 128, 4096, 4, 2): (0.34417875, 0.084321729),
+    ("prefill", 128, 4096, 8, 1): (0.25254875, 0.145336134), ("prefill", 128, 4096, 8, 4): (0.50654375, 0.145752701),
+    ("prefill", 256, 1024, 4, 1): (0.03286125, 0.014686675), ("prefill", 256, 1024, 4, 2): (0.0571225, 0.015236495),
+    ("prefill", 256, 1024, 8, 1): (0.043765, 0.022472989), ("prefill", 256, 1024, 8, 4): (0.0829025, 0.023372149),
+    ("prefill", 256, 4096, 4, 1): (0.19131, 0.079831933), ("prefill", 256, 4096, 4, 2): (0.34008, 0.084252101),
+    ("prefill", 256, 4096, 8, 1): (0.25009625, 0.144997599), ("prefill", 256, 4096, 8, 4): (0.50262875, 0.145212485),
+    ("decode", 128, 128, 4, 1): (0.58231125, 0.15942617), ("decode", 128, 128, 4, 2): (0.3259175, 0.226237695),
+    ("decode", 128, 128, 8, 1): (0.5799825, 0.159394958), ("decode", 128, 128, 8, 4): (0.55449, 0.331831933),
+    ("decode", 128, 256, 4, 1): (1.1546875, 0.313444178), ("decode", 128, 256, 4, 2): (0.64474375, 0.452889556),
+    ("decode", 128, 256, 8, 1): (1.150025, 0.313991597), ("decode", 128, 256, 8, 4): (1.1009563, 0.649698679),
+    ("decode", 256, 128, 4, 1): (0.54297, 0.15329892), ("decode", 256, 128, 4, 2): (0.28788125, 0.207255702),
+    ("decode", 256, 128, 8, 1): (0.5406875, 0.152806723), ("decode", 256, 128, 8, 4): (0.42053875, 0.313996399),
+    ("decode", 256, 256, 4, 1): (1.0762225, 0.303966387), ("decode", 256, 256, 4, 2): (0.56767875, 0.415367347),
+    ("decode", 256, 256, 8, 1): (1.0714862, 0.303222089), ("decode", 256, 256, 8, 4): (None, 0.610410564),
+}
+
+
+def reference_suite(pkg, wl, dev, reps=50):
+    """The reference's perf-guard workloads on this GPU, timed the way its harness times them: device time
+    of the whole op, new-token cache write included (its kernel fuses the write; here rpa_kv_write +
+    rpa_attention).  Prefill = N tokens cut into 2048-token sequences with q_len == kv_len
+    (benchmark/kernels/flash_attention/utils.py:61-68, bench_flashattention.py:59-62); decode = N rows of one
+    token on 1025..2048 cached tokens (utils.py:131-132; numpy draws here, jax draws there).  `reps` steps are
+    captured in ONE HIP graph so that the figure is kernels back to back, not launch overhead."""
+    import numpy as np
+    import torch
+
+    m = importlib.import_module("sglang_jax_amd.ragged_paged_attention")
+    rows = []
+    for (mode, P, N, Hq, Hkv), (v6e, v7) in REFERENCE_PUBLISHED_MS.items():
+        if mode == "prefill":
+            q_lens = [2048] * (N // 2048) + ([N % 2048] if N % 2048 else [])
+            kv_lens = list(q_lens)
+        else:
+            kv_lens = (np.random.default_rng(42).integers(1024, 2048, size=N) + 1).tolist()
+            q_lens = [1] * N
+        b = wl.make_batch(f"reference_{mode}", q_lens, kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=128,
+                          page_size=P, seed=42, device=dev, pool_pages=600000 // P)
+        T, n = sum(q_lens), len(q_lens)
+        dec = n if mode == "decode" else 0
+        keys = torch.randn(T, Hkv, 128, device=dev, dtype=torch.bfloat16)
+        vals = torch.randn(T, Hkv, 128, device=dev, dtype=torch.bfloat16)
+        call = m.RpaCall(b.q, b.kv_cache, None, b.kv_lens, b.page_indices, b.cu_q_lens, b.cu_kv_lens, num_seqs=n,
+                         decode_end=dec, sm_scale=b.sm_scale, max_kv_len=max(kv_lens), max_q_len=max(q_lens),
+                         sum_decode_kv_len=sum(kv_lens) if dec else 0, own_workspace=True)
+
+        def step():
+            call.kv_write(keys, vals)
+            call.attention()
+
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(reps):
+                step()
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = _events(2)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        rows.append({"mode": mode, "page_size": P, "tokens_or_batch": N, "q_heads": Hq, "kv_heads": Hkv, "ms": ms,
+                     "tpu_v6e_ms": v6e, "tpu_v7_ms": v7, "speedup_vs_v6e": None if v6e is None else v6e / ms,
+                     "speedup_vs_v7": v7 / ms})
+        del call, b, keys, vals, graph
+    return rows
+
+
 def cpu_baseline(wl, budget_s=15.0):
     """CPU oracle on a bounded sample of the default workload: its first decode rows
     (same seeded lengths and layout, values drawn on the host)."""
@@ -267,6 +350,8 @@ def main():
                          "c5fp8: C5 on an e4m3 latent cache")
     ap.add_argument("--all", action="store_true", help="(default) also time the other configurations")
     ap.add_argument("--main-only", action="store_true", help="skip the other configurations")
+    ap.add_argument("--reference-suite", action="store_true",
+                    help="with --main-only: still run the reference's own perf-guard workloads")
     ap.add_argument("--static-shapes", action="store_true",
                     help="run the main configuration with the batch composition read on the device (grids sized "
                          "from static shapes only)")
@@ -391,6 +476,11 @@ def main():
                                          "avg_launch_ms": r["prefill_ms"], "flops_per_launch": r["prefill_flops"]}
             others[name] = r
         line["other_configs"] = others
+    if args.reference_suite or not args.main_only:
+        line["reference_suite"] = {
+            "what": "the reference's published perf-guard workloads (bench_flashattention.py:264-328), device ms per op "
+                    "with the new-token cache write, this GPU against its TPU v6e / v7 baselines",
+            "rows": reference_suite(pkg, wl, dev)}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(line))
