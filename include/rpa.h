@@ -95,7 +95,9 @@ typedef struct RpaParams {
   int32_t num_seqs;           /* S = distribution[2]: sequences to process */
   int32_t num_q_heads;        /* Hq */
   int32_t num_kv_heads;       /* Hkv, Hq % Hkv == 0 */
-  int32_t head_dim;           /* D: 128 or 256 */
+  int32_t head_dim;           /* D: 128 or 256.  Narrower heads (64, 80, 96, 192 ...) run zero-padded to the next
+                               * multiple of 128 exactly as in the reference (rpa_v3:1187-1241 pads the queries,
+                               * memory_pool.py:70 stores aligned rows); the caller pads, as the host mirror does */
   int32_t page_size;          /* P */
   int32_t total_pages;
   int32_t pages_per_seq;      /* row stride of the padded table (cu_kv_lens == NULL) */

@@ -395,12 +395,35 @@ def ragged_paged_attention(
         kv_cache_fused = kv_cache_fused.view(s[0], s[1], s[2] * s[3], s[4])
     if not (queries.is_contiguous() and kv_cache_fused.is_contiguous()):
         raise ValueError("queries and kv_cache_fused must be contiguous")
-    if queries.dtype != torch.bfloat16:
-        raise ValueError(f"Expected bfloat16 queries, got {queries.dtype}")
+    # rpa_v3 sets no query dtype; the engine hands over the model's (bf16, f16 or f32).  The matrix
+    # units here take bf16 operands: wider queries are rounded to bf16 once (2^-9 relative, inside
+    # the parity tolerance) and the output comes back in the query dtype as in rpa_v3:1788
+    q_dtype = queries.dtype
+    if q_dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise ValueError(f"Expected bfloat16, float16 or float32 queries, got {queries.dtype}")
+    if q_dtype != torch.bfloat16:
+        queries = queries.to(torch.bfloat16)
+    if out_dtype is None:
+        out_dtype = q_dtype
+
+    # rpa_v3:1187-1241, 1270-1296: head dims that are not a multiple of 128 (64, 80, 96, 192 ...) run
+    # zero-padded.  The engine's pool already stores aligned rows (memory_pool.py:70): then only the
+    # queries and the new tokens are padded here.  A cache with narrow rows is padded, run and copied
+    # back, as the reference does.
+    actual_head_dim = queries.shape[2]
+    caller_cache = kv_cache_fused
+    if kv_cache_fused.shape[3] % 128 != 0:
+        kv_cache_fused = torch.nn.functional.pad(kv_cache_fused, (0, -kv_cache_fused.shape[3] % 128))
     total_pages, page_size, h2, head_dim = kv_cache_fused.shape
     num_kv_heads = h2 // 2
-    if head_dim != queries.shape[2]:
-        raise ValueError(f"Expected cache head_dim={head_dim} to equal q head_dim={queries.shape[2]}")
+    if not (actual_head_dim <= head_dim < actual_head_dim + 128):
+        raise ValueError(f"Expected cache head_dim={caller_cache.shape[3]} to be q head_dim={actual_head_dim}, "
+                         "or that rounded up to a multiple of 128")
+    if actual_head_dim != head_dim:
+        queries = torch.nn.functional.pad(queries, (0, head_dim - actual_head_dim))
+        if keys is not None:
+            keys = torch.nn.functional.pad(keys, (0, head_dim - actual_head_dim))
+            values = torch.nn.functional.pad(values, (0, head_dim - actual_head_dim))
     i, j, k = (int(x) for x in dist)
     if not (i <= j <= k):
         raise ValueError(f"distribution must satisfy i <= j <= k, got {i}, {j}, {k}")
@@ -410,8 +433,8 @@ def ragged_paged_attention(
     # rpa_v3:1788: bfloat16 unless asked otherwise.  The kernels normalise in f32 and round the
     # finished row to bf16 once; float32 output is those values widened (one bf16 rounding more
     # than the reference's f32 accumulator leaves, far inside the parity tolerance)
-    if out_dtype not in (None, torch.bfloat16, torch.float32):
-        raise NotImplementedError("out_dtype must be bfloat16 or float32")
+    if out_dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise NotImplementedError("out_dtype must be bfloat16, float16 or float32")
     call = RpaCall(queries, kv_cache_fused, None, kv_lens_d, page_d, cu_q_d, cu_kv_d, num_seqs=k, decode_end=i,
                    sm_scale=sm_scale, sliding_window=sliding_window, soft_cap=soft_cap, mask_value=mask_value,
                    k_scale=k_scale, v_scale=v_scale,
@@ -435,9 +458,16 @@ def ragged_paged_attention(
             raise ValueError(f"Expected keys/values dtype {kv_cache_fused.dtype}, got {keys.dtype}/{values.dtype}")
         call.kv_write(keys.contiguous(), values.contiguous())
     call.attention()
-    if out_dtype == torch.float32:
-        return call.out.float(), kv_cache_fused
-    return call.out, kv_cache_fused
+    out = call.out
+    if actual_head_dim != head_dim:
+        out = out[:, :, :actual_head_dim].contiguous()
+    if out_dtype != torch.bfloat16:
+        out = out.to(out_dtype)
+    if kv_cache_fused is not caller_cache:  # narrow rows: the new tokens go back into the caller's cache
+        if keys is not None:
+            caller_cache.copy_(kv_cache_fused[..., : caller_cache.shape[3]])
+        kv_cache_fused = caller_cache
+    return out, kv_cache_fused
 
 
 def ragged_paged_attention_ref_surface(

@@ -275,7 +275,63 @@ def test_new_tokens_are_written_into_the_cache(pkg, wl, gpu):
     assert_parity(out32[:T].cpu(), want.float(), **BF16_TOL)
     with pytest.raises(NotImplementedError):
         pkg.ragged_paged_attention(g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
-                                   b.distribution.numpy(), None, sm_scale=b.sm_scale, out_dtype=torch.float16)
+                                   b.distribution.numpy(), None, sm_scale=b.sm_scale, out_dtype=torch.float64)
+
+
+@pytest.mark.parametrize("q_dtype", [torch.float32, torch.float16])
+def test_wider_query_dtypes_come_back_in_their_own_type(pkg, wl, gpu, q_dtype):
+    """rpa_v3 sets no query dtype and returns the queries' (rpa_v3:1788).  Here they are rounded to bf16
+    once: the oracle runs on the rounded queries' source values, the tolerance is the bf16 one."""
+    b = wl.make_batch("qdtype", [1, 1, 33, 130], [300, 17, 33, 400], num_q_heads=8, num_kv_heads=2, head_dim=128,
+                      page_size=16, seed=71)
+    want = oracle_out(b)
+    g = b.to(gpu)
+    out, _ = pkg.ragged_paged_attention(
+        g.q.to(q_dtype), None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+        b.distribution.numpy(), None, sm_scale=b.sm_scale, max_kv_len=400, max_q_len=130)
+    assert out.dtype == q_dtype
+    assert_parity(out.cpu().float(), want.float(), **BF16_TOL)
+
+
+@pytest.mark.parametrize("head_dim,aligned_pool", [(64, True), (64, False), (96, True), (80, False), (192, True), (192, False)])
+def test_head_dims_that_are_not_a_multiple_of_128(pkg, wl, gpu, head_dim, aligned_pool):
+    """rpa_v3:1187-1241, 1270-1296: queries, new tokens and narrow caches run zero-padded to the next
+    multiple of 128 and come back at their own width.  `aligned_pool`: the cache already stores padded
+    rows, as the engine's pool does (memory_pool.py:70), and only queries and new tokens are narrow."""
+    q_lens, kv_lens = [1, 1, 20, 70], [64, 200, 20, 300]
+    Hq, Hkv, P = 8, 2, 16
+    b = wl.make_batch("narrow", q_lens, kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=head_dim, page_size=P, seed=72)
+    want = oracle_out(b)
+    kp, vp = split_fused_cache(b.kv_cache)
+    table = b.padded_page_table()
+    T = sum(q_lens)
+    keys = torch.empty(T, Hkv, head_dim, dtype=torch.bfloat16)
+    vals = torch.empty(T, Hkv, head_dim, dtype=torch.bfloat16)
+    holed = b.kv_cache.clone()
+    t = 0
+    for i, (ql, kv) in enumerate(zip(q_lens, kv_lens)):
+        for j in range(ql):
+            pos = kv - ql + j
+            page, row = int(table[i, pos // P]), pos % P
+            keys[t], vals[t] = kp[page, row], vp[page, row]
+            holed[page, row] = 0
+            t += 1
+    wide = -head_dim % 128
+    cache_in = torch.nn.functional.pad(holed, (0, wide)) if aligned_pool else holed
+    # whatever an aligned pool holds in the padding of its rows cannot reach the result: the padded
+    # query dims are zero and the padded value dims are cut off
+    if aligned_pool:
+        cache_in[..., head_dim:] = 3.0
+    g = b.to(gpu)
+    cache_in = cache_in.to(gpu)
+    out, cache = pkg.ragged_paged_attention(
+        g.q, keys.to(gpu), vals.to(gpu), cache_in, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+        b.distribution.numpy(), None, sm_scale=b.sm_scale, max_kv_len=300, max_q_len=70)
+    torch.cuda.synchronize()
+    assert out.shape == (g.q.shape[0], Hq, head_dim)
+    assert cache.data_ptr() == cache_in.data_ptr()
+    assert torch.equal(cache[..., :head_dim].cpu().view(torch.int16), b.kv_cache.view(torch.int16))
+    assert_parity(out[:T].cpu().float(), want.float(), **BF16_TOL)
 
 
 def test_dynamic_validation_through_the_wrapper(pkg, wl, gpu):
