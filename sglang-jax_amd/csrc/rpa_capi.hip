@@ -579,9 +579,9 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   const bool dyn = p->distribution != nullptr;
   if (!dyn && p->num_seqs <= p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) return RPA_OK;
   if (dyn && p->num_seqs <= 0) return RPA_OK;
-  // 256-wide heads: bf16 caches take the flash kernel (two 128-dim halves per row, one workgroup
-  // per CU); fp8 caches and rows the caller masks itself stay on the row kernel
-  if (p->head_dim == 256 && (p->kv_dtype == RPA_KV_FP8_E4M3 || env_int("RPA_PREFILL_ROWS256", 0) != 0))
+  // 256-wide heads take the flash kernel (two 128-dim halves per row, one workgroup per CU; e4m3
+  // caches staged through registers); RPA_PREFILL_ROWS256=1 sends them through the row kernel
+  if (p->head_dim == 256 && env_int("RPA_PREFILL_ROWS256", 0) != 0)
     return rows256(p, (p->mask_mode == RPA_MASK_CUSTOM) ? 0 : p->decode_end, p->num_seqs, stream);
   rpa::PrefillArgs a;
   a.head_dim = p->head_dim;

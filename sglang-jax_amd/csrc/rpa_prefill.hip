@@ -36,11 +36,67 @@ using namespace pf;
 namespace {
 
 
+// ---- fp8 rows into the same LDS layout (the 256-wide heads' fp8 path) ----
+// Thread tid stages a quarter of K row and V row (tid >> 2): HD / 4 bytes of e4m3 each, loaded
+// two tiles ahead into registers, widened to bf16 and written one tile ahead to the chunk
+// positions the asynchronous copy would have used, so the products read both caches alike.
+template <int HD>
+struct Fp8Stage {
+  u32x4_t k[HD / 64], v[HD / 64];
+};
+
+template <bool UNIFORM>
+__device__ __forceinline__ int32_t fp8_fetch_page(const TileSrc& s, int tb, int tid) {
+  tb = min(tb, s.last_tok & ~(kBN - 1));
+  if constexpr (UNIFORM) {
+    return scalar_load_i32(s.pages + __builtin_amdgcn_readfirstlane(page_slot(s, tb)));
+  } else {
+    return s.pages[page_slot(s, min(tb + (tid >> 2), s.last_tok))];
+  }
+}
+
+template <bool UNIFORM, int HD>
+__device__ __forceinline__ void fp8_gload(Fp8Stage<HD>& st, const TileSrc& s, const KvAddr& kv, const char* kh,
+                                          const char* vh, int tb, int tid, int32_t page) {
+  tb = min(tb, s.last_tok & ~(kBN - 1));  // past the end: re-read the last tile
+  const int64_t ro = row_offset<UNIFORM>(s, kv, tb, tb + (tid >> 2), page) + (tid & 3) * (HD / 4);
+#pragma unroll
+  for (int i = 0; i < HD / 64; ++i) {
+    st.k[i] = ld16(kh + ro + i * 16);
+    st.v[i] = ld16(vh + ro + i * 16);
+  }
+}
+
+template <int HD>
+__device__ __forceinline__ void fp8_lstore(const Fp8Stage<HD>& st, char* lds_k, char* lds_v, int tid) {
+  const int t = tid >> 2;
+  char* kr = lds_k + t * Tile<HD>::kRowB;
+  char* vr = lds_v + t * Tile<HD>::kRowB;
+  const int ks = t & 15, vs = (t & 3) << 2;
+#pragma unroll
+  for (int i = 0; i < HD / 64; ++i) {
+    const int j = (tid & 3) * (HD / 32) + 2 * i;  // the first of the two bf16 chunks these 16 bytes widen to
+    {
+      const u32x2_t a = fp8x4_to_bf16x4(st.k[i][0]), b = fp8x4_to_bf16x4(st.k[i][1]);
+      const u32x2_t c = fp8x4_to_bf16x4(st.k[i][2]), d = fp8x4_to_bf16x4(st.k[i][3]);
+      lds_st16(kr + ((j ^ ks) << 4), u32x4_t{a[0], a[1], b[0], b[1]});
+      lds_st16(kr + (((j + 1) ^ ks) << 4), u32x4_t{c[0], c[1], d[0], d[1]});
+    }
+    {
+      const u32x2_t a = fp8x4_to_bf16x4(st.v[i][0]), b = fp8x4_to_bf16x4(st.v[i][1]);
+      const u32x2_t c = fp8x4_to_bf16x4(st.v[i][2]), d = fp8x4_to_bf16x4(st.v[i][3]);
+      lds_st16(vr + ((j ^ vs) << 4), u32x4_t{a[0], a[1], b[0], b[1]});
+      lds_st16(vr + (((j + 1) ^ vs) << 4), u32x4_t{c[0], c[1], d[0], d[1]});
+    }
+  }
+}
+
 // EXT compiles in the rarely used options (temperature factor, custom mask / no mask); the
 // plain causal instantiation keeps its scale in a scalar register and its mask test to one compare.
 // HD = 256 doubles the rows in LDS (two 64 KiB slots), the Q^T operands and the accumulators: one
 // workgroup per CU, one wave per SIMD with up to 512 registers.
-template <bool UNIFORM, bool CAP, bool EXT, int HD = 128>
+// FP8: an e4m3 cache staged through registers into the same LDS layout (see above).
+template <bool UNIFORM, bool CAP, bool EXT, int HD = 128, bool FP8 = false>
 __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_kernel(const PrefillArgs a_in, int tiles, int nseq,
                                                                                   bool by_level) {
   PrefillArgs a = a_in;  // static-shape mode: the sequences to process come from the device
@@ -85,7 +141,7 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
     for (int ks = 0; ks < T::kSteps; ++ks) qB[ks] = ld16(qp + ks * 16);
     if (EXT && a.sm.q_scale > 0.f) {
 #pragma unroll
-      for (int ks = 0; ks < T::kSteps; ++ks) qB[ks] = requantise_q(qB[ks], a.sm.q_scale, false);
+      for (int ks = 0; ks < T::kSteps; ++ks) qB[ks] = requantise_q(qB[ks], a.sm.q_scale, FP8);
     }
   }
   Softmax<CAP> sm;
@@ -143,20 +199,38 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
   }
 
   // ---- pipeline: page ids two tiles ahead, the asynchronous copy one tile ahead ----
-  const AsyncOffsets<HD> ofs = make_async_offsets<HD>(a.kv, wave, lane);
+  AsyncOffsets<HD> ofs;
   AsyncPages<UNIFORM, HD> pg;
-  async_fetch_pages<UNIFORM, HD>(pg, src, t_lo, wave, lane);
-  async_copy_tile<UNIFORM, HD>(lds_k0, lds_v0, src, a.kv, kh, vh, t_lo, wave, lane, pg, ofs);
-  async_fetch_pages<UNIFORM, HD>(pg, src, t_lo + kBN, wave, lane);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the copies have landed in LDS
+  Fp8Stage<HD> stg;     // FP8: rows of the tile after the next one
+  int32_t fp8_page = 0;  // FP8: page of this thread's row in the tile loaded next
+  if constexpr (FP8) {
+    fp8_page = fp8_fetch_page<UNIFORM>(src, t_lo, tid);
+    fp8_gload<UNIFORM, HD>(stg, src, a.kv, kh, vh, t_lo, tid, fp8_page);
+    fp8_page = fp8_fetch_page<UNIFORM>(src, t_lo + kBN, tid);
+    fp8_lstore<HD>(stg, lds_k0, lds_v0, tid);
+    fp8_gload<UNIFORM, HD>(stg, src, a.kv, kh, vh, t_lo + kBN, tid, fp8_page);
+    fp8_page = fp8_fetch_page<UNIFORM>(src, t_lo + 2 * kBN, tid);
+  } else {
+    ofs = make_async_offsets<HD>(a.kv, wave, lane);
+    async_fetch_pages<UNIFORM, HD>(pg, src, t_lo, wave, lane);
+    async_copy_tile<UNIFORM, HD>(lds_k0, lds_v0, src, a.kv, kh, vh, t_lo, wave, lane, pg, ofs);
+    async_fetch_pages<UNIFORM, HD>(pg, src, t_lo + kBN, wave, lane);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the copies have landed in LDS
+  }
   __syncthreads();
 
   // one tile: consume (lds_k, lds_v), fill (nxt_k, nxt_v) with the tile after it
   auto tile_step = [&](const char* lds_k, const char* lds_v, char* nxt_k, char* nxt_v, int tb) {
     if (tb + kBN < t_hi) {
       // the other slot was last read before the barrier that ended the previous tile
-      async_copy_tile<UNIFORM, HD>(nxt_k, nxt_v, src, a.kv, kh, vh, tb + kBN, wave, lane, pg, ofs);
-      async_fetch_pages<UNIFORM, HD>(pg, src, tb + 2 * kBN, wave, lane);
+      if constexpr (FP8) {
+        fp8_lstore<HD>(stg, nxt_k, nxt_v, tid);
+        fp8_gload<UNIFORM, HD>(stg, src, a.kv, kh, vh, tb + 2 * kBN, tid, fp8_page);
+        fp8_page = fp8_fetch_page<UNIFORM>(src, tb + 3 * kBN, tid);
+      } else {
+        async_copy_tile<UNIFORM, HD>(nxt_k, nxt_v, src, a.kv, kh, vh, tb + kBN, wave, lane, pg, ofs);
+        async_fetch_pages<UNIFORM, HD>(pg, src, tb + 2 * kBN, wave, lane);
+      }
     }
     // visible to this wave?  causal: some token <= last row's position; window: some token
     // newer than the first row's horizon
@@ -191,7 +265,7 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
             }
       }
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // the next tile has landed
+    if constexpr (!FP8) __builtin_amdgcn_s_waitcnt(0x0F70);  // the next tile has landed
     __syncthreads();
   };
   for (int tb = t_lo; tb < t_hi; tb += 2 * kBN) {
@@ -462,6 +536,8 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
 #define RPA_ASYNC(U, C, E) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_ASYNC256(U, C, E) \
   hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E, 256>), g, blk, 0, stream, a, tiles, nseq, by_level)
+#define RPA_ASYNC256_FP8(U, C, E) \
+  hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E, 256, true>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_PICK(M, ...)                                            \
   switch ((uniform ? 4 : 0) | (cap ? 2 : 0) | (ext ? 1 : 0)) {        \
     case 0: M(__VA_ARGS__ false, false, false); break;              \
@@ -476,8 +552,11 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
 #define RPA_STAGED_FP8(U, C, E) RPA_STAGED(true, U, C, E)
 #define RPA_STAGED_BF16(U, C, E) RPA_STAGED(false, U, C, E)
   if (a.head_dim == 256) {
-    if (a.fp8) return hipErrorInvalidValue;  // 256-wide fp8 rows go through the row kernel
-    RPA_PICK(RPA_ASYNC256, )
+    if (a.fp8) {
+      RPA_PICK(RPA_ASYNC256_FP8, )
+    } else {
+      RPA_PICK(RPA_ASYNC256, )
+    }
   } else if (!staged) {
     RPA_PICK(RPA_ASYNC, )
   } else if (a.fp8) {
@@ -491,6 +570,7 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
 #undef RPA_STAGED
 #undef RPA_ASYNC
 #undef RPA_ASYNC256
+#undef RPA_ASYNC256_FP8
   return hipGetLastError();
 }
 

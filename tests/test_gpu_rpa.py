@@ -435,6 +435,8 @@ NEEDLE_CASES = {
     "wide_heads_rows": ([1] * 6, [9000, 4097, 12000, 30000, 5000, 7000], 8, 2, 256, 64, torch.bfloat16, None),
     "wide_heads_rows_fp8": ([1] * 6, [9000, 4097, 12000, 30000, 5000, 7000], 8, 2, 256, 64, torch.float8_e4m3fn, None),
     "wide_heads_chunks": ([200, 300], [4296, 8000], 16, 4, 256, 64, torch.bfloat16, None),
+    "wide_heads_chunks_fp8": ([200, 300, 70], [4296, 8000, 70], 16, 4, 256, 64, torch.float8_e4m3fn, None),
+    "wide_heads_chunks_fp8_small_pages": ([130, 65], [2130, 4000], 8, 2, 256, 16, torch.float8_e4m3fn, 1500),
 }
 
 
@@ -820,7 +822,7 @@ def test_head_dim_256_options(pkg, wl, gpu, window, cap, kv_dtype):
     assert_parity(got.float(), want.float(), **tol)
     # full attention (causal = 0 without a mask)
     assert_parity(gpu_out(pkg, b, gpu, causal=False).float(), oracle_out(b, causal=False).float(), **tol)
-    # custom masks: every row goes through the flash kernel (bf16 caches) or the row kernel (fp8)
+    # custom masks: every row goes through the flash kernel
     rng = np.random.default_rng(11)
     masks = []
     for ql, kv in zip(q_lens, kv_lens):
@@ -858,6 +860,25 @@ def test_head_dim_256_long_decode_rows_are_split(pkg, wl, gpu, kv_dtype, window)
     sink = torch.from_numpy(np.random.RandomState(101).randn(8).astype(np.float32))
     assert_parity(gpu_out(pkg, b, gpu, attention_sink=sink).float(),
                                oracle_out(b, attention_sink=sink).float(), **tol)
+
+
+@pytest.mark.parametrize("P,window", [(64, None), (16, None), (24, 100)])
+def test_head_dim_256_fp8_chunks_flash_kernel_against_row_kernel(pkg, wl, gpu, P, window, monkeypatch):
+    """e4m3 caches with 256-wide heads: chunks take the flash kernel (rows staged through registers
+    into the bf16 kernel's LDS layout); the row kernel (RPA_PREFILL_ROWS256=1) reads the same cache
+    one query token per wave.  Both against the oracle, and against each other more tightly."""
+    q_lens, kv_lens = [1, 1, 129, 64, 300, 5], [70, 257, 129, 1000, 3000, 600]
+    b = batch256(wl, "d256f8", q_lens, kv_lens, 95, Hq=8, Hkv=2, P=P, kv_dtype=torch.float8_e4m3fn, sliding_window=window)
+    say(f"case d256 fp8 chunks P={P} window={window}")
+    want = oracle_out(b)
+    flash = gpu_out(pkg, b, gpu)
+    monkeypatch.setenv("RPA_PREFILL_ROWS256", "1")
+    rows = gpu_out(pkg, b, gpu)
+    monkeypatch.delenv("RPA_PREFILL_ROWS256")
+    assert_parity(flash.float(), want.float(), **FP8_TOL)
+    assert_parity(rows.float(), want.float(), **FP8_TOL)
+    torch.testing.assert_close(flash.float(), rows.float(), rtol=1e-2, atol=4e-3)
+    assert not torch.equal(flash, rows)  # two kernels: the last bits differ somewhere
 
 
 def test_head_dim_256_cache_write_and_gather(pkg, wl, gpu):
