@@ -57,11 +57,11 @@ DECODE_KERNEL = {
 PREFILL_KERNEL = "rpa_prefill_pipe_kernel"
 
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", PREFILL_KERNEL): 326.1e6 + 77.2e6,
+    ("c2", PREFILL_KERNEL): 325.9e6 + 77.2e6,
     ("c2", "rpa_decode_balanced_kernel"): 501.0e6 + 2.7e6,
     ("c3", "rpa_decode_splitkv_kernel"): 2148.6e6 + 1.9e6,
-    ("c5", "rpa_mla_balanced_kernel"): 816.1e6 + 81.1e6,
-    ("c5p", "rpa_mla_decode_kernel (one row per query token)"): 632.7e6 + 268.5e6,
+    ("c5", "rpa_mla_balanced_kernel"): 824.0e6 + 49.3e6,
+    ("c5p", "rpa_mla_decode_kernel (one row per query token)"): 632.9e6 + 268.5e6,
 }
 
 
