@@ -44,13 +44,15 @@ ACC = 1000                                # register ids >= ACC name accumulatio
 # Experiment switches (timing probes only: results are wrong with any of them set)
 X = set(os.environ.get("RPA_PIPE_X", "").split(","))
 AHEAD = int(os.environ.get("RPA_PIPE_AHEAD", 3))   # fragments requested ahead of the MFMAs that use them
+STAGGER = int(os.environ.get("RPA_PIPE_STAGGER", 4))  # matrix slots a wave spreads its copies over (with X = stagger)
 NBUF = 4                                  # operand fragment buffers per matrix
 
 # scalar registers used inside the block (all listed as clobbers)
 KB, VB = 60, 62                           # s[60:61], s[62:63]: global base of the K / V tile being copied
 ST = [64, 65, 66, 67]                     # temporaries
 PGC = 68                                  # page id of tile t + 2
-SGPR_CLOBBERS = list(range(60, 69))
+WV = 69                                   # this wave's index in its workgroup (staggered copies)
+SGPR_CLOBBERS = list(range(60, 70 if "stagger" in X else 69))
 
 K_SLOT = [0, 16384]                       # byte offsets of the ring slots from the LDS array's start
 V_SLOT = [32768, 49152]
@@ -126,7 +128,7 @@ class Ins:
 def wait_states(ins):
     if ins.kind == "nop":
         return int(ins.text.split()[1]) + 1
-    if ins.kind == "label":
+    if ins.kind in ("label", "skip"):  # "skip": inside a branch some waves jump over: counts for nothing
         return 0
     return 1
 
@@ -301,7 +303,7 @@ class Gen:
                 Ins(f"global_load_lds_dwordx4 {vr(ofs)}, s[{sb}:{sb + 1}]", "vmem", [ofs], [])]
 
     # ---------------------------------------------------------------- one iteration
-    def iteration(self, em, it, ks, vs, copies):
+    def iteration(self, em, it, ks, vs, copies, uid=""):
         """Iteration `it` (0 / 1) of a step.  it = 0: softmax of the odd-half scores into the odd-half
         probabilities, scores of the tile's first half into the even buffers, second product with the
         even-half probabilities; it = 1: the mirror image on the tile's second half."""
@@ -348,7 +350,19 @@ class Gen:
                 em.emit(self.mfma_pv(f, q, pp))
                 if q == nq - 1:
                     frag_reads("v", f + AHEAD)
-                    if copies:
+                    if copies and "stagger" in X:
+                        # wave w of the workgroup issues its eight copies at matrix slots 4w .. 4w+3 of the
+                        # step (two per slot): the four waves never queue for the texture path together
+                        j = 8 * it + k
+                        if j < 4 * STAGGER:
+                            per_slot = 8 // STAGGER
+                            em.raw(f"s_cmp_eq_u32 s{WV}, {j // STAGGER}", "skip")
+                            em.raw(f"s_cbranch_scc0 L_nc_{uid}{j}_%=", "skip")
+                            for g in range(per_slot * (j % STAGGER), per_slot * (j % STAGGER + 1)):
+                                for x in copies[g]:
+                                    em.raw(x.text, "skip")
+                            em.label(f"L_nc_{uid}{j}_%=")
+                    elif copies:
                         for x in copies.pop(0):
                             em.emit(x)
                 deal(per[s])
@@ -431,15 +445,17 @@ class Gen:
                 for x in grp:
                     em.emit(x)
             copies = []
+        if "stagger" in X:
+            em.raw(f"s_bfe_u32 s{WV}, %[lds_wave], 0x2000c")      # (lds_wave >> 12) & 3
         for it in (0, 1):
-            self.iteration(em, it, ks, vs, copies)
+            self.iteration(em, it, ks, vs, copies, uid)
             tag = uid + "ab"[it]
             if "norare" not in X:
                 em.raw(f"s_cbranch_vccnz L_rare_{tag}_%=")
             em.label(f"L_back_{tag}_%=")
             for q in range(self.nq):
                 em.emit(valu(f"v_add_f32 {vr(t.L[q])}, {vr(t.L[q])}, {vr(t.PS[q][0])}", [t.L[q], t.PS[q][0]], [t.L[q]]))
-        assert not copies and not em.lds_queue
+        assert ("stagger" in X or not copies) and not em.lds_queue
         # ---- end of step: the copies have landed, everybody has finished reading the slots they overwrite next
         em.raw("s_waitcnt lgkmcnt(0)" if "novmwait" in X else "s_waitcnt vmcnt(0) lgkmcnt(0)", "wait")
         em.raw("s_mov_b32 %[pg_a], %[pg_b]")
