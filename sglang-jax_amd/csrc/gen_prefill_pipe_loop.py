@@ -298,6 +298,11 @@ class Gen:
         base = (V_SLOT if is_v else K_SLOT)[fill_slot] + n * 1024
         ofs = (t.OFSV if is_v else t.OFSK) + n
         sb = VB if is_v else KB
+        if "copyexec0" in X:  # probe: the instruction is issued, no lane moves data
+            return [Ins(f"s_add_u32 m0, %[lds_wave], {base}", "salu"),
+                    Ins("s_mov_b64 exec, 0", "salu"),
+                    Ins(f"global_load_lds_dwordx4 {vr(ofs)}, s[{sb}:{sb + 1}]", "vmem", [ofs], []),
+                    Ins("s_mov_b64 exec, -1", "salu")]
         return [Ins(f"s_add_u32 m0, %[lds_wave], {base}", "salu"),
                 Ins("s_nop 0", "nop"),
                 Ins(f"global_load_lds_dwordx4 {vr(ofs)}, s[{sb}:{sb + 1}]", "vmem", [ofs], [])]
@@ -440,6 +445,8 @@ class Gen:
         copies = [self.copy_ins(n, False, 1 - ks) for n in range(4)] + [self.copy_ins(n, True, 1 - vs) for n in range(4)]
         if "nocopy" in X:
             copies = []
+        if "halfcopy" in X:  # probe: half of the tile bytes (what a tile shared by 256 rows would move per wave)
+            copies = [c if i % 2 == 0 else [] for i, c in enumerate(copies)]
         if "copyfirst" in X:
             for grp in copies:
                 for x in grp:
@@ -458,8 +465,9 @@ class Gen:
         assert ("stagger" in X or not copies) and not em.lds_queue
         # ---- end of step: the copies have landed, everybody has finished reading the slots they overwrite next
         em.raw("s_waitcnt lgkmcnt(0)" if "novmwait" in X else "s_waitcnt vmcnt(0) lgkmcnt(0)", "wait")
-        em.raw("s_mov_b32 %[pg_a], %[pg_b]")
-        em.raw(f"s_mov_b32 %[pg_b], s{PGC}")
+        if "copysame" not in X:  # probe: every step copies the same pages (cache hits)
+            em.raw("s_mov_b32 %[pg_a], %[pg_b]")
+            em.raw(f"s_mov_b32 %[pg_b], s{PGC}")
         if "nobarrier" not in X:
             em.raw("s_barrier")
         em.raw("s_add_u32 %[t], %[t], 1")
