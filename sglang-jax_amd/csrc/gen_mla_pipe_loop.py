@@ -97,7 +97,7 @@ def ring(f):
 def frag_read(f):
     """operand fragment f of the tile: 0..35 K of (k-step f >> 1, token block f & 1), 36..67 V^T of dim chunk f - 36"""
     dst = ring(f)
-    if "nolds" in X:
+    if "nolds" in X or ("halflds" in X and f % 2 == 1):  # halflds: what fragments shared by 32 heads would read
         return []
     if f < 36:
         ks, b = f >> 1, f & 1
@@ -113,11 +113,11 @@ def frag_mfma(f):
     if f < 36:
         ks, b = f >> 1, f & 1
         ins = mfma(S[b], ring(f), Q + 4 * ks, None if ks == 0 else S[b])
-        ins.lds_need = None if "nolds" in X else [("k", f)]
+        ins.lds_need = None if "nolds" in X or ("halflds" in X and f % 2 == 1) else [("k", f)]
     else:
         j = f - 36
         ins = mfma(O + 4 * j, ring(f), P, O + 4 * j)
-        ins.lds_need = None if "nolds" in X else [("vlo", f), ("vhi", f)]
+        ins.lds_need = None if "nolds" in X or ("halflds" in X and f % 2 == 1) else [("vlo", f), ("vhi", f)]
     return ins
 
 
