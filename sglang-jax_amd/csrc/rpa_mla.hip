@@ -27,6 +27,7 @@
 #include "rpa_common.h"
 #include "rpa_kernels.h"
 #include "rpa_mla_pipe_loop.inc"
+#include "rpa_mla_wide_loop.inc"
 
 namespace rpa {
 
@@ -49,6 +50,8 @@ __device__ __forceinline__ u32x4_t lds_ld16(const char* p) { return *reinterpret
 
 typedef uint32_t u32x32_t __attribute__((ext_vector_type(32)));
 typedef uint32_t u32x8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x32_t __attribute__((ext_vector_type(32)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ u32x2_t lds_tr16(const char* p) {
   typedef __attribute__((address_space(3))) s16x4_t* lds_ptr_t;
@@ -89,20 +92,23 @@ __device__ __forceinline__ int page_slot(const Src& s, int tok) {
 // The 8 x 5 = 40 copy instructions of a tile cover 37 blocks: the last three repeat block 0
 // (same source, same destination, same bytes), so every wave has the same number of copies
 // in flight and the slot is exactly 37 KiB.
+// CPW: copy instructions per wave and tile -- 5 with eight waves, 10 with four (wide workgroups).
+template <int CPW = kCopiesPerWave>
 __device__ __forceinline__ int copy_block(int wave, int n) {
-  const int blk = wave * kCopiesPerWave + n;
+  const int blk = wave * CPW + n;
   return blk < kUsedBlocks ? blk : 0;
 }
 
+template <int CPW = kCopiesPerWave>
 __device__ __forceinline__ void chunk_of(const Src& s, int wave, int lane, int n, int& row, int& inner) {
-  const int p = copy_block(wave, n) * 64 + lane;
+  const int p = copy_block<CPW>(wave, n) * 64 + lane;
   row = p / kChunks;
   int j = p - row * kChunks;
   if (j >= 72) { row = 0; j = 0; }
   inner = j < 64 ? j * 16 : s.rope_byte + (j - 64) * 16;
 }
 
-template <bool UNIFORM>
+template <bool UNIFORM, int CPW = kCopiesPerWave>
 __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* cache, int tb, int wave, int lane,
                                           int page) {
   tb = min(tb, s.last_tok & ~(kTok - 1));  // past the end: re-copy the last tile
@@ -116,24 +122,24 @@ __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* 
       int ln = lane;
       asm volatile("" : "+v"(ln));  // opaque: keeps the offset arithmetic inside the loop
 #pragma unroll
-      for (int n = 0; n < kCopiesPerWave; ++n) {
+      for (int n = 0; n < CPW; ++n) {
         int row, inner;
-        chunk_of(s, wave, ln, n, row, inner);
-        async_copy16(base + (uint32_t)(row * s.row_bytes + inner), slot + copy_block(wave, n) * 1024);
+        chunk_of<CPW>(s, wave, ln, n, row, inner);
+        async_copy16(base + (uint32_t)(row * s.row_bytes + inner), slot + copy_block<CPW>(wave, n) * 1024);
       }
       return;
     }
   }
   // last, partial tile (rows clamped to the last valid token) or pages smaller than a tile
 #pragma unroll
-  for (int n = 0; n < kCopiesPerWave; ++n) {
+  for (int n = 0; n < CPW; ++n) {
     int row, inner;
-    chunk_of(s, wave, lane, n, row, inner);
+    chunk_of<CPW>(s, wave, lane, n, row, inner);
     const int tok = min(tb + row, s.last_tok);
     const int ps = page_slot(s, tok);
     const int pg = UNIFORM ? page : s.pages[ps];
     const char* src = cache + (int64_t)pg * s.page_stride + (int64_t)(tok - ps * s.page_size) * s.row_bytes + inner;
-    async_copy16(src, slot + copy_block(wave, n) * 1024);
+    async_copy16(src, slot + copy_block<CPW>(wave, n) * 1024);
   }
 }
 
@@ -538,7 +544,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
         asm volatile(RPA_MLA_PIPE_F8_ASM
                      : "+" C(O0)(o[0]), "+" C(O1)(o[1]), "+" C(O2)(o[2]), "+" C(O3)(o[3]), "+" C(O4)(o[4]),
                        "+" C(O5)(o[5]), "+" C(O6)(o[6]), "+" C(O7)(o[7]), "+" C(ML)(ml), "+" C(OFS)(ofs),
-                       [t] "+s"(k), [pg] "+s"(pg_next)
+                       [t] "+&s"(k), [pg] "+&s"(pg_next)
                      : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), [t_end] "s"(k1), [t_begin] "s"(t_begin),
                        [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),
                        [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2_bits),
@@ -550,7 +556,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
         asm volatile(RPA_MLA_PIPE_ASM
                      : "+" C(O0)(o[0]), "+" C(O1)(o[1]), "+" C(O2)(o[2]), "+" C(O3)(o[3]), "+" C(O4)(o[4]),
                        "+" C(O5)(o[5]), "+" C(O6)(o[6]), "+" C(O7)(o[7]), "+" C(ML)(ml), "+" C(OFS)(ofs),
-                       [t] "+s"(k), [pg] "+s"(pg_next)
+                       [t] "+&s"(k), [pg] "+&s"(pg_next)
                      : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), [t_end] "s"(k1), [t_begin] "s"(t_begin),
                        [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),
                        [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2_bits),
@@ -634,6 +640,220 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   mla_segment<UNIFORM, CAP, PIPE, FP8>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
 }
 
+// immediate of s_waitcnt vmcnt(n) (n < 64) with the other counters left alone
+constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
+
+// ---- wide workgroups: FOUR waves, each owning two blocks of 16 heads, so that every K and V^T operand read
+// from LDS feeds two matrix instructions (LDS reads, not the matrix pipe, are what the eight-wave
+// workgroups wait for).  256 accumulators in the accumulation registers, 144 registers of Q^T, one wave per
+// SIMD.  Every tile of the segment runs inside the assembly loop of rpa_mla_wide_loop.inc (masks and the
+// clamped copies of the row's last tile included); compiled code only loads the queries, starts the ring,
+// takes the first tile's maxima as the reference and writes the result.  bf16 caches, pages of a
+// power-of-two size >= 32, no soft cap, Hq a multiple of 128.  `ring`: the four slots, contiguous.
+__device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
+                                                 int t_begin, int t_end, const MlaDest dest, char* ring) {
+  constexpr int CPW = 2 * kCopiesPerWave;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 15, g = lane >> 4;
+  const int head0 = head_base + wave * 32;
+  const int seq = mr.seq;
+  const int kv_len = mr.kv_len;
+  const int tq = mr.tq;
+
+  Src src;
+  src.page_size = a.pt.page_size;
+  src.page_shift = 31 - __builtin_clz(src.page_size);
+  src.last_tok = kv_len - 1;
+  src.pages = a.pt.page_indices + (a.pt.cu_kv_lens ? (a.pt.cu_kv_lens[seq] / a.pt.page_size)
+                                                  : (int64_t)seq * a.pt.pages_per_seq);
+  src.row_bytes = a.row_stride * 2;
+  src.page_stride = (int64_t)src.row_bytes * a.pt.page_size;
+  src.rope_byte = a.rope_offset * 2;
+  auto page_of = [&](int tb) -> int {
+    tb = min(tb, src.last_tok & ~(kTok - 1));
+    return scalar_load_i32(src.pages + __builtin_amdgcn_readfirstlane(page_slot(src, tb)));
+  };
+
+  // ---- Q^T operands: column c of block hb = head head0 + 16 hb + c, k-step ks covers dims 32ks + 8g .. ----
+  u32x4_t qB[2][18];
+#pragma unroll
+  for (int hb = 0; hb < 2; ++hb) {
+    const int head = min(head0 + 16 * hb + c, a.Hq - 1);
+    const uint16_t* qn = a.ql_nope + ((int64_t)tq * a.Hq + head) * 512 + g * 8;
+    const uint16_t* qr = a.q_pe + ((int64_t)tq * a.Hq + head) * 64 + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < 16; ++ks) qB[hb][ks] = ld16(qn + ks * 32);
+    qB[hb][16] = ld16(qr);
+    qB[hb][17] = ld16(qr + 32);
+  }
+  const float scale2 = a.sm.sm_scale * kLog2e;
+
+  int pg_next = page_of(t_begin + 3 * kTok);
+  copy_tile<true, CPW>(ring, src, a.cache, t_begin, wave, lane, page_of(t_begin));
+  copy_tile<true, CPW>(ring + kSlotB, src, a.cache, t_begin + kTok, wave, lane, page_of(t_begin + kTok));
+  copy_tile<true, CPW>(ring + 2 * kSlotB, src, a.cache, t_begin + 2 * kTok, wave, lane, page_of(t_begin + 2 * kTok));
+#pragma unroll
+  for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+    for (int ks = 0; ks < 18; ++ks) asm volatile("" ::"v"(qB[hb][ks]));
+  // the tiles the first step reads have landed once only the newest copies are outstanding (the generated
+  // loop says how many: the same count its own end-of-step wait uses)
+  __builtin_amdgcn_s_waitcnt(vmcnt_imm(RPA_MLA_WIDE_COPIES_AHEAD));
+  __syncthreads();
+
+  // ---- the reference of the probabilities: per head, the maximum of the first tile's visible scores ----
+  float m_init[2];
+  {
+    f32x4_t s[2][2];
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) s[hb][0] = s[hb][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const char* kp = ring + c * kRowB + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < 18; ++ks) {
+      const u32x4_t k0 = lds_ld16(kp + ks * 64);
+      const u32x4_t k1 = lds_ld16(kp + 16 * kRowB + ks * 64);
+#pragma unroll
+      for (int hb = 0; hb < 2; ++hb) {
+        s[hb][0] = mfma16(k0, qB[hb][ks], s[hb][0]);
+        s[hb][1] = mfma16(k1, qB[hb][ks], s[hb][1]);
+      }
+    }
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) {
+      float mx = -3.0e38f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int tok = t_begin + tok_of(g, i);
+        if (tok < kv_len && tok >= t_lo) mx = fmaxf(mx, s[hb][i >> 2][i & 3] * scale2);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      m_init[hb] = mx;
+    }
+  }
+
+  // ---- the loop ----
+  typedef __attribute__((address_space(3))) char* lds_ptr_t;
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)ring);
+  const int nT = (t_end - t_begin + kTok - 1) / kTok;
+  f32x32_t o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int e = 0; e < 32; ++e) o[i][e] = 0.f;
+  u32x32_t q0, q1, q2, q3;
+  u32x16_t q4;
+#pragma unroll
+  for (int e = 0; e < 32; ++e) {
+    q0[e] = qB[0][e >> 2][e & 3];
+    q1[e] = qB[0][8 + (e >> 2)][e & 3];
+    q3[e] = qB[1][6 + (e >> 2)][e & 3];           // registers 96 .. 127 = block 1, operands 6 .. 13
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) q2[e] = qB[0][16 + (e >> 2)][e & 3];                 // registers 64 .. 71
+#pragma unroll
+  for (int e = 8; e < 32; ++e) q2[e] = qB[1][(e - 8) >> 2][(e - 8) & 3];            // registers 72 .. 95 = block 1, operands 0 .. 5
+#pragma unroll
+  for (int e = 0; e < 16; ++e) q4[e] = qB[1][14 + (e >> 2)][e & 3];                // registers 128 .. 143
+  const int ln = fresh_lane();  // lane parts are worked out here, not carried from the top
+  const int cc = ln & 15, gg = ln >> 4;
+  u32x8_t ml = {__float_as_uint(m_init[0]), 0u, __float_as_uint(m_init[1]), 0u,
+                lds_base + (uint32_t)(cc * kRowB + gg * 16),
+                lds_base + (uint32_t)((4 * gg + (cc >> 2)) * kRowB + (cc & 3) * 8),
+                (uint32_t)(t_lo - t_begin - 4 * gg), (uint32_t)(kv_len - t_begin - 4 * gg)};
+  u32x16_t ofs, ofsl;
+#pragma unroll
+  for (int n = 0; n < 16; ++n) ofs[n] = ofsl[n] = 0;
+  const int last_row = src.last_tok & (kTok - 1);  // last valid row of the row's last tile
+#pragma unroll
+  for (int n = 0; n < CPW; ++n) {
+    int row, inner;
+    chunk_of<CPW>(src, wave, ln, n, row, inner);
+    ofs[n] = (uint32_t)(row * src.row_bytes + inner);
+    ofsl[n] = (uint32_t)(min(row, last_row) * src.row_bytes + inner);
+  }
+  const uint32_t cache_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)a.cache);
+  const uint32_t cache_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)a.cache >> 32));
+  const int last_tile_tok = __builtin_amdgcn_readfirstlane(src.last_tok & ~(kTok - 1));
+  const uint32_t scale2_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(scale2));
+  const int wave_blk = wave * CPW * 1024;
+  // `t` and `pg` change inside the block while the inputs are still being read: early-clobber, or the compiler
+  // may give an input that happens to hold the same value on entry (the LDS base, 0, and t = 0) the same register
+  int k = 0;
+#define C(n) RPA_MLA_WIDE_C_##n
+  asm volatile(RPA_MLA_WIDE_ASM
+               : "+" C(O0)(o[0]), "+" C(O1)(o[1]), "+" C(O2)(o[2]), "+" C(O3)(o[3]), "+" C(O4)(o[4]), "+" C(O5)(o[5]),
+                 "+" C(O6)(o[6]), "+" C(O7)(o[7]), "+" C(ML)(ml), "+" C(OFS)(ofs), [t] "+&s"(k), [pg] "+&s"(pg_next)
+               : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), C(Q3)(q3), C(Q4)(q4), C(OFSL)(ofsl), [t_end] "s"(nT),
+                 [t_begin] "s"(t_begin), [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes),
+                 [pshift] "s"(src.page_shift), [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages),
+                 [scale2] "s"(scale2_bits), [wave_blk] "s"(wave_blk), [slot0] "s"(lds_base)
+               : RPA_MLA_WIDE_CLOBBERS);
+#undef C
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the copies issued past the end
+
+  // ---- epilogue: lane (c, g) holds head head0 + 16 hb + c, dims 16j + 4g + r in accumulator 128 hb + 4 j + r ----
+  const int lo_ = fresh_lane();
+  const int c_out = lo_ & 15, g_out = lo_ >> 4;
+#pragma unroll
+  for (int hb = 0; hb < 2; ++hb) {
+    const float m = __uint_as_float(ml[2 * hb]);
+    float l = __uint_as_float(ml[2 * hb + 1]);
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    const int head = head0 + 16 * hb + c_out;
+    if (head >= a.Hq) continue;
+    if (dest.final_rows) {
+      const float inv = a.out_scale / l;
+      uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 512 + g_out * 4;
+#pragma unroll
+      for (int j = 0; j < 32; ++j) {
+        const int e = (4 * j) & 31, i = 4 * hb + (j >> 3);
+        u32x2_t w = {pack_bf16x2(o[i][e] * inv, o[i][e + 1] * inv), pack_bf16x2(o[i][e + 2] * inv, o[i][e + 3] * inv)};
+        *reinterpret_cast<u32x2_t*>(op + j * 16) = w;
+      }
+    } else {
+      const int64_t slot = dest.base + head;
+      uint16_t* wo = a.ws_o + slot * 512 + g_out * 4;
+#pragma unroll
+      for (int j = 0; j < 32; ++j) {
+        const int e = (4 * j) & 31, i = 4 * hb + (j >> 3);
+        u32x2_t w = {pack_bf16x2(o[i][e], o[i][e + 1]), pack_bf16x2(o[i][e + 2], o[i][e + 3])};
+        *reinterpret_cast<u32x2_t*>(wo + j * 16) = w;
+      }
+      if (g_out == 0) {
+        a.ws_ml[slot * 2 + 0] = m;
+        a.ws_ml[slot * 2 + 1] = l;
+      }
+    }
+  }
+  // every wave has left the loop behind its last barrier; the next segment's first copies overwrite slots
+  // 0 .. 2, whose last readers (this segment's last steps) may still be running in another wave
+  __syncthreads();
+}
+
+// ---- fixed split plan, wide workgroups: grid = (max_splits, rows, head groups of 128); block = 256 threads
+__global__ __launch_bounds__(256, 1) void rpa_mla_decode_wide_kernel(const MlaDecodeArgs a) {
+  __shared__ __attribute__((aligned(1024))) char ring[4 * kSlotB];
+  const int row_id = blockIdx.y;
+  const int split = blockIdx.x;
+  const MlaRow mr = mla_row(a, row_id);
+  if (!mr.valid) return;
+  const int kv_len = mr.kv_len;
+  if (kv_len <= 0) return;
+  const int t_lo = (a.sm.window > 0) ? max(0, kv_len - a.sm.window) : 0;
+  const int t0 = t_lo & ~(kTok - 1);
+  const int t_begin = t0 + split * a.chunk;
+  if (t_begin >= kv_len) return;
+  const int t_end = (split == a.max_splits - 1) ? kv_len : min(kv_len, t_begin + a.chunk);
+  MlaDest dest;
+  dest.final_rows = a.max_splits == 1;
+  dest.base = ((int64_t)row_id * a.max_splits + split) * a.Hq;
+  mla_segment_wide(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, ring);
+}
+
 // ---- balanced plan (one row per sequence): the 32-token tiles of the whole batch, sequence by
 // sequence and inside a sequence head group by head group, are dealt evenly to the workgroups;
 // workgroup j takes tiles [j * pw, (j + 1) * pw).  Pieces that are whole rows are finished in
@@ -664,12 +884,9 @@ __device__ __forceinline__ int mla_tiles_per_wg(const MlaDecodeArgs& a, int tota
   return max(a.forced_tiles_per_wg > 0 ? a.forced_tiles_per_wg : a.min_tiles_per_wg, even);
 }
 
-template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false>
-__global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecodeArgs a) {
-  __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
-  __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
-  __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
-  __shared__ __attribute__((aligned(1024))) char slot3[kSlotB];
+// `segment(mr, head_base, t_lo, t_begin, t_end, dest)` runs one piece on the workgroup's LDS ring.
+template <class Segment>
+__device__ __forceinline__ void mla_balanced_body(const MlaDecodeArgs& a, Segment segment) {
   const int lane = threadIdx.x & 63;
   const int wg = blockIdx.x;
   const int units = (a.Hq + 127) / 128;
@@ -754,8 +971,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
     dest.final_rows = (tile == 0) && (take == nt);
     dest.base = ((int64_t)wg * 2 + (first_piece ? 0 : 1)) * 128 - unit * 128;  // + head
     first_piece = false;
-    mla_segment<UNIFORM, CAP, PIPE, FP8>(a, mr, unit * 128, t_lo, t0 + tile * kTok,
-                                    min(kv_len, t0 + (tile + take) * kTok), dest, slot0, slot1, slot2, slot3);
+    segment(mr, unit * 128, t_lo, t0 + tile * kTok, min(kv_len, t0 + (tile + take) * kTok), dest);
     x += take;
     if (x < x_end && tile + take == nt && unit == units - 1) {
       seq_first += (nt + pad) * units;
@@ -766,6 +982,28 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
       } while (nt == 0);
     }
   }
+}
+
+
+template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false>
+__global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecodeArgs a) {
+  __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot3[kSlotB];
+  mla_balanced_body(a, [&](const MlaRow& mr, int head_base, int t_lo, int t_begin, int t_end, const MlaDest& dest)
+                        __attribute__((always_inline)) {
+    mla_segment<UNIFORM, CAP, PIPE, FP8>(a, mr, head_base, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
+  });
+}
+
+// the same plan on wide workgroups (four waves of 32 heads)
+__global__ __launch_bounds__(256, 1) void rpa_mla_balanced_wide_kernel(const MlaDecodeArgs a) {
+  __shared__ __attribute__((aligned(1024))) char ring[4 * kSlotB];
+  mla_balanced_body(a, [&](const MlaRow& mr, int head_base, int t_lo, int t_begin, int t_end, const MlaDest& dest)
+                        __attribute__((always_inline)) {
+    mla_segment_wide(a, mr, head_base, t_lo, t_begin, t_end, dest, ring);
+  });
 }
 
 // Merge the n partial rows of one (row, head): 128 threads, 4 dims each.  Partials are taken eight at
@@ -923,6 +1161,27 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
       ef = hipGetLastError();
     }
     return ef;
+  }
+  // wide workgroups (four waves of 32 heads) wherever the assembly loop applies; RPA_MLA_WIDE=0 keeps the
+  // eight-wave kernels (read per call: tests switch it)
+  const char* wide_env = getenv("RPA_MLA_WIDE");
+  const bool wide = !(wide_env && *wide_env == '0') && pipe;
+  if (wide && a.balanced) {
+    hipLaunchKernelGGL(rpa_mla_balanced_wide_kernel, dim3(a.num_wgs), dim3(256), 0, stream, a);
+    hipError_t eb = hipGetLastError();
+    if (eb != hipSuccess) return eb;
+    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+    return hipGetLastError();
+  }
+  if (wide) {
+    hipLaunchKernelGGL(rpa_mla_decode_wide_kernel, grid, dim3(256), 0, stream, a);
+    hipError_t ew = hipGetLastError();
+    if (ew != hipSuccess) return ew;
+    if (a.max_splits > 1) {
+      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      ew = hipGetLastError();
+    }
+    return ew;
   }
   if (a.balanced) {
     const dim3 bgrid(a.num_wgs);

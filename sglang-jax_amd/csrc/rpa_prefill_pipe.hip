@@ -235,11 +235,13 @@ struct LoopScalars {
 __device__ __forceinline__ void pipe_loop(RowBlock (&b)[1], const Shared& sh, int& t, int& pg_a, int& pg_b,
                                           const LoopScalars& sc) {
 #define C(n) RPA_PIPE_NQ1_C_##n
+  // t and the page ids change inside the block while inputs are still being read: early-clobber, so that no
+  // input that happens to hold the same value on entry can share their registers
   asm volatile(RPA_PIPE_NQ1_ASM
                : "+" C(O00)(b[0].O[0]), "+" C(O01)(b[0].O[1]), "+" C(O02)(b[0].O[2]), "+" C(O03)(b[0].O[3]),
                  "+" C(S00)(b[0].S[0]), "+" C(S01)(b[0].S[1]), "+" C(P00)(b[0].P[0]), "+" C(P01)(b[0].P[1]),
                  "+" C(NM0)(b[0].NM), "+" C(M0)(b[0].m), "+" C(L0)(b[0].l),
-                 [t] "+s"(t), [pg_a] "+s"(pg_a), [pg_b] "+s"(pg_b)
+                 [t] "+&s"(t), [pg_a] "+&s"(pg_a), [pg_b] "+&s"(pg_b)
                : C(Q0)(b[0].Q), C(KOFF)(sh.koff), C(VOFF)(sh.voff), C(OFSK)(sh.ofs_k), C(OFSV)(sh.ofs_v),
                  RPA_PIPE_SCALARS(sc)
                : RPA_PIPE_NQ1_CLOBBERS);
@@ -256,7 +258,7 @@ __device__ __forceinline__ void pipe_loop(RowBlock (&b)[2], const Shared& sh, in
                  "+" C(S10)(b[1].S[0]), "+" C(S11)(b[1].S[1]), "+" C(P10)(b[1].P[0]), "+" C(P11)(b[1].P[1]),
                  "+" C(NM0)(b[0].NM), "+" C(M0)(b[0].m), "+" C(L0)(b[0].l),
                  "+" C(NM1)(b[1].NM), "+" C(M1)(b[1].m), "+" C(L1)(b[1].l),
-                 [t] "+s"(t), [pg_a] "+s"(pg_a), [pg_b] "+s"(pg_b)
+                 [t] "+&s"(t), [pg_a] "+&s"(pg_a), [pg_b] "+&s"(pg_b)
                : C(Q0)(b[0].Q), C(Q1)(b[1].Q), C(KOFF)(sh.koff), C(VOFF)(sh.voff), C(OFSK)(sh.ofs_k), C(OFSV)(sh.ofs_v),
                  RPA_PIPE_SCALARS(sc)
                : RPA_PIPE_NQ2_CLOBBERS);

@@ -372,6 +372,38 @@ def test_mla_assembly_loop_against_compiled_loop(pkg, wl, gpu, window, monkeypat
     assert_parity(run_gpu(pkg, b, gpu)[:sum(q_lens)].float(), oracle(b).float(), **TOL)
 
 
+@pytest.mark.parametrize("window", [None, 3000])
+def test_mla_wide_workgroups_against_eight_wave_workgroups(pkg, wl, gpu, window, monkeypatch):
+    """128 heads, 64-token pages, bf16 cache: by default four waves of 32 heads run every tile of a
+    segment inside the assembly loop of rpa_mla_wide_loop.inc (masks of the first and last tile, clamped
+    copies of the row's last tile and the reference-raising path included); RPA_MLA_WIDE=0 keeps the
+    eight-wave kernels.  Rows from one token to 12800, ends on and off tile borders, with and without
+    planted keys, every plan: against the oracle and against each other."""
+    kv_lens = [1, 31, 32, 33, 96, 127, 128, 129, 160, 161, 256, 416, 1000, 2048, 4097, 6001, 12800, 9999]
+    for needles in (False, True):
+        b = wl.make_mla_batch("mla_wide", [1] * len(kv_lens), kv_lens, num_q_heads=128, lkv_dim=512, rope_dim=64,
+                              page_size=64, seed=8620 + needles, sliding_window=window)
+        if needles:
+            wl.plant_mla_needles(b, seed=6)
+        want = oracle(b)
+        for kw in ({}, {"num_splits": 1}, {"num_splits": 3}, {"num_splits": 40}):
+            say(f"mla wide workgroups window={window} needles={needles} {kw}")
+            monkeypatch.delenv("RPA_MLA_WIDE", raising=False)
+            on = run_gpu(pkg, b, gpu, **kw)[:len(kv_lens)]
+            monkeypatch.setenv("RPA_MLA_WIDE", "0")
+            off = run_gpu(pkg, b, gpu, **kw)[:len(kv_lens)]
+            monkeypatch.delenv("RPA_MLA_WIDE")
+            assert_parity(on.float(), want.float(), **TOL)
+            assert_parity(off.float(), want.float(), **TOL)
+            assert float(row_rel_error(on.float(), off.float()).max()) < 1e-2
+            assert not torch.equal(on, off)  # two kernels: the last bits differ somewhere
+    # chunks on long prefixes (one row per query token), 256 heads (two workgroups per row), 32-token pages
+    for Hq, P, q_lens, kv_lens in ((128, 64, [1, 70, 33], [5000, 4170, 1033]), (256, 32, [40, 1], [1500, 700])):
+        b = wl.make_mla_batch("mla_wide_chunks", q_lens, kv_lens, num_q_heads=Hq, lkv_dim=512, rope_dim=64, page_size=P,
+                              seed=8630, sliding_window=window)
+        assert_parity(run_gpu(pkg, b, gpu)[:sum(q_lens)].float(), oracle(b).float(), **TOL)
+
+
 FP8 = torch.float8_e4m3fn
 FP8_TOL = dict(rtol=5e-2, atol=5e-2)
 
