@@ -89,7 +89,8 @@ PGN = 66                     # page id of tile t + 4
 ONES, LIMIT, DELTA, PASS = 67, 68, 69, 70
 PMASK, PSTR = 71, 72         # page_size - 1, bytes per page
 LASTK = 73                   # index of the row's last tile inside the segment
-SGPR_CLOBBERS = list(range(60, 74))
+CPB, CPL = 74, 75            # LDS addresses for the step's copies (see copy_group)
+SGPR_CLOBBERS = list(range(60, 76))
 
 NEG_BIG = "0xf149f2ca"       # -1e30
 
@@ -156,15 +157,18 @@ def softmax(hb, sc, check=True):
 
 
 def copy_group(n, fill_slot):
-    """copy n of this wave: block 10 * wave + n of the slot (blocks past the 37th repeat block 0)"""
-    a = f"s{ST[0]}"
-    return [Ins(f"s_add_u32 {a}, %[wave_blk], {n * 1024}", "salu"),
-            Ins(f"s_cmp_lt_u32 {a}, {BLOCKS * 1024}", "salu"),
-            Ins(f"s_cselect_b32 {a}, {a}, 0", "salu"),
-            Ins(f"s_add_u32 {a}, {a}, {fill_slot * SLOT_B}", "salu"),
-            Ins(f"s_add_u32 m0, {a}, %[slot0]", "salu"),
+    """copy n of this wave: block 10 * wave + n of the slot (blocks past the 37th repeat the last one); s[CPB] is
+    the LDS address of the wave's first block in the slot being filled, s[CPL] that of the slot's last block"""
+    return [Ins(f"s_add_u32 m0, s{CPB}, {n * 1024}", "salu"),
+            Ins(f"s_min_u32 m0, m0, s{CPL}", "salu"),
             Ins("s_nop 0", "nop"),
             Ins(f"global_load_lds_dwordx4 {vr(OFS + n)}, s[{SB}:{SB + 1}]", "vmem", [OFS + n], [])]
+
+
+def copy_bases(em, fill_slot):
+    em.raw(f"s_add_u32 s{CPL}, %[slot0], {fill_slot * SLOT_B + (BLOCKS - 1) * 1024}")
+    em.raw(f"s_add_u32 s{CPB}, %[slot0], {fill_slot * SLOT_B}")
+    em.raw(f"s_add_u32 s{CPB}, s{CPB}, %[wave_blk]")
 
 
 def tile_scalars(em, k):
@@ -340,6 +344,7 @@ def step_plain(em, k):
     """tile t in slot k: scores, softmax, second product; tile t + 3 goes to slot (k + 3) & 3"""
     fill = (k + 3) & 3
     tile_scalars(em, k)
+    copy_bases(em, fill)
     em.emit(valu(f"v_add_u32 {vr(KADDR)}, {k * SLOT_B}, {vr(KBASE)}", [KBASE], [KADDR]))
     em.emit(valu(f"v_add_u32 {vr(VADDR)}, {k * SLOT_B}, {vr(VBASE)}", [VBASE], [VADDR]))
     copies = [] if "nocopy" in X else [copy_group(n, fill) for n in range(COPIES)]
@@ -357,6 +362,7 @@ def step_pipelined(em, k):
     fill = (k + 3) & 3
     cur, nxt = (SC, SC2) if k % 2 == 0 else (SC2, SC)
     tile_scalars(em, k)
+    copy_bases(em, fill)
     em.emit(valu(f"v_add_u32 {vr(KADDR2)}, {((k + 1) & 3) * SLOT_B}, {vr(KBASE)}", [KBASE], [KADDR2]))
     em.emit(valu(f"v_add_u32 {vr(VADDR)}, {k * SLOT_B}, {vr(VBASE)}", [VBASE], [VADDR]))
     copies = [] if "nocopy" in X else [copy_group(n, fill) for n in range(COPIES)]

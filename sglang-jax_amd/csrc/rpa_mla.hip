@@ -96,7 +96,8 @@ __device__ __forceinline__ int page_slot(const Src& s, int tok) {
 template <int CPW = kCopiesPerWave>
 __device__ __forceinline__ int copy_block(int wave, int n) {
   const int blk = wave * CPW + n;
-  return blk < kUsedBlocks ? blk : 0;
+  if constexpr (CPW == kCopiesPerWave) return blk < kUsedBlocks ? blk : 0;
+  else return min(blk, kUsedBlocks - 1);  // wide workgroups: the spare copies repeat the last block
 }
 
 template <int CPW = kCopiesPerWave>
