@@ -28,6 +28,7 @@
 #include "rpa_kernels.h"
 #include "rpa_mla_pipe_loop.inc"
 #include "rpa_mla_wide_loop.inc"
+#include "rpa_mla_wide32_loop.inc"
 
 namespace rpa {
 
@@ -651,13 +652,17 @@ constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 // clamped copies of the row's last tile included); compiled code only loads the queries, starts the ring,
 // takes the first tile's maxima as the reference and writes the result.  bf16 caches, pages of a
 // power-of-two size >= 32, no soft cap, Hq a multiple of 128.  `ring`: the four slots, contiguous.
+// M32: the loop of rpa_mla_wide32_loop.inc (32x32x16 matrix instructions, one head per lane and half: lane c of
+// half h = lane / 32 owns head head0 + c and the tokens 8 (i / 4) + 4 h + i % 4 of a tile) instead of two blocks of
+// 16 heads on 16x16x32 instructions.
+template <bool M32>
 __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
                                                  int t_begin, int t_end, const MlaDest dest, char* ring) {
   constexpr int CPW = 2 * kCopiesPerWave;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int c = lane & 15, g = lane >> 4;
+  const int c = M32 ? (lane & 31) : (lane & 15), g = M32 ? (lane >> 5) : (lane >> 4);
   const int head0 = head_base + wave * 32;
   const int seq = mr.seq;
   const int kv_len = mr.kv_len;
@@ -678,16 +683,26 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   };
 
   // ---- Q^T operands: column c of block hb = head head0 + 16 hb + c, k-step ks covers dims 32ks + 8g .. ----
+  // 16x16x32: qB[hb][ks], k-step ks covers dims 32ks + 8g ..; 32x32x16: the same 36 registers of 4 as
+  // qB[ks / 18][ks % 18], k-step ks covers dims 16ks + 8g .. of head head0 + c
   u32x4_t qB[2][18];
-#pragma unroll
-  for (int hb = 0; hb < 2; ++hb) {
-    const int head = min(head0 + 16 * hb + c, a.Hq - 1);
+  if constexpr (M32) {
+    const int head = min(head0 + c, a.Hq - 1);
     const uint16_t* qn = a.ql_nope + ((int64_t)tq * a.Hq + head) * 512 + g * 8;
     const uint16_t* qr = a.q_pe + ((int64_t)tq * a.Hq + head) * 64 + g * 8;
 #pragma unroll
-    for (int ks = 0; ks < 16; ++ks) qB[hb][ks] = ld16(qn + ks * 32);
-    qB[hb][16] = ld16(qr);
-    qB[hb][17] = ld16(qr + 32);
+    for (int ks = 0; ks < 36; ++ks) qB[ks / 18][ks % 18] = ld16(ks < 32 ? qn + ks * 16 : qr + (ks - 32) * 16);
+  } else {
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) {
+      const int head = min(head0 + 16 * hb + c, a.Hq - 1);
+      const uint16_t* qn = a.ql_nope + ((int64_t)tq * a.Hq + head) * 512 + g * 8;
+      const uint16_t* qr = a.q_pe + ((int64_t)tq * a.Hq + head) * 64 + g * 8;
+#pragma unroll
+      for (int ks = 0; ks < 16; ++ks) qB[hb][ks] = ld16(qn + ks * 32);
+      qB[hb][16] = ld16(qr);
+      qB[hb][17] = ld16(qr + 32);
+    }
   }
   const float scale2 = a.sm.sm_scale * kLog2e;
 
@@ -701,12 +716,26 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
     for (int ks = 0; ks < 18; ++ks) asm volatile("" ::"v"(qB[hb][ks]));
   // the tiles the first step reads have landed once only the newest copies are outstanding (the generated
   // loop says how many: the same count its own end-of-step wait uses)
+  static_assert(RPA_MLA_WIDE_COPIES_AHEAD == RPA_MLA_WIDE32_COPIES_AHEAD, "one prologue for both loops");
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(RPA_MLA_WIDE_COPIES_AHEAD));
   __syncthreads();
 
   // ---- the reference of the probabilities: per head, the maximum of the first tile's visible scores ----
   float m_init[2];
-  {
+  if constexpr (M32) {
+    f32x16_t s = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const char* kp = ring + c * kRowB + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < 36; ++ks) s = mfma32(lds_ld16(kp + ks * 32), qB[ks / 18][ks % 18], s);
+    float mx = -3.0e38f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int tok = t_begin + 8 * (i >> 2) + 4 * g + (i & 3);
+      if (tok < kv_len && tok >= t_lo) mx = fmaxf(mx, s[i] * scale2);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    m_init[0] = m_init[1] = mx;
+  } else {
     f32x4_t s[2][2];
 #pragma unroll
     for (int hb = 0; hb < 2; ++hb) s[hb][0] = s[hb][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -759,11 +788,23 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
 #pragma unroll
   for (int e = 0; e < 16; ++e) q4[e] = qB[1][14 + (e >> 2)][e & 3];                // registers 128 .. 143
   const int ln = fresh_lane();  // lane parts are worked out here, not carried from the top
-  const int cc = ln & 15, gg = ln >> 4;
-  u32x8_t ml = {__float_as_uint(m_init[0]), 0u, __float_as_uint(m_init[1]), 0u,
-                lds_base + (uint32_t)(cc * kRowB + gg * 16),
-                lds_base + (uint32_t)((4 * gg + (cc >> 2)) * kRowB + (cc & 3) * 8),
-                (uint32_t)(t_lo - t_begin - 4 * gg), (uint32_t)(kv_len - t_begin - 4 * gg)};
+  u32x8_t ml;
+  if constexpr (M32) {
+    // K operand: row c, bytes 32ks + 16g.  V^T operand of (dim block d, k-step kk): the lane points at token
+    // 16kk + 4g + (r >> 2) (+ 8 for the second read), dims 32d + 16 (b & 1) + 8 ((r & 3) >> 1) + 4 (r & 1), with
+    // r = lane & 15, b = lane >> 4 (what the transposing read hands to lane dim = lane % 32)
+    const int cc = ln & 31, gg = ln >> 5, r16 = ln & 15, b16 = ln >> 4;
+    const int v_in = ((b16 & 1) << 5) + (((r16 & 3) >> 1) << 4) + ((r16 & 1) << 3);
+    ml = u32x8_t{__float_as_uint(m_init[0]), 0u, lds_base + (uint32_t)(cc * kRowB + gg * 16),
+                 lds_base + (uint32_t)((4 * gg + (r16 >> 2)) * kRowB + v_in), (uint32_t)(t_lo - t_begin - 4 * gg),
+                 (uint32_t)(kv_len - t_begin - 4 * gg), 0u, 0u};
+  } else {
+    const int cc = ln & 15, gg = ln >> 4;
+    ml = u32x8_t{__float_as_uint(m_init[0]), 0u, __float_as_uint(m_init[1]), 0u,
+                 lds_base + (uint32_t)(cc * kRowB + gg * 16),
+                 lds_base + (uint32_t)((4 * gg + (cc >> 2)) * kRowB + (cc & 3) * 8),
+                 (uint32_t)(t_lo - t_begin - 4 * gg), (uint32_t)(kv_len - t_begin - 4 * gg)};
+  }
   u32x16_t ofs, ofsl;
 #pragma unroll
   for (int n = 0; n < 16; ++n) ofs[n] = ofsl[n] = 0;
@@ -783,20 +824,52 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   // `t` and `pg` change inside the block while the inputs are still being read: early-clobber, or the compiler
   // may give an input that happens to hold the same value on entry (the LDS base, 0, and t = 0) the same register
   int k = 0;
+  // both loops bind their operands to the same registers
 #define C(n) RPA_MLA_WIDE_C_##n
-  asm volatile(RPA_MLA_WIDE_ASM
-               : "+" C(O0)(o[0]), "+" C(O1)(o[1]), "+" C(O2)(o[2]), "+" C(O3)(o[3]), "+" C(O4)(o[4]), "+" C(O5)(o[5]),
-                 "+" C(O6)(o[6]), "+" C(O7)(o[7]), "+" C(ML)(ml), "+" C(OFS)(ofs), [t] "+&s"(k), [pg] "+&s"(pg_next)
-               : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), C(Q3)(q3), C(Q4)(q4), C(OFSL)(ofsl), [t_end] "s"(nT),
-                 [t_begin] "s"(t_begin), [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes),
-                 [pshift] "s"(src.page_shift), [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages),
-                 [scale2] "s"(scale2_bits), [wave_blk] "s"(wave_blk), [slot0] "s"(lds_base)
-               : RPA_MLA_WIDE_CLOBBERS);
+#define RPA_WIDE_OPERANDS                                                                                              \
+  : "+" C(O0)(o[0]), "+" C(O1)(o[1]), "+" C(O2)(o[2]), "+" C(O3)(o[3]), "+" C(O4)(o[4]), "+" C(O5)(o[5]),                \
+    "+" C(O6)(o[6]), "+" C(O7)(o[7]), "+" C(ML)(ml), "+" C(OFS)(ofs), [t] "+&s"(k), [pg] "+&s"(pg_next)                 \
+  : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), C(Q3)(q3), C(Q4)(q4), C(OFSL)(ofsl), [t_end] "s"(nT), [t_begin] "s"(t_begin),     \
+    [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),                  \
+    [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2_bits),             \
+    [wave_blk] "s"(wave_blk), [slot0] "s"(lds_base)
+  if constexpr (M32) {
+    asm volatile(RPA_MLA_WIDE32_ASM RPA_WIDE_OPERANDS : RPA_MLA_WIDE32_CLOBBERS);
+  } else {
+    asm volatile(RPA_MLA_WIDE_ASM RPA_WIDE_OPERANDS : RPA_MLA_WIDE_CLOBBERS);
+  }
+#undef RPA_WIDE_OPERANDS
 #undef C
   __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the copies issued past the end
 
-  // ---- epilogue: lane (c, g) holds head head0 + 16 hb + c, dims 16j + 4g + r in accumulator 128 hb + 4 j + r ----
+  // ---- epilogue ----
   const int lo_ = fresh_lane();
+  if constexpr (M32) {
+    // lane (c, h) holds head head0 + c, dims 32d + 8q + 4h + r in accumulator 16d + 4q + r
+    const int c_out = lo_ & 31, h_out = lo_ >> 5;
+    const float m = __uint_as_float(ml[0]);
+    float l = __uint_as_float(ml[1]);
+    l += __shfl_xor(l, 32);
+    const int head = head0 + c_out;
+    if (head < a.Hq) {
+      const float inv = dest.final_rows ? a.out_scale / l : 1.0f;
+      uint16_t* op = dest.final_rows ? a.out + ((int64_t)tq * a.Hq + head) * 512 + h_out * 4
+                                     : a.ws_o + (dest.base + head) * 512 + h_out * 4;
+#pragma unroll
+      for (int d = 0; d < 16; ++d)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int e = (16 * d + 4 * q) & 31, i = d >> 1;
+          u32x2_t w = {pack_bf16x2(o[i][e] * inv, o[i][e + 1] * inv), pack_bf16x2(o[i][e + 2] * inv, o[i][e + 3] * inv)};
+          *reinterpret_cast<u32x2_t*>(op + 32 * d + 8 * q) = w;
+        }
+      if (!dest.final_rows && h_out == 0) {
+        a.ws_ml[(dest.base + head) * 2 + 0] = m;
+        a.ws_ml[(dest.base + head) * 2 + 1] = l;
+      }
+    }
+  } else {
+  // lane (c, g) holds head head0 + 16 hb + c, dims 16j + 4g + r in accumulator 128 hb + 4 j + r
   const int c_out = lo_ & 15, g_out = lo_ >> 4;
 #pragma unroll
   for (int hb = 0; hb < 2; ++hb) {
@@ -830,12 +903,14 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
       }
     }
   }
+  }
   // every wave has left the loop behind its last barrier; the next segment's first copies overwrite slots
   // 0 .. 2, whose last readers (this segment's last steps) may still be running in another wave
   __syncthreads();
 }
 
 // ---- fixed split plan, wide workgroups: grid = (max_splits, rows, head groups of 128); block = 256 threads
+template <bool M32>
 __global__ __launch_bounds__(256, 1) void rpa_mla_decode_wide_kernel(const MlaDecodeArgs a) {
   __shared__ __attribute__((aligned(1024))) char ring[4 * kSlotB];
   const int row_id = blockIdx.y;
@@ -852,7 +927,7 @@ __global__ __launch_bounds__(256, 1) void rpa_mla_decode_wide_kernel(const MlaDe
   MlaDest dest;
   dest.final_rows = a.max_splits == 1;
   dest.base = ((int64_t)row_id * a.max_splits + split) * a.Hq;
-  mla_segment_wide(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, ring);
+  mla_segment_wide<M32>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, ring);
 }
 
 // ---- balanced plan (one row per sequence): the 32-token tiles of the whole batch, sequence by
@@ -999,11 +1074,12 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
 }
 
 // the same plan on wide workgroups (four waves of 32 heads)
+template <bool M32>
 __global__ __launch_bounds__(256, 1) void rpa_mla_balanced_wide_kernel(const MlaDecodeArgs a) {
   __shared__ __attribute__((aligned(1024))) char ring[4 * kSlotB];
   mla_balanced_body(a, [&](const MlaRow& mr, int head_base, int t_lo, int t_begin, int t_end, const MlaDest& dest)
                         __attribute__((always_inline)) {
-    mla_segment_wide(a, mr, head_base, t_lo, t_begin, t_end, dest, ring);
+    mla_segment_wide<M32>(a, mr, head_base, t_lo, t_begin, t_end, dest, ring);
   });
 }
 
@@ -1167,15 +1243,22 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   // eight-wave kernels (read per call: tests switch it)
   const char* wide_env = getenv("RPA_MLA_WIDE");
   const bool wide = !(wide_env && *wide_env == '0') && pipe;
+  // RPA_MLA_WIDE=32: the wide loop on 32x32x16 matrix instructions (one head per lane and half).  Half the matrix
+  // instructions, and 8 % faster than the default loop when neither reads its operands -- but its 32-row LDS
+  // reads collide on the 1184-byte row pitch that suits the 16-row reads (7 % slower as a whole): opt-in until
+  // it has a row layout of its own
+  const bool m32 = wide_env && wide_env[0] == '3' && wide_env[1] == '2';
   if (wide && a.balanced) {
-    hipLaunchKernelGGL(rpa_mla_balanced_wide_kernel, dim3(a.num_wgs), dim3(256), 0, stream, a);
+    if (m32) hipLaunchKernelGGL(rpa_mla_balanced_wide_kernel<true>, dim3(a.num_wgs), dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(rpa_mla_balanced_wide_kernel<false>, dim3(a.num_wgs), dim3(256), 0, stream, a);
     hipError_t eb = hipGetLastError();
     if (eb != hipSuccess) return eb;
     hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
     return hipGetLastError();
   }
   if (wide) {
-    hipLaunchKernelGGL(rpa_mla_decode_wide_kernel, grid, dim3(256), 0, stream, a);
+    if (m32) hipLaunchKernelGGL(rpa_mla_decode_wide_kernel<true>, grid, dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(rpa_mla_decode_wide_kernel<false>, grid, dim3(256), 0, stream, a);
     hipError_t ew = hipGetLastError();
     if (ew != hipSuccess) return ew;
     if (a.max_splits > 1) {

@@ -208,12 +208,12 @@ def test_generated_assembly_is_up_to_date(tmp_path):
     csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "sglang-jax_amd", "csrc")
     work = tmp_path / "csrc"
     work.mkdir()
-    for name in ("gen_prefill_pipe_loop.py", "gen_mla_pipe_loop.py", "gen_mla_wide_loop.py"):
+    for name in ("gen_prefill_pipe_loop.py", "gen_mla_pipe_loop.py", "gen_mla_wide_loop.py", "gen_mla_wide32_loop.py"):
         shutil.copy(os.path.join(csrc, name), work / name)
     env = {k: v for k, v in os.environ.items() if not k.startswith(("RPA_PIPE_", "RPA_MLA_PIPE_", "RPA_MLA_WIDE_"))}
     env["PYTHONDONTWRITEBYTECODE"] = "1"
     for gen, inc in (("gen_prefill_pipe_loop.py", "rpa_prefill_pipe_loop.inc"), ("gen_mla_pipe_loop.py", "rpa_mla_pipe_loop.inc"),
-                     ("gen_mla_wide_loop.py", "rpa_mla_wide_loop.inc")):
+                     ("gen_mla_wide_loop.py", "rpa_mla_wide_loop.inc"), ("gen_mla_wide32_loop.py", "rpa_mla_wide32_loop.inc")):
         subprocess.run([sys.executable, str(work / gen)], check=True, env=env, stdout=subprocess.DEVNULL)
         with open(work / inc) as f, open(os.path.join(csrc, inc)) as g:
             assert f.read() == g.read(), f"{inc} is stale: run {gen}"

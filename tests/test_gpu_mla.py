@@ -404,6 +404,33 @@ def test_mla_wide_workgroups_against_eight_wave_workgroups(pkg, wl, gpu, window,
         assert_parity(run_gpu(pkg, b, gpu)[:sum(q_lens)].float(), oracle(b).float(), **TOL)
 
 
+@pytest.mark.parametrize("window", [None, 3000])
+def test_mla_wide_workgroups_on_32x32_matrix_instructions(pkg, wl, gpu, window, monkeypatch):
+    """RPA_MLA_WIDE=32: the wide loop generated for 32x32x16 matrix instructions (one head per lane and half,
+    rpa_mla_wide32_loop.inc; opt-in): same cases, against the oracle and the default loop."""
+    kv_lens = [1, 31, 32, 33, 96, 127, 128, 129, 160, 161, 256, 416, 1000, 2048, 4097, 6001, 12800, 9999]
+    for needles in (False, True):
+        b = wl.make_mla_batch("mla_wide32", [1] * len(kv_lens), kv_lens, num_q_heads=128, lkv_dim=512, rope_dim=64,
+                              page_size=64, seed=8640 + needles, sliding_window=window)
+        if needles:
+            wl.plant_mla_needles(b, seed=7)
+        want = oracle(b)
+        for kw in ({}, {"num_splits": 1}, {"num_splits": 3}):
+            say(f"mla wide 32x32 window={window} needles={needles} {kw}")
+            monkeypatch.setenv("RPA_MLA_WIDE", "32")
+            on = run_gpu(pkg, b, gpu, **kw)[:len(kv_lens)]
+            monkeypatch.delenv("RPA_MLA_WIDE")
+            off = run_gpu(pkg, b, gpu, **kw)[:len(kv_lens)]
+            assert_parity(on.float(), want.float(), **TOL)
+            assert float(row_rel_error(on.float(), off.float()).max()) < 1e-2
+            assert not torch.equal(on, off)
+    monkeypatch.setenv("RPA_MLA_WIDE", "32")
+    q_lens, kv_lens = [1, 70, 33], [5000, 4170, 1033]
+    b = wl.make_mla_batch("mla_wide32_chunks", q_lens, kv_lens, num_q_heads=128, lkv_dim=512, rope_dim=64, page_size=64,
+                          seed=8650, sliding_window=window)
+    assert_parity(run_gpu(pkg, b, gpu)[:sum(q_lens)].float(), oracle(b).float(), **TOL)
+
+
 FP8 = torch.float8_e4m3fn
 FP8_TOL = dict(rtol=5e-2, atol=5e-2)
 
