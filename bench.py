@@ -44,24 +44,24 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # kernel that streams the KV bytes of each workload's decode rows: ragged batches that need
 # splitting take the balanced plan, equal-length and tiny ones the fixed split plan
 DECODE_KERNEL = {
-    "c5p": "rpa_mla_decode_kernel",
+    "c5p": "rpa_mla_decode_wide_kernel",
     "c1": "rpa_decode_splitkv_kernel",
     "c2": "rpa_decode_balanced_kernel",
     "c3": "rpa_decode_splitkv_kernel",
     "c4": "rpa_decode_balanced_kernel",
     "c4swa": "rpa_decode_splitkv_kernel",
-    "c5": "rpa_mla_balanced_kernel",
+    "c5": "rpa_mla_balanced_wide_kernel",
     "c5fp8": "rpa_mla_balanced_kernel",
 }
 
 PREFILL_KERNEL = "rpa_prefill_pipe_kernel"
 
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", PREFILL_KERNEL): 325.9e6 + 77.2e6,
+    ("c2", PREFILL_KERNEL): 327.2e6 + 77.2e6,
     ("c2", "rpa_decode_balanced_kernel"): 501.0e6 + 2.7e6,
     ("c3", "rpa_decode_splitkv_kernel"): 2148.6e6 + 1.9e6,
-    ("c5", "rpa_mla_balanced_kernel"): 824.0e6 + 49.3e6,
-    ("c5p", "rpa_mla_decode_kernel (one row per query token)"): 632.9e6 + 268.5e6,
+    ("c5", "rpa_mla_balanced_wide_kernel"): 820.3e6 + 44.8e6,
+    ("c5p", "rpa_mla_decode_wide_kernel (one row per query token)"): 633.5e6 + 268.5e6,
 }
 
 
@@ -424,7 +424,7 @@ def main():
     pre_tflops = main_res.get("prefill_tflops")
     # dominant kernel of the workload (largest average launch time inside the timed region)
     roofline_decode = decode_roofline(args.config, main_res) if dec_gbps is not None else None
-    prefill_kernel = "rpa_mla_decode_kernel (one row per query token)" if args.config == "c5p" else PREFILL_KERNEL
+    prefill_kernel = "rpa_mla_decode_wide_kernel (one row per query token)" if args.config == "c5p" else PREFILL_KERNEL
     if pre_tflops is not None and main_res.get("prefill_ms", 0) >= main_res.get("decode_ms", 0):
         roofline = {"kernel": prefill_kernel, "bound": "mfma", "achieved": pre_tflops,
                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": pre_tflops / MFMA_BF16_PEAK_TFLOPS,
@@ -460,7 +460,7 @@ def main():
                 continue
             r = run(name)
             if name == "c5p":
-                r["roofline"] = {"kernel": "rpa_mla_decode_kernel (one row per query token)", "bound": "mfma",
+                r["roofline"] = {"kernel": "rpa_mla_decode_wide_kernel (one row per query token)", "bound": "mfma",
                                  "achieved": r["prefill_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                  "frac": r["prefill_tflops"] / MFMA_BF16_PEAK_TFLOPS, "avg_launch_ms": r["prefill_ms"],
                                  "flops_per_launch": r["prefill_flops"]}
