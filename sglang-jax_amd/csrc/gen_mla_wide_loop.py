@@ -49,6 +49,7 @@ PIPELINED = "pipe" in X      # scores of tile t + 1 under the softmax of tile t 
 NBUF = 4 if PIPELINED else 8  # operand fragment buffers (the second set of score registers of the pipelined loop pays for four)
 AHEAD = int(os.environ.get("RPA_MLA_WIDE_AHEAD", 3 if PIPELINED else 6))
 assert AHEAD < NBUF
+PAIRWAIT = "nopairwait" not in X
 
 ROW_B = 1184                 # bytes of a latent row in LDS
 SLOT_B = 37 * 1024           # one ring slot
@@ -123,18 +124,25 @@ def frag_read(f, kaddr=None):
                 rng(dst + 2, 2), lds_tag=("vhi", f))]
 
 
+def frag_tags(f):
+    return [("k", f)] if f < 36 else [("vlo", f), ("vhi", f)]
+
+
 def frag_mfmas(f, sc):
-    """the two matrix instructions (one per block of heads) that consume fragment f; scores go to `sc`"""
+    """the two matrix instructions (one per block of heads) that consume fragment f; scores go to `sc`.  With
+    PAIRWAIT the first instruction of an even fragment also waits for the odd fragment behind it (requested long
+    before): one wait instruction per two fragments."""
     out = []
     for hb in range(2):
         if f < 36:
             ks, b = f >> 1, f & 1
             ins = mfma(sc[hb][b], ring(f), Q[hb] + 4 * ks, None if ks == 0 else sc[hb][b])
-            ins.lds_need = None if "nolds" in X else [("k", f)]
         else:
             j = f - 36
             ins = mfma(O[hb] + 4 * j, ring(f), P[hb], O[hb] + 4 * j)
-            ins.lds_need = None if "nolds" in X else [("vlo", f), ("vhi", f)]
+        ins.lds_need = None if "nolds" in X else list(frag_tags(f))
+        if PAIRWAIT and hb == 0 and f % 2 == 0 and ins.lds_need is not None and AHEAD >= 2:
+            ins.lds_need += frag_tags(f + 1)
         out.append(ins)
     return out
 
@@ -299,8 +307,10 @@ def softmax_and_check(em, k, hb, sc):
         em.emit(valu(f"v_add_f32 {vr(L[hb])}, {vr(L[hb])}, {vr(PS)}", [L[hb], PS], [L[hb]]))
 
 
-def qk_phase(em, sc, kaddr, copies, extra=None):
-    """the 72 matrix instructions of a tile's scores; copy groups and (pipelined loop) vector work in between"""
+def qk_phase(em, sc, kaddr, copies, extra=None, into_pv=False):
+    """the 72 matrix instructions of a tile's scores; copy groups and (pipelined loop) vector work in between.
+    `into_pv`: the operand requests run on into the second product's first fragments, which then travel under the
+    softmax"""
     extra = list(extra or [])
     copy_at = {2 + 3 * n: n for n in range(COPIES)}
     for f in range(AHEAD):
@@ -310,16 +320,17 @@ def qk_phase(em, sc, kaddr, copies, extra=None):
             em.emit(ins)
             if extra:
                 em.emit(extra.pop(0))
-        if f + AHEAD < 36:
+        if f + AHEAD < (68 if into_pv else 36):
             emit_all(em, frag_read(f + AHEAD, kaddr))
         if f in copy_at and copies:
             emit_all(em, copies[copy_at[f]])
     emit_all(em, extra)
 
 
-def pv_phase(em):
-    for f in range(36, 36 + AHEAD):
-        emit_all(em, frag_read(f))
+def pv_phase(em, prefetched=False):
+    if not prefetched:
+        for f in range(36, 36 + AHEAD):
+            emit_all(em, frag_read(f))
     for f in range(36, 68):
         emit_all(em, frag_mfmas(f, None))
         if f + AHEAD < 68:
@@ -348,11 +359,11 @@ def step_plain(em, k):
     em.emit(valu(f"v_add_u32 {vr(KADDR)}, {k * SLOT_B}, {vr(KBASE)}", [KBASE], [KADDR]))
     em.emit(valu(f"v_add_u32 {vr(VADDR)}, {k * SLOT_B}, {vr(VBASE)}", [VBASE], [VADDR]))
     copies = [] if "nocopy" in X else [copy_group(n, fill) for n in range(COPIES)]
-    qk_phase(em, SC, KADDR, copies)
+    qk_phase(em, SC, KADDR, copies, into_pv=True)
     mask_check(em, f"{k}")
     for hb in range(2):
         softmax_and_check(em, k, hb, SC)
-    pv_phase(em)
+    pv_phase(em, prefetched=True)
     end_of_step(em)
 
 
