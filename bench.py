@@ -57,11 +57,11 @@ DECODE_KERNEL = {
 PREFILL_KERNEL = "rpa_prefill_pipe_kernel"
 
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", PREFILL_KERNEL): 327.2e6 + 77.2e6,
+    ("c2", PREFILL_KERNEL): 326.5e6 + 77.2e6,
     ("c2", "rpa_decode_balanced_kernel"): 501.0e6 + 2.7e6,
     ("c3", "rpa_decode_splitkv_kernel"): 2148.6e6 + 1.9e6,
     ("c5", "rpa_mla_balanced_wide_kernel"): 820.3e6 + 44.8e6,
-    ("c5p", "rpa_mla_decode_wide_kernel (one row per query token)"): 633.5e6 + 268.5e6,
+    ("c5p", "rpa_mla_decode_wide_kernel (one row per query token)"): 633.0e6 + 268.4e6,
 }
 
 
