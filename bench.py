@@ -308,9 +308,10 @@ def reference_suite(pkg, wl, dev, reps=50):
     return rows
 
 
-def cpu_baseline(wl, budget_s=15.0):
+def cpu_baseline(wl, budget_s=10.0, prefill_budget_s=8.0):
     """CPU oracle on a bounded sample of the default workload: its first decode rows
-    (same seeded lengths and layout, values drawn on the host)."""
+    (same seeded lengths and layout, values drawn on the host), and -- reported under `prefill` -- one
+    256-token chunk on a 512-token prefix with the same heads."""
     import torch
 
     from oracle.ref_rpa import ref_ragged_paged_attention_fused
@@ -335,9 +336,26 @@ def cpu_baseline(wl, budget_s=15.0):
             break
     dt = (time.perf_counter() - t0) / reps
     nbytes = wl.decode_bytes(b)
+    # the prefill side of the same workload
+    pb = wl.make_batch("c2_prefill_sample", [256], [768], num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=64,
+                       seed=1003)
+    ptable = pb.padded_page_table()
+    g = lambda: ref_ragged_paged_attention_fused(pb.q, pb.kv_cache, pb.kv_lens, ptable, pb.cu_q_lens, [1],
+                                                 sm_scale=pb.sm_scale)
+    g()
+    preps, t1 = 0, time.perf_counter()
+    while True:
+        g()
+        preps += 1
+        if time.perf_counter() - t1 > prefill_budget_s or preps >= 200:
+            break
+    pdt = (time.perf_counter() - t1) / preps
     return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"CPU oracle (torch f32) on decode rows 0..{rows - 1} of c2_llama3_8b_mixed "
-                      f"(kv_lens {kv_d[:rows].tolist()}), {reps} reps, {dt * 1e3:.1f} ms each"}
+                      f"(kv_lens {kv_d[:rows].tolist()}), {reps} reps, {dt * 1e3:.1f} ms each",
+            "prefill": {"value": wl.prefill_flops(pb) / pdt / 1e12, "unit": "TFLOP/s",
+                        "sample": f"the same oracle on one 256-token chunk on a 512-token prefix (32 / 8 heads of 128), "
+                                  f"{preps} reps, {pdt * 1e3:.1f} ms each"}}
 
 
 def main():
