@@ -88,7 +88,7 @@ typedef struct RpaParams {
   const int32_t* cu_kv_lens;  /* i32[S+1] cumulative page-aligned kv lens; NULL => padded 2-D table */
   const float* k_scale;       /* f32[Hkv] dequantisation scale of K, or NULL (= 1) */
   const float* v_scale;       /* f32[Hkv] or NULL */
-  void* workspace;            /* split-KV partials; >= rpa_workspace_bytes() */
+  void* workspace;            /* partial rows of cut K/V ranges; >= rpa_workspace_bytes() */
   size_t workspace_bytes;
   /* ---- static shape ---- */
   int32_t num_tokens;         /* T */
@@ -225,7 +225,12 @@ int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t*
                       int64_t num_page_indices, const int32_t* cu_q_lens,
                       const int32_t* cu_kv_lens, const int32_t* distribution);
 
-/* Bytes of split-KV workspace rpa_decode / rpa_attention need for `p`. */
+/*
+ * Bytes of workspace for `p`: what the decode rows' split-KV plan needs (rpa_decode fails without
+ * it), or, if larger, the room that lets a prefill launch which would leave most of the GPU idle
+ * (one long prompt on a few heads, a verify step on a long context) cut its K/V ranges into pieces
+ * and merge them; rpa_prefill uses that room when it is there and runs whole ranges when it is not.
+ */
 size_t rpa_workspace_bytes(const RpaParams* p);
 size_t rpa_mla_workspace_bytes(const RpaMlaParams* p);
 
@@ -261,8 +266,10 @@ int rpa_attention(const RpaParams* p, void* stream);
  * tight serving loops, harnesses that forbid it).  No counterpart in the reference, where XLA owns
  * every buffer.  Same arguments and results as rpa_attention, except that p->workspace and
  * p->workspace_bytes are ignored: the split-KV workspace is an array the library holds itself on
- * every GPU, rpa_noalloc_max_workspace_bytes() (40 MiB) long.  A batch whose rpa_workspace_bytes()
- * exceeds it is refused with RPA_EINVAL_WORKSPACE.  The call allocates and frees nothing.  All
+ * every GPU, rpa_noalloc_max_workspace_bytes() (40 MiB) long.  A batch whose decode rows need more
+ * than that is refused with RPA_EINVAL_WORKSPACE; a prefill launch that would cut its K/V ranges
+ * does so only if its partial rows fit the array (otherwise it runs whole ranges: the same rows to
+ * the tolerance of the path, not bit for bit).  The call allocates and frees nothing.  All
  * calls on one GPU share the array: calls that overlap on one GPU (two streams, a graph replay next
  * to eager work) race on it; order them on one stream.
  */

@@ -470,7 +470,10 @@ BalancedLayout balanced_layout(const RpaParams* p) {
 std::atomic<unsigned long long> g_decode_generation{1};
 }  // namespace
 
-size_t rpa_workspace_bytes(const RpaParams* p_in) {
+static size_t prefill_optional_workspace(const RpaParams* p);
+
+// What the decode partition cannot run without.
+static size_t required_workspace_bytes(const RpaParams* p_in) {
   if (!p_in) return 0;
   const RpaParams pv = planning_view(p_in);
   const RpaParams* p = &pv;
@@ -481,6 +484,11 @@ size_t rpa_workspace_bytes(const RpaParams* p_in) {
     return balanced_layout(p).total;
   if (sp.splits <= 1) return 0;
   return (size_t)p->decode_end * sp.splits * p->num_q_heads * (p->head_dim + 2) * sizeof(float);
+}
+
+size_t rpa_workspace_bytes(const RpaParams* p) {
+  if (!p) return 0;
+  return std::max(required_workspace_bytes(p), prefill_optional_workspace(p));
 }
 
 int rpa_gather_pages(const RpaParams* p, int32_t seq, void* k_out, void* v_out, int32_t max_tokens,
@@ -545,7 +553,7 @@ int rpa_decode(const RpaParams* p_in, void* stream) {
     a.forced_blocks_per_wave = (int32_t)std::max<int64_t>(1, ((bound + 31) / 32 + p->num_splits - 1) / p->num_splits);
   }
   if (a.balanced) {
-    const size_t need = rpa_workspace_bytes(p);
+    const size_t need = required_workspace_bytes(p);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
     const BalancedLayout lay = balanced_layout(p);
@@ -564,7 +572,7 @@ int rpa_decode(const RpaParams* p_in, void* stream) {
       a.generation = (g_decode_generation.fetch_add(1, std::memory_order_relaxed) % ((1ull << 48) - 1)) + 1;
     }
   } else if (sp.splits > 1) {
-    const size_t need = rpa_workspace_bytes(p);
+    const size_t need = required_workspace_bytes(p);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(RPA_EINVAL_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, p->workspace_bytes);
     a.ws_o = static_cast<float*>(p->workspace);
@@ -573,17 +581,11 @@ int rpa_decode(const RpaParams* p_in, void* stream) {
   return check_hip(rpa::launch_decode(a, static_cast<hipStream_t>(stream)), "rpa_decode");
 }
 
-int rpa_prefill(const RpaParams* p, void* stream) {
-  int rc = rpa_validate(p);
-  if (rc != RPA_OK) return rc;
+// The prefill kernels' view of a call; false when the call has no chunk for them.
+static bool prefill_args(const RpaParams* p, rpa::PrefillArgs& a) {
   const bool dyn = p->distribution != nullptr;
-  if (!dyn && p->num_seqs <= p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) return RPA_OK;
-  if (dyn && p->num_seqs <= 0) return RPA_OK;
-  // 256-wide heads take the flash kernel (two 128-dim halves per row, one workgroup per CU; e4m3
-  // caches staged through registers); RPA_PREFILL_ROWS256=1 sends them through the row kernel
-  if (p->head_dim == 256 && env_int("RPA_PREFILL_ROWS256", 0) != 0)
-    return rows256(p, (p->mask_mode == RPA_MASK_CUSTOM) ? 0 : p->decode_end, p->num_seqs, stream);
-  rpa::PrefillArgs a;
+  if (!dyn && p->num_seqs <= p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) return false;
+  if (dyn && p->num_seqs <= 0) return false;
   a.head_dim = p->head_dim;
   a.q = static_cast<const uint16_t*>(p->q);
   a.out = static_cast<uint16_t*>(p->out);
@@ -601,6 +603,40 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   a.max_q_len = p->max_q_len > 0 ? p->max_q_len : p->num_tokens;
   a.max_kv_len = p->max_kv_len > 0 ? p->max_kv_len : 0;
   a.fp8 = p->kv_dtype == RPA_KV_FP8_E4M3;
+  a.kv_splits = 1;
+  a.num_tokens = p->num_tokens;
+  a.ws_o = nullptr;
+  a.ws_ml = nullptr;
+  return true;
+}
+
+// Workspace that lets a prefill launch which would leave most of the GPU idle cut its K/V ranges into
+// pieces; never required: without it the launch runs whole ranges.
+static size_t prefill_optional_workspace(const RpaParams* p) {
+  rpa::PrefillArgs a;
+  if (p->head_dim != 128 || !prefill_args(p, a)) return 0;
+  return rpa::prefill_split_workspace_bytes(a, rpa::prefill_kv_splits(a));
+}
+
+int rpa_prefill(const RpaParams* p, void* stream) {
+  int rc = rpa_validate(p);
+  if (rc != RPA_OK) return rc;
+  rpa::PrefillArgs a;
+  if (!prefill_args(p, a)) return RPA_OK;
+  // 256-wide heads take the flash kernel (two 128-dim halves per row, one workgroup per CU; e4m3
+  // caches staged through registers); RPA_PREFILL_ROWS256=1 sends them through the row kernel
+  if (p->head_dim == 256 && env_int("RPA_PREFILL_ROWS256", 0) != 0)
+    return rows256(p, (p->mask_mode == RPA_MASK_CUSTOM) ? 0 : p->decode_end, p->num_seqs, stream);
+  if (p->head_dim == 128) {
+    // the decode partition is done with the workspace by the time these kernels run (same stream)
+    const int splits = rpa::prefill_kv_splits(a);
+    const size_t need = rpa::prefill_split_workspace_bytes(a, splits);
+    if (splits > 1 && p->workspace && p->workspace_bytes >= need && (reinterpret_cast<uintptr_t>(p->workspace) & 15) == 0) {
+      a.kv_splits = splits;
+      a.ws_o = static_cast<float*>(p->workspace);
+      a.ws_ml = a.ws_o + (size_t)p->num_tokens * p->num_q_heads * splits * 128;
+    }
+  }
   return check_hip(rpa::launch_prefill(a, static_cast<hipStream_t>(stream)), "rpa_prefill");
 }
 
@@ -615,7 +651,7 @@ size_t rpa_noalloc_max_workspace_bytes(void) { return kNoAllocScratchBytes; }
 int rpa_attention_noalloc(const RpaParams* p, void* stream) {
   int rc = rpa_validate(p);
   if (rc != RPA_OK) return rc;
-  const size_t need = rpa_workspace_bytes(p);
+  const size_t need = required_workspace_bytes(p);  // (a prefill launch cuts its K/V ranges only if the array has the room)
   if (need > kNoAllocScratchBytes)
     return fail(RPA_EINVAL_WORKSPACE,
                 "this batch needs a split-KV workspace of %zu bytes, the built-in one holds %zu: call rpa_attention "
@@ -624,7 +660,7 @@ int rpa_attention_noalloc(const RpaParams* p, void* stream) {
   RpaParams q = *p;
   q.workspace = nullptr;
   q.workspace_bytes = 0;
-  if (need > 0) {
+  if (need > 0 || prefill_optional_workspace(p) > 0) {
     void* ptr = nullptr;
     if ((rc = noalloc_scratch(&ptr)) != RPA_OK) return rc;
     q.workspace = ptr;  // the device address, never the array's name

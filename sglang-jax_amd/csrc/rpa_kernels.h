@@ -92,6 +92,13 @@ struct PrefillArgs {
   // device i32[3] or nullptr: when given, seq_end is only a bound and the sequences to process are
   // [dist[0], min(seq_end, dist[2])) (custom-mask calls: [0, ...))
   const int32_t* dist;
+  // K/V range of every workgroup cut into kv_splits pieces (pipelined kernel, launches that would leave most
+  // of the GPU idle; 0 or 1 = whole ranges): partial rows f32 [token][Hq][piece][128] in ws_o, their
+  // (reference, sum) pairs in ws_ml, merged by a second launch over num_tokens x Hq rows
+  int32_t kv_splits;
+  int32_t num_tokens;  // bound on the query tokens of the call (rows of q)
+  float* ws_o;
+  float* ws_ml;
 };
 
 struct GatherArgs {
@@ -163,6 +170,10 @@ struct MlaWriteArgs {
 
 hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream);
 hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream);
+// How many pieces launch_prefill would cut the K/V ranges into if it had the workspace (1 = no cut), and the
+// bytes of workspace that takes.
+int prefill_kv_splits(const PrefillArgs& a);
+size_t prefill_split_workspace_bytes(const PrefillArgs& a, int splits);
 hipError_t launch_gather(const GatherArgs& a, hipStream_t stream);
 // head_dim 256: every query token of sequences [seq_begin, seq_end) as a row of its own; at most
 // max_token_rows tokens (a host bound) are covered

@@ -509,6 +509,22 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
 
 }  // namespace
 
+namespace {
+bool takes_pipe_kernel(const PrefillArgs& a) {
+  static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
+  static const bool use_pipe = [] { const char* v = getenv("RPA_PREFILL_PIPE"); return !(v && *v == '0'); }();
+  return use_pipe && !force_staged && prefill_pipe_applies(a);
+}
+}  // namespace
+
+int prefill_kv_splits(const PrefillArgs& a) {
+  return takes_pipe_kernel(a) ? prefill_pipe_kv_splits(a, a.seq_end - a.seq_begin) : 1;
+}
+
+size_t prefill_split_workspace_bytes(const PrefillArgs& a, int splits) {
+  return splits > 1 ? (size_t)a.num_tokens * a.Hq * splits * (128 + 2) * sizeof(float) : 0;
+}
+
 hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const int nseq = a.seq_end - a.seq_begin;
   if (nseq <= 0 || a.max_q_len <= 0) return hipSuccess;
@@ -527,8 +543,7 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const bool cap = a.sm.soft_cap != 0.f || a.sm.round_logits != 0;
   static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
   const bool staged = a.fp8 || force_staged;
-  static const bool use_pipe = [] { const char* v = getenv("RPA_PREFILL_PIPE"); return !(v && *v == '0'); }();
-  if (use_pipe && !force_staged && prefill_pipe_applies(a)) return launch_prefill_pipe(a, nseq, level_order, stream);
+  if (takes_pipe_kernel(a)) return launch_prefill_pipe(a, nseq, level_order, stream);
   const dim3 g((unsigned)grid), blk(256);
   const bool ext = a.sm.xai_len > 0.f || a.sm.mask_mode != 0 || a.sm.q_scale > 0.f;
 #define RPA_STAGED(F, U, C, E) \

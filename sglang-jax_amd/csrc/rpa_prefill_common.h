@@ -375,5 +375,6 @@ __device__ __forceinline__ void async_copy_tile(char* lds_k, char* lds_v, const 
 // rpa_prefill_pipe.hip: the software-pipelined kernel for the plain causal bf16 case
 bool prefill_pipe_applies(const PrefillArgs& a);
 hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order, hipStream_t stream);
+int prefill_pipe_kv_splits(const PrefillArgs& a, int nseq);
 
 }  // namespace rpa

@@ -173,6 +173,50 @@ def test_workspace_size_is_deterministic(pkg):
     assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
 
 
+def test_workspace_for_prefill_launches_that_leave_the_gpu_idle(pkg, monkeypatch):
+    """rpa_workspace_bytes also reports the room that lets an under-filled prefill launch cut its K/V
+    ranges into pieces: (tokens x heads x pieces) partial rows of 128 + 2 floats.  Nothing for launches
+    that fill the GPU, for calls whose composition is on the device, without a bound on the lengths,
+    or with RPA_PREFILL_SPLITS=0; the forced count is honoured."""
+    lib = pkg._lib.load()
+    monkeypatch.delenv("RPA_PREFILL_SPLITS", raising=False)
+
+    def params(tokens, hq, hkv, max_kv):
+        p = base_params(pkg)
+        p.num_seqs, p.decode_end, p.num_tokens = 1, 0, tokens
+        p.num_q_heads, p.num_kv_heads, p.page_size, p.total_pages = hq, hkv, 64, 8192
+        p.max_q_len, p.max_kv_len = tokens, max_kv
+        return p
+
+    row = (128 + 2) * 4
+    p = params(512, 8, 2, 16384)  # one 512-token chunk on a long prefix, 32 workgroups
+    need = lib.rpa_workspace_bytes(ctypes.byref(p))
+    assert need > 0 and need % (512 * 8 * row) == 0
+    pieces = need // (512 * 8 * row)
+    assert 2 <= pieces <= 64
+    p.max_kv_len = 0  # no bound on the lengths: no cut
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+    p = params(512, 8, 2, 16384)
+    p.distribution = 0x1000  # composition on the device: no cut, only what the decode plan of such a call asks for
+    dyn = lib.rpa_workspace_bytes(ctypes.byref(p))
+    monkeypatch.setenv("RPA_PREFILL_SPLITS", "7")
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == dyn
+    monkeypatch.delenv("RPA_PREFILL_SPLITS")
+    p = params(2048, 32, 8, 8192)  # 512 workgroups: the GPU is full
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+    p = params(1000, 8, 4, 1000)  # a short range: the merge would cost what the cut saves
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+    p = params(16, 8, 2, 32768)  # a verify step on a long context: the short-chunk tile, many pieces
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) // (16 * 8 * row) >= 16
+    p.kv_dtype = 1  # e4m3 caches take the other kernels
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+    p = params(512, 8, 2, 16384)
+    monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+    monkeypatch.setenv("RPA_PREFILL_SPLITS", "5")
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 512 * 8 * 5 * row
+
+
 def test_python_wrapper_raises_like_the_reference(pkg):
     import torch
 

@@ -1106,3 +1106,48 @@ def test_device_side_distribution_matches_host_integers(pkg, wl, gpu, kv_dtype):
                                             sm_scale=c.sm_scale, k_scale=gc.k_scale, v_scale=gc.v_scale)
         torch.cuda.synchronize()
         assert_parity(out[: sum(sub_q)].cpu().float(), oracle_out(c).float(), **tol)
+
+
+# ---- prefill launches that would leave most of the GPU idle: K/V ranges cut into pieces + merge ----
+KV_PIECE_CASES = [
+    # name, q_lens, kv_lens, Hq, Hkv, P, window, sink, whether the automatic plan cuts the launch
+    ("one_prompt_4_heads", [1024], [1024], 4, 1, 128, None, False, True),
+    ("one_prompt_8_heads", [1000], [1000], 8, 4, 64, None, True, False),  # the merge would cost what the cut saves
+    ("chunk_on_long_prefix", [300], [5300], 8, 2, 64, None, False, True),
+    ("two_chunks_and_decode_rows", [1, 1, 200, 77], [900, 40, 3000, 77], 4, 1, 64, None, False, True),
+    ("window", [1, 260], [700, 4100], 8, 2, 64, 1000, False, True),
+    ("verify_step_long_context", [16], [9000], 8, 2, 256, None, False, True),
+    ("verify_steps_window_sink", [1, 5, 33], [100, 6000, 2100], 4, 1, 64, 1500, True, True),
+    ("full_gpu", [600, 900], [2000, 900], 32, 8, 64, None, False, False),
+]
+
+
+@pytest.mark.parametrize("name,q_lens,kv_lens,Hq,Hkv,P,window,sink,cuts", KV_PIECE_CASES, ids=[c[0] for c in KV_PIECE_CASES])
+def test_prefill_launches_that_leave_the_gpu_idle_cut_their_kv_ranges(pkg, wl, gpu, monkeypatch, name, q_lens, kv_lens,
+                                                                      Hq, Hkv, P, window, sink, cuts):
+    for needles in (False, True):
+        say(f"prefill pieces {name} needles={needles}")
+        b = wl.make_batch(name, q_lens, kv_lens, num_q_heads=Hq, num_kv_heads=Hkv, head_dim=128, page_size=P, seed=77,
+                          sliding_window=window)
+        if needles:
+            wl.plant_needles(b, seed=5)
+        kw = {}
+        if sink:
+            kw["attention_sink"] = torch.linspace(-1.0, 2.0, Hq)
+        want = oracle_out(b, **kw)
+        monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
+        whole = gpu_out(pkg, b, gpu, **kw)
+        monkeypatch.delenv("RPA_PREFILL_SPLITS")
+        auto = gpu_out(pkg, b, gpu, **kw)
+        assert_parity(whole.float(), want.float(), **BF16_TOL)
+        assert_parity(auto.float(), want.float(), **BF16_TOL)
+        assert torch.equal(auto, whole) != cuts, "the automatic plan: cut expected" if cuts else "no cut expected"
+        assert float(row_rel_error(auto.float(), whole.float()).max()) < 1e-2
+        for forced in ("2", "7", "32"):  # more pieces than some row blocks have tiles: empty pieces
+            monkeypatch.setenv("RPA_PREFILL_SPLITS", forced)
+            cut = gpu_out(pkg, b, gpu, **kw)
+            monkeypatch.delenv("RPA_PREFILL_SPLITS")
+            assert torch.isfinite(cut.float()).all()
+            assert_parity(cut.float(), want.float(), **BF16_TOL)
+            assert float(row_rel_error(cut.float(), whole.float()).max()) < 1e-2
+        assert torch.equal(auto, gpu_out(pkg, b, gpu, **kw))
