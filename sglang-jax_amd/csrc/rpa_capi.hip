@@ -614,7 +614,8 @@ static bool prefill_args(const RpaParams* p, rpa::PrefillArgs& a) {
 // pieces; never required: without it the launch runs whole ranges.
 static size_t prefill_optional_workspace(const RpaParams* p) {
   rpa::PrefillArgs a;
-  if (p->head_dim != 128 || !prefill_args(p, a)) return 0;
+  if (!prefill_args(p, a)) return 0;
+  if (p->head_dim == 256 && env_int("RPA_PREFILL_ROWS256", 0) != 0) return 0;  // the row kernel has its own plan
   return rpa::prefill_split_workspace_bytes(a, rpa::prefill_kv_splits(a));
 }
 
@@ -627,14 +628,14 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   // caches staged through registers); RPA_PREFILL_ROWS256=1 sends them through the row kernel
   if (p->head_dim == 256 && env_int("RPA_PREFILL_ROWS256", 0) != 0)
     return rows256(p, (p->mask_mode == RPA_MASK_CUSTOM) ? 0 : p->decode_end, p->num_seqs, stream);
-  if (p->head_dim == 128) {
+  {
     // the decode partition is done with the workspace by the time these kernels run (same stream)
     const int splits = rpa::prefill_kv_splits(a);
     const size_t need = rpa::prefill_split_workspace_bytes(a, splits);
     if (splits > 1 && p->workspace && p->workspace_bytes >= need && (reinterpret_cast<uintptr_t>(p->workspace) & 15) == 0) {
       a.kv_splits = splits;
       a.ws_o = static_cast<float*>(p->workspace);
-      a.ws_ml = a.ws_o + (size_t)p->num_tokens * p->num_q_heads * splits * 128;
+      a.ws_ml = a.ws_o + (size_t)p->num_tokens * p->num_q_heads * splits * p->head_dim;
     }
   }
   return check_hip(rpa::launch_prefill(a, static_cast<hipStream_t>(stream)), "rpa_prefill");

@@ -168,9 +168,14 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
   MaskCtx mc;
   mc.mode = 0;
   if constexpr (EXT) mc = make_mask_ctx(a, w, wr.row);
-  const int t_hi = causal ? min(w.kv_len, w.prefix + wg_r_hi + 1) : w.kv_len;  // exclusive
+  int t_hi = causal ? min(w.kv_len, w.prefix + wg_r_hi + 1) : w.kv_len;  // exclusive
   int t_lo = 0;
   if (W_ > 0) t_lo = max(0, w.prefix + w.q_start - W_ + 1) & ~(kBN - 1);
+  int split = 0;
+  if (a.kv_splits > 1 && !kv_piece(a, t_lo, t_hi, split)) {  // under-filled launch, nothing left for this piece
+    write_empty_partial_rows<T::kDimTiles>(a, w, wr, h, split);
+    return;
+  }
 
   // ---- operand addresses inside a tile (bytes) ----
   // K operand of (m-tile mt, k-step ks): row 32mt + c, chunk (2ks + h) ^ (c & 15)
@@ -273,7 +278,8 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
     if (tb + kBN >= t_hi) break;
     tile_step(lds_k1, lds_v1, lds_k0, lds_v0, tb + kBN);
   }
-  write_rows<T::kDimTiles>(a, w, wr, O, l, h, m * sm.sc2);
+  if (a.kv_splits > 1) write_partial_rows<T::kDimTiles>(a, w, wr, O, l, h, m * sm.sc2, split);
+  else write_rows<T::kDimTiles>(a, w, wr, O, l, h, m * sm.sc2);
 }
 
 // ==================================================================== staged path (fp8 cache)
@@ -452,9 +458,14 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
   MaskCtx mc;
   mc.mode = 0;
   if constexpr (EXT) mc = make_mask_ctx(a, w, wr.row);
-  const int t_hi = causal ? min(w.kv_len, w.prefix + wg_r_hi + 1) : w.kv_len;  // exclusive
+  int t_hi = causal ? min(w.kv_len, w.prefix + wg_r_hi + 1) : w.kv_len;  // exclusive
   int t_lo = 0;
   if (W_ > 0) t_lo = max(0, w.prefix + w.q_start - W_ + 1) & ~(kBN - 1);
+  int split = 0;
+  if (a.kv_splits > 1 && !kv_piece(a, t_lo, t_hi, split)) {  // under-filled launch, nothing left for this piece
+    write_empty_partial_rows<4>(a, w, wr, h, split);
+    return;
+  }
 
   // ---- pipeline: page ids run two tiles ahead, rows one tile ahead (in registers), LDS one
   // tile ahead of the MFMAs.  Loads past the last tile re-read the last tile.
@@ -504,7 +515,8 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
     }
     __syncthreads();
   }
-  write_rows(a, w, wr, O, l, h, m * sm.sc2);
+  if (a.kv_splits > 1) write_partial_rows<4>(a, w, wr, O, l, h, m * sm.sc2, split);
+  else write_rows(a, w, wr, O, l, h, m * sm.sc2);
 }
 
 }  // namespace
@@ -518,11 +530,15 @@ bool takes_pipe_kernel(const PrefillArgs& a) {
 }  // namespace
 
 int prefill_kv_splits(const PrefillArgs& a) {
-  return takes_pipe_kernel(a) ? prefill_pipe_kv_splits(a, a.seq_end - a.seq_begin) : 1;
+  const int nseq = a.seq_end - a.seq_begin;
+  if (takes_pipe_kernel(a)) return prefill_pipe_kv_splits(a, nseq);
+  // the compiled kernels: 128 positions of one head per workgroup, a tile takes about 1.1 us alone on its CU
+  // (2.2 us for 256-wide heads)
+  return kv_pieces(a, nseq, kBM, 1, a.head_dim == 256 ? 2.2 : 1.1);
 }
 
 size_t prefill_split_workspace_bytes(const PrefillArgs& a, int splits) {
-  return splits > 1 ? (size_t)a.num_tokens * a.Hq * splits * (128 + 2) * sizeof(float) : 0;
+  return splits > 1 ? (size_t)a.num_tokens * a.Hq * splits * (a.head_dim + 2) * sizeof(float) : 0;
 }
 
 hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
@@ -544,7 +560,9 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
   const bool staged = a.fp8 || force_staged;
   if (takes_pipe_kernel(a)) return launch_prefill_pipe(a, nseq, level_order, stream);
-  const dim3 g((unsigned)grid), blk(256);
+  const bool cut = a.kv_splits > 1;  // pieces of the K/V ranges on the second grid dimension, then the merge
+  if (cut && (!a.ws_o || !a.ws_ml || a.kv_splits > 64)) return hipErrorInvalidValue;
+  const dim3 g((unsigned)grid, cut ? (unsigned)a.kv_splits : 1u), blk(256);
   const bool ext = a.sm.xai_len > 0.f || a.sm.mask_mode != 0 || a.sm.q_scale > 0.f;
 #define RPA_STAGED(F, U, C, E) \
   hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
@@ -586,7 +604,7 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
 #undef RPA_ASYNC
 #undef RPA_ASYNC256
 #undef RPA_ASYNC256_FP8
-  return hipGetLastError();
+  return cut ? launch_prefill_combine(a, stream) : hipGetLastError();
 }
 
 }  // namespace rpa

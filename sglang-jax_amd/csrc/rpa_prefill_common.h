@@ -274,6 +274,152 @@ __device__ __forceinline__ void write_rows(const PrefillArgs& a, const Work& w, 
     }
 }
 
+// -------------------------------------------------- K/V ranges cut into pieces (under-filled launches)
+// A launch with far fewer workgroups than CUs (one long prompt on a few heads, a chunk on a long prefix, a
+// verify step on a long context) cuts every workgroup's run of K/V tiles into a.kv_splits pieces; blockIdx.y
+// picks the piece, which leaves its rows as they stand -- unnormalised accumulators, (reference, sum) of the
+// probabilities in log2 units -- in workspace slot ((token, head), piece), and rpa_prefill_combine_kernel
+// finishes them.
+constexpr float kNoReference = -1.0e30f;  // reference of a row that met no visible token: weighs nothing in the merge
+
+// The piece of [t_lo, t_hi) that this workgroup runs; false when nothing is left for it.
+__device__ __forceinline__ bool kv_piece(const PrefillArgs& a, int& t_lo, int& t_hi, int& split) {
+  split = blockIdx.y;
+  const int nT = (t_hi - t_lo + kBN - 1) / kBN;
+  // (the division runs on the vector pipe: say that its result is the same in every lane)
+  const int per = __builtin_amdgcn_readfirstlane((nT + a.kv_splits - 1) / a.kv_splits);
+  const int lo = split * per, hi = min(nT, lo + per);
+  if (lo >= hi) return false;
+  t_hi = min(t_hi, t_lo + hi * kBN);
+  t_lo += lo * kBN;
+  return true;
+}
+
+// lane (c, h) holds query row c, dims 32d + 8*(v/4) + 4h + v%4 in O[d][v]
+template <int ND>
+__device__ __forceinline__ void write_partial_rows(const PrefillArgs& a, const Work& w, const WaveRows& wr,
+                                                   const f32x16_t (&O)[ND], float l, int h, float m2, int split) {
+  typedef float f32x4_t __attribute__((ext_vector_type(4)));
+  l += __shfl_xor(l, 32);
+  if (!wr.active || wr.row >= w.q_len) return;
+  const int64_t slot = ((int64_t)(w.qg0 + wr.row) * a.Hq + w.head) * a.kv_splits + split;
+  float* op = a.ws_o + slot * (ND * 32) + 4 * h;
+#pragma unroll
+  for (int d = 0; d < ND; ++d)
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq)
+      *reinterpret_cast<f32x4_t*>(op + d * 32 + vq * 8) =
+          f32x4_t{O[d][4 * vq + 0], O[d][4 * vq + 1], O[d][4 * vq + 2], O[d][4 * vq + 3]};
+  if (h == 0) {
+    a.ws_ml[slot * 2] = fmaxf(m2, kNoReference);
+    a.ws_ml[slot * 2 + 1] = l;
+  }
+}
+
+template <int ND>
+__device__ __forceinline__ void write_empty_partial_rows(const PrefillArgs& a, const Work& w, const WaveRows& wr, int h,
+                                                         int split) {
+  f32x16_t zero[ND];
+#pragma unroll
+  for (int d = 0; d < ND; ++d) zero[d] = kZero16;
+  write_partial_rows<ND>(a, w, wr, zero, 0.f, h, kNoReference, split);
+}
+
+// Merge the kv_splits partial rows of one (query token, query head): out = sum_j O_j 2^(m_j - m*) /
+// sum_j l_j 2^(m_j - m*).  grid = (tokens, Hq); one wave, HD / 64 dims per lane; lane j fetches (m_j, l_j).
+template <int HD>
+__global__ __launch_bounds__(64) void rpa_prefill_combine_kernel(const PrefillArgs a) {
+  constexpr int kDpl = HD / 64;
+  typedef float fvec_t __attribute__((ext_vector_type(kDpl)));
+  const int tok0 = scalar_load_i32(a.pt.cu_q_lens + a.seq_begin);
+  const int tok1 = scalar_load_i32(a.pt.cu_q_lens + a.seq_end);
+  const int token = tok0 + (int)blockIdx.x;
+  if (token >= tok1) return;
+  const int head = blockIdx.y, lane = threadIdx.x, n = a.kv_splits;
+  const int64_t base = ((int64_t)token * a.Hq + head) * n;
+  float mj = -INFINITY, lj = 0.f;
+  if (lane < n) {
+    mj = a.ws_ml[(base + lane) * 2];
+    lj = a.ws_ml[(base + lane) * 2 + 1];
+  }
+  float mstar = mj;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mstar = fmaxf(mstar, __shfl_xor(mstar, off));
+  const float wj = (lane < n) ? fast_exp2(mj - mstar) : 0.f;
+  float den = lj * wj;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) den += __shfl_xor(den, off);
+  float acc[kDpl];
+#pragma unroll
+  for (int e = 0; e < kDpl; ++e) acc[e] = 0.f;
+  for (int j0 = 0; j0 < n; j0 += 8) {  // eight partial rows requested at a time
+    fvec_t o[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      o[u] = *reinterpret_cast<const fvec_t*>(a.ws_o + (base + min(j0 + u, n - 1)) * HD + kDpl * lane);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float wu = (j0 + u < n) ? __shfl(wj, j0 + u) : 0.f;  // the repeated last row does not count
+#pragma unroll
+      for (int e = 0; e < kDpl; ++e) acc[e] += o[u][e] * wu;
+    }
+  }
+  const float vs = a.v_scale ? a.v_scale[head / a.G] : 1.0f;
+  const float inv = a.sm.sink ? vs * sink_inverse(mstar, den, sink_logit(a.sm.sink, a.sm.round_logits, head)) : vs / den;
+  uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)token * a.Hq + head) * HD + kDpl * lane);
+#pragma unroll
+  for (int e = 0; e < kDpl; e += 2) op[e / 2] = pack_bf16x2(acc[e] * inv, acc[e + 1] * inv);
+}
+
+inline hipError_t launch_prefill_combine(const PrefillArgs& a, hipStream_t stream) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const int64_t tokens = std::max<int64_t>(1, (int64_t)a.num_tokens - a.seq_begin);  // decode rows hold one token each
+  const dim3 g((unsigned)tokens, (unsigned)a.Hq);
+  if (a.head_dim == 256) hipLaunchKernelGGL(rpa_prefill_combine_kernel<256>, g, dim3(64), 0, stream, a);
+  else hipLaunchKernelGGL(rpa_prefill_combine_kernel<128>, g, dim3(64), 0, stream, a);
+  return hipGetLastError();
+}
+
+// How many pieces (1 = whole ranges): the count that minimises a small model of the launch, fitted to
+// measurements of the pipelined kernel.  The critical path is the longest range, chain / n tiles per piece; a
+// tile takes ~tile_us while every workgroup has a CU to itself (up to ~192 workgroups: the dispatcher does
+// not spread them perfectly), 2.6 x that once two share every CU (512), in proportion in between, and the
+// launch runs in rounds of 512 workgroups beyond; the merge costs a launch (~1.5 us) plus the partial rows'
+// way to memory and back (~0.29 ns per (token, head, piece) of 128 dims).  A cut must save at least 2 us,
+// leaves no piece under four tiles and makes at most 64 pieces.  bm / heads: query positions and query heads
+// per workgroup.  RPA_PREFILL_SPLITS: 0 / 1 never, n forces n (read per call).
+inline int kv_pieces(const PrefillArgs& a, int nseq, int bm, int heads, double tile_us) {
+  if (a.dist || nseq <= 0 || a.max_q_len <= 0 || a.max_kv_len <= 0 || a.num_tokens <= 0) return 1;
+  const char* env = getenv("RPA_PREFILL_SPLITS");
+  const int forced = env ? atoi(env) : -1;
+  if (forced == 0 || forced == 1) return 1;
+  if (forced > 1) return std::min(forced, 64);
+  const int64_t tokens = std::max<int64_t>(1, (int64_t)a.num_tokens - a.seq_begin);
+  const int64_t blocks = std::min<int64_t>((int64_t)nseq * ((a.max_q_len + bm - 1) / bm), tokens / bm + nseq);
+  const int64_t wgs = blocks * a.Hkv * (a.G / heads);
+  int64_t longest = a.max_kv_len;  // tokens of the longest range
+  if (a.sm.window > 0) longest = std::min<int64_t>(longest, (int64_t)a.sm.window + bm + kBN);
+  const int64_t chain = (longest + kBN - 1) / kBN;
+  const int64_t cap = std::min<int64_t>(64, chain / 4);
+  const double per_piece = 0.29e-3 * (double)tokens * a.Hq * (a.head_dim / 128);  // us per piece for the partial rows
+  auto launch_us = [&](int n) {
+    const double w = (double)wgs * n;
+    const double rate = w <= 192 ? 1.0 : w <= 512 ? 1.0 + (w - 192) * (1.6 / 320) : 2.6 * (w / 512);
+    return tile_us * rate * chain / n + (n > 1 ? 1.5 + per_piece * n : 0.0);
+  };
+  int best = 1;
+  double best_us = launch_us(1) - 2.0;
+  for (int n = 2; n <= cap; ++n) {
+    const double us = launch_us(n);
+    if (us < best_us) {
+      best_us = us;
+      best = n;
+    }
+  }
+  return best;
+}
+
 // ==================================================================== async path (bf16 cache)
 // Geometry of a tile for head dim HD (128 or 256): rows stay row-major and unpadded in LDS.
 template <int HD>

@@ -265,29 +265,6 @@ __device__ __forceinline__ void pipe_loop(RowBlock (&b)[2], const Shared& sh, in
 #undef C
 }
 
-// A piece's rows as they stand: the unnormalised accumulators, and (reference, sum) of the probabilities, in
-// workspace slot ((token, head), piece).  A row that met no visible token in the piece gets a reference far
-// below any real one, so it weighs nothing in the merge.  Lane (c, h) holds row c, dims 32d + 8(v/4) + 4h + v%4.
-__device__ __forceinline__ void write_partial_rows(const PrefillArgs& a, const Work& w, const WaveRows& wr,
-                                                   const f32x16_t (&O)[4], float l, int h, float m2, bool seen,
-                                                   int split) {
-  typedef float f32x4_t __attribute__((ext_vector_type(4)));
-  l += __shfl_xor(l, 32);
-  if (!wr.active || wr.row >= w.q_len) return;
-  const int64_t slot = ((int64_t)(w.qg0 + wr.row) * a.Hq + w.head) * a.kv_splits + split;
-  float* op = a.ws_o + slot * 128 + 4 * h;
-#pragma unroll
-  for (int d = 0; d < 4; ++d)
-#pragma unroll
-    for (int vq = 0; vq < 4; ++vq)
-      *reinterpret_cast<f32x4_t*>(op + d * 32 + vq * 8) =
-          f32x4_t{O[d][4 * vq + 0], O[d][4 * vq + 1], O[d][4 * vq + 2], O[d][4 * vq + 3]};
-  if (h == 0) {
-    a.ws_ml[slot * 2] = seen ? m2 : kSeenFloor;
-    a.ws_ml[slot * 2 + 1] = l;
-  }
-}
-
 // HEADS4: the short-chunk tile.  A workgroup owns 32 query positions of FOUR query heads of a kv head, one
 // head per wave, instead of 128 positions of one head: chunks of a few dozen tokens (a verify step, a short
 // prompt, the tail of a long one) then fill their tiles, and the four waves still share every K/V tile.
@@ -332,14 +309,9 @@ __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kerne
   int t_hi = min(w.kv_len, w.prefix + wg_r_hi + 1);  // exclusive
   int t_lo = 0;
   if (W_ > 0) t_lo = max(0, w.prefix + w.q_start - W_ + 1) & ~(kBN - 1);
-  int nT = (t_hi - t_lo + kBN - 1) / kBN;  // K/V tiles of the workgroup
   int split = 0;
   if constexpr (SPLIT) {
-    split = blockIdx.y;
-    const int per = (nT + a.kv_splits - 1) / a.kv_splits;
-    const int lo = split * per, hi = min(nT, lo + per);
-    if (lo >= hi) {  // nothing left for this piece: rows that weigh nothing in the merge
-      const f32x16_t zero[4] = {kZero16, kZero16, kZero16, kZero16};
+    if (!kv_piece(a, t_lo, t_hi, split)) {  // nothing left for this piece
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         WaveRows wr;
@@ -348,14 +320,15 @@ __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kerne
         wr.active = wr.r_lo < w.q_len;
         wr.row = wr.r_lo + c;
         wr.qpos = w.prefix + wr.row;
-        write_partial_rows(a, w, wr, zero, 0.f, h, 0.f, false, split);
+        write_empty_partial_rows<4>(a, w, wr, h, split);
       }
       return;
     }
-    t_hi = min(t_hi, t_lo + hi * kBN);
-    t_lo += lo * kBN;
-    nT = hi - lo;
+    // the piece's bounds went through the vector pipe (a division); the assembly loop takes scalars
+    t_lo = __builtin_amdgcn_readfirstlane(t_lo);
+    t_hi = __builtin_amdgcn_readfirstlane(t_hi);
   }
+  const int nT = (t_hi - t_lo + kBN - 1) / kBN;  // K/V tiles of the workgroup (of its piece)
 
   RowBlock b[NQ];
 #pragma unroll
@@ -500,51 +473,9 @@ __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kerne
     wr.active = wr.r_lo < w.q_len;
     wr.row = wr.r_lo + c;
     wr.qpos = b[q].qpos;
-    if constexpr (SPLIT) write_partial_rows(a, w, wr, b[q].O, b[q].l, h, b[q].m, b[q].seen != 0.f, split);
+    if constexpr (SPLIT) write_partial_rows<4>(a, w, wr, b[q].O, b[q].l, h, b[q].seen != 0.f ? b[q].m : kNoReference, split);
     else write_rows<4>(a, w, wr, b[q].O, b[q].l, h, b[q].m);
   }
-}
-
-// Merge the kv_splits partial rows of one (query token, query head): out = sum_j O_j 2^(m_j - m*) /
-// sum_j l_j 2^(m_j - m*).  grid = (tokens, Hq); one wave, 2 dims per lane; lane j fetches (m_j, l_j).
-__global__ __launch_bounds__(64) void rpa_prefill_combine_kernel(const PrefillArgs a) {
-  const int tok0 = scalar_load_i32(a.pt.cu_q_lens + a.seq_begin);
-  const int tok1 = scalar_load_i32(a.pt.cu_q_lens + a.seq_end);
-  const int token = tok0 + (int)blockIdx.x;
-  if (token >= tok1) return;
-  const int head = blockIdx.y, lane = threadIdx.x, n = a.kv_splits;
-  const int64_t base = ((int64_t)token * a.Hq + head) * n;
-  float mj = -INFINITY, lj = 0.f;
-  if (lane < n) {
-    mj = a.ws_ml[(base + lane) * 2];
-    lj = a.ws_ml[(base + lane) * 2 + 1];
-  }
-  typedef float f32x2_t __attribute__((ext_vector_type(2)));
-  float mstar = mj;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) mstar = fmaxf(mstar, __shfl_xor(mstar, off));
-  const float wj = (lane < n) ? fast_exp2(mj - mstar) : 0.f;
-  float den = lj * wj;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) den += __shfl_xor(den, off);
-  float acc0 = 0.f, acc1 = 0.f;
-  for (int j0 = 0; j0 < n; j0 += 8) {  // eight partial rows requested at a time
-    f32x2_t o[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u)
-      o[u] = *reinterpret_cast<const f32x2_t*>(a.ws_o + (base + min(j0 + u, n - 1)) * 128 + 2 * lane);
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const float wu = (j0 + u < n) ? __shfl(wj, j0 + u) : 0.f;  // the repeated last row does not count
-      acc0 += o[u][0] * wu;
-      acc1 += o[u][1] * wu;
-    }
-  }
-  const int hk = head / a.G;
-  const float vs = a.v_scale ? a.v_scale[hk] : 1.0f;
-  const float inv = a.sm.sink ? vs * sink_inverse(mstar, den, sink_logit(a.sm.sink, a.sm.round_logits, head)) : vs / den;
-  uint32_t* op = reinterpret_cast<uint32_t*>(a.out + ((int64_t)token * a.Hq + head) * 128 + 2 * lane);
-  *op = pack_bf16x2(acc0 * inv, acc1 * inv);
 }
 
 }  // namespace
@@ -569,45 +500,11 @@ bool short_chunk_tile(const PrefillArgs& a, int nq) {
 }
 }  // namespace
 
-// Pieces per K/V range for a launch of the pipelined kernel (1 = whole ranges): the count that minimises a
-// small model of the launch, fitted to measurements.  The critical path is the longest range, chain / n tiles
-// per piece; a tile takes ~0.8 us while every workgroup has a CU to itself (up to ~192 workgroups: the
-// dispatcher does not spread them perfectly), ~2.06 us once two share every CU (512), in proportion in between,
-// and the launch runs in rounds of 512 workgroups beyond that; the merge costs a launch (~1.5 us) plus the partial
-// rows' way to memory and back (~0.29 ns per (token, head, piece)).  A cut must save at least 2 us, leaves no
-// piece under four tiles and makes at most 64 pieces.  RPA_PREFILL_SPLITS: 0 / 1 never, n forces n (read per
-// call).
+// Pieces per K/V range for a launch of the pipelined kernel (1 = whole ranges).
 int prefill_pipe_kv_splits(const PrefillArgs& a, int nseq) {
-  if (a.dist || nseq <= 0 || a.max_q_len <= 0 || a.max_kv_len <= 0 || a.num_tokens <= 0 || forced_nq() == 2) return 1;
-  const char* env = getenv("RPA_PREFILL_SPLITS");
-  const int forced = env ? atoi(env) : -1;
-  if (forced == 0 || forced == 1) return 1;
-  if (forced > 1) return std::min(forced, 64);
+  if (forced_nq() == 2) return 1;
   const bool heads4 = short_chunk_tile(a, 1);
-  const int bm = heads4 ? 32 : 128;
-  const int64_t tokens = std::max<int64_t>(1, (int64_t)a.num_tokens - a.seq_begin);  // decode rows hold one token each
-  const int64_t blocks = std::min<int64_t>((int64_t)nseq * ((a.max_q_len + bm - 1) / bm), tokens / bm + nseq);
-  const int64_t wgs = blocks * a.Hkv * (heads4 ? a.G / 4 : a.G);
-  int64_t longest = a.max_kv_len;  // tokens of the longest range
-  if (a.sm.window > 0) longest = std::min<int64_t>(longest, (int64_t)a.sm.window + bm + kBN);
-  const int64_t chain = (longest + kBN - 1) / kBN;
-  const int64_t cap = std::min<int64_t>(64, chain / 4);
-  const double per_piece = 0.29e-3 * (double)tokens * a.Hq;  // us per piece for the partial rows
-  auto launch_us = [&](int n) {
-    const double w = (double)wgs * n;
-    const double tile_us = w <= 192 ? 0.8 : w <= 512 ? 0.8 + (w - 192) * (1.26 / 320) : 2.06 * (w / 512);
-    return tile_us * chain / n + (n > 1 ? 1.5 + per_piece * n : 0.0);
-  };
-  int best = 1;
-  double best_us = launch_us(1) - 2.0;
-  for (int n = 2; n <= cap; ++n) {
-    const double us = launch_us(n);
-    if (us < best_us) {
-      best_us = us;
-      best = n;
-    }
-  }
-  return best;
+  return kv_pieces(a, nseq, heads4 ? 32 : 128, heads4 ? 4 : 1, 0.8);
 }
 
 hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order, hipStream_t stream) {
@@ -641,11 +538,7 @@ hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order,
       else RPA_LAUNCH_SPLIT(false, false);
     }
 #undef RPA_LAUNCH_SPLIT
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    const int64_t tokens = std::max<int64_t>(1, (int64_t)a.num_tokens - a.seq_begin);
-    hipLaunchKernelGGL(rpa_prefill_combine_kernel, dim3((unsigned)tokens, (unsigned)a.Hq), dim3(64), 0, stream, a);
-    return hipGetLastError();
+    return launch_prefill_combine(a, stream);
   }
 #define RPA_LAUNCH(W, N) \
   hipLaunchKernelGGL((rpa_prefill_pipe_kernel<W, N>), g, blk, 0, stream, a, tiles, nseq, by_level, limit)

@@ -208,8 +208,12 @@ def test_workspace_for_prefill_launches_that_leave_the_gpu_idle(pkg, monkeypatch
     assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
     p = params(16, 8, 2, 32768)  # a verify step on a long context: the short-chunk tile, many pieces
     assert lib.rpa_workspace_bytes(ctypes.byref(p)) // (16 * 8 * row) >= 16
-    p.kv_dtype = 1  # e4m3 caches take the other kernels
-    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+    p.kv_dtype = 1  # e4m3 caches take the compiled kernels (128 positions per workgroup), which cut too
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) // (16 * 8 * row) >= 16
+    p = params(200, 4, 1, 3000)  # 256-wide heads: rows of 256 + 2 floats
+    p.head_dim = 256
+    need = lib.rpa_workspace_bytes(ctypes.byref(p))
+    assert need > 0 and need % (200 * 4 * (256 + 2) * 4) == 0
     p = params(512, 8, 2, 16384)
     monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
     assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0

@@ -1151,3 +1151,47 @@ def test_prefill_launches_that_leave_the_gpu_idle_cut_their_kv_ranges(pkg, wl, g
             assert_parity(cut.float(), want.float(), **BF16_TOL)
             assert float(row_rel_error(cut.float(), whole.float()).max()) < 1e-2
         assert torch.equal(auto, gpu_out(pkg, b, gpu, **kw))
+
+
+@pytest.mark.parametrize("kind", ["fp8", "soft_cap", "d256", "d256_fp8", "custom_mask", "no_mask"])
+def test_kv_range_pieces_in_the_compiled_prefill_kernels(pkg, wl, gpu, monkeypatch, kind):
+    """The same cut for the launches the pipelined kernel does not take: e4m3 caches, soft cap, 256-wide heads,
+    custom masks and unmasked attention.  Automatic and forced piece counts against the oracle and against whole
+    ranges; one row block of the batch is shorter than the others, so forced counts leave empty pieces."""
+    fp8 = kind in ("fp8", "d256_fp8")
+    D = 256 if kind.startswith("d256") else 128
+    q_lens, kv_lens = ([1, 40, 260], [500, 40, 4300]) if kind not in ("custom_mask", "no_mask") else ([6, 12], [3000, 700])
+    b = wl.make_batch("pieces_" + kind, q_lens, kv_lens, num_q_heads=8, num_kv_heads=2, head_dim=D, page_size=64, seed=91,
+                      kv_dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16, soft_cap=30.0 if kind == "soft_cap" else None)
+    if kind not in ("custom_mask", "no_mask"):
+        wl.plant_needles(b, seed=3)
+    okw, gkw = {}, {}
+    if kind == "custom_mask":
+        rng = np.random.default_rng(5)
+        masks = []
+        for ql, kv in zip(q_lens, kv_lens):
+            m = (rng.random((ql, kv)) < 0.5).astype(np.int32)
+            m[:, kv - 1] = 1  # every row keeps a token; row 0 keeps nothing else: one piece holds all it sees
+            m[0, : kv - 1] = 0
+            masks.append(m)
+        cm = flat_mask(masks)
+        okw, gkw = dict(causal=False, custom_mask=cm), dict(causal=0, custom_mask=cm.to(gpu))
+    elif kind == "no_mask":
+        okw, gkw = dict(causal=False), dict(causal=0)
+    tol = FP8_TOL if fp8 else BF16_TOL
+    say(f"compiled-kernel pieces {kind}")
+    want = oracle_out(b, **okw)
+    monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
+    whole = gpu_out(pkg, b, gpu, **gkw)
+    monkeypatch.delenv("RPA_PREFILL_SPLITS")
+    auto = gpu_out(pkg, b, gpu, **gkw)
+    assert_parity(whole.float(), want.float(), **tol)
+    assert_parity(auto.float(), want.float(), **tol)
+    assert not torch.equal(auto, whole), "the automatic plan was expected to cut this launch"
+    assert float(row_rel_error(auto.float(), whole.float()).max()) < (3e-2 if fp8 else 1e-2)
+    for forced in ("3", "64"):
+        monkeypatch.setenv("RPA_PREFILL_SPLITS", forced)
+        cut = gpu_out(pkg, b, gpu, **gkw)
+        monkeypatch.delenv("RPA_PREFILL_SPLITS")
+        assert torch.isfinite(cut.float()).all()
+        assert_parity(cut.float(), want.float(), **tol)
