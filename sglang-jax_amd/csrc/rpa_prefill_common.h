@@ -198,6 +198,16 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[ND]
                                              const Softmax<CAP>& sm, bool need_mask, int tb, int h, int qpos,
                                              int window, u32x4_t (&pB)[2][2], const MaskCtx& mc) {
   if constexpr (CAP) {
+    if (sm.cap != 0.f && !sm.round_mode) {
+      // soft cap alone (the usual case), constants folded: five instructions per score.
+      // cap tanh(s scale / cap) temp log2e = k2 - 2 k2 / (2^(s k1) + 1)
+      const float k1 = sm.scale * sm.inv_cap * (2.0f * kLog2e), k2 = sm.cap * sm.temp * kLog2e;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          S[mt][v] = __builtin_fmaf(__builtin_amdgcn_rcpf(fast_exp2(S[mt][v] * k1) + 1.0f), -2.0f * k2, k2);
+    } else
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
