@@ -59,12 +59,39 @@ __device__ __forceinline__ int page_slot_of(const SeqView& s, int tok) {
   return s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
 }
 
+// A window of consecutive page ids of a row, copied asynchronously into a wave's own LDS slice
+// (global_load_lds_dword, no register in between): 64 ids per copy instruction, entry i = page slot
+// first_slot + i, clamped to the row's last page.  The copy is issued as inline assembly and its completion
+// is the caller's business: loads complete in order, so it has landed once any load issued after it has been
+// waited for.
+constexpr int kWinSmallPages = 256;  // entries of a window when pages are smaller than a block
+
+template <int ENTRIES>
+__device__ __forceinline__ void copy_page_window(const int32_t* row_pages, int last_slot, int32_t* lds, int first_slot,
+                                                 int lane) {
+  typedef const __attribute__((address_space(3))) char* lds_ptr_t;
+  const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds));
+#pragma unroll
+  for (int k = 0; k < ENTRIES / 64; ++k) {
+    const int32_t* src = row_pages + min(first_slot + 64 * k + lane, last_slot);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(base + 256u * k), "v"(src) : "memory", "m0");
+  }
+}
+
+__device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // Issue the global loads of one 32-token block.  Token indices are clamped to
 // the last valid token so that nothing past kv_len (and nothing past the
 // sequence's page list) is ever dereferenced; clamped rows are masked later.
-template <bool FP8, bool UNIFORM_PAGE>
+// WINDOW, win / win_first: for pages that do not hold whole blocks, the LDS window the caller keeps of this
+// row's page ids (entry 0 = page slot win_first); without it every lane fetches the ids of its tokens from
+// memory, a dependent round trip in front of the block's loads.
+// (A compile-time choice: with both lookups in the code the compiler's wait-count bookkeeping sees a possible
+// page-id load behind every block and drains the whole queue in front of each block's use.)
+template <bool FP8, bool UNIFORM_PAGE, bool WINDOW = false>
 __device__ __forceinline__ void load_block(KvRegs<FP8>& r, const SeqView& s, const KvAddr& kv,
-                                           const char* kh, const char* vh, int tb, int page, int c, int g) {
+                                           const char* kh, const char* vh, int tb, int page, int c, int g,
+                                           const int32_t* win = nullptr, int win_first = 0) {
   constexpr int kLaneK = FP8 ? 32 : 16;  // byte offset step of lane group g inside a K row
   constexpr int kLaneV = FP8 ? 8 : 16;   // byte offset step of lane c inside a V row
   if constexpr (UNIFORM_PAGE) {
@@ -97,7 +124,7 @@ __device__ __forceinline__ void load_block(KvRegs<FP8>& r, const SeqView& s, con
     for (int b = 0; b < 2; ++b) {
       const int tok = min(tb + b * 16 + c, s.last_tok);
       const int slot = page_slot_of(s, tok);
-      const int page = s.pages[slot];
+      const int page = WINDOW ? win[slot - win_first] : s.pages[slot];
       const char* kp = kh + (int64_t)page * kv.page_stride +
                        (int64_t)((tok - slot * s.page_size) * kv.tok_stride + g * kLaneK);
       if constexpr (FP8) {
@@ -112,7 +139,7 @@ __device__ __forceinline__ void load_block(KvRegs<FP8>& r, const SeqView& s, con
     for (int i = 0; i < 8; ++i) {
       const int tok = min(tb + tok_slot(g, i), s.last_tok);
       const int slot = page_slot_of(s, tok);
-      const int page = s.pages[slot];
+      const int page = WINDOW ? win[slot - win_first] : s.pages[slot];
       const char* vp = vh + (int64_t)page * kv.page_stride +
                        (int64_t)((tok - slot * s.page_size) * kv.tok_stride + c * kLaneV);
       if constexpr (FP8) r.v[i] = ld8(vp);
@@ -422,15 +449,38 @@ __device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int
     if constexpr (UNIFORM_PAGE) return scalar_load_i32(sv.pages + __builtin_amdgcn_readfirstlane(page_slot_of(sv, tb)));
     else return 0;
   };
+  // Pages smaller than a block: the ids of the next kWinSmallPages pages wait in the wave's LDS window and
+  // every lane looks its token rows up there; fetched from memory per block they were a dependent round
+  // trip in front of every block's loads, behind which the loads already in flight had to drain (page size
+  // 16: 2.6 TB/s where pages of 64 stream 5.8).  The window moves on every kWinSmallPages pages, at the
+  // price of one drained queue.
+  __shared__ int32_t seg_windows[UNIFORM_PAGE ? 1 : 4][UNIFORM_PAGE ? 1 : kWinSmallPages];  // [wave][entry]
+  const int32_t* win = nullptr;
+  int win_first = 0;
+  auto cover = [&](int tb) __attribute__((always_inline)) {  // make the window hold the pages of block tb
+    if constexpr (!UNIFORM_PAGE) {
+      const int last_slot = page_slot_of(sv, sv.last_tok);
+      if (!win || page_slot_of(sv, min(tb + kBlk - 1, sv.last_tok)) - win_first >= kWinSmallPages) {
+        int32_t* mine = seg_windows[__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)];
+        win_first = __builtin_amdgcn_readfirstlane(page_slot_of(sv, tb));
+        copy_page_window<kWinSmallPages>(sv.pages, last_slot, mine, win_first, lane);
+        wait_all_loads();
+        win = mine;
+      }
+    }
+  };
   KvRegs<FP8> ra, rb;
   int pg_next = page_of(block_tok(1));
-  load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, t_begin, page_of(t_begin), c, g);
+  cover(t_begin);
+  load_block<FP8, UNIFORM_PAGE, !UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, t_begin, page_of(t_begin), c, g, win, win_first);
   for (int blk = 0; blk < nblk; blk += 2) {
-    load_block<FP8, UNIFORM_PAGE>(rb, sv, a.kv, kh, vh, block_tok(blk + 1), pg_next, c, g);
+    cover(block_tok(blk + 1));
+    load_block<FP8, UNIFORM_PAGE, !UNIFORM_PAGE>(rb, sv, a.kv, kh, vh, block_tok(blk + 1), pg_next, c, g, win, win_first);
     pg_next = page_of(block_tok(blk + 2));
     compute_block<MT, FP8, CAP>(ra, qB, acc, m, l, so, t_begin + blk * kBlk, g);
     if (blk + 1 >= nblk) break;
-    load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, block_tok(blk + 2), pg_next, c, g);
+    cover(block_tok(blk + 2));
+    load_block<FP8, UNIFORM_PAGE, !UNIFORM_PAGE>(ra, sv, a.kv, kh, vh, block_tok(blk + 2), pg_next, c, g, win, win_first);
     pg_next = page_of(block_tok(blk + 3));
     compute_block<MT, FP8, CAP>(rb, qB, acc, m, l, so, t_begin + (blk + 1) * kBlk, g);
   }
@@ -567,29 +617,23 @@ __device__ __forceinline__ RowMeta row_resolve(const DecodeArgs& a, int seq, con
   return m;
 }
 
-// A window of 64 consecutive page ids of a row, copied asynchronously into the wave's own LDS
-// slice (global_load_lds_dword, no register in between) and looked up with a uniform LDS read:
+// The balanced plan's window of a row's page ids (copy_page_window), looked up with a uniform LDS read
+// when pages hold whole blocks and with one LDS read per lane and token row when they are smaller:
 // the steady state of a wave issues no small dependent global loads at all, and because no
 // register ever waits for the copy, the compiler never drains the vector-memory queue for it.
-// The copy is issued as inline assembly and its completion is the caller's business: loads
-// complete in order, so it has landed once any load issued after it has been waited for.
 struct PageWindow {
-  int32_t* lds;  // 64 ids of this wave
+  int32_t* lds;  // ids of this wave: 64 (whole blocks per page, one uniform lookup per block) or kWinSmallPages
   int first;     // slot of entry 0
 };
 
+template <int ENTRIES>
 __device__ __forceinline__ void request_window(const DecodeArgs& a, const RowMeta& row, PageWindow& w,
                                                int first_slot, int page_shift, int lane) {
   w.first = first_slot;
   const int last_tok = max(row.kv_len - 1, 0);
   const int last_slot = page_shift >= 0 ? (last_tok >> page_shift) : (last_tok / a.pt.page_size);
-  const int32_t* src = a.pt.page_indices + row.page0 + min(first_slot + lane, last_slot);
-  typedef const __attribute__((address_space(3))) char* lds_ptr_t;
-  const uint32_t m0v = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)w.lds));
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(m0v), "v"(src) : "memory", "m0");
+  copy_page_window<ENTRIES>(a.pt.page_indices + row.page0, last_slot, w.lds, first_slot, lane);
 }
-
-__device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // One piece of work of a wave: tokens of one (row, kv head, group of 16 query heads).
 struct Piece {
@@ -804,22 +848,25 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
     cur = make_piece(row, unit, blk, min(row.nb - blk, x_end - x));
   }
   int cur_unit = (x - row_first) / row.nb;
-  __shared__ int32_t lds_windows[4][2][64];  // [wave][current / next piece][entry]
+  constexpr int kWin = UNIFORM_PAGE ? 64 : kWinSmallPages;
+  __shared__ int32_t lds_windows[4][2][kWin];  // [wave][current / next piece][entry]
   PageWindow win = {lds_windows[wave][0], 0};
   PageWindow nwin = {lds_windows[wave][1], 0};
-  if constexpr (UNIFORM_PAGE) request_window(a, cur.row, win, slot_of_tok(cur.t_first), page_shift, lane);
+  // what load_block takes besides the uniform page id: the window itself when pages are smaller than a block
+  auto lanes_win = [&](const PageWindow& pwn) -> const int32_t* { return UNIFORM_PAGE ? nullptr : pwn.lds; };
+  request_window<kWin>(a, cur.row, win, slot_of_tok(cur.t_first), page_shift, lane);
   u32x4_t qB[MT][4];
   load_queries<MT, FP8>(a, cur.row.tq, min(cur.hk, a.Hkv - 1), cur.rg * 16 * MT, c, g, qB);
-  if constexpr (UNIFORM_PAGE) wait_all_loads();  // the window (and the queries behind it)
+  wait_all_loads();  // the window (and the queries behind it)
 
   KvRegs<FP8> ra, rb;
   bool in_b = false;  // which register set holds the block about to be consumed
   {
     const SeqView sv = view_of(cur.row);
     const int hk = min(cur.hk, a.Hkv - 1);
-    load_block<FP8, UNIFORM_PAGE>(ra, sv, a.kv, a.kv.k_base + (int64_t)hk * a.kv.head_stride,
+    load_block<FP8, UNIFORM_PAGE, !UNIFORM_PAGE>(ra, sv, a.kv, a.kv.k_base + (int64_t)hk * a.kv.head_stride,
                                   a.kv.v_base + (int64_t)hk * a.kv.head_stride, cur.t_first,
-                                  page_in(win, cur.t_first), c, g);
+                                  page_in(win, cur.t_first), c, g, lanes_win(win), win.first);
   }
 
   PendingMerge pm_first = {}, pm_last = {};
@@ -882,7 +929,7 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
         }
         const int x_next = x + cur.nblk;
         nxt = make_piece(nrow, nunit, 0, min(nrow.nb, x_end - x_next));
-        if constexpr (UNIFORM_PAGE) request_window(a, nrow, nwin, slot_of_tok(nxt.t_first), page_shift, lane);
+        request_window<kWin>(a, nrow, nwin, slot_of_tok(nxt.t_first), page_shift, lane);
         nsv = view_of(nrow);
         const int nhk = min(nxt.hk, a.Hkv - 1);
         nkh = a.kv.k_base + (int64_t)nhk * a.kv.head_stride;
@@ -892,22 +939,22 @@ __global__ __launch_bounds__(256, 2) void rpa_decode_balanced_kernel(const Decod
       const bool last = (i + 1 == cur.nblk);
       // the block to request now: the next one of this piece, the first one of the next piece,
       // or (nothing left) this block again, so that every path has the same loads in flight
-      if constexpr (UNIFORM_PAGE) {
-        if (!last && slot_of_tok(tb + kBlk) - win.first >= 64) {  // every 64 pages
-          request_window(a, cur.row, win, slot_of_tok(tb + kBlk), page_shift, lane);
-          wait_all_loads();
-        }
+      // the window moves on when the next block's last page lies beyond it
+      if (!last && slot_of_tok(tb + kBlk + (UNIFORM_PAGE ? 0 : kBlk - 1)) - win.first >= kWin) {
+        request_window<kWin>(a, cur.row, win, slot_of_tok(tb + kBlk), page_shift, lane);
+        wait_all_loads();
       }
       // real branches, not selects: looking a page up in the next piece's window must not make
       // every block wait for that window
       if (last && has_next) {
         // The next piece's window was requested at block resolve_at, in front of that block's
         // prefetch.  Two blocks later a wait for younger loads has passed; earlier it has not.
-        if (UNIFORM_PAGE && i <= resolve_at + 1) wait_all_loads();
-        load_block<FP8, UNIFORM_PAGE>(fill, nsv, a.kv, nkh, nvh, nxt.t_first, page_in(nwin, nxt.t_first), c, g);
+        if (i <= resolve_at + 1) wait_all_loads();
+        load_block<FP8, UNIFORM_PAGE, !UNIFORM_PAGE>(fill, nsv, a.kv, nkh, nvh, nxt.t_first, page_in(nwin, nxt.t_first), c, g,
+                                      lanes_win(nwin), nwin.first);
       } else {
         const int ptb = last ? tb : tb + kBlk;
-        load_block<FP8, UNIFORM_PAGE>(fill, sv, a.kv, kh, vh, ptb, page_in(win, ptb), c, g);
+        load_block<FP8, UNIFORM_PAGE, !UNIFORM_PAGE>(fill, sv, a.kv, kh, vh, ptb, page_in(win, ptb), c, g, lanes_win(win), win.first);
       }
       compute_block<MT, FP8, CAP>(use, qB, acc, m, l, so, tb, g);
     };

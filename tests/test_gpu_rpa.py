@@ -103,6 +103,31 @@ def test_decode_irregular_lengths_small_pages(pkg, wl, gpu):
     check(pkg, wl, gpu, "decode_irregular", [1] * len(lens), lens, P=8, seed=33)
 
 
+@pytest.mark.parametrize("P", [1, 4, 16, 24])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_decode_long_rows_on_pages_smaller_than_a_block(pkg, wl, gpu, P, fp8):
+    """Pages that do not hold whole 32-token blocks: every lane looks the pages of its token rows up in the wave's
+    LDS window of 256 page ids, which moves on several times along these rows (P = 1: every 8 blocks).  One long row
+    cut over the GPU (fixed plan, forced counts included), a ragged batch (balanced plan: pieces end inside windows
+    and the next piece's window is another row's), planted keys, a sliding window."""
+    tol = FP8_TOL if fp8 else BF16_TOL
+    kw = dict(num_q_heads=16, num_kv_heads=4, head_dim=128, page_size=P, kv_dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16)
+    say(f"small pages P={P} fp8={fp8}: one long row")
+    b = wl.make_batch("small_pages_long", [1], [3000 if P == 1 else 9001], seed=340 + P, **kw)
+    wl.plant_needles(b, seed=2)
+    want = oracle_out(b)
+    for ns in (0, 1, 5):
+        got = gpu_out(pkg, b, gpu, **({"num_splits": ns} if ns else {}))
+        assert_parity(got.float(), want.float(), **tol)
+    say(f"small pages P={P} fp8={fp8}: ragged batch")
+    rng = np.random.default_rng(P)
+    lens = [int(x) for x in rng.integers(1, 700 if P == 1 else 2500, size=40)] + [1, 31, 32, 33, 255, 257]
+    for window in (None, 300):
+        b = wl.make_batch("small_pages_ragged", [1] * len(lens), lens, seed=350 + P, sliding_window=window, **kw)
+        wl.plant_needles(b, seed=3)
+        assert_parity(gpu_out(pkg, b, gpu).float(), oracle_out(b).float(), **tol)
+
+
 def test_decode_single_long_sequence(pkg, wl, gpu):
     check(pkg, wl, gpu, "decode_16384", [1], [16384], Hq=32, Hkv=8, P=64, seed=34)
 
