@@ -153,4 +153,25 @@ __device__ __forceinline__ u32x2_t fp8x4_to_bf16x4(uint32_t w) {
   return u32x2_t{fp8x2_to_bf16x2(w, false), fp8x2_to_bf16x2(w, true)};
 }
 
+// A window of consecutive page ids of a row, copied asynchronously into a wave's own LDS slice
+// (global_load_lds_dword, no register in between): 64 ids per copy instruction, entry i = page slot
+// first_slot + i, clamped to the row's last page.  The copy is issued as inline assembly and its completion
+// is the caller's business: loads complete in order, so it has landed once any load issued after it has been
+// waited for.
+constexpr int kWinSmallPages = 256;  // entries of a window when pages are smaller than a block
+
+template <int ENTRIES>
+__device__ __forceinline__ void copy_page_window(const int32_t* row_pages, int last_slot, int32_t* lds, int first_slot,
+                                                 int lane) {
+  typedef const __attribute__((address_space(3))) char* lds_ptr_t;
+  const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds));
+#pragma unroll
+  for (int k = 0; k < ENTRIES / 64; ++k) {
+    const int32_t* src = row_pages + min(first_slot + 64 * k + lane, last_slot);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(base + 256u * k), "v"(src) : "memory", "m0");
+  }
+}
+
+__device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 }  // namespace rpa

@@ -59,27 +59,6 @@ __device__ __forceinline__ int page_slot_of(const SeqView& s, int tok) {
   return s.page_shift >= 0 ? (tok >> s.page_shift) : (tok / s.page_size);
 }
 
-// A window of consecutive page ids of a row, copied asynchronously into a wave's own LDS slice
-// (global_load_lds_dword, no register in between): 64 ids per copy instruction, entry i = page slot
-// first_slot + i, clamped to the row's last page.  The copy is issued as inline assembly and its completion
-// is the caller's business: loads complete in order, so it has landed once any load issued after it has been
-// waited for.
-constexpr int kWinSmallPages = 256;  // entries of a window when pages are smaller than a block
-
-template <int ENTRIES>
-__device__ __forceinline__ void copy_page_window(const int32_t* row_pages, int last_slot, int32_t* lds, int first_slot,
-                                                 int lane) {
-  typedef const __attribute__((address_space(3))) char* lds_ptr_t;
-  const uint32_t base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds));
-#pragma unroll
-  for (int k = 0; k < ENTRIES / 64; ++k) {
-    const int32_t* src = row_pages + min(first_slot + 64 * k + lane, last_slot);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(base + 256u * k), "v"(src) : "memory", "m0");
-  }
-}
-
-__device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
 // Issue the global loads of one 32-token block.  Token indices are clamped to
 // the last valid token so that nothing past kv_len (and nothing past the
 // sequence's page list) is ever dereferenced; clamped rows are masked later.
@@ -1256,12 +1235,23 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
     if (tb_begin >= t_hi) return;  // the merge pass knows how many pieces a row has
     if (split < nsplit - 1) tb_end = min(t_hi, tb_begin + a.chunk);
   }
+  // pages smaller than a block: the lanes look their token rows' pages up in an LDS window of the row's page
+  // ids (see decode_segment) instead of fetching them from memory in front of every block
+  __shared__ int32_t win_ids[UNIFORM_PAGE ? 1 : kWinSmallPages];
+  const int32_t* win = nullptr;
+  int win_first = 0;
   for (int tb = tb_begin; tb < tb_end; tb += kBlk) {
     int page = 0;
     if constexpr (UNIFORM_PAGE) page = __builtin_amdgcn_readfirstlane(sv.pages[page_slot_of(sv, tb)]);
+    else if (!win || page_slot_of(sv, min(tb + kBlk - 1, sv.last_tok)) - win_first >= kWinSmallPages) {
+      win_first = __builtin_amdgcn_readfirstlane(page_slot_of(sv, tb));
+      copy_page_window<kWinSmallPages>(sv.pages, page_slot_of(sv, sv.last_tok), win_ids, win_first, lane);
+      wait_all_loads();
+      win = win_ids;
+    }
     KvRegs<FP8> r0, r1;
-    load_block<FP8, UNIFORM_PAGE>(r0, sv, a.kv, kh, vh, tb, page, c, g);
-    load_block<FP8, UNIFORM_PAGE>(r1, sv, a.kv, kh + kHalfB, vh + kHalfB, tb, page, c, g);
+    load_block<FP8, UNIFORM_PAGE, !UNIFORM_PAGE>(r0, sv, a.kv, kh, vh, tb, page, c, g, win, win_first);
+    load_block<FP8, UNIFORM_PAGE, !UNIFORM_PAGE>(r1, sv, a.kv, kh + kHalfB, vh + kHalfB, tb, page, c, g, win, win_first);
     f32x4_t s[2];
     {
       u32x4_t kA[2][4];

@@ -78,6 +78,11 @@ __device__ __forceinline__ int tok_of(int g, int i) {
 
 struct Src {
   const int32_t* pages;
+  // pages smaller than a tile: the wave's LDS window of this row's page ids (entry 0 = page slot win_first),
+  // which the lanes look their rows' pages up in; fetched from memory per tile they would be a load the next
+  // tile's copies depend on, behind which the copies in flight drain
+  const int32_t* win;
+  int32_t win_first;
   int32_t page_size, page_shift, last_tok;
   int64_t page_stride;  // bytes
   int32_t row_bytes;    // bytes between tokens of a page
@@ -139,7 +144,7 @@ __device__ __forceinline__ void copy_tile(char* slot, const Src& s, const char* 
     chunk_of<CPW>(s, wave, lane, n, row, inner);
     const int tok = min(tb + row, s.last_tok);
     const int ps = page_slot(s, tok);
-    const int pg = UNIFORM ? page : s.pages[ps];
+    const int pg = UNIFORM ? page : s.win[ps - s.win_first];
     const char* src = cache + (int64_t)pg * s.page_stride + (int64_t)(tok - ps * s.page_size) * s.row_bytes + inner;
     async_copy16(src, slot + copy_block<CPW>(wave, n) * 1024);
   }
@@ -178,7 +183,7 @@ __device__ __forceinline__ void copy_tile_f8(char* stage, const Src& s, const ch
     } else {  // last, partial tile (rows clamped to the last valid token) or pages smaller than a tile
       const int tok = min(tb + row, s.last_tok);
       const int ps = page_slot(s, tok);
-      const int pg = UNIFORM ? page : s.pages[ps];
+      const int pg = UNIFORM ? page : s.win[ps - s.win_first];
       async_copy16(cache + (int64_t)pg * s.page_stride + (int64_t)(tok - ps * s.page_size) * s.row_bytes + inner,
                    stage + blk * 1024);
     }
@@ -295,6 +300,20 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   src.row_bytes = a.row_stride * (FP8 ? 1 : 2);
   src.page_stride = (int64_t)src.row_bytes * a.pt.page_size;
   src.rope_byte = a.rope_offset * (FP8 ? 1 : 2);
+  src.win = nullptr;
+  src.win_first = 0;
+  __shared__ int32_t page_windows[UNIFORM ? 1 : 8][UNIFORM ? 1 : kWinSmallPages];  // [wave][entry]
+  auto cover = [&](int tb) __attribute__((always_inline)) {  // make the wave's window hold the pages of tile tb
+    if constexpr (!UNIFORM) {
+      tb = min(tb, src.last_tok & ~(kTok - 1));
+      if (!src.win || page_slot(src, min(tb + kTok - 1, src.last_tok)) - src.win_first >= kWinSmallPages) {
+        src.win_first = __builtin_amdgcn_readfirstlane(page_slot(src, tb));
+        copy_page_window<kWinSmallPages>(src.pages, page_slot(src, src.last_tok), page_windows[wave], src.win_first, lane);
+        wait_all_loads();
+        src.win = page_windows[wave];
+      }
+    }
+  };
   auto page_of = [&](int tb) -> int {
     if constexpr (UNIFORM) {
       tb = min(tb, src.last_tok & ~(kTok - 1));
@@ -339,6 +358,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   // 111 KiB per CU in flight, which is what HBM latency under load asks for) ----
   int pg_next = page_of(t_begin + 3 * kTok);
   auto stage_of = [&](int i) -> char* { return i == 0 ? slot2 : (i == 1 ? slot2 + kF8StageB : slot3); };
+  cover(t_begin);  // (the first three tiles never span a window's 256 pages)
   if constexpr (FP8) {
     copy_tile_f8<UNIFORM>(stage_of(0), src, a.cache, t_begin, wave, lane, page_of(t_begin));
     copy_tile_f8<UNIFORM>(stage_of(1), src, a.cache, t_begin + kTok, wave, lane, page_of(t_begin + kTok));
@@ -379,6 +399,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     const int k_off_t = PIPE ? (c_t * kRowB + g_t * 16) : k_off;
     const int v_off_t = PIPE ? ((4 * g_t + (c_t >> 2)) * kRowB + (c_t & 3) * 8) : v_off;
     // `fill` held tile tb - 32, which every wave finished before the last barrier
+    cover(tb + 3 * kTok);
     if constexpr (FP8) copy_tile_f8<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane_t, pg_next);
     else copy_tile<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane_t, pg_next);
     pg_next = page_of(tb + 4 * kTok);

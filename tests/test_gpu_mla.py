@@ -52,6 +52,29 @@ def test_mla_decode_page_sizes(pkg, wl, gpu, P, Hq):
     assert_parity(got.float(), oracle(b).float(), **TOL)
 
 
+@pytest.mark.parametrize("P", [4, 8, 16])
+@pytest.mark.parametrize("f8", [False, True])
+def test_mla_long_rows_on_pages_smaller_than_a_tile(pkg, wl, gpu, P, f8):
+    """Pages that do not hold whole 32-token tiles: the lanes look their rows' pages up in the wave's LDS window of
+    256 page ids, which moves on several times along these rows.  One long row (cut over the GPU, forced counts
+    included) and a ragged batch on the balanced plan, planted keys."""
+    kw = dict(num_q_heads=128, lkv_dim=512, rope_dim=64, page_size=P, sm_scale=192 ** -0.5,
+              kv_dtype=torch.float8_e4m3fn if f8 else torch.bfloat16)
+    ref = fp8_oracle if f8 else oracle
+    say(f"mla small pages P={P} f8={f8}: one long row")
+    b = wl.make_mla_batch("mla_small_pages", [1], [6001], seed=410 + P, **kw)
+    wl.plant_mla_needles(b, seed=4)
+    want = ref(b)
+    for ns in (0, 1, 5):
+        got = run_gpu(pkg, b, gpu, **({"num_splits": ns} if ns else {}))
+        assert_parity(got.float(), want.float(), **TOL)
+    say(f"mla small pages P={P} f8={f8}: ragged batch")
+    lens = [int(x) for x in np.random.default_rng(P).integers(1, 3000, size=24)] + [1, 31, 32, 33, 2049]
+    b = wl.make_mla_batch("mla_small_pages_ragged", [1] * len(lens), lens, seed=420 + P, **kw)
+    wl.plant_mla_needles(b, seed=5)
+    assert_parity(run_gpu(pkg, b, gpu).float(), ref(b).float(), **TOL)
+
+
 @pytest.mark.parametrize("window,cap", [(128, None), (None, 30.0), (128, 30.0)])
 def test_mla_window_and_soft_cap(pkg, wl, gpu, window, cap):
     kv_lens = [100, 128, 129, 700]

@@ -128,6 +128,19 @@ def test_decode_long_rows_on_pages_smaller_than_a_block(pkg, wl, gpu, P, fp8):
         assert_parity(gpu_out(pkg, b, gpu).float(), oracle_out(b).float(), **tol)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_decode_256_wide_heads_on_pages_smaller_than_a_block(pkg, wl, gpu, fp8):
+    """The row kernel of the 256-wide heads with the same LDS window of page ids: long decode rows (cut into
+    pieces, the window moves along each) and a short chunk on a long prefix (one row per query token)."""
+    tol = FP8_TOL if fp8 else BF16_TOL
+    for P, q_lens, kv_lens in ((16, [1, 1, 1], [9001, 300, 4100]), (4, [1, 7], [2500, 1900])):
+        say(f"256-wide heads small pages P={P} fp8={fp8}")
+        b = wl.make_batch("d256_small_pages", q_lens, kv_lens, num_q_heads=8, num_kv_heads=2, head_dim=256, page_size=P,
+                          seed=360 + P, kv_dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16)
+        wl.plant_needles(b, seed=6)
+        assert_parity(gpu_out(pkg, b, gpu).float(), oracle_out(b).float(), **tol)
+
+
 def test_decode_single_long_sequence(pkg, wl, gpu):
     check(pkg, wl, gpu, "decode_16384", [1], [16384], Hq=32, Hkv=8, P=64, seed=34)
 
