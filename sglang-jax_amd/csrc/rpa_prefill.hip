@@ -107,6 +107,7 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
   using T = Tile<HD>;
   constexpr int kRowB = T::kRowB;
   constexpr int kTileB = T::kTileB;
+  constexpr bool kMaskPre = EXT && HD == 128 && !FP8;
   // Four separate arrays (not one indexed array): the compiler can then prove that the
   // asynchronous copy into one ring slot does not alias the LDS reads of the other slot and
   // does not drain the vector-memory queue in the middle of a tile.
@@ -226,6 +227,12 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
 
   // one tile: consume (lds_k, lds_v), fill (nxt_k, nxt_v) with the tile after it
   auto tile_step = [&](const char* lds_k, const char* lds_v, char* nxt_k, char* nxt_v, int tb) {
+    // a caller's mask: the tile's words are requested before the next tile's copy (128-wide heads on bf16 caches,
+    // where the registers for them exist)
+    MaskTile mtile;
+    if constexpr (kMaskPre) {
+      if (mc.mode == 1) load_mask_tile(mtile, mc, tb, h);
+    }
     if (tb + kBN < t_hi) {
       // the other slot was last read before the barrier that ended the previous tile
       if constexpr (FP8) {
@@ -255,7 +262,7 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
           S[1] = mfma32(lds_ld16(lds_k + koff[ks] + 32 * kRowB), qB[ks], S[1]);
         }
         u32x4_t pB[2][2];
-        softmax_tile<CAP, EXT, T::kDimTiles>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc);
+        softmax_tile<CAP, EXT, T::kDimTiles, kMaskPre>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc, &mtile);
         // independent accumulator chains (dim tiles), issued round-robin
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)

@@ -193,10 +193,40 @@ __device__ __forceinline__ MaskCtx make_mask_ctx(const PrefillArgs& a, const Wor
   return mc;
 }
 
-template <bool CAP, bool EXT, int ND = 4>
+// The mask words of one lane for a whole 64-token tile: group 4 mt + j holds tokens tb + 32 mt + 8 j + 4 h .. + 3,
+// the lane's scores v = 4 j .. 4 j + 3 of half mt.  Requested at the top of a tile's step, in FRONT of the next
+// tile's copy: loads return in order, so the wait for these words then leaves the copy in flight.  (One
+// 4-byte load per score behind the first product, as before, waited for the copy as well on every tile and
+// cost 32 load instructions per lane: a verify step of 16 draft tokens on 4096-token prefixes ran 5.6 x slower
+// with a tree mask than without.)
+typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
+struct MaskTile {
+  i32x4_t g[8];
+};
+
+__device__ __forceinline__ void load_mask_tile(MaskTile& t, const MaskCtx& mc, int tb, int h) {
+  if (tb + kBN <= mc.kv_len) {  // the tile lies inside the row
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        __builtin_memcpy(&t.g[4 * mt + j], mc.row + tb + 32 * mt + 8 * j + 4 * h, 16);  // rows are 4-byte aligned only
+  } else {  // the row's last tile: word by word, clamped (tokens beyond kv_len are hidden whatever they read)
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t.g[4 * mt + j][e] = mc.row[min(tb + 32 * mt + 8 * j + 4 * h + e, mc.kv_len - 1)];
+  }
+}
+
+// PRE: the caller's mask comes from `pre` instead of one load per score.
+template <bool CAP, bool EXT, int ND = 4, bool PRE = false>
 __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[ND], float& m, float& l,
                                              const Softmax<CAP>& sm, bool need_mask, int tb, int h, int qpos,
-                                             int window, u32x4_t (&pB)[2][2], const MaskCtx& mc) {
+                                             int window, u32x4_t (&pB)[2][2], const MaskCtx& mc,
+                                             const MaskTile* pre = nullptr) {
   if constexpr (CAP) {
     if (sm.cap != 0.f && !sm.round_mode) {
       // soft cap alone (the usual case), constants folded: five instructions per score.
@@ -207,18 +237,31 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[ND]
 #pragma unroll
         for (int v = 0; v < 16; ++v)
           S[mt][v] = __builtin_fmaf(__builtin_amdgcn_rcpf(fast_exp2(S[mt][v] * k1) + 1.0f), -2.0f * k2, k2);
-    } else
+    } else {
+      // the general path: soft cap (if any), temperature, then the logit rounded to the softmax dtype.  One loop
+      // per combination, so that no score pays for a choice that is the same for the whole call.
+      const bool capped = sm.cap != 0.f;
+      const float k1 = sm.scale * sm.inv_cap * (2.0f * kLog2e), k2 = (capped ? sm.cap : sm.scale) * sm.temp;
+      auto all_scores = [&](auto logit, auto rounded) __attribute__((always_inline)) {
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+        for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        // the general path: soft cap (if any), temperature, rounding of the logit (if asked)
-        float x = S[mt][v] * sm.scale;
-        if (sm.cap != 0.f) x = soft_cap_f(x, sm.cap, sm.inv_cap);
-        x = x * sm.temp;
-        if (sm.round_mode) x = round_logit(x, sm.round_mode);
-        S[mt][v] = x * kLog2e;
+          for (int v = 0; v < 16; ++v) S[mt][v] = rounded(logit(S[mt][v])) * kLog2e;
+      };
+      auto with_cap = [&](float s) { return __builtin_fmaf(__builtin_amdgcn_rcpf(fast_exp2(s * k1) + 1.0f), -2.0f * k2, k2); };
+      auto no_cap = [&](float s) { return s * k2; };
+      auto as_is = [](float x) { return x; };
+      auto to_bf16 = [](float x) { return bf16_round(x); };
+      auto to_f16 = [](float x) { return f16_round(x); };
+      if (capped) {  // (rounded: the unrounded capped case is the branch above)
+        if (sm.round_mode == 1) all_scores(with_cap, to_bf16);
+        else all_scores(with_cap, to_f16);
+      } else {
+        if (sm.round_mode == 1) all_scores(no_cap, to_bf16);
+        else if (sm.round_mode == 2) all_scores(no_cap, to_f16);
+        else all_scores(no_cap, as_is);
       }
+    }
   }
   if (need_mask) {
 #pragma unroll
@@ -228,6 +271,7 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[ND]
         const int tok = tb + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
         bool masked;
         if (!EXT || mc.mode == 0) masked = tok > qpos;
+        else if constexpr (PRE) masked = (tok >= mc.kv_len) || (mc.mode == 1 && pre->g[4 * mt + (v >> 2)][v & 3] < 1);
         else masked = (tok >= mc.kv_len) || (mc.mode == 1 && mc.row[tok] < 1);
         masked = masked || (window > 0 && tok <= qpos - window);
         S[mt][v] = masked ? kMaskRaw : S[mt][v];
