@@ -229,7 +229,9 @@ int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t*
  * Bytes of workspace for `p`: what the decode rows' split-KV plan needs (rpa_decode fails without
  * it), or, if larger, the room that lets a prefill launch which would leave most of the GPU idle
  * (one long prompt on a few heads, a verify step on a long context) cut its K/V ranges into pieces
- * and merge them; rpa_prefill uses that room when it is there and runs whole ranges when it is not.
+ * and merge them, and that holds a custom mask as one bit per (query token, kv token); rpa_prefill uses
+ * that room when it is there and otherwise runs whole ranges and reads the mask's i32 words (slower,
+ * same results to the tolerance of the path).
  */
 size_t rpa_workspace_bytes(const RpaParams* p);
 size_t rpa_mla_workspace_bytes(const RpaMlaParams* p);

@@ -607,8 +607,35 @@ static bool prefill_args(const RpaParams* p, rpa::PrefillArgs& a) {
   a.num_tokens = p->num_tokens;
   a.ws_o = nullptr;
   a.ws_ml = nullptr;
+  a.mask_bits = nullptr;
+  a.mask_pitch = 0;
   return true;
 }
+
+// What a prefill launch can use of the workspace, none of it required: the partial rows of K/V ranges cut into
+// pieces (launches that would leave most of the GPU idle), and a custom mask turned into bits by a pre-pass
+// (needs a bound on the lengths; RPA_MASK_BITS=0 keeps the kernels on the caller's i32 words).
+namespace {
+struct PrefillWorkspace {
+  int splits;
+  int pitch;  // 64-bit words per bit row
+  size_t split_bytes, bits_offset, bits_bytes, total;
+};
+PrefillWorkspace prefill_workspace(const RpaParams* p, const rpa::PrefillArgs& a) {
+  PrefillWorkspace w = {};
+  w.splits = rpa::prefill_kv_splits(a);
+  w.split_bytes = rpa::prefill_split_workspace_bytes(a, w.splits);
+  w.bits_offset = (w.split_bytes + 255) & ~(size_t)255;
+  if (p->mask_mode == RPA_MASK_CUSTOM && p->head_dim == 128 && !p->distribution && p->max_kv_len > 0 && p->num_tokens > 0 &&
+      env_int("RPA_MASK_BITS", 1) != 0) {
+    w.pitch = (p->max_kv_len + 63) / 64;
+    w.bits_bytes = (size_t)p->num_tokens * w.pitch * sizeof(uint64_t);
+    if (w.bits_bytes > ((size_t)256 << 20)) w.bits_bytes = 0;  // a batch this large keeps the i32 words
+  }
+  w.total = w.bits_bytes ? w.bits_offset + w.bits_bytes : w.split_bytes;
+  return w;
+}
+}  // namespace
 
 // Workspace that lets a prefill launch which would leave most of the GPU idle cut its K/V ranges into
 // pieces; never required: without it the launch runs whole ranges.
@@ -616,7 +643,7 @@ static size_t prefill_optional_workspace(const RpaParams* p) {
   rpa::PrefillArgs a;
   if (!prefill_args(p, a)) return 0;
   if (p->head_dim == 256 && env_int("RPA_PREFILL_ROWS256", 0) != 0) return 0;  // the row kernel has its own plan
-  return rpa::prefill_split_workspace_bytes(a, rpa::prefill_kv_splits(a));
+  return prefill_workspace(p, a).total;
 }
 
 int rpa_prefill(const RpaParams* p, void* stream) {
@@ -628,14 +655,29 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   // caches staged through registers); RPA_PREFILL_ROWS256=1 sends them through the row kernel
   if (p->head_dim == 256 && env_int("RPA_PREFILL_ROWS256", 0) != 0)
     return rows256(p, (p->mask_mode == RPA_MASK_CUSTOM) ? 0 : p->decode_end, p->num_seqs, stream);
-  {
+  if (p->workspace && (reinterpret_cast<uintptr_t>(p->workspace) & 15) == 0) {
     // the decode partition is done with the workspace by the time these kernels run (same stream)
-    const int splits = rpa::prefill_kv_splits(a);
-    const size_t need = rpa::prefill_split_workspace_bytes(a, splits);
-    if (splits > 1 && p->workspace && p->workspace_bytes >= need && (reinterpret_cast<uintptr_t>(p->workspace) & 15) == 0) {
-      a.kv_splits = splits;
-      a.ws_o = static_cast<float*>(p->workspace);
-      a.ws_ml = a.ws_o + (size_t)p->num_tokens * p->num_q_heads * splits * p->head_dim;
+    const PrefillWorkspace w = prefill_workspace(p, a);
+    char* ws = static_cast<char*>(p->workspace);
+    size_t bits_at = 0;
+    bool cut = false, bits = false;
+    if (w.bits_bytes && p->workspace_bytes >= w.total) {
+      bits = true;
+      bits_at = w.bits_offset;
+      cut = w.splits > 1;
+    } else if (w.bits_bytes && p->workspace_bytes >= w.bits_bytes) {
+      bits = true;  // room for the bits alone: they save more than the pieces
+    } else if (w.splits > 1 && p->workspace_bytes >= w.split_bytes) {
+      cut = true;
+    }
+    if (cut) {
+      a.kv_splits = w.splits;
+      a.ws_o = reinterpret_cast<float*>(ws);
+      a.ws_ml = a.ws_o + (size_t)p->num_tokens * p->num_q_heads * w.splits * p->head_dim;
+    }
+    if (bits) {
+      a.mask_bits = reinterpret_cast<uint64_t*>(ws + bits_at);
+      a.mask_pitch = w.pitch;
     }
   }
   return check_hip(rpa::launch_prefill(a, static_cast<hipStream_t>(stream)), "rpa_prefill");

@@ -99,6 +99,10 @@ struct PrefillArgs {
   int32_t num_tokens;  // bound on the query tokens of the call (rows of q)
   float* ws_o;
   float* ws_ml;
+  // Custom masks: one bit per (query token, kv token), mask_pitch 64-bit words per token row, written by
+  // rpa_mask_bits_kernel in front of the attention kernels; nullptr: the kernels read the caller's i32 words
+  uint64_t* mask_bits;
+  int32_t mask_pitch;
 };
 
 struct GatherArgs {

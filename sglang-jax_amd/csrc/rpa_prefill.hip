@@ -96,7 +96,10 @@ __device__ __forceinline__ void fp8_lstore(const Fp8Stage<HD>& st, char* lds_k, 
 // HD = 256 doubles the rows in LDS (two 64 KiB slots), the Q^T operands and the accumulators: one
 // workgroup per CU, one wave per SIMD with up to 512 registers.
 // FP8: an e4m3 cache staged through registers into the same LDS layout (see above).
-template <bool UNIFORM, bool CAP, bool EXT, int HD = 128, bool FP8 = false>
+// HEADS4: the short-chunk tile (chunks of at most 64 tokens: a verify step, a short prompt).  A workgroup owns 32
+// query positions of FOUR query heads of a kv head, one head per wave, instead of 128 positions of one head:
+// such chunks then fill their tiles, and the four waves still share every K/V tile.
+template <bool UNIFORM, bool CAP, bool EXT, int HD = 128, bool FP8 = false, bool HEADS4 = false>
 __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_kernel(const PrefillArgs a_in, int tiles, int nseq,
                                                                                   bool by_level) {
   PrefillArgs a = a_in;  // static-shape mode: the sequences to process come from the device
@@ -107,7 +110,6 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
   using T = Tile<HD>;
   constexpr int kRowB = T::kRowB;
   constexpr int kTileB = T::kTileB;
-  constexpr bool kMaskPre = EXT && HD == 128 && !FP8;
   // Four separate arrays (not one indexed array): the compiler can then prove that the
   // asynchronous copy into one ring slot does not alias the LDS reads of the other slot and
   // does not drain the vector-memory queue in the middle of a tile.
@@ -116,18 +118,21 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
   __shared__ __attribute__((aligned(1024))) char lds_v0[kTileB];
   __shared__ __attribute__((aligned(1024))) char lds_v1[kTileB];
 
-  const Work w = decompose(a, tiles, nseq, by_level);
+  static_assert(!HEADS4 || (HD == 128 && !FP8), "the short-chunk tile exists for 128-wide heads on bf16 caches");
+  constexpr int BM = HEADS4 ? 32 : kBM;  // query positions per workgroup
+  Work w = decompose(a, tiles, nseq, by_level, BM, HEADS4 ? 4 : 1);
   if (!w.valid) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if constexpr (HEADS4) w.head += wave;  // this wave's head
   const int c = lane & 31, h = lane >> 5;
   const TileSrc src = make_src(a, w);
   const char* kh = a.kv.k_base + (int64_t)w.hk * a.kv.head_stride;
   const char* vh = a.kv.v_base + (int64_t)w.hk * a.kv.head_stride;
 
   WaveRows wr;
-  wr.r_lo = w.q_start + wave * 32;
+  wr.r_lo = w.q_start + (HEADS4 ? 0 : wave * 32);
   wr.r_hi = min(wr.r_lo + 31, w.q_len - 1);
   wr.active = wr.r_lo < w.q_len;
   wr.row = wr.r_lo + c;
@@ -164,7 +169,7 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
     for (int v = 0; v < 16; ++v) O[d][v] = 0.f;
   float m = kMaxFloor, l = 0.f;
 
-  const int wg_r_hi = min(w.q_start + kBM, w.q_len) - 1;
+  const int wg_r_hi = min(w.q_start + BM, w.q_len) - 1;
   const bool causal = !EXT || a.sm.mask_mode == 0;
   MaskCtx mc;
   mc.mode = 0;
@@ -227,11 +232,9 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
 
   // one tile: consume (lds_k, lds_v), fill (nxt_k, nxt_v) with the tile after it
   auto tile_step = [&](const char* lds_k, const char* lds_v, char* nxt_k, char* nxt_v, int tb) {
-    // a caller's mask: the tile's words are requested before the next tile's copy (128-wide heads on bf16 caches,
-    // where the registers for them exist)
-    MaskTile mtile;
-    if constexpr (kMaskPre) {
-      if (mc.mode == 1) load_mask_tile(mtile, mc, tb, h);
+    uint64_t mask_word = 0;  // a caller's mask turned into bits by the pre-pass: one word per lane and tile
+    if constexpr (EXT && HD == 128) {
+      if (mc.mode == 1 && mc.bits) mask_word = mc.bits[min(tb >> 6, mc.bit_words - 1)];
     }
     if (tb + kBN < t_hi) {
       // the other slot was last read before the barrier that ended the previous tile
@@ -262,7 +265,7 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void rpa_prefill_async_ke
           S[1] = mfma32(lds_ld16(lds_k + koff[ks] + 32 * kRowB), qB[ks], S[1]);
         }
         u32x4_t pB[2][2];
-        softmax_tile<CAP, EXT, T::kDimTiles, kMaskPre>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc, &mtile);
+        softmax_tile<CAP, EXT, T::kDimTiles>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc, mask_word);
         // independent accumulator chains (dim tiles), issued round-robin
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -489,6 +492,10 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
   for (int tb = t_lo; tb < t_hi; tb += kBN, buf ^= 1) {
     const char* lds_k = lds_k_buf[buf];
     const char* lds_v = lds_v_buf[buf];
+    uint64_t mask_word = 0;  // a caller's mask turned into bits by the pre-pass: one word per lane and tile
+    if constexpr (EXT) {
+      if (mc.mode == 1 && mc.bits) mask_word = mc.bits[min(tb >> 6, mc.bit_words - 1)];
+    }
     if (tb + kBN < t_hi) {
       // the other buffer was last read before the barrier that ended the previous tile
       tile_lstore<FP8>(stg, lds_k_buf[buf ^ 1], lds_v_buf[buf ^ 1], tid);
@@ -509,7 +516,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
         for (int ks = 1; ks < 8; ++ks) S[mt] = mfma32(lds_ld16(kp + ks * 32), qB[ks], S[mt]);
       }
       u32x4_t pB[2][2];
-      softmax_tile<CAP, EXT>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc);
+      softmax_tile<CAP, EXT>(S, O, m, l, sm, need_mask, tb, h, wr.qpos, W_, pB, mc, mask_word);
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
         const char* vp = lds_v + (d * 32 + c) * kVPitch + h * 16;
@@ -529,6 +536,45 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
 }  // namespace
 
 namespace {
+// ---------------------------------------------------------------- custom masks as bits
+// The caller's mask is one i32 per (query token, kv token).  Read where the scores are, a wave's 32 rows are 32
+// separate 256-byte runs per tile -- four times the cache lines of the K/V tile itself, per query head.  This
+// pre-pass reads it once, coalesced, and leaves one bit per pair (>= 1 keeps): bit t % 64 of word t / 64 of
+// row `token`, mask_pitch words per row; tokens from kv_len on read as hidden.  grid = query tokens, 4 waves,
+// wave w takes words w, w + 4, ...
+__device__ __forceinline__ int mask_owner_of_token(const int32_t* cu_q_lens, int num_seqs, int tok) {
+  int lo = 0, hi = num_seqs;  // last i with cu_q_lens[i] <= tok (zero-length sequences are skipped)
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu_q_lens[mid] <= tok) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+__global__ __launch_bounds__(256) void rpa_mask_bits_kernel(const PrefillArgs a) {
+  const int token = a.pt.cu_q_lens[a.seq_begin] + (int)blockIdx.x;
+  if (token >= a.pt.cu_q_lens[a.seq_end]) return;
+  const int seq = mask_owner_of_token(a.pt.cu_q_lens, a.seq_end, token);
+  const int kv_len = a.pt.kv_lens[seq];
+  const int width = a.sm.mask_rows_page_aligned ? (a.pt.cu_kv_lens[seq + 1] - a.pt.cu_kv_lens[seq]) : kv_len;
+  const int32_t* row = a.sm.custom_mask + a.sm.cu_mask_lens[seq] + (int64_t)(token - a.pt.cu_q_lens[seq]) * width;
+  uint64_t* out = a.mask_bits + (int64_t)token * a.mask_pitch;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int words = min((kv_len + 63) >> 6, a.mask_pitch);
+  for (int k = wave; k < words; k += 4) {
+    const int t = 64 * k + lane;
+    const int v = (t < kv_len) ? row[t] : 0;
+    const uint64_t keep = __ballot(v >= 1);
+    if (lane == 0) out[k] = keep;
+  }
+}
+
+hipError_t launch_mask_bits(const PrefillArgs& a, hipStream_t stream) {
+  if (!a.mask_bits || a.num_tokens <= 0) return hipSuccess;
+  hipLaunchKernelGGL(rpa_mask_bits_kernel, dim3((unsigned)a.num_tokens), dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
 bool takes_pipe_kernel(const PrefillArgs& a) {
   static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
   static const bool use_pipe = [] { const char* v = getenv("RPA_PREFILL_PIPE"); return !(v && *v == '0'); }();
@@ -536,12 +582,24 @@ bool takes_pipe_kernel(const PrefillArgs& a) {
 }
 }  // namespace
 
+namespace {
+// The compiled flash kernel's short-chunk tile: 32 positions x 4 heads per workgroup for chunks of at most 64
+// tokens (128-wide heads on bf16 caches, heads in fours; RPA_PREFILL_PIPE_TILE=32|128 forces either, read per call).
+bool compiled_short_chunk_tile(const PrefillArgs& a) {
+  static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
+  if (a.fp8 || force_staged || a.head_dim != 128 || (a.G % 4) != 0) return false;
+  const char* tile_env = getenv("RPA_PREFILL_PIPE_TILE");
+  const int force_tile = tile_env ? atoi(tile_env) : 0;
+  return force_tile ? force_tile == 32 : a.max_q_len <= 64;
+}
+}  // namespace
+
 int prefill_kv_splits(const PrefillArgs& a) {
   const int nseq = a.seq_end - a.seq_begin;
   if (takes_pipe_kernel(a)) return prefill_pipe_kv_splits(a, nseq);
-  // the compiled kernels: 128 positions of one head per workgroup, a tile takes about 1.1 us alone on its CU
-  // (2.2 us for 256-wide heads)
-  return kv_pieces(a, nseq, kBM, 1, a.head_dim == 256 ? 2.2 : 1.1);
+  // the compiled kernels: a tile takes about 1.1 us alone on its CU (2.2 us for 256-wide heads)
+  const bool heads4 = compiled_short_chunk_tile(a);
+  return kv_pieces(a, nseq, heads4 ? 32 : kBM, heads4 ? 4 : 1, a.head_dim == 256 ? 2.2 : 1.1);
 }
 
 size_t prefill_split_workspace_bytes(const PrefillArgs& a, int splits) {
@@ -551,22 +609,31 @@ size_t prefill_split_workspace_bytes(const PrefillArgs& a, int splits) {
 hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const int nseq = a.seq_end - a.seq_begin;
   if (nseq <= 0 || a.max_q_len <= 0) return hipSuccess;
-  int tiles = (a.max_q_len + kBM - 1) / kBM;
+  if (takes_pipe_kernel(a)) {
+    static const bool lo = [] { const char* v = getenv("RPA_PREFILL_LEVEL_ORDER"); return !(v && *v == '0'); }();
+    return launch_prefill_pipe(a, nseq, lo, stream);
+  }
+  const bool heads4 = compiled_short_chunk_tile(a);
+  const int bm = heads4 ? 32 : kBM;
+  int tiles = (a.max_q_len + bm - 1) / bm;
   // levels 0 .. ceil(max_kv_len / rows): only worth their empty workgroups when prefixes are
   // not much longer than the chunks (else every tile of a sequence costs about the same anyway)
   static const bool level_order = [] { const char* v = getenv("RPA_PREFILL_LEVEL_ORDER"); return !(v && *v == '0'); }();
-  const int levels = a.max_kv_len > 0 ? (a.max_kv_len + kBM - 1) / kBM + 1 : 0;
+  const int levels = a.max_kv_len > 0 ? (a.max_kv_len + bm - 1) / bm + 1 : 0;
   const bool by_level = level_order && a.sm.mask_mode == 0 && levels > tiles && levels <= 2 * tiles + 2;
   if (by_level) tiles = levels;
   const int64_t units = (int64_t)nseq * a.Hkv;
-  const int64_t grid = (units >= 8 ? ((units + 7) / 8) * 8 : units) * a.G * tiles;
+  const int64_t grid = (units >= 8 ? ((units + 7) / 8) * 8 : units) * (heads4 ? a.G / 4 : a.G) * tiles;
   if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
   const bool uniform = (a.pt.page_size % kBN) == 0;
   // soft cap and logit rounding share the general score path
   const bool cap = a.sm.soft_cap != 0.f || a.sm.round_logits != 0;
   static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
   const bool staged = a.fp8 || force_staged;
-  if (takes_pipe_kernel(a)) return launch_prefill_pipe(a, nseq, level_order, stream);
+  if (a.sm.mask_mode == 1) {
+    hipError_t e = launch_mask_bits(a, stream);
+    if (e != hipSuccess) return e;
+  }
   const bool cut = a.kv_splits > 1;  // pieces of the K/V ranges on the second grid dimension, then the merge
   if (cut && (!a.ws_o || !a.ws_ml || a.kv_splits > 64)) return hipErrorInvalidValue;
   const dim3 g((unsigned)grid, cut ? (unsigned)a.kv_splits : 1u), blk(256);
@@ -574,6 +641,8 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
 #define RPA_STAGED(F, U, C, E) \
   hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_ASYNC(U, C, E) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
+#define RPA_ASYNC_HEADS4(U, C, E) \
+  hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E, 128, false, true>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_ASYNC256(U, C, E) \
   hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E, 256>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_ASYNC256_FP8(U, C, E) \
@@ -597,6 +666,8 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
     } else {
       RPA_PICK(RPA_ASYNC256, )
     }
+  } else if (heads4) {
+    RPA_PICK(RPA_ASYNC_HEADS4, )
   } else if (!staged) {
     RPA_PICK(RPA_ASYNC, )
   } else if (a.fp8) {
@@ -609,6 +680,7 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
 #undef RPA_PICK
 #undef RPA_STAGED
 #undef RPA_ASYNC
+#undef RPA_ASYNC_HEADS4
 #undef RPA_ASYNC256
 #undef RPA_ASYNC256_FP8
   return cut ? launch_prefill_combine(a, stream) : hipGetLastError();

@@ -178,7 +178,9 @@ __device__ __forceinline__ float swap_max(float x) {
 struct MaskCtx {
   int mode;
   int kv_len;
-  const int32_t* row;  // mode 1: this lane's mask row (token t at row[t])
+  const int32_t* row;    // mode 1: this lane's mask row (token t at row[t])
+  const uint64_t* bits;  // mode 1: the same row as bits (token t = bit t % 64 of word t / 64), or nullptr
+  int bit_words;         // words per bit row
 };
 
 __device__ __forceinline__ MaskCtx make_mask_ctx(const PrefillArgs& a, const Work& w, int row) {
@@ -186,6 +188,9 @@ __device__ __forceinline__ MaskCtx make_mask_ctx(const PrefillArgs& a, const Wor
   mc.mode = a.sm.mask_mode;
   mc.kv_len = w.kv_len;
   mc.row = nullptr;
+  mc.bits = nullptr;
+  mc.bit_words = a.mask_pitch;
+  if (mc.mode == 1 && a.mask_bits) mc.bits = a.mask_bits + (int64_t)(w.qg0 + min(row, w.q_len - 1)) * a.mask_pitch;
   if (mc.mode == 1) {
     const int width = a.sm.mask_rows_page_aligned ? (a.pt.cu_kv_lens[w.seq + 1] - a.pt.cu_kv_lens[w.seq]) : w.kv_len;
     mc.row = a.sm.custom_mask + a.sm.cu_mask_lens[w.seq] + (int64_t)min(row, w.q_len - 1) * width;
@@ -193,41 +198,28 @@ __device__ __forceinline__ MaskCtx make_mask_ctx(const PrefillArgs& a, const Wor
   return mc;
 }
 
-// The mask words of one lane for a whole 64-token tile: group 4 mt + j holds tokens tb + 32 mt + 8 j + 4 h .. + 3,
-// the lane's scores v = 4 j .. 4 j + 3 of half mt.  Requested at the top of a tile's step, in FRONT of the next
-// tile's copy: loads return in order, so the wait for these words then leaves the copy in flight.  (One
-// 4-byte load per score behind the first product, as before, waited for the copy as well on every tile and
-// cost 32 load instructions per lane: a verify step of 16 draft tokens on 4096-token prefixes ran 5.6 x slower
-// with a tree mask than without.)
-typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
-struct MaskTile {
-  i32x4_t g[8];
-};
-
-__device__ __forceinline__ void load_mask_tile(MaskTile& t, const MaskCtx& mc, int tb, int h) {
-  if (tb + kBN <= mc.kv_len) {  // the tile lies inside the row
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        __builtin_memcpy(&t.g[4 * mt + j], mc.row + tb + 32 * mt + 8 * j + 4 * h, 16);  // rows are 4-byte aligned only
-  } else {  // the row's last tile: word by word, clamped (tokens beyond kv_len are hidden whatever they read)
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) t.g[4 * mt + j][e] = mc.row[min(tb + 32 * mt + 8 * j + 4 * h + e, mc.kv_len - 1)];
-  }
-}
-
-// PRE: the caller's mask comes from `pre` instead of one load per score.
-template <bool CAP, bool EXT, int ND = 4, bool PRE = false>
+// mask_word: with a caller's mask turned into bits (mc.bits), the word of this tile's 64 tokens, which the
+// caller fetches at the top of the tile's step, in FRONT of the next tile's copy: loads return in order, so
+// the wait for it leaves the copy in flight.  Without the bits, one 4-byte load per score, here, behind the
+// first product (which waits for the copy as well).
+template <bool CAP, bool EXT, int ND = 4>
 __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[ND], float& m, float& l,
                                              const Softmax<CAP>& sm, bool need_mask, int tb, int h, int qpos,
                                              int window, u32x4_t (&pB)[2][2], const MaskCtx& mc,
-                                             const MaskTile* pre = nullptr) {
-  if constexpr (CAP) {
+                                             uint64_t mask_word = 0) {
+  if constexpr (CAP && ND != 4) {
+    // 256-wide heads: one loop with run-time choices (those kernels have no register to spare for variants)
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float x = S[mt][v] * sm.scale;
+        if (sm.cap != 0.f) x = soft_cap_f(x, sm.cap, sm.inv_cap);
+        x = x * sm.temp;
+        if (sm.round_mode) x = round_logit(x, sm.round_mode);
+        S[mt][v] = x * kLog2e;
+      }
+  } else if constexpr (CAP) {
     if (sm.cap != 0.f && !sm.round_mode) {
       // soft cap alone (the usual case), constants folded: five instructions per score.
       // cap tanh(s scale / cap) temp log2e = k2 - 2 k2 / (2^(s k1) + 1)
@@ -263,7 +255,19 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[ND]
       }
     }
   }
-  if (need_mask) {
+  if (EXT && ND == 4 && need_mask && mc.mode == 1 && mc.bits) {  // (128-wide heads: the 256-wide kernels have no register to spare)
+    // the caller's mask as bits: the tile's 64 tokens are one word, fetched by the caller at the top of the step
+    const uint32_t half[2] = {(uint32_t)mask_word >> (4 * h), (uint32_t)(mask_word >> 32) >> (4 * h)};
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int tok = tb + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        bool masked = (tok >= mc.kv_len) || !((half[mt] >> (8 * (v >> 2) + (v & 3))) & 1u);
+        masked = masked || (window > 0 && tok <= qpos - window);
+        S[mt][v] = masked ? kMaskRaw : S[mt][v];
+      }
+  } else if (need_mask) {
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -271,7 +275,6 @@ __device__ __forceinline__ void softmax_tile(f32x16_t (&S)[2], f32x16_t (&O)[ND]
         const int tok = tb + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
         bool masked;
         if (!EXT || mc.mode == 0) masked = tok > qpos;
-        else if constexpr (PRE) masked = (tok >= mc.kv_len) || (mc.mode == 1 && pre->g[4 * mt + (v >> 2)][v & 3] < 1);
         else masked = (tok >= mc.kv_len) || (mc.mode == 1 && mc.row[tok] < 1);
         masked = masked || (window > 0 && tok <= qpos - window);
         S[mt][v] = masked ? kMaskRaw : S[mt][v];

@@ -221,6 +221,37 @@ def test_workspace_for_prefill_launches_that_leave_the_gpu_idle(pkg, monkeypatch
     assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 512 * 8 * 5 * row
 
 
+def test_workspace_for_a_custom_mask_as_bits(pkg, monkeypatch):
+    """Custom masks: rpa_workspace_bytes adds one bit per (query token, kv token up to the bound on the lengths),
+    rows of whole 64-bit words, behind the partial rows of a cut launch (256-byte aligned).  Not without a bound on
+    the lengths, not for 256-wide heads, not with RPA_MASK_BITS=0."""
+    lib = pkg._lib.load()
+    monkeypatch.delenv("RPA_PREFILL_SPLITS", raising=False)
+    monkeypatch.delenv("RPA_MASK_BITS", raising=False)
+    p = base_params(pkg)
+    p.num_seqs, p.decode_end, p.num_tokens = 64, 0, 1024
+    p.num_q_heads, p.num_kv_heads, p.page_size, p.total_pages = 32, 8, 64, 8192
+    p.max_q_len, p.max_kv_len = 16, 4112
+    p.mask_mode = 1
+    p.custom_mask = 0x1000
+    p.cu_mask_lens = 0x1000
+    bits = 1024 * ((4112 + 63) // 64) * 8
+    monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == bits
+    monkeypatch.setenv("RPA_PREFILL_SPLITS", "3")
+    partial = 1024 * 32 * 3 * (128 + 2) * 4
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == ((partial + 255) // 256) * 256 + bits
+    monkeypatch.setenv("RPA_MASK_BITS", "0")
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == partial
+    monkeypatch.delenv("RPA_MASK_BITS")
+    monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
+    p.max_kv_len = 0
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+    p.max_kv_len = 4112
+    p.head_dim = 256
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+
+
 def test_python_wrapper_raises_like_the_reference(pkg):
     import torch
 

@@ -1233,3 +1233,80 @@ def test_kv_range_pieces_in_the_compiled_prefill_kernels(pkg, wl, gpu, monkeypat
         monkeypatch.delenv("RPA_PREFILL_SPLITS")
         assert torch.isfinite(cut.float()).all()
         assert_parity(cut.float(), want.float(), **tol)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("aligned", [False, True])
+def test_custom_mask_as_bits_equals_the_callers_words(pkg, wl, gpu, monkeypatch, fp8, aligned):
+    """A pre-pass turns the caller's i32 mask into one bit per (query token, kv token) and the kernels read one
+    word per lane and tile; RPA_MASK_BITS=0 keeps them on the i32 words.  Same rows bit for bit, and the oracle's:
+    a verify step on long contexts, a chunk, decode rows, rows kv_len wide and rows padded to whole pages,
+    with and without a sliding window."""
+    P = 64
+    q_lens, kv_lens = [1, 9, 16, 1, 130], [700, 3009, 64, 65, 1000]
+    rng = np.random.default_rng(12)
+    masks = []
+    for ql, kv in zip(q_lens, kv_lens):
+        m = (rng.random((ql, kv)) < 0.5).astype(np.int32) * rng.integers(1, 4, size=(ql, kv)).astype(np.int32)
+        m[:, kv - 1] = 1   # every row keeps a token
+        m[0, : kv - 1] = 0  # and one row nothing else
+        if aligned:
+            w = -(-kv // P) * P
+            mp = np.full((ql, w), 7, dtype=np.int32)  # the padding says "keep": tokens from kv_len on stay hidden
+            mp[:, :kv] = m
+            m = mp
+        masks.append(m)
+    cm = flat_mask(masks)
+    want_masks = flat_mask([m[:, :kv] for m, kv in zip(masks, kv_lens)])
+    for window in (None, 900):
+        say(f"mask bits fp8={fp8} aligned={aligned} window={window}")
+        b = wl.make_batch("mask_bits", q_lens, kv_lens, num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=P, seed=93,
+                          kv_dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16, sliding_window=window)
+        kw = dict(causal=0, custom_mask=cm.to(gpu), mask_aligned_to_cu_kv=aligned)
+        monkeypatch.setenv("RPA_MASK_BITS", "0")
+        words = gpu_out(pkg, b, gpu, **kw)
+        monkeypatch.delenv("RPA_MASK_BITS")
+        bits = gpu_out(pkg, b, gpu, **kw)
+        assert torch.equal(bits, words)
+        assert_parity(bits.float(), oracle_out(b, causal=False, custom_mask=want_masks).float(), **(FP8_TOL if fp8 else BF16_TOL))
+
+
+@pytest.mark.parametrize("kind", ["soft_cap", "xai_temperature", "custom_mask", "no_mask", "softmax_bf16"])
+def test_short_chunks_take_the_four_head_tile_in_the_compiled_kernel(pkg, wl, gpu, monkeypatch, kind):
+    """The compiled flash kernel (every option the pipelined one does not take) with the same short-chunk tile:
+    32 positions x 4 query heads per workgroup for chunks of at most 64 tokens.  Against the oracle and against
+    the same call forced onto the 128-position tile (RPA_PREFILL_PIPE_TILE)."""
+    q_lens = [1, 1, 2, 5, 16, 31, 32, 33, 64, 47]
+    kv_lens = [300, 5000, 2, 5, 4016, 31, 1056, 97, 64, 5047]
+    for window in (None, 700):
+        say(f"short chunks, compiled kernel, {kind} window={window}")
+        b = wl.make_batch("short_chunks_" + kind, q_lens, kv_lens, num_q_heads=16, num_kv_heads=2, head_dim=128, page_size=64,
+                          seed=4300, sliding_window=window, soft_cap=30.0 if kind == "soft_cap" else None)
+        wl.plant_needles(b, seed=9)
+        okw, gkw = {}, {}
+        if kind == "xai_temperature":
+            okw = gkw = dict(xai_temperature_len=512.0)
+        elif kind == "softmax_bf16":
+            okw = gkw = dict(softmax_dtype=torch.bfloat16)
+        elif kind == "no_mask":
+            okw, gkw = dict(causal=False), dict(causal=0)
+        elif kind == "custom_mask":
+            rng = np.random.default_rng(8)
+            masks = []
+            for ql, kv in zip(q_lens, kv_lens):
+                m = (rng.random((ql, kv)) < 0.6).astype(np.int32)
+                m[:, kv - 1] = 1
+                masks.append(m)
+            cm = flat_mask(masks)
+            okw, gkw = dict(causal=False, custom_mask=cm), dict(causal=0, custom_mask=cm.to(gpu))
+        want = oracle_out(b, **okw)
+        monkeypatch.setenv("RPA_PREFILL_PIPE_TILE", "32")
+        small = gpu_out(pkg, b, gpu, **gkw)
+        monkeypatch.setenv("RPA_PREFILL_PIPE_TILE", "128")
+        big = gpu_out(pkg, b, gpu, **gkw)
+        monkeypatch.delenv("RPA_PREFILL_PIPE_TILE")
+        auto = gpu_out(pkg, b, gpu, **gkw)
+        assert_parity(small.float(), want.float(), **BF16_TOL)
+        assert_parity(big.float(), want.float(), **BF16_TOL)
+        assert torch.equal(auto, small)  # every chunk here is at most 64 tokens long
+        assert float(row_rel_error(small.float(), big.float()).max()) < 1e-2
