@@ -406,7 +406,7 @@ __device__ __forceinline__ void tile_lstore(const Stage<FP8>& st, char* lds_k, c
   }
 }
 
-template <bool FP8, bool UNIFORM, bool CAP, bool EXT>
+template <bool FP8, bool UNIFORM, bool CAP, bool EXT, bool HEADS4 = false>
 __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const PrefillArgs a_in, int tiles, int nseq, bool by_level) {
   PrefillArgs a = a_in;  // static-shape mode: the sequences to process come from the device
   if (a.dist) {
@@ -416,17 +416,19 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
   __shared__ __attribute__((aligned(16))) char lds_k_buf[2][kBN * kKPitch];
   __shared__ __attribute__((aligned(16))) char lds_v_buf[2][128 * kVPitch];
 
-  const Work w = decompose(a, tiles, nseq, by_level);
+  constexpr int BM = HEADS4 ? 32 : kBM;  // the short-chunk tile: 32 positions x 4 heads, one head per wave
+  Work w = decompose(a, tiles, nseq, by_level, BM, HEADS4 ? 4 : 1);
   if (!w.valid) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
+  if constexpr (HEADS4) w.head += wave;
   const int c = lane & 31, h = lane >> 5;
   const TileSrc src = make_src(a, w);
   const char* kh = a.kv.k_base + (int64_t)w.hk * a.kv.head_stride;
   const char* vh = a.kv.v_base + (int64_t)w.hk * a.kv.head_stride;
 
   WaveRows wr;
-  wr.r_lo = w.q_start + wave * 32;
+  wr.r_lo = w.q_start + (HEADS4 ? 0 : wave * 32);
   wr.r_hi = min(wr.r_lo + 31, w.q_len - 1);
   wr.active = wr.r_lo < w.q_len;
   wr.row = wr.r_lo + c;
@@ -463,7 +465,7 @@ __global__ __launch_bounds__(256, 2) void rpa_prefill_staged_kernel(const Prefil
     for (int v = 0; v < 16; ++v) O[d][v] = 0.f;
   float m = kMaxFloor, l = 0.f;
 
-  const int wg_r_hi = min(w.q_start + kBM, w.q_len) - 1;
+  const int wg_r_hi = min(w.q_start + BM, w.q_len) - 1;
   const bool causal = !EXT || a.sm.mask_mode == 0;
   MaskCtx mc;
   mc.mode = 0;
@@ -584,10 +586,10 @@ bool takes_pipe_kernel(const PrefillArgs& a) {
 
 namespace {
 // The compiled flash kernel's short-chunk tile: 32 positions x 4 heads per workgroup for chunks of at most 64
-// tokens (128-wide heads on bf16 caches, heads in fours; RPA_PREFILL_PIPE_TILE=32|128 forces either, read per call).
+// tokens (128-wide heads, heads in fours; RPA_PREFILL_PIPE_TILE=32|128 forces either, read per call).
 bool compiled_short_chunk_tile(const PrefillArgs& a) {
   static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
-  if (a.fp8 || force_staged || a.head_dim != 128 || (a.G % 4) != 0) return false;
+  if ((force_staged && !a.fp8) || a.head_dim != 128 || (a.G % 4) != 0) return false;
   const char* tile_env = getenv("RPA_PREFILL_PIPE_TILE");
   const int force_tile = tile_env ? atoi(tile_env) : 0;
   return force_tile ? force_tile == 32 : a.max_q_len <= 64;
@@ -640,6 +642,8 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const bool ext = a.sm.xai_len > 0.f || a.sm.mask_mode != 0 || a.sm.q_scale > 0.f;
 #define RPA_STAGED(F, U, C, E) \
   hipLaunchKernelGGL((rpa_prefill_staged_kernel<F, U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
+#define RPA_STAGED_FP8_HEADS4(U, C, E) \
+  hipLaunchKernelGGL((rpa_prefill_staged_kernel<true, U, C, E, true>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_ASYNC(U, C, E) hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E>), g, blk, 0, stream, a, tiles, nseq, by_level)
 #define RPA_ASYNC_HEADS4(U, C, E) \
   hipLaunchKernelGGL((rpa_prefill_async_kernel<U, C, E, 128, false, true>), g, blk, 0, stream, a, tiles, nseq, by_level)
@@ -666,6 +670,8 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
     } else {
       RPA_PICK(RPA_ASYNC256, )
     }
+  } else if (heads4 && a.fp8) {
+    RPA_PICK(RPA_STAGED_FP8_HEADS4, )
   } else if (heads4) {
     RPA_PICK(RPA_ASYNC_HEADS4, )
   } else if (!staged) {
@@ -681,6 +687,7 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
 #undef RPA_STAGED
 #undef RPA_ASYNC
 #undef RPA_ASYNC_HEADS4
+#undef RPA_STAGED_FP8_HEADS4
 #undef RPA_ASYNC256
 #undef RPA_ASYNC256_FP8
   return cut ? launch_prefill_combine(a, stream) : hipGetLastError();
