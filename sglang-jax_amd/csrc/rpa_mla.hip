@@ -24,6 +24,8 @@
 // too.  So no address swizzle and no row permutation: MFMA row m of a score tile is token
 // 16b + m, and every LDS address is a per-lane base plus a compile-time offset.
 
+#include <type_traits>
+
 #include "rpa_common.h"
 #include "rpa_kernels.h"
 #include "rpa_mla_pipe_loop.inc"
@@ -278,7 +280,13 @@ struct MlaDest {
 // FP8: the cache holds e4m3 bytes.  Slots 0 and 1 are the bf16 ring, slot 2 (two halves) and slot 3 three
 // staging areas; a step copies the bytes of tile k + 3, multiplies tile k, and ends by expanding tile
 // k + 1 between two barriers.
-template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false>
+// DS: with at most 64 heads (a tensor-parallel share) most waves of the workgroup would have no heads, and a step
+// would last as long as one wave's serial chain through the tile (36 + 32 dependent matrix instructions with
+// their LDS reads) while the others only copy.  With DS = 8 / 4 / 2 (at most 16 / 32 / 64 heads) the DS waves of a
+// block of 16 heads share its tile instead: wave `sub` of the block takes token half sub & 1 and k-step group
+// sub >> 1 of the first product, leaves its partial scores in LDS, every wave of the block sums them and takes
+// the (same) probabilities, and the second product's 32 output chunks are dealt out 32 / DS per wave.
+template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false, int DS = 1>
 __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
                                             int t_begin, int t_end, const MlaDest dest, char* slot0, char* slot1,
                                             char* slot2, char* slot3) {
@@ -286,8 +294,12 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, g = lane >> 4;
-  const int head0 = head_base + wave * 16;
+  static_assert(DS == 1 || (UNIFORM && !PIPE), "shared tiles: compiled loop, whole tiles per page (LDS for the partial scores)");
+  const int sub = wave % DS;                       // this wave's place among the DS waves of its block of heads
+  const int head0 = head_base + (wave / DS) * 16;
   const bool wave_on = head0 < a.Hq;
+  constexpr int kChunksPerWave = 32 / DS;          // output chunks of 16 dims per wave
+  __shared__ __attribute__((aligned(16))) float partial_scores[DS == 1 ? 1 : 8][DS == 1 ? 4 : 256];  // [wave][lane x 4]
   const int seq = mr.seq;
   const int kv_len = mr.kv_len;
 
@@ -403,11 +415,48 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     if constexpr (FP8) copy_tile_f8<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane_t, pg_next);
     else copy_tile<UNIFORM>(fill, src, a.cache, tb + 3 * kTok, wave, lane_t, pg_next);
     pg_next = page_of(tb + 4 * kTok);
+    if constexpr (DS > 1) {
+      // this wave's share of the first product: one token half, one group of k-steps
+      f32x4_t sp = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (wave_on) {
+        const char* kp = cur + k_off_t + (sub & 1) * 16 * kRowB;
+        constexpr int kGroups = DS / 2;  // 4 groups of 5, 5, 4, 4 k-steps; 2 of 9; 1 of 18
+        auto chain = [&](auto lo, auto hi) __attribute__((always_inline)) {
+#pragma unroll
+          for (int ks = decltype(lo)::value; ks < decltype(hi)::value; ++ks) sp = mfma16(lds_ld16(kp + ks * 64), qB[ks], sp);
+        };
+        using std::integral_constant;
+        const int kg = sub >> 1;
+        if constexpr (kGroups == 4) {
+          if (kg == 0) chain(integral_constant<int, 0>{}, integral_constant<int, 5>{});
+          else if (kg == 1) chain(integral_constant<int, 5>{}, integral_constant<int, 10>{});
+          else if (kg == 2) chain(integral_constant<int, 10>{}, integral_constant<int, 14>{});
+          else chain(integral_constant<int, 14>{}, integral_constant<int, 18>{});
+        } else if constexpr (kGroups == 2) {
+          if (kg == 0) chain(integral_constant<int, 0>{}, integral_constant<int, 9>{});
+          else chain(integral_constant<int, 9>{}, integral_constant<int, 18>{});
+        } else {
+          chain(integral_constant<int, 0>{}, integral_constant<int, 18>{});
+        }
+      }
+      *reinterpret_cast<f32x4_t*>(&partial_scores[wave][lane_t * 4]) = sp;
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the partial scores are written
+      bare_barrier();
+    }
     if (wave_on) {
       // two independent accumulator chains (token halves), issued alternately
       f32x4_t s[2];
       s[0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       s[1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if constexpr (DS > 1) {
+        // the block's scores: the partial sums of its DS waves (wave sub' holds half sub' & 1, group sub' >> 1)
+        const int w0 = (wave / DS) * DS;
+#pragma unroll
+        for (int u = 0; u < DS; ++u) {
+          const f32x4_t part = *reinterpret_cast<const f32x4_t*>(&partial_scores[w0 + u][lane_t * 4]);
+          s[u & 1] += part;
+        }
+      } else {
       const char* kp = cur + k_off_t;
 #pragma unroll
       for (int ks = 0; ks < 18; ++ks) {
@@ -416,6 +465,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
         // fence the scheduler every few MFMAs: it would otherwise hoist all LDS reads of the
         // tile, run out of registers and spill (a spill reload drains the copy queue)
         if (ks % 3 == 2) __builtin_amdgcn_sched_barrier(0);
+      }
       }
       float x[8];
 #pragma unroll
@@ -449,11 +499,12 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
                                  pack_bf16x2(p[6], p[7])};
       if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-        for (int j = 0; j < 32; ++j) acc[j] = acc[j] * alpha;
+        for (int j = 0; j < kChunksPerWave; ++j) acc[j] = acc[j] * alpha;
       }
-      const char* vp = cur + v_off_t;
+      // (shared tiles: this wave's chunks are sub * kChunksPerWave .. of the 32)
+      const char* vp = cur + v_off_t + (DS > 1 ? sub * kChunksPerWave * 32 : 0);
 #pragma unroll
-      for (int j = 0; j < 32; ++j) {
+      for (int j = 0; j < kChunksPerWave; ++j) {
         const char* vt = vp + j * 32;
         const u32x2_t lo = lds_tr16(vt);
         const u32x2_t hi = lds_tr16(vt + 16 * kRowB);
@@ -612,11 +663,12 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   asm volatile("" : "+v"(c_out), "+v"(g_out));
   const int head = head0 + c_out;
   if (!wave_on || head >= a.Hq) return;
+  const int chunk0 = DS > 1 ? sub * kChunksPerWave : 0;  // shared tiles: this wave's output chunks
   if (dest.final_rows) {
     const float inv = a.out_scale / l;
-    uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 512 + g_out * 4;
+    uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 512 + g_out * 4 + chunk0 * 16;
 #pragma unroll
-    for (int j = 0; j < 32; ++j) {
+    for (int j = 0; j < kChunksPerWave; ++j) {
       u32x2_t w = {pack_bf16x2(acc[j][0] * inv, acc[j][1] * inv), pack_bf16x2(acc[j][2] * inv, acc[j][3] * inv)};
       *reinterpret_cast<u32x2_t*>(op + j * 16) = w;
     }
@@ -624,13 +676,13 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     const int64_t slot = dest.base + head;
     // partial rows are left as bf16: the merge reads half the bytes, and the result is rounded to
     // bf16 anyway
-    uint16_t* wo = a.ws_o + slot * 512 + g_out * 4;
+    uint16_t* wo = a.ws_o + slot * 512 + g_out * 4 + chunk0 * 16;
 #pragma unroll
-    for (int j = 0; j < 32; ++j) {
+    for (int j = 0; j < kChunksPerWave; ++j) {
       u32x2_t w = {pack_bf16x2(acc[j][0], acc[j][1]), pack_bf16x2(acc[j][2], acc[j][3])};
       *reinterpret_cast<u32x2_t*>(wo + j * 16) = w;
     }
-    if (g_out == 0) {
+    if (g_out == 0 && (DS == 1 || sub == 0)) {
       a.ws_ml[slot * 2 + 0] = m;
       a.ws_ml[slot * 2 + 1] = l;
     }
@@ -638,7 +690,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
 }
 
 // ---- fixed split plan: grid = (max_splits, rows, head groups of 128); block = 512 threads
-template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false>
+template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false, int DS = 1>
 __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeArgs a) {
   // three separate arrays: lets the compiler see that a copy into one slot does not alias the
   // reads of another, so it does not drain the vector-memory queue before LDS reads
@@ -660,7 +712,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   MlaDest dest;
   dest.final_rows = a.max_splits == 1;
   dest.base = ((int64_t)row_id * a.max_splits + split) * a.Hq;
-  mla_segment<UNIFORM, CAP, PIPE, FP8>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
+  mla_segment<UNIFORM, CAP, PIPE, FP8, DS>(a, mr, blockIdx.z * 128, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
 }
 
 // immediate of s_waitcnt vmcnt(n) (n < 64) with the other counters left alone
@@ -1082,7 +1134,7 @@ __device__ __forceinline__ void mla_balanced_body(const MlaDecodeArgs& a, Segmen
 }
 
 
-template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false>
+template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false, int DS = 1>
 __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecodeArgs a) {
   __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
@@ -1090,7 +1142,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
   __shared__ __attribute__((aligned(1024))) char slot3[kSlotB];
   mla_balanced_body(a, [&](const MlaRow& mr, int head_base, int t_lo, int t_begin, int t_end, const MlaDest& dest)
                         __attribute__((always_inline)) {
-    mla_segment<UNIFORM, CAP, PIPE, FP8>(a, mr, head_base, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
+    mla_segment<UNIFORM, CAP, PIPE, FP8, DS>(a, mr, head_base, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
   });
 }
 
@@ -1226,6 +1278,38 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   const int P = a.pt.page_size;
   const bool pipe = use_pipe && uniform && !cap && (P & (P - 1)) == 0 && (a.Hq % 128) == 0 &&
                     (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);
+  // at most 64 heads (a tensor-parallel share): the waves of a workgroup share each tile of a block of 16 heads
+  // (mla_segment, DS) instead of leaving most of them without heads.  RPA_MLA_SHARED_TILES=0: one wave per block,
+  // as with 128 heads (read per call).
+  const char* ds_env = getenv("RPA_MLA_SHARED_TILES");
+  const int ds = (uniform && !cap && a.Hq <= 64 && !(ds_env && *ds_env == '0')) ? (a.Hq <= 16 ? 8 : (a.Hq <= 32 ? 4 : 2)) : 1;
+  if (ds != 1) {
+#define RPA_MLA_DS(KERNEL, GRID, F8)                                                                                  \
+  do {                                                                                                                \
+    if (ds == 8) hipLaunchKernelGGL((KERNEL<true, false, false, F8, 8>), GRID, block, 0, stream, a);                 \
+    else if (ds == 4) hipLaunchKernelGGL((KERNEL<true, false, false, F8, 4>), GRID, block, 0, stream, a);            \
+    else hipLaunchKernelGGL((KERNEL<true, false, false, F8, 2>), GRID, block, 0, stream, a);                         \
+  } while (0)
+    if (a.balanced) {
+      const dim3 bgrid(a.num_wgs);
+      if (a.fp8) RPA_MLA_DS(rpa_mla_balanced_kernel, bgrid, true);
+      else RPA_MLA_DS(rpa_mla_balanced_kernel, bgrid, false);
+      hipError_t eb = hipGetLastError();
+      if (eb != hipSuccess) return eb;
+      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      return hipGetLastError();
+    }
+    if (a.fp8) RPA_MLA_DS(rpa_mla_decode_kernel, grid, true);
+    else RPA_MLA_DS(rpa_mla_decode_kernel, grid, false);
+#undef RPA_MLA_DS
+    hipError_t es = hipGetLastError();
+    if (es != hipSuccess) return es;
+    if (a.max_splits > 1) {
+      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      es = hipGetLastError();
+    }
+    return es;
+  }
   if (a.fp8) {  // e4m3 caches
     if (a.balanced) {
       const dim3 bgrid(a.num_wgs);

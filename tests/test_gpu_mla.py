@@ -75,6 +75,33 @@ def test_mla_long_rows_on_pages_smaller_than_a_tile(pkg, wl, gpu, P, f8):
     assert_parity(run_gpu(pkg, b, gpu).float(), ref(b).float(), **TOL)
 
 
+@pytest.mark.parametrize("Hq", [8, 16, 32, 48, 64])
+@pytest.mark.parametrize("f8", [False, True])
+def test_mla_waves_share_tiles_when_heads_are_few(pkg, wl, gpu, monkeypatch, Hq, f8):
+    """At most 64 heads (a tensor-parallel share of the 128): the eight waves of a workgroup share each tile of a
+    block of 16 heads -- partial scores per (token half, k-step group) summed through LDS, output chunks dealt out
+    -- instead of one wave per block.  Against the oracle and against RPA_MLA_SHARED_TILES=0: a long row cut over
+    the GPU, a ragged batch on the balanced plan, a sliding window, planted keys, a short chunk (token rows)."""
+    kw = dict(num_q_heads=Hq, lkv_dim=512, rope_dim=64, page_size=64, sm_scale=192 ** -0.5,
+              kv_dtype=torch.float8_e4m3fn if f8 else torch.bfloat16)
+    ref = fp8_oracle if f8 else oracle
+    lens = [int(x) for x in np.random.default_rng(Hq).integers(1, 3000, size=20)] + [1, 31, 32, 33, 7001]
+    for name, q_lens, kv_lens, window in (("long", [1], [9001], None), ("ragged", [1] * len(lens), lens, None),
+                                          ("window", [1, 1, 1], [100, 700, 5000], 600), ("chunk", [1, 9], [800, 2100], None)):
+        say(f"mla shared tiles Hq={Hq} f8={f8} {name}")
+        b = wl.make_mla_batch("mla_shared_" + name, q_lens, kv_lens, seed=430 + Hq, sliding_window=window, **kw)
+        wl.plant_mla_needles(b, seed=6)
+        want = ref(b)
+        T = sum(q_lens)
+        shared = run_gpu(pkg, b, gpu)[:T]
+        monkeypatch.setenv("RPA_MLA_SHARED_TILES", "0")
+        single = run_gpu(pkg, b, gpu)[:T]
+        monkeypatch.delenv("RPA_MLA_SHARED_TILES")
+        assert_parity(shared.float(), want.float(), **TOL)
+        assert_parity(single.float(), want.float(), **TOL)
+        assert torch.equal(shared, run_gpu(pkg, b, gpu)[:T])
+
+
 @pytest.mark.parametrize("window,cap", [(128, None), (None, 30.0), (128, 30.0)])
 def test_mla_window_and_soft_cap(pkg, wl, gpu, window, cap):
     kv_lens = [100, 128, 129, 700]
