@@ -52,6 +52,7 @@ DECODE_KERNEL = {
     "c4swa": "rpa_decode_splitkv_kernel",
     "c5": "rpa_mla_balanced_wide_kernel",
     "c5fp8": "rpa_mla_balanced_kernel",
+    "c5tp8": "rpa_mla_balanced_kernel (shared tiles)",
 }
 
 PREFILL_KERNEL = "rpa_prefill_pipe_kernel"
@@ -363,9 +364,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5", "c5fp8", "c5p"],
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5", "c5fp8", "c5tp8", "c5p"],
                     help="c5p: absorbed-MLA prefill chunks (512 tokens on 4096-token prefixes), DeepSeek-V3 shape; "
-                         "c5fp8: C5 on an e4m3 latent cache")
+                         "c5fp8: C5 on an e4m3 latent cache; c5tp8: C5 with 16 of the 128 heads (one GPU's share at tensor-parallel 8)")
     ap.add_argument("--all", action="store_true", help="(default) also time the other configurations")
     ap.add_argument("--main-only", action="store_true", help="skip the other configurations")
     ap.add_argument("--reference-suite", action="store_true",
@@ -406,11 +407,12 @@ def main():
         return {"c1": lambda: wl.config_c1(dev), "c2": lambda: wl.config_c2(dev), "c3": lambda: wl.config_c3(dev),
                 "c4": lambda: wl.config_c4(dev), "c4swa": lambda: wl.config_c4(dev, window=True),
                 "c5": lambda: wl.config_c5(dev), "c5p": lambda: wl.config_c5_prefill(dev),
-                "c5fp8": lambda: wl.config_c5(dev, kv_dtype=torch.float8_e4m3fn)}[name]()
+                "c5fp8": lambda: wl.config_c5(dev, kv_dtype=torch.float8_e4m3fn),
+                "c5tp8": lambda: wl.config_c5(dev, num_q_heads=16)}[name]()
 
     def run(name, keep=False):
         b = build(name)
-        if name in ("c5", "c5p", "c5fp8"):
+        if name in ("c5", "c5p", "c5fp8", "c5tp8"):
             r = run_mla_config(pkg, wl, b, args.steps, args.warmup)
         elif keep:
             r, call = run_rpa_config(pkg, wl, b, args.steps, args.warmup, keep_call=True,
@@ -434,7 +436,7 @@ def main():
                 "frac_back_to_back": (res["decode_gbps_back_to_back"] / HBM_PEAK_GBPS
                                       if "decode_gbps_back_to_back" in res else None)}
 
-    if args.config in ("c5", "c5p", "c5fp8"):
+    if args.config in ("c5", "c5p", "c5fp8", "c5tp8"):
         main_res, sample = run(args.config), None
     else:
         main_res, sample = run(args.config, keep=True)
@@ -473,7 +475,7 @@ def main():
     }
     if not args.main_only:
         others = {}
-        for name in ("c1", "c2", "c3", "c4", "c4swa", "c5", "c5fp8", "c5p"):
+        for name in ("c1", "c2", "c3", "c4", "c4swa", "c5", "c5fp8", "c5tp8", "c5p"):
             if name == args.config:
                 continue
             r = run(name)
@@ -485,7 +487,7 @@ def main():
                 others[name] = r
                 continue
             r["roofline"] = decode_roofline(name, r)
-            if name in ("c5", "c5fp8"):
+            if name in ("c5", "c5fp8", "c5tp8"):
                 r["roofline"]["mfma_frac"] = r["tflops"] / MFMA_BF16_PEAK_TFLOPS
             if "prefill_tflops" in r:
                 r["roofline_prefill"] = {"kernel": PREFILL_KERNEL, "bound": "mfma", "achieved": r["prefill_tflops"],

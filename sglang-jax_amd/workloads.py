@@ -311,7 +311,8 @@ def config_c5(device="cpu", scale: float = 1.0, num_q_heads: int = 128, kv_dtype
     rng = np.random.Generator(np.random.PCG64(seed))
     S = 64
     kv = rng.integers(_scaled(2048, scale), _scaled(16384, scale), size=S, endpoint=True)
-    name = "c5_deepseek_v3_mla_decode" + ("" if kv_dtype == torch.bfloat16 else "_fp8")
+    name = ("c5_deepseek_v3_mla_decode" + ("" if kv_dtype == torch.bfloat16 else "_fp8") +
+            ("" if num_q_heads == 128 else f"_{num_q_heads}_heads"))
     return make_mla_batch(name, np.ones(S, int), kv, num_q_heads=num_q_heads,
                           lkv_dim=512, rope_dim=64, page_size=64, seed=seed, device=device,
                           sm_scale=1.0 / math.sqrt(192.0), kv_dtype=kv_dtype)
