@@ -465,9 +465,12 @@ inline int kv_pieces(const PrefillArgs& a, int nseq, int bm, int heads, double t
     const double rate = w <= 192 ? 1.0 : w <= 512 ? 1.0 + (w - 192) * (1.6 / 320) : 2.6 * (w / 512);
     return tile_us * rate * chain / n + (n > 1 ? 1.5 + per_piece * n : 0.0);
   };
+  // (and the partial rows stay under 256 MB)
+  const int64_t row_bytes = (int64_t)a.num_tokens * a.Hq * (a.head_dim + 2) * 4;
+  const int64_t cap_ws = row_bytes > 0 ? ((int64_t)256 << 20) / row_bytes : 64;
   int best = 1;
   double best_us = launch_us(1) - 2.0;
-  for (int n = 2; n <= cap; ++n) {
+  for (int n = 2; n <= cap && n <= cap_ws; ++n) {
     const double us = launch_us(n);
     if (us < best_us) {
       best_us = us;
