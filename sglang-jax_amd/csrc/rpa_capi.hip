@@ -626,7 +626,7 @@ PrefillWorkspace prefill_workspace(const RpaParams* p, const rpa::PrefillArgs& a
   w.splits = rpa::prefill_kv_splits(a);
   w.split_bytes = rpa::prefill_split_workspace_bytes(a, w.splits);
   w.bits_offset = (w.split_bytes + 255) & ~(size_t)255;
-  if (p->mask_mode == RPA_MASK_CUSTOM && p->head_dim == 128 && !p->distribution && p->max_kv_len > 0 && p->num_tokens > 0 &&
+  if (p->mask_mode == RPA_MASK_CUSTOM && p->head_dim == 128 && p->max_kv_len > 0 && p->num_tokens > 0 &&
       env_int("RPA_MASK_BITS", 1) != 0) {
     w.pitch = (p->max_kv_len + 63) / 64;
     w.bits_bytes = (size_t)p->num_tokens * w.pitch * sizeof(uint64_t);

@@ -554,9 +554,12 @@ __device__ __forceinline__ int mask_owner_of_token(const int32_t* cu_q_lens, int
 }
 
 __global__ __launch_bounds__(256) void rpa_mask_bits_kernel(const PrefillArgs a) {
+  // (masked calls run every sequence through the prefill kernels; with the composition on the device the number
+  // of sequences is only a bound)
+  const int seq_end = a.dist ? min(a.seq_end, a.dist[2]) : a.seq_end;
   const int token = a.pt.cu_q_lens[a.seq_begin] + (int)blockIdx.x;
-  if (token >= a.pt.cu_q_lens[a.seq_end]) return;
-  const int seq = mask_owner_of_token(a.pt.cu_q_lens, a.seq_end, token);
+  if (token >= a.pt.cu_q_lens[seq_end]) return;
+  const int seq = mask_owner_of_token(a.pt.cu_q_lens, seq_end, token);
   const int kv_len = a.pt.kv_lens[seq];
   const int width = a.sm.mask_rows_page_aligned ? (a.pt.cu_kv_lens[seq + 1] - a.pt.cu_kv_lens[seq]) : kv_len;
   const int32_t* row = a.sm.custom_mask + a.sm.cu_mask_lens[seq] + (int64_t)(token - a.pt.cu_q_lens[seq]) * width;

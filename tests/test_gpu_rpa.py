@@ -1269,6 +1269,17 @@ def test_custom_mask_as_bits_equals_the_callers_words(pkg, wl, gpu, monkeypatch,
         bits = gpu_out(pkg, b, gpu, **kw)
         assert torch.equal(bits, words)
         assert_parity(bits.float(), oracle_out(b, causal=False, custom_mask=want_masks).float(), **(FP8_TOL if fp8 else BF16_TOL))
+        # the composition on the device (the jitted caller's mode): the pre-pass reads the number of sequences there
+        g = b.to(gpu)
+        out, _ = pkg.ragged_paged_attention(
+            g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+            b.distribution.to(torch.int32).to(gpu), cm.to(gpu), sm_scale=b.sm_scale, sliding_window=window, k_scale=g.k_scale,
+            v_scale=g.v_scale, causal=0, mask_aligned_to_cu_kv=aligned, max_kv_len=max(kv_lens), max_q_len=max(q_lens))
+        torch.cuda.synchronize()
+        monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")  # (that mode never cuts K/V ranges into pieces)
+        whole = gpu_out(pkg, b, gpu, **kw)
+        monkeypatch.delenv("RPA_PREFILL_SPLITS")
+        assert torch.equal(out[: sum(q_lens)].cpu(), whole)
 
 
 @pytest.mark.parametrize("kind", ["soft_cap", "xai_temperature", "custom_mask", "no_mask", "softmax_bf16", "fp8", "fp8_custom_mask"])
