@@ -343,8 +343,11 @@ constexpr float kNoReference = -1.0e30f;  // reference of a row that met no visi
 __device__ __forceinline__ bool kv_piece(const PrefillArgs& a, int& t_lo, int& t_hi, int& split) {
   split = blockIdx.y;
   const int nT = (t_hi - t_lo + kBN - 1) / kBN;
+  // The host chose the number of pieces for the longest range it knew a bound of; a shorter range is cut into
+  // fewer (no piece under four tiles), the workgroups of the others leave rows that weigh nothing.
+  const int pieces = max(1, min(a.kv_splits, nT >> 2));
   // (the division runs on the vector pipe: say that its result is the same in every lane)
-  const int per = __builtin_amdgcn_readfirstlane((nT + a.kv_splits - 1) / a.kv_splits);
+  const int per = __builtin_amdgcn_readfirstlane((nT + pieces - 1) / pieces);
   const int lo = split * per, hi = min(nT, lo + per);
   if (lo >= hi) return false;
   t_hi = min(t_hi, t_lo + hi * kBN);
@@ -388,8 +391,14 @@ template <int HD>
 __global__ __launch_bounds__(64) void rpa_prefill_combine_kernel(const PrefillArgs a) {
   constexpr int kDpl = HD / 64;
   typedef float fvec_t __attribute__((ext_vector_type(kDpl)));
-  const int tok0 = scalar_load_i32(a.pt.cu_q_lens + a.seq_begin);
-  const int tok1 = scalar_load_i32(a.pt.cu_q_lens + a.seq_end);
+  // (with the call's composition on the device the sequences to process are read there, as in the kernels)
+  int seq_begin = a.seq_begin, seq_end = a.seq_end;
+  if (a.dist) {
+    seq_begin = (a.sm.mask_mode == 1) ? 0 : scalar_load_i32(a.dist);
+    seq_end = min(seq_end, scalar_load_i32(a.dist + 2));
+  }
+  const int tok0 = scalar_load_i32(a.pt.cu_q_lens + seq_begin);
+  const int tok1 = scalar_load_i32(a.pt.cu_q_lens + seq_end);
   const int token = tok0 + (int)blockIdx.x;
   if (token >= tok1) return;
   const int head = blockIdx.y, lane = threadIdx.x, n = a.kv_splits;
@@ -447,7 +456,9 @@ inline hipError_t launch_prefill_combine(const PrefillArgs& a, hipStream_t strea
 // leaves no piece under four tiles and makes at most 64 pieces.  bm / heads: query positions and query heads
 // per workgroup.  RPA_PREFILL_SPLITS: 0 / 1 never, n forces n (read per call).
 inline int kv_pieces(const PrefillArgs& a, int nseq, int bm, int heads, double tile_us) {
-  if (a.dist || nseq <= 0 || a.max_q_len <= 0 || a.max_kv_len <= 0 || a.num_tokens <= 0) return 1;
+  // (with the composition on the device nseq, max_q_len, max_kv_len and num_tokens are bounds: a launch that is
+  // under-filled even by its bounds is cut, and every workgroup fits the piece count to its own range)
+  if (nseq <= 0 || a.max_q_len <= 0 || a.max_kv_len <= 0 || a.num_tokens <= 0) return 1;
   const char* env = getenv("RPA_PREFILL_SPLITS");
   const int forced = env ? atoi(env) : -1;
   if (forced == 0 || forced == 1) return 1;

@@ -197,11 +197,13 @@ def test_workspace_for_prefill_launches_that_leave_the_gpu_idle(pkg, monkeypatch
     p.max_kv_len = 0  # no bound on the lengths: no cut
     assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
     p = params(512, 8, 2, 16384)
-    p.distribution = 0x1000  # composition on the device: no cut, only what the decode plan of such a call asks for
-    dyn = lib.rpa_workspace_bytes(ctypes.byref(p))
+    p.distribution = 0x1000  # composition on the device: the same rule on the bounds (every workgroup fits the count to its range)
+    monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
+    dyn = lib.rpa_workspace_bytes(ctypes.byref(p))  # what the decode plan of such a call asks for
     monkeypatch.setenv("RPA_PREFILL_SPLITS", "7")
-    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == dyn
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == max(dyn, 512 * 8 * 7 * row)
     monkeypatch.delenv("RPA_PREFILL_SPLITS")
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == max(dyn, need)
     p = params(2048, 32, 8, 8192)  # 512 workgroups: the GPU is full
     assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
     p = params(1000, 8, 4, 1000)  # a short range: the merge would cost what the cut saves

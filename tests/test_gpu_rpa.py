@@ -1271,15 +1271,21 @@ def test_custom_mask_as_bits_equals_the_callers_words(pkg, wl, gpu, monkeypatch,
         assert_parity(bits.float(), oracle_out(b, causal=False, custom_mask=want_masks).float(), **(FP8_TOL if fp8 else BF16_TOL))
         # the composition on the device (the jitted caller's mode): the pre-pass reads the number of sequences there
         g = b.to(gpu)
-        out, _ = pkg.ragged_paged_attention(
-            g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
-            b.distribution.to(torch.int32).to(gpu), cm.to(gpu), sm_scale=b.sm_scale, sliding_window=window, k_scale=g.k_scale,
-            v_scale=g.v_scale, causal=0, mask_aligned_to_cu_kv=aligned, max_kv_len=max(kv_lens), max_q_len=max(q_lens))
-        torch.cuda.synchronize()
-        monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")  # (that mode never cuts K/V ranges into pieces)
+
+        def on_device():
+            out, _ = pkg.ragged_paged_attention(
+                g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+                b.distribution.to(torch.int32).to(gpu), cm.to(gpu), sm_scale=b.sm_scale, sliding_window=window,
+                k_scale=g.k_scale, v_scale=g.v_scale, causal=0, mask_aligned_to_cu_kv=aligned, max_kv_len=max(kv_lens),
+                max_q_len=max(q_lens))
+            torch.cuda.synchronize()
+            return out[: sum(q_lens)].cpu()
+
+        assert_parity(on_device().float(), bits.float(), **(FP8_TOL if fp8 else BF16_TOL))  # (K/V pieces chosen from bounds)
+        monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
         whole = gpu_out(pkg, b, gpu, **kw)
+        assert torch.equal(on_device(), whole)
         monkeypatch.delenv("RPA_PREFILL_SPLITS")
-        assert torch.equal(out[: sum(q_lens)].cpu(), whole)
 
 
 @pytest.mark.parametrize("kind", ["soft_cap", "xai_temperature", "custom_mask", "no_mask", "softmax_bf16", "fp8", "fp8_custom_mask"])
@@ -1324,3 +1330,32 @@ def test_short_chunks_take_the_four_head_tile_in_the_compiled_kernel(pkg, wl, gp
         assert_parity(big.float(), want.float(), **tol)
         assert torch.equal(auto, small)  # every chunk here is at most 64 tokens long
         assert float(row_rel_error(small.float(), big.float()).max()) < (3e-2 if fp8 else 1e-2)
+
+
+def test_kv_range_pieces_with_the_composition_on_the_device(pkg, wl, gpu, monkeypatch):
+    """The jitted caller's mode: only bounds on the host (padded sequence slots, the longest context the page table
+    allows).  A launch that is under-filled even by its bounds is cut, and every workgroup fits the piece count to
+    its own range (no piece under four tiles): a verify step and a chunk whose real lengths are far below the
+    bounds, against the oracle and against whole ranges."""
+    for q_lens, kv_lens, bound in (([16, 16], [9000, 300], 32768), ([1, 1, 200], [700, 40, 1300], 16384)):
+        say(f"pieces, composition on the device: q={q_lens} kv={kv_lens} bound={bound}")
+        b = wl.make_batch("pieces_on_device", q_lens, kv_lens, num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=64, seed=97)
+        wl.plant_needles(b, seed=4)
+        want = oracle_out(b)
+        g = b.to(gpu)
+        T = sum(q_lens)
+
+        def run():
+            out, _ = pkg.ragged_paged_attention(
+                g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+                b.distribution.to(torch.int32).to(gpu), None, sm_scale=b.sm_scale, max_kv_len=bound, max_q_len=max(q_lens))
+            torch.cuda.synchronize()
+            return out[:T].cpu()
+
+        cut = run()
+        monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
+        whole = run()
+        monkeypatch.delenv("RPA_PREFILL_SPLITS")
+        assert_parity(cut.float(), want.float(), **BF16_TOL)
+        assert_parity(whole.float(), want.float(), **BF16_TOL)
+        assert not torch.equal(cut, whole), "the bounds were expected to cut this launch"
