@@ -18,8 +18,17 @@ One JSON line is printed:
   parity_sample  a few rows of the timed output against the CPU oracle (outside the timed region)
   other_configs  the remaining configurations (C1, C3, C4, C4 windowed, C5), each with its kernel,
               average / median / minimum launch time, algorithmic bytes or FLOPs and roofline fraction
-              (--main-only skips them)
+              (--main-only skips them); roofline.configs repeats kernel time and fractions of each, compactly
+  ceilings    what this device delivers to the simplest kernels of the same shape, measured in this run: a
+              streaming read (contiguous and through a random table of 256 KiB pages) and a matrix-instruction
+              issue loop at two waves per SIMD; every roofline object carries frac (of the published peak) and
+              frac_of_achievable (of these)
+  settle_ms   untimed steps of the same workload run before the warm-up so that the device's clocks have
+              left their idle state when the W warm-up and K timed steps start (--settle-ms 0 switches it off)
   cpu_baseline  the CPU oracle timed on this box's host cores on a bounded sample
+
+The reference's published perf-guard workloads (32 rows) go to stderr as a JSON line of their own; the line on
+stdout keeps their summary.
 """
 
 from __future__ import annotations
@@ -78,9 +87,34 @@ def _stats(ms):
     return {"mean": sum(ms) / n, "median": ms[n // 2] if n % 2 else 0.5 * (ms[n // 2 - 1] + ms[n // 2]), "min": ms[0]}
 
 
-def time_partitions(call, steps, warmup, has_decode, has_prefill):
-    """W warm-up steps, then exactly `steps` timed steps; returns wall ms per step and
-    mean / median / min of the event-timed duration of each partition inside the timed region."""
+def settle(step, ms):
+    """Untimed steps for about `ms` milliseconds of wall time (at most 2000 steps): a device that starts from
+    idle runs its first milliseconds at other clocks than the rest.  Returns what it did."""
+    import torch
+
+    if ms <= 0:
+        return {"ms": 0.0, "steps": 0}
+    torch.cuda.synchronize()
+    t0, n = time.perf_counter(), 0
+    while (time.perf_counter() - t0) * 1e3 < ms and n < 2000:
+        for _ in range(5):
+            step()
+        n += 5
+        torch.cuda.synchronize()
+    return {"ms": (time.perf_counter() - t0) * 1e3, "steps": n}
+
+
+def _series(ms):
+    """Per-step durations of the timed region in microseconds, in step order, with the means of the first and
+    the last quarter: a drift over the region (clocks, caches) shows here."""
+    q = max(1, len(ms) // 4)
+    return {"us": [round(x * 1e3, 1) for x in ms], "first_quarter_mean_us": sum(ms[:q]) / q * 1e3,
+            "last_quarter_mean_us": sum(ms[-q:]) / q * 1e3}
+
+
+def time_partitions(call, steps, warmup, has_decode, has_prefill, settle_ms=0.0):
+    """`settle_ms` of untimed steps, W warm-up steps, then exactly `steps` timed steps; returns wall ms per
+    step and mean / median / min of the event-timed duration of each partition inside the timed region."""
     import torch
 
     def one(ev=None):
@@ -95,6 +129,7 @@ def time_partitions(call, steps, warmup, has_decode, has_prefill):
         if ev is not None:
             ev[2].record()
 
+    settled = settle(one, settle_ms)
     for _ in range(warmup):
         one()
     evs = [_events(3) for _ in range(steps)]
@@ -104,8 +139,11 @@ def time_partitions(call, steps, warmup, has_decode, has_prefill):
         one(evs[i])
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    dec = _stats([e[0].elapsed_time(e[1]) for e in evs])
-    pre = _stats([e[1].elapsed_time(e[2]) for e in evs])
+    dec_ms = [e[0].elapsed_time(e[1]) for e in evs]
+    pre_ms = [e[1].elapsed_time(e[2]) for e in evs]
+    dec, pre = _stats(dec_ms), _stats(pre_ms)
+    dec["series"], pre["series"] = _series(dec_ms), _series(pre_ms)
+    dec["settle"] = pre["settle"] = settled
     # After the timed region: each partition again as `steps` launches in a row between ONE pair of
     # events.  An event recorded between two kernels is a packet of its own that the next kernel
     # waits for, so the per-step figures above carry a few microseconds of the measurement itself;
@@ -147,11 +185,16 @@ def make_call(pkg, b, static_shapes=False):
                      sum_decode_kv_len=int(sum(b.meta["kv_lens"][:dec_end])))
 
 
-def run_rpa_config(pkg, wl, b, steps, warmup, keep_call=False, static_shapes=False):
+def run_rpa_config(pkg, wl, b, steps, warmup, keep_call=False, static_shapes=False, settle_ms=0.0, series=False):
     dec_end, n = int(b.distribution[0]), int(b.distribution[2])
     call = make_call(pkg, b, static_shapes)
-    ms, dec, pre = time_partitions(call, steps, warmup, dec_end > 0, n > dec_end)
-    res = {"workload": b.name, "ms_per_step": ms}
+    ms, dec, pre = time_partitions(call, steps, warmup, dec_end > 0, n > dec_end, settle_ms)
+    res = {"workload": b.name, "ms_per_step": ms, "settle": dec["settle"]}
+    if series:
+        if dec_end > 0:
+            res["decode_series"] = dec["series"]
+        if n > dec_end:
+            res["prefill_series"] = pre["series"]
     if dec_end > 0:
         nbytes = wl.decode_bytes(b, 0, dec_end)
         res.update(decode_ms=dec["mean"], decode_ms_median=dec["median"], decode_ms_min=dec["min"], decode_bytes=nbytes,
@@ -192,7 +235,7 @@ def parity_sample(wl, b, call):
             "max_row_rel_err": float(rel), "tolerance": "rtol = atol = 2e-2 (5e-2 fp8 KV), row-relative 1e-2 (3e-2)"}
 
 
-def run_mla_config(pkg, wl, b, steps, warmup):
+def run_mla_config(pkg, wl, b, steps, warmup, settle_ms=0.0):
     import torch
 
     n = int(b.distribution[2])
@@ -203,6 +246,7 @@ def run_mla_config(pkg, wl, b, steps, warmup):
         pkg.mla_ragged_paged_attention(b.ql_nope, b.q_pe, None, None, b.cache_kv, b.kv_lens, b.page_indices,
                                        b.cu_q_lens, b.cu_kv_lens, dist, **kw)
 
+    settled = settle(one, settle_ms)
     for _ in range(warmup):
         one()
     evs = [_events(2) for _ in range(steps)]
@@ -218,10 +262,10 @@ def run_mla_config(pkg, wl, b, steps, warmup):
     ms = st["mean"]
     if any(q != 1 for q in b.meta["q_lens"]):  # prefill chunks: a FLOP figure, no decode bytes
         flops = wl.mla_attention_flops(b)
-        return {"workload": b.name, "ms_per_step": (t1 - t0) * 1e3 / steps, "prefill_ms": ms, "prefill_ms_median": st["median"],
+        return {"workload": b.name, "ms_per_step": (t1 - t0) * 1e3 / steps, "settle": settled, "prefill_ms": ms, "prefill_ms_median": st["median"],
                 "prefill_ms_min": st["min"], "prefill_flops": flops, "prefill_tflops": flops / (ms * 1e-3) / 1e12}
     nbytes, flops = wl.mla_decode_bytes(b), wl.mla_decode_flops(b)
-    return {"workload": b.name, "ms_per_step": (t1 - t0) * 1e3 / steps, "decode_ms": ms, "decode_ms_median": st["median"],
+    return {"workload": b.name, "ms_per_step": (t1 - t0) * 1e3 / steps, "settle": settled, "decode_ms": ms, "decode_ms_median": st["median"],
             "decode_ms_min": st["min"], "decode_bytes": nbytes, "decode_gbps": nbytes / (ms * 1e-3) / 1e9,
             "tflops": flops / (ms * 1e-3) / 1e12}
 
@@ -309,6 +353,81 @@ def reference_suite(pkg, wl, dev, reps=50):
     return rows
 
 
+def measure_ceilings(dev, nbytes=2 << 30, reps=5):
+    """What this device delivers to the simplest kernels of the attention kernels' shape (csrc/rpa_ceilings.hip,
+    lib/librpa_ceilings.so), event-timed on the current stream:
+      * a streaming read of `nbytes` of random data, every wave sixteen 16-byte loads per lane in flight, over
+        wave counts from the decode plan's (3.5 per CU) to 32 per CU, contiguous and through a random table of
+        256 KiB pages (one page = 64 tokens of 8 kv heads x 128 dims, bf16 K and V), each wave on a contiguous
+        run of blocks or the waves interleaved block by block;
+      * v_mfma_f32_32x32x16_bf16 into four independent accumulators, two waves per SIMD.
+    `achievable` holds the best of each: the denominators of frac_of_achievable."""
+    import ctypes
+
+    import torch
+
+    path = os.path.join(ROOT, "sglang-jax_amd", "lib", "librpa_ceilings.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is not built: run __graft_entry__.build()")
+    lib = ctypes.CDLL(path)
+    lib.rpa_ceiling_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64,
+                                            ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    lib.rpa_ceiling_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    page_bytes = 256 << 10
+    src = torch.empty(nbytes // 8, dtype=torch.int64, device=dev).random_()
+    table = torch.randperm(nbytes // page_bytes, generator=torch.Generator().manual_seed(7)).to(torch.int32).to(dev)
+    sink = torch.zeros(64, dtype=torch.int32, device=dev)
+
+    def timed(launch, n):
+        for _ in range(2):
+            launch()
+        a, b = _events(2)
+        a.record()
+        for _ in range(n):
+            launch()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n
+
+    rows = []
+    plan_waves = cus * 4 - cus // 2  # the decode plan's resident waves on 16-bit caches
+    for waves in (plan_waves, cus * 4, cus * 8, cus * 16, cus * 32):
+        for order in (0, 1):
+            for paged in (False, True):
+                def launch():
+                    rc = lib.rpa_ceiling_stream_read(src.data_ptr(), nbytes, table.data_ptr() if paged else None, page_bytes,
+                                                     waves, order, sink.data_ptr(), stream)
+                    if rc != 0:
+                        raise RuntimeError(f"rpa_ceiling_stream_read: hip error {rc}")
+                ms = timed(launch, reps)
+                rows.append({"waves": waves, "order": "contiguous runs" if order == 0 else "interleaved", "paged": paged,
+                             "ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9})
+    iters = 2000
+    wgs = 2 * cus
+
+    def launch_mfma():
+        rc = lib.rpa_ceiling_mfma(wgs, iters, sink.data_ptr(), stream)
+        if rc != 0:
+            raise RuntimeError(f"rpa_ceiling_mfma: hip error {rc}")
+    mfma_ms = timed(launch_mfma, reps)
+    mfma_tflops = wgs * 4 * iters * 16 * 32768 / (mfma_ms * 1e-3) / 1e12
+    best = lambda paged, waves=None: max(r["gbps"] for r in rows if r["paged"] == paged and (waves is None or r["waves"] == waves))
+    del src, table
+    torch.cuda.empty_cache()
+    return {
+        "what": "streaming read of %d MiB (16 KiB per wave in flight) and a v_mfma_f32_32x32x16_bf16 issue loop at two "
+                "waves per SIMD, measured in this run" % (nbytes >> 20),
+        "achievable": {"hbm_read_gbps_contiguous": best(False), "hbm_read_gbps_paged_256KiB": best(True),
+                       "hbm_read_gbps_paged_at_decode_plan_waves": best(True, plan_waves),
+                       "mfma_bf16_tflops": mfma_tflops},
+        "frac_of_published_peak": {"hbm_contiguous": best(False) / HBM_PEAK_GBPS, "hbm_paged": best(True) / HBM_PEAK_GBPS,
+                                   "mfma_bf16": mfma_tflops / MFMA_BF16_PEAK_TFLOPS},
+        "mfma_loop_ms": mfma_ms, "stream_read": rows,
+    }
+
+
 def cpu_baseline(wl, budget_s=10.0, prefill_budget_s=8.0):
     """CPU oracle on a bounded sample of the default workload: its first decode rows
     (same seeded lengths and layout, values drawn on the host), and -- reported under `prefill` -- one
@@ -375,6 +494,13 @@ def main():
                     help="run the main configuration with the batch composition read on the device (grids sized "
                          "from static shapes only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="untimed steps of the same workload for this many milliseconds before the warm-up (reported "
+                         "as settle_ms; 0 = none): the first milliseconds after idle run at other clocks")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="only measure what the device delivers to a plain streaming read and to a matrix-instruction "
+                         "issue loop (the denominators of frac_of_achievable) and print them")
+    ap.add_argument("--no-ceilings", action="store_true", help="skip those measurements (no frac_of_achievable)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy (10 launches): the known-size kernel "
                          "against which rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled")
@@ -403,6 +529,24 @@ def main():
         print(json.dumps({"copy_calibration_bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4, "launches": 10}))
         return
 
+    if args.ceilings:
+        print(json.dumps({"ceilings": measure_ceilings(dev, reps=10)}))
+        return
+    ceilings = None if args.no_ceilings else measure_ceilings(dev)
+
+    def achievable(bound):
+        if ceilings is None:
+            return None
+        return ceilings["achievable"]["hbm_read_gbps_paged_256KiB" if bound == "hbm" else "mfma_bf16_tflops"]
+
+    def with_achievable(r):
+        """frac_of_achievable next to frac: the same figure against what a plain kernel reaches on this device"""
+        top = achievable(r["bound"])
+        r["frac_of_achievable"] = None if top is None else r["achieved"] / top
+        if r.get("frac_back_to_back") is not None and top is not None:
+            r["frac_of_achievable_back_to_back"] = r["frac_back_to_back"] * r["peak"] / top
+        return r
+
     def build(name):
         return {"c1": lambda: wl.config_c1(dev), "c2": lambda: wl.config_c2(dev), "c3": lambda: wl.config_c3(dev),
                 "c4": lambda: wl.config_c4(dev), "c4swa": lambda: wl.config_c4(dev, window=True),
@@ -413,14 +557,14 @@ def main():
     def run(name, keep=False):
         b = build(name)
         if name in ("c5", "c5p", "c5fp8", "c5tp8"):
-            r = run_mla_config(pkg, wl, b, args.steps, args.warmup)
+            r = run_mla_config(pkg, wl, b, args.steps, args.warmup, settle_ms=args.settle_ms)
         elif keep:
             r, call = run_rpa_config(pkg, wl, b, args.steps, args.warmup, keep_call=True,
-                                     static_shapes=args.static_shapes)
+                                     static_shapes=args.static_shapes, settle_ms=args.settle_ms, series=True)
             r = (r, parity_sample(wl, b, call))
             del call
         else:
-            r = run_rpa_config(pkg, wl, b, args.steps, args.warmup)
+            r = run_rpa_config(pkg, wl, b, args.steps, args.warmup, settle_ms=args.settle_ms)
         del b
         torch.cuda.empty_cache()
         return r
@@ -443,28 +587,36 @@ def main():
     dec_gbps = main_res.get("decode_gbps")
     pre_tflops = main_res.get("prefill_tflops")
     # dominant kernel of the workload (largest average launch time inside the timed region)
-    roofline_decode = decode_roofline(args.config, main_res) if dec_gbps is not None else None
+    roofline_decode = with_achievable(decode_roofline(args.config, main_res)) if dec_gbps is not None else None
     prefill_kernel = "rpa_mla_decode_wide_kernel (one row per query token)" if args.config == "c5p" else PREFILL_KERNEL
+
+    def prefill_roofline(name, res, kernel):
+        return with_achievable({
+            "kernel": kernel, "bound": "mfma", "achieved": res["prefill_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": res["prefill_tflops"] / MFMA_BF16_PEAK_TFLOPS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((name, kernel)), "avg_launch_ms": res["prefill_ms"],
+            "median_launch_ms": res["prefill_ms_median"], "min_launch_ms": res["prefill_ms_min"],
+            "flops_per_launch": res["prefill_flops"], "back_to_back_launch_ms": res.get("prefill_ms_back_to_back"),
+            "frac_back_to_back": (res["prefill_tflops_back_to_back"] / MFMA_BF16_PEAK_TFLOPS
+                                  if "prefill_tflops_back_to_back" in res else None)})
+
+    roofline_prefill = prefill_roofline(args.config, main_res, prefill_kernel) if pre_tflops is not None else None
     if pre_tflops is not None and main_res.get("prefill_ms", 0) >= main_res.get("decode_ms", 0):
-        roofline = {"kernel": prefill_kernel, "bound": "mfma", "achieved": pre_tflops,
-                    "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": pre_tflops / MFMA_BF16_PEAK_TFLOPS,
-                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, prefill_kernel)),
-                    "avg_launch_ms": main_res["prefill_ms"], "median_launch_ms": main_res["prefill_ms_median"],
-                    "min_launch_ms": main_res["prefill_ms_min"], "flops_per_launch": main_res["prefill_flops"],
-                    "back_to_back_launch_ms": main_res.get("prefill_ms_back_to_back"),
-                    "frac_back_to_back": (main_res["prefill_tflops_back_to_back"] / MFMA_BF16_PEAK_TFLOPS
-                                          if "prefill_tflops_back_to_back" in main_res else None)}
+        roofline = dict(roofline_prefill)
     else:
-        roofline = roofline_decode
+        roofline = dict(roofline_decode)
     line = {
         "metric": "ragged paged attn: decode HBM GB/s (% of peak), prefill TFLOP/s; 1 MI355X",
         "value": dec_gbps if dec_gbps is not None else pre_tflops,
         "unit": "GB/s" if dec_gbps is not None else "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
+        "settle_ms": main_res["settle"]["ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.config not in ("c4", "c4swa", "c5fp8") else "bf16 (fp8-e4m3 KV)", "data": "synthetic",
         "config": {"workload": main_res["workload"], "value_is": "decode partition (split-KV + combine) algorithmic bytes / time",
-                   "call_mode": "static shapes, composition read on the device" if args.static_shapes else "host integers"},
+                   "call_mode": "static shapes, composition read on the device" if args.static_shapes else "host integers",
+                   "settle": "%d untimed steps (%.0f ms) before the %d warm-up steps" % (
+                       main_res["settle"]["steps"], main_res["settle"]["ms"], args.warmup)},
         "decode_frac_of_hbm_peak": None if dec_gbps is None else dec_gbps / HBM_PEAK_GBPS,
         "prefill_tflops": pre_tflops,
         "prefill_frac_of_mfma_peak": None if pre_tflops is None else pre_tflops / MFMA_BF16_PEAK_TFLOPS,
@@ -472,7 +624,17 @@ def main():
         "roofline": roofline,
         "roofline_decode": roofline_decode,
         "parity_sample": sample,
+        "ceilings": ceilings,
     }
+    # every configuration's dominant kernel in one compact map inside `roofline`:
+    # name -> [kernel, bound, average launch ms, fraction of the published peak, fraction of the achievable]
+    compact = lambda r: [r["kernel"], r["bound"], round(r["avg_launch_ms"], 5), round(r["frac"], 4),
+                         None if r["frac_of_achievable"] is None else round(r["frac_of_achievable"], 4)]
+    configs = {}
+    if roofline_decode is not None:
+        configs[args.config + (" decode rows" if roofline_prefill is not None else "")] = compact(roofline_decode)
+    if roofline_prefill is not None:
+        configs[args.config + (" prefill rows" if roofline_decode is not None else "")] = compact(roofline_prefill)
     if not args.main_only:
         others = {}
         for name in ("c1", "c2", "c3", "c4", "c4swa", "c5", "c5fp8", "c5tp8", "c5p"):
@@ -480,27 +642,37 @@ def main():
                 continue
             r = run(name)
             if name == "c5p":
-                r["roofline"] = {"kernel": "rpa_mla_decode_wide_kernel (one row per query token)", "bound": "mfma",
-                                 "achieved": r["prefill_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                 "frac": r["prefill_tflops"] / MFMA_BF16_PEAK_TFLOPS, "avg_launch_ms": r["prefill_ms"],
-                                 "flops_per_launch": r["prefill_flops"]}
+                r["roofline"] = with_achievable({
+                    "kernel": "rpa_mla_decode_wide_kernel (one row per query token)", "bound": "mfma",
+                    "achieved": r["prefill_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": r["prefill_tflops"] / MFMA_BF16_PEAK_TFLOPS, "avg_launch_ms": r["prefill_ms"],
+                    "flops_per_launch": r["prefill_flops"]})
                 others[name] = r
+                configs[name] = compact(r["roofline"])
                 continue
-            r["roofline"] = decode_roofline(name, r)
+            r["roofline"] = with_achievable(decode_roofline(name, r))
+            configs[name + (" decode rows" if "prefill_tflops" in r else "")] = compact(r["roofline"])
             if name in ("c5", "c5fp8", "c5tp8"):
                 r["roofline"]["mfma_frac"] = r["tflops"] / MFMA_BF16_PEAK_TFLOPS
             if "prefill_tflops" in r:
-                r["roofline_prefill"] = {"kernel": PREFILL_KERNEL, "bound": "mfma", "achieved": r["prefill_tflops"],
-                                         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                         "frac": r["prefill_tflops"] / MFMA_BF16_PEAK_TFLOPS,
-                                         "avg_launch_ms": r["prefill_ms"], "flops_per_launch": r["prefill_flops"]}
+                r["roofline_prefill"] = prefill_roofline(name, r, PREFILL_KERNEL)
+                configs[name + " prefill rows"] = compact(r["roofline_prefill"])
             others[name] = r
         line["other_configs"] = others
+    roofline["configs"] = configs
+    roofline["configs_columns"] = ["kernel", "bound", "avg_launch_ms", "frac", "frac_of_achievable"]
     if args.reference_suite or not args.main_only:
+        rows = reference_suite(pkg, wl, dev)
+        what = ("the reference's published perf-guard workloads (bench_flashattention.py:264-328), device ms per op "
+                "with the new-token cache write, this GPU against its TPU v6e / v7 baselines")
+        # the 32 rows go to stderr as a line of their own: stdout holds the one line with the headline
+        print(json.dumps({"reference_suite": {"what": what, "rows": rows}}), file=sys.stderr)
+        v6 = [r["speedup_vs_v6e"] for r in rows if r["speedup_vs_v6e"] is not None]
+        v7 = [r["speedup_vs_v7"] for r in rows]
         line["reference_suite"] = {
-            "what": "the reference's published perf-guard workloads (bench_flashattention.py:264-328), device ms per op "
-                    "with the new-token cache write, this GPU against its TPU v6e / v7 baselines",
-            "rows": reference_suite(pkg, wl, dev)}
+            "what": what + "; the rows are on stderr", "workloads": len(rows),
+            "speedup_vs_v6e_min_max": [min(v6), max(v6)], "speedup_vs_v7_min_max": [min(v7), max(v7)],
+            "ahead_of_v6e": sum(x > 1 for x in v6), "ahead_of_v7": sum(x > 1 for x in v7)}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(line))

@@ -29,6 +29,14 @@ extern "C" {
 
 #define RPA_VERSION 100 /* 0.1.0 */
 
+/* The entry points below are the library's ONLY dynamic symbols: it is built with hidden default
+ * visibility, so nothing else of it can collide with, or be interposed by, a host process. */
+#if defined(__GNUC__) || defined(__clang__)
+#define RPA_API __attribute__((visibility("default")))
+#else
+#define RPA_API
+#endif
+
 typedef enum RpaStatus {
   RPA_OK = 0,
   RPA_EINVAL_SHAPE = -1,
@@ -204,24 +212,24 @@ typedef struct RpaMlaParams {
 } RpaMlaParams;
 
 /* Library version (RPA_VERSION of the build). */
-int rpa_version(void);
+RPA_API int rpa_version(void);
 
 /* Thread-local description of the last error returned on this thread. */
-const char* rpa_last_error(void);
+RPA_API const char* rpa_last_error(void);
 
 /*
  * Static contract check: static_validate_inputs,
  * ragged_paged_attention_v3.py:1314-1439 (3-D q, Hq % Hkv == 0,
  * sliding_window > 0, soft_cap != 0, ...).  Called by every entry point.
  */
-int rpa_validate(const RpaParams* p);
+RPA_API int rpa_validate(const RpaParams* p);
 
 /*
  * Value check on HOST copies of the metadata: dynamic_validate_inputs,
  * ragged_paged_attention_v3.py:1442-1487 (0 < q_len <= kv_len, page count and
  * page index ranges, distribution ordering).  Pointers are host memory.
  */
-int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t* page_indices,
+RPA_API int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t* page_indices,
                       int64_t num_page_indices, const int32_t* cu_q_lens,
                       const int32_t* cu_kv_lens, const int32_t* distribution);
 
@@ -233,8 +241,8 @@ int rpa_validate_host(const RpaParams* p, const int32_t* kv_lens, const int32_t*
  * that room when it is there and otherwise runs whole ranges and reads the mask's i32 words (slower,
  * same results to the tolerance of the path).
  */
-size_t rpa_workspace_bytes(const RpaParams* p);
-size_t rpa_mla_workspace_bytes(const RpaMlaParams* p);
+RPA_API size_t rpa_workspace_bytes(const RpaParams* p);
+RPA_API size_t rpa_mla_workspace_bytes(const RpaMlaParams* p);
 
 /*
  * Page-table gather of one sequence (the indexing expression
@@ -242,26 +250,26 @@ size_t rpa_mla_workspace_bytes(const RpaMlaParams* p);
  * ragged_paged_attention_v3.py:138-139).  Copies, bit for bit, the K rows and
  * V rows of sequence `seq` into k_out / v_out [kv_len, Hkv, D] (kv dtype).
  */
-int rpa_gather_pages(const RpaParams* p, int32_t seq, void* k_out, void* v_out,
+RPA_API int rpa_gather_pages(const RpaParams* p, int32_t seq, void* k_out, void* v_out,
                      int32_t max_tokens, void* stream);
 
 /*
  * Decode rows [0, decode_end): split-KV pass + combine pass.  Stands in for the
  * DECODE pallas_call of ragged_paged_attention_v3.py:2065-2072.
  */
-int rpa_decode(const RpaParams* p, void* stream);
+RPA_API int rpa_decode(const RpaParams* p, void* stream);
 
 /*
  * Prefill / mixed rows [decode_end, num_seqs): flash-style MFMA kernel.  Stands
  * in for the PREFILL and MIXED pallas_calls, ragged_paged_attention_v3.py:2074-2090.
  */
-int rpa_prefill(const RpaParams* p, void* stream);
+RPA_API int rpa_prefill(const RpaParams* p, void* stream);
 
 /*
  * Whole call: dispatch by distribution exactly as
  * ragged_paged_attention_v3.py:2060-2090 does (decode rows, then the rest).
  */
-int rpa_attention(const RpaParams* p, void* stream);
+RPA_API int rpa_attention(const RpaParams* p, void* stream);
 
 /*
  * rpa_attention for callers that cannot allocate device memory (code under HIP graph capture,
@@ -275,8 +283,8 @@ int rpa_attention(const RpaParams* p, void* stream);
  * calls on one GPU share the array: calls that overlap on one GPU (two streams, a graph replay next
  * to eager work) race on it; order them on one stream.
  */
-size_t rpa_noalloc_max_workspace_bytes(void);
-int rpa_attention_noalloc(const RpaParams* p, void* stream);
+RPA_API size_t rpa_noalloc_max_workspace_bytes(void);
+RPA_API int rpa_attention_noalloc(const RpaParams* p, void* stream);
 
 /*
  * Scatter the new K/V rows of every sequence into the paged cache: the fused
@@ -285,10 +293,10 @@ int rpa_attention_noalloc(const RpaParams* p, void* stream);
  * sequence i goes to position kv_len_i - q_len_i + j.  keys/values are
  * [T, Hkv, D] in the cache dtype.
  */
-int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void* stream);
+RPA_API int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void* stream);
 
 /* Absorbed-MLA decode, see RpaMlaParams: every sequence contributes exactly one query token. */
-int rpa_mla_decode(const RpaMlaParams* p, void* stream);
+RPA_API int rpa_mla_decode(const RpaMlaParams* p, void* stream);
 
 /*
  * Absorbed-MLA attention for any batch composition (decode, prefill chunks, mixed): the three
@@ -297,15 +305,15 @@ int rpa_mla_decode(const RpaMlaParams* p, void* stream);
  * Workspace: rpa_mla_attention_workspace_bytes(); max_kv_len / sum_kv_len bound, resp. sum, the
  * per-token visible lengths.
  */
-size_t rpa_mla_attention_workspace_bytes(const RpaMlaParams* p);
-int rpa_mla_attention(const RpaMlaParams* p, void* stream);
+RPA_API size_t rpa_mla_attention_workspace_bytes(const RpaMlaParams* p);
+RPA_API int rpa_mla_attention(const RpaMlaParams* p, void* stream);
 
 /*
  * Write the new latent rows into the paged cache: update_kv_cache of kernels/mla/v1/ref.py:56-105
  * (the fused cache update of kernels/mla/v2/kernel.py).  new_kv_c bf16 [T, lkv_dim], new_k_pe bf16
  * [T, rope_dim]; token j of sequence i goes to position kv_len_i - q_len_i + j.
  */
-int rpa_mla_kv_write(const RpaMlaParams* p, const void* new_kv_c, const void* new_k_pe, void* stream);
+RPA_API int rpa_mla_kv_write(const RpaMlaParams* p, const void* new_kv_c, const void* new_k_pe, void* stream);
 
 #ifdef __cplusplus
 }

@@ -18,6 +18,10 @@ LIB_PATH = os.path.join(OUT_DIR, "librpa_mi355.so")
 HASH_PATH = os.path.join(OUT_DIR, "librpa_mi355.srchash")
 
 SOURCES = ["rpa_capi.hip", "rpa_decode.hip", "rpa_prefill.hip", "rpa_prefill_pipe.hip", "rpa_mla.hip"]
+# bench.py's measurement kernels (a streaming read, a matrix-instruction issue loop): a library of their own,
+# so that the attention library carries nothing but the attention path
+CEILINGS_SOURCE = "rpa_ceilings.hip"
+CEILINGS_LIB_PATH = os.path.join(OUT_DIR, "librpa_ceilings.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -26,6 +30,9 @@ FLAGS = [
     "-fPIC",
     "-std=c++17",
     "-ffp-contract=fast",
+    # only the RPA_API entry points of include/rpa.h are dynamic symbols
+    "-fvisibility=hidden",
+    "-fvisibility-inlines-hidden",
     # never let the compiler form packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
@@ -68,10 +75,13 @@ def build(verbose: bool = False, extra_flags=()) -> str:
         return obj
 
     with ThreadPoolExecutor(max_workers=4) as pool:
-        objs = list(pool.map(compile_one, SOURCES))
-    tmp = LIB_PATH + ".tmp"
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp])
-    os.replace(tmp, LIB_PATH)
+        objs = list(pool.map(compile_one, SOURCES + [CEILINGS_SOURCE]))
+    ceil_obj = objs.pop()
+    for path, members in ((LIB_PATH, objs), (CEILINGS_LIB_PATH, [ceil_obj])):
+        tmp = path + ".tmp"
+        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *members, "-o", tmp])
+        os.replace(tmp, path)
+    objs.append(ceil_obj)
     if not extra_flags:
         with open(HASH_PATH, "w") as f:
             f.write(source_hash() + "\n")

@@ -388,7 +388,7 @@ __device__ __forceinline__ void write_empty_partial_rows(const PrefillArgs& a, c
 // Merge the kv_splits partial rows of one (query token, query head): out = sum_j O_j 2^(m_j - m*) /
 // sum_j l_j 2^(m_j - m*).  grid = (tokens, Hq); one wave, HD / 64 dims per lane; lane j fetches (m_j, l_j).
 template <int HD>
-__global__ __launch_bounds__(64) void rpa_prefill_combine_kernel(const PrefillArgs a) {
+static __global__ __launch_bounds__(64) void rpa_prefill_combine_kernel(const PrefillArgs a) {
   constexpr int kDpl = HD / 64;
   typedef float fvec_t __attribute__((ext_vector_type(kDpl)));
   // (with the call's composition on the device the sequences to process are read there, as in the kernels)

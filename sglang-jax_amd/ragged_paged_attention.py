@@ -84,6 +84,27 @@ def _host_max(t):
     return 0
 
 
+def _prefill_q_bound(cu_q_lens, dist, chunk_prefill_size, static_shapes):
+    """Bound on the query length of the sequences behind the decode rows, which sizes the prefill grid (0 = the
+    token count).  A host copy of ``cu_q_lens`` gives the exact maximum.  Without one, ``chunk_prefill_size`` is
+    a bound only where the reference itself takes it for one: on the PREFILL partition [i, j), launched with
+    ``static_q_len = chunk_prefill_size`` (rpa_v3:2074-2082).  Sequences of the MIXED partition [j, k) may be of
+    any length (``static_q_len = None``, rpa_v3:2083-2090), and with the composition on the device j and k are
+    unknown here: then only the token count bounds a chunk."""
+    i, j, k = (int(x) for x in dist)
+    host = None
+    if isinstance(cu_q_lens, np.ndarray):
+        host = cu_q_lens
+    elif isinstance(cu_q_lens, torch.Tensor) and cu_q_lens.device.type == "cpu":
+        host = cu_q_lens.numpy()
+    if host is not None and not static_shapes:
+        q = np.diff(host[i:k + 1])
+        return int(q.max()) if q.size else 0
+    if static_shapes or not chunk_prefill_size or j != k:
+        return 0
+    return int(chunk_prefill_size)
+
+
 def static_validate_inputs(queries, keys, values, kv_cache_fused, kv_lens, page_indices, cu_q_lens,
                            cu_kv_lens, distribution, *, causal=1, sliding_window=None, soft_cap=None,
                            chunk_prefill_size=None, skip_kv_mask=False):
@@ -364,7 +385,11 @@ def ragged_paged_attention(
     Mirrors rpa_v3:1667-1733.  TPU tuning knobs (block sizes, vmem limit, semaphore
     checks, debug mode) are accepted and ignored.  ``k_scale``/``v_scale`` may be a
     float (reference) or one value per kv head.  ``distribution`` and the optional
-    ``max_kv_len``/``max_q_len`` are host values used only to size launch grids;
+    ``max_kv_len``/``max_q_len`` are host values used only to size launch grids
+    (``max_q_len`` left out: the exact maximum when ``cu_q_lens`` is a host array; else
+    ``chunk_prefill_size`` when the batch has no MIXED partition, whose sequences the reference lets be
+    of any length; else the token count).  A sequence longer than a ``max_q_len`` the caller passes
+    loses its rows past the bound: it is a promise, like a static shape.
     ``host_kv_lens`` is an optional host copy of ``kv_lens`` (the split plan balances on its
     sum) for callers that pass ``kv_lens`` as a device tensor.
 
@@ -440,8 +465,8 @@ def ragged_paged_attention(
                    k_scale=k_scale, v_scale=v_scale,
                    max_kv_len=max_kv_len if max_kv_len is not None else _host_max(
                        host_kv_lens if host_kv_lens is not None else kv_lens),
-                   # the static chunk size bounds a chunk's length (rpa_v3:1691): it sizes the prefill grid
-                   max_q_len=max_q_len if max_q_len is not None else (chunk_prefill_size or 0), num_splits=num_splits,
+                   max_q_len=max_q_len if max_q_len is not None else _prefill_q_bound(
+                       cu_q_lens, dist, chunk_prefill_size, static_shapes), num_splits=num_splits,
                    sum_decode_kv_len=_host_decode_sum(host_kv_lens if host_kv_lens is not None else kv_lens, i),
                    attention_sink=attention_sink, xai_temperature_len=xai_temperature_len, causal=bool(causal),
                    custom_mask=custom_mask, mask_aligned_to_cu_kv=mask_aligned_to_cu_kv,

@@ -457,6 +457,40 @@ def sub_batch(b: Batch, seqs, last_rows: int | None = None) -> Batch:
         meta={"q_lens": q_lens, "kv_lens": kv_lens, "rows": q_rows.tolist()})
 
 
+def mla_sub_batch(b: MlaBatch, seqs) -> MlaBatch:
+    """`sub_batch` for the latent cache: the sequences `seqs` of `b` as a compact CPU batch of their own
+    (pages renumbered 0..n-1, same page contents, every query token kept)."""
+    P = b.page_size
+    kv = b.kv_lens.cpu().numpy()
+    cu_q = b.cu_q_lens.cpu().numpy()
+    cu_kv = b.cu_kv_lens.cpu().numpy()
+    pages = b.page_indices.cpu().numpy()
+    q_rows, new_pages, q_lens, kv_lens = [], [], [], []
+    for i in seqs:
+        q_rows.append(torch.arange(int(cu_q[i]), int(cu_q[i + 1])))
+        cnt = -(-int(kv[i]) // P)
+        new_pages.append(pages[cu_kv[i] // P: cu_kv[i] // P + cnt])
+        q_lens.append(int(cu_q[i + 1] - cu_q[i]))
+        kv_lens.append(int(kv[i]))
+    q_rows = torch.cat(q_rows)
+    old = np.concatenate(new_pages).astype(np.int64)
+    cu_kv_new = np.zeros(len(seqs) + 1, dtype=np.int32)
+    cu_kv_new[1:] = np.cumsum(np.array([len(x) for x in new_pages]) * P)
+    cu_q_new = np.zeros(len(seqs) + 1, dtype=np.int32)
+    cu_q_new[1:] = np.cumsum(q_lens)
+    dec = 0
+    while dec < len(seqs) and q_lens[dec] == 1:
+        dec += 1
+    dev = b.ql_nope.device
+    return MlaBatch(
+        name=b.name + "_sample", ql_nope=b.ql_nope[q_rows.to(dev)].cpu(), q_pe=b.q_pe[q_rows.to(dev)].cpu(),
+        cache_kv=b.cache_kv[torch.from_numpy(old).to(dev)].cpu(), kv_lens=torch.tensor(kv_lens, dtype=torch.int32),
+        page_indices=torch.arange(len(old), dtype=torch.int32), cu_q_lens=torch.from_numpy(cu_q_new),
+        cu_kv_lens=torch.from_numpy(cu_kv_new), distribution=torch.tensor([dec, dec, len(seqs)], dtype=torch.int32),
+        sm_scale=b.sm_scale, page_size=P, sliding_window=b.sliding_window, soft_cap=b.soft_cap,
+        meta={"q_lens": q_lens, "kv_lens": kv_lens, "rows": q_rows.tolist()})
+
+
 # --------------------------------------------------------------------------
 # Algorithmic bytes / FLOPs of a batch (the numerators of every roofline figure)
 # --------------------------------------------------------------------------

@@ -47,21 +47,63 @@ def test_header_links_from_two_translation_units(tmp_path):
         assert subprocess.run([str(out)]).returncode == 0
 
 
-def test_library_exports_no_stray_data_symbol(pkg):
+def test_library_exports_nothing_but_the_declared_entry_points(pkg):
+    """The library is built with hidden visibility: its dynamic symbol table holds the functions rpa.h
+    declares and nothing else (no data object, no C++ helper a host process could collide with or interpose)."""
     import subprocess
 
     r = subprocess.run(["nm", "-D", "--defined-only", pkg._lib.LIB_PATH], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
-    data = [ln.split()[-1] for ln in r.stdout.splitlines() if len(ln.split()) == 3 and ln.split()[1] in "BDCbd"]
-    assert not [n for n in data if n.startswith("Rpa")], data
+    defined = {}
+    for ln in r.stdout.splitlines():
+        parts = ln.split()
+        if len(parts) == 3:
+            defined[parts[2]] = parts[1]
+    stray = {n: k for n, k in defined.items() if n not in header_functions() and not n.startswith("__hip_")}
+    assert not stray, stray
+    assert all(defined[n] == "T" for n in header_functions())
 
 
-def test_struct_layout_matches_header(pkg):
-    # 11 pointers + size_t + 15 int32 + 3 float + int64
-    # ... and the device-side distribution pointer at the end
-    assert ctypes.sizeof(pkg._lib.RpaParams) == 12 * 8 + 18 * 4 + 8 + 3 * 8 + 5 * 4 + 4 + 8  # incl. padding
-    # 10 pointers / size_t + 13 int32 + 3 float + int64 + 3 float (+ tail padding)
-    assert ctypes.sizeof(pkg._lib.RpaMlaParams) == 10 * 8 + 13 * 4 + 3 * 4 + 8 + 3 * 4 + 4 + 8 + 2 * 4
+def _header_struct_fields(name):
+    """Field names of a struct of rpa.h, in declaration order, read from the header's text."""
+    text = open(os.path.join(ROOT, "include", "rpa.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (name, name), text, flags=re.S).group(1)
+    fields = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if decl:
+            fields.append(re.search(r"([A-Za-z_][A-Za-z0-9_]*)$", decl).group(1))
+    return fields
+
+
+@pytest.mark.parametrize("struct", ["RpaParams", "RpaMlaParams"])
+def test_struct_layout_matches_header(pkg, tmp_path, struct):
+    """sizeof and every offsetof as the C compiler lays the header's struct out, against the ctypes mirror:
+    a field reordered or retyped on one side only fails here even when the total size stays the same."""
+    import subprocess
+
+    fields = _header_struct_fields(struct)
+    mirror = getattr(pkg._lib, struct)
+    assert fields == [f[0] for f in mirror._fields_]
+    src = tmp_path / "layout.c"
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "rpa.h"', "int main(void) {",
+             '  printf("sizeof %%zu\\n", sizeof(%s));' % struct]
+    for f in fields:
+        lines.append('  printf("%s %%zu %%zu\\n", offsetof(%s, %s), sizeof(((%s*)0)->%s));' % (f, struct, f, struct, f))
+    lines += ["  return 0;", "}"]
+    src.write_text("\n".join(lines) + "\n")
+    exe = tmp_path / "layout"
+    r = subprocess.run(["gcc", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    out = subprocess.run([str(exe)], capture_output=True, text=True).stdout.split("\n")
+    assert int(out[0].split()[1]) == ctypes.sizeof(mirror)
+    for ln in out[1:]:
+        if ln:
+            name, off, size = ln.split()
+            assert getattr(mirror, name).offset == int(off), name
+            assert getattr(mirror, name).size == int(size), name
 
 
 def base_params(pkg):
