@@ -14,6 +14,55 @@
 
 #include "../../include/rpa.h"
 #include "rpa_kernels.h"
+#include "rpa_tuning.h"
+
+extern char** environ;
+
+namespace rpa {
+
+// One parse of the RPA_* switches per change of the environment (per thread): see rpa_tuning.h.
+const Tuning& tuning() {
+  thread_local Tuning t;
+  thread_local uint64_t seen = 0;
+  thread_local bool valid = false;
+  // setenv() never edits a string in place: a changed variable is a changed pointer in environ
+  uint64_t h = 1469598103934665603ull;
+  for (char** e = environ; e && *e; ++e) h = (h ^ reinterpret_cast<uintptr_t>(*e)) * 1099511628211ull;
+  if (valid && h == seen) return t;
+  t = Tuning();
+  auto geti = [](const char* name, int& dst) {
+    const char* v = getenv(name);
+    if (v && *v) dst = atoi(v);
+  };
+  geti("RPA_DECODE_MIN_CHUNK", t.decode_min_chunk);
+  geti("RPA_DECODE_BALANCED", t.decode_balanced);
+  geti("RPA_DECODE_WAVES_PER_WG", t.decode_waves_per_wg);
+  geti("RPA_DECODE_WAVE_CAPACITY", t.decode_wave_capacity);
+  geti("RPA_DECODE_MERGE_IN_KERNEL", t.decode_merge_in_kernel);
+  geti("RPA_MASK_BITS", t.mask_bits);
+  geti("RPA_PREFILL_ROWS256", t.prefill_rows256);
+  geti("RPA_PREFILL_STAGED", t.prefill_staged);
+  geti("RPA_PREFILL_PIPE", t.prefill_pipe);
+  geti("RPA_PREFILL_PIPE_TILE", t.prefill_pipe_tile);
+  geti("RPA_PREFILL_LEVEL_ORDER", t.prefill_level_order);
+  geti("RPA_PREFILL_PIPE_NQ", t.prefill_pipe_nq);
+  geti("RPA_PREFILL_SPLITS", t.prefill_splits);
+  geti("RPA_MLA_MIN_CHUNK", t.mla_min_chunk);
+  geti("RPA_MLA_WG_CAPACITY", t.mla_wg_capacity);
+  geti("RPA_MLA_BALANCED", t.mla_balanced);
+  geti("RPA_MLA_PIECE_PAD", t.mla_piece_pad);
+  geti("RPA_MLA_PIPE", t.mla_pipe);
+  geti("RPA_MLA_SHARED_TILES", t.mla_shared_tiles);
+  geti("RPA_MLA_WIDE", t.mla_wide);
+  if (const char* v = getenv("RPA_PREFILL_PIPE_LIMIT")) {
+    if (*v) t.prefill_pipe_limit = (float)atof(v);
+  }
+  seen = h;
+  valid = true;
+  return t;
+}
+
+}  // namespace rpa
 
 namespace {
 
@@ -25,12 +74,6 @@ int fail(int code, const char* fmt, ...) {
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
   return code;
-}
-
-int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
-  if (!v || !*v) return dflt;
-  return atoi(v);
 }
 
 constexpr float kDefaultMask = -0.7f * 3.4028234663852886e38f;
@@ -168,15 +211,12 @@ SplitPlan decode_plan(const RpaParams* p) {
   int64_t work = p->sum_decode_kv_len > 0 ? p->sum_decode_kv_len * per_row : 0;
   if (p->sliding_window > 0) work = 0;  // visible lengths are not the raw lengths
   return plan_splits(bound, p->sliding_window, units, work, p->num_splits,
-                     env_int("RPA_DECODE_MIN_CHUNK", 64), decode_wave_capacity(p));
+                     rpa::tuning().decode_min_chunk, decode_wave_capacity(p));
 }
 
 // Balanced decode plan: a fixed number of waves (every wave slot of the GPU once) share the
 // 32-token blocks of the batch evenly; the device works the partition out from kv_lens.
-bool decode_balanced() {
-  static const bool on = env_int("RPA_DECODE_BALANCED", 1) != 0;
-  return on;
-}
+bool decode_balanced() { return rpa::tuning().decode_balanced != 0; }
 
 // The balanced plan pays for itself on ragged batches.  Rows of one known length (the host's
 // sum equals rows x bound) split evenly under the fixed plan already, and small batches the
@@ -199,7 +239,7 @@ bool use_balanced(const RpaParams* p, const SplitPlan& fixed) {
                                      p->cu_kv_lens != nullptr);
   const int nw = decode_waves_per_wg(p);
   const int64_t units = (int64_t)((p->num_kv_heads + nw - 1) / nw) * ((p->num_q_heads / p->num_kv_heads + 15) / 16);
-  const int64_t min_blocks = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 64) / 32);
+  const int64_t min_blocks = std::max(1, rpa::tuning().decode_min_chunk / 32);
   if ((int64_t)p->decode_end * ((bound + 31) / 32) * units <= (int64_t)decode_wgs(p) * min_blocks)
     return false;
   const bool equal_lengths = p->sum_decode_kv_len > 0 && p->max_kv_len > 0 &&
@@ -228,7 +268,8 @@ int64_t decode_kv_bytes(const RpaParams* p) {
 // more CUs (C1 14.0 against 15.9 us).
 int decode_waves_per_wg(const RpaParams* p) {
   const int dflt = decode_kv_bytes(p) >= (32ll << 20) ? 4 : 2;
-  const int nw = env_int("RPA_DECODE_WAVES_PER_WG", dflt);
+  const int forced = rpa::tuning().decode_waves_per_wg;
+  const int nw = forced > 0 ? forced : dflt;
   return std::max(1, std::min(std::min(nw, 4), p->num_kv_heads));
 }
 
@@ -241,7 +282,7 @@ int decode_waves_per_wg(const RpaParams* p) {
 // never a workgroup count between one and two per CU, which the dispatcher spreads unevenly
 // (1152 waves in 4-wave workgroups: 133 us on C2).
 int decode_wave_capacity(const RpaParams* p) {
-  const int env = env_int("RPA_DECODE_WAVE_CAPACITY", 0);
+  const int env = rpa::tuning().decode_wave_capacity;
   if (env > 0) return env;
   const int cus = wave_capacity() / 8;
   if (esize_of(p->kv_dtype) == 1) return cus * 8;
@@ -277,7 +318,7 @@ size_t rows256_workspace(const RpaParams* p) {
 }
 
 // head_dim 256: every query token of sequences [seq_begin, seq_end) is a row of the row kernel
-int rows256(const RpaParams* p, int seq_begin, int seq_end, void* stream) {
+int rows256(const RpaParams* p, int seq_begin, int seq_end, void* stream, int dist_role = 0) {
   if (seq_end <= seq_begin) return RPA_OK;
   rpa::DecodeArgs a = {};
   a.q = static_cast<const uint16_t*>(p->q);
@@ -292,8 +333,9 @@ int rows256(const RpaParams* p, int seq_begin, int seq_end, void* stream) {
   a.Hkv = p->num_kv_heads;
   a.G = p->num_q_heads / p->num_kv_heads;
   a.fp8 = p->kv_dtype == RPA_KV_FP8_E4M3;
+  a.dist = dist_role ? p->distribution : nullptr;
   // decode rows are one token each; other sequences are bounded by the tokens of the call
-  const int rows = (seq_end <= p->decode_end) ? (seq_end - seq_begin) : p->num_tokens;
+  const int rows = (dist_role != 2 && seq_end <= p->decode_end) ? (seq_end - seq_begin) : p->num_tokens;
   if (seq_begin == 0 && seq_end == p->decode_end && p->mask_mode != RPA_MASK_CUSTOM) {
     const SplitPlan sp = rows256_plan(p);
     if (sp.splits > 1) {
@@ -306,7 +348,8 @@ int rows256(const RpaParams* p, int seq_begin, int seq_end, void* stream) {
       a.ws_ml = a.ws_o + (size_t)p->decode_end * sp.splits * p->num_q_heads * p->head_dim;
     }
   }
-  return check_hip(rpa::launch_rows256(a, seq_begin, seq_end, rows, static_cast<hipStream_t>(stream)), "rpa rows256");
+  return check_hip(rpa::launch_rows256(a, seq_begin, seq_end, rows, dist_role, static_cast<hipStream_t>(stream)),
+                   "rpa rows256");
 }
 
 }  // namespace
@@ -360,8 +403,6 @@ int rpa_validate(const RpaParams* p) {
     return fail(RPA_EINVAL_NULL, "split layout needs v_pages");
   if (p->sliding_window < 0) return fail(RPA_EINVAL_WINDOW, "sliding_window=%d must be positive", p->sliding_window);
   if (std::isnan(p->soft_cap)) return fail(RPA_EINVAL_SOFTCAP, "soft_cap must not be NaN");
-  if (p->distribution && p->head_dim != 128)
-    return fail(RPA_EUNSUPPORTED, "a device-side distribution is built for head_dim 128 only, got %d", p->head_dim);
   if (!p->distribution && (p->decode_end < 0 || p->decode_end > p->num_seqs))
     return fail(RPA_EINVAL_DISTRIBUTION, "distribution must satisfy 0 <= decode_end=%d <= num_seqs=%d",
                 p->decode_end, p->num_seqs);
@@ -517,9 +558,7 @@ int rpa_decode(const RpaParams* p_in, void* stream) {
   const RpaParams* p = &pv;
   if (p->decode_end <= 0) return RPA_OK;
   if (p->mask_mode == RPA_MASK_CUSTOM) return RPA_OK;  // masked rows all go through the prefill kernel
-  if (p->head_dim == 256) return rows256(p, 0, p->decode_end, stream);
-  if (p->decode_end > 65535)  // rows sit on the second grid dimension
-    return fail(RPA_EUNSUPPORTED, "at most 65535 decode rows per call, got %d", p->decode_end);
+  if (p->head_dim == 256) return rows256(p, 0, p->decode_end, stream, p->distribution ? 1 : 0);
   const SplitPlan sp = decode_plan(p);
   rpa::DecodeArgs a;
   a.q = static_cast<const uint16_t*>(p->q);
@@ -545,7 +584,7 @@ int rpa_decode(const RpaParams* p_in, void* stream) {
   a.balanced = use_balanced(p, sp) ? 1 : 0;
   a.num_wgs = decode_wgs(p);
   a.waves_per_wg = decode_waves_per_wg(p);
-  a.min_blocks_per_wave = std::max(1, env_int("RPA_DECODE_MIN_CHUNK", 64) / 32);
+  a.min_blocks_per_wave = std::max(1, rpa::tuning().decode_min_chunk / 32);
   a.forced_blocks_per_wave = 0;
   if (p->num_splits > 0) {  // the caller pins the partition: about num_splits pieces for the longest row
     const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
@@ -565,7 +604,7 @@ int rpa_decode(const RpaParams* p_in, void* stream) {
     // Every workgroup of the balanced grid is resident from the start and ends with its cut
     // piece, so all merges fall at the very end of the kernel, where they cost what the second
     // launch costs, and the written-through partial rows cost more: it measures slower.
-    if (env_int("RPA_DECODE_MERGE_IN_KERNEL", 0) != 0 && (reinterpret_cast<uintptr_t>(ws) & 7) == 0) {
+    if (rpa::tuning().decode_merge_in_kernel != 0 && (reinterpret_cast<uintptr_t>(ws) & 7) == 0) {
       a.merge_counters = reinterpret_cast<unsigned long long*>(ws + lay.counters);
       // 48 bits, never zero: the arrival words are never cleared, and a word of zeros must not
       // look like this call's
@@ -627,7 +666,7 @@ PrefillWorkspace prefill_workspace(const RpaParams* p, const rpa::PrefillArgs& a
   w.split_bytes = rpa::prefill_split_workspace_bytes(a, w.splits);
   w.bits_offset = (w.split_bytes + 255) & ~(size_t)255;
   if (p->mask_mode == RPA_MASK_CUSTOM && p->head_dim == 128 && p->max_kv_len > 0 && p->num_tokens > 0 &&
-      env_int("RPA_MASK_BITS", 1) != 0) {
+      rpa::tuning().mask_bits != 0) {
     w.pitch = (p->max_kv_len + 63) / 64;
     w.bits_bytes = (size_t)p->num_tokens * w.pitch * sizeof(uint64_t);
     if (w.bits_bytes > ((size_t)256 << 20)) w.bits_bytes = 0;  // a batch this large keeps the i32 words
@@ -642,7 +681,7 @@ PrefillWorkspace prefill_workspace(const RpaParams* p, const rpa::PrefillArgs& a
 static size_t prefill_optional_workspace(const RpaParams* p) {
   rpa::PrefillArgs a;
   if (!prefill_args(p, a)) return 0;
-  if (p->head_dim == 256 && env_int("RPA_PREFILL_ROWS256", 0) != 0) return 0;  // the row kernel has its own plan
+  if (p->head_dim == 256 && rpa::tuning().prefill_rows256 != 0) return 0;  // the row kernel has its own plan
   return prefill_workspace(p, a).total;
 }
 
@@ -653,8 +692,9 @@ int rpa_prefill(const RpaParams* p, void* stream) {
   if (!prefill_args(p, a)) return RPA_OK;
   // 256-wide heads take the flash kernel (two 128-dim halves per row, one workgroup per CU; e4m3
   // caches staged through registers); RPA_PREFILL_ROWS256=1 sends them through the row kernel
-  if (p->head_dim == 256 && env_int("RPA_PREFILL_ROWS256", 0) != 0)
-    return rows256(p, (p->mask_mode == RPA_MASK_CUSTOM) ? 0 : p->decode_end, p->num_seqs, stream);
+  if (p->head_dim == 256 && rpa::tuning().prefill_rows256 != 0)
+    return rows256(p, (p->mask_mode == RPA_MASK_CUSTOM || p->distribution) ? 0 : p->decode_end, p->num_seqs, stream,
+                   p->distribution ? 2 : 0);
   if (p->workspace && (reinterpret_cast<uintptr_t>(p->workspace) & 15) == 0) {
     // the decode partition is done with the workspace by the time these kernels run (same stream)
     const PrefillWorkspace w = prefill_workspace(p, a);
@@ -733,6 +773,8 @@ int rpa_kv_write(const RpaParams* p, const void* keys, const void* values, void*
 
 // ---------------------------------------------------------------- MLA ----
 
+static int mla_wgs();
+
 static SplitPlan mla_plan(const RpaMlaParams* p, int64_t rows) {
   const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                      p->cu_kv_lens != nullptr);
@@ -743,7 +785,7 @@ static SplitPlan mla_plan(const RpaMlaParams* p, int64_t rows) {
   int64_t work = p->sum_kv_len > 0 ? p->sum_kv_len * groups : 0;
   if (p->sliding_window > 0) work = 0;
   return plan_splits(bound, p->sliding_window, units, work, p->num_splits,
-                     env_int("RPA_MLA_MIN_CHUNK", 256), env_int("RPA_MLA_WG_CAPACITY", wave_capacity() / 8));
+                     rpa::tuning().mla_min_chunk, mla_wgs());
 }
 
 static int mla_validate(const RpaMlaParams* p) {
@@ -768,11 +810,14 @@ static int mla_validate(const RpaMlaParams* p) {
   return RPA_OK;
 }
 
-static int mla_wgs() { return std::max(1, env_int("RPA_MLA_WG_CAPACITY", wave_capacity() / 8)); }
+static int mla_wgs() {
+  const int forced = rpa::tuning().mla_wg_capacity;
+  return std::max(1, forced > 0 ? forced : wave_capacity() / 8);
+}
 
 // same criteria as the MHA decode path: ragged sequence rows that need splitting
 static bool mla_use_balanced(const RpaMlaParams* p, const SplitPlan& fixed, bool token_rows) {
-  static const bool on = env_int("RPA_MLA_BALANCED", 1) != 0;
+  const bool on = rpa::tuning().mla_balanced != 0;
   if (!on || token_rows || p->num_splits == 1) return false;
   // Rows the fixed plan leaves whole: one workgroup job per row.  With many more jobs than
   // workgroup slots the dispatcher evens them out by itself; with up to two per slot the kernel
@@ -784,7 +829,7 @@ static bool mla_use_balanced(const RpaMlaParams* p, const SplitPlan& fixed, bool
   const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                      p->cu_kv_lens != nullptr);
   const int64_t units = (p->num_q_heads + 127) / 128;
-  const int64_t min_tiles = std::max(1, env_int("RPA_MLA_MIN_CHUNK", 256) / 32);
+  const int64_t min_tiles = std::max(1, rpa::tuning().mla_min_chunk / 32);
   if ((int64_t)p->num_seqs * ((bound + 31) / 32) * units <= (int64_t)mla_wgs() * min_tiles) return false;
   const bool equal_lengths = p->sum_kv_len > 0 && p->max_kv_len > 0 &&
                              p->sum_kv_len == (int64_t)p->num_seqs * p->max_kv_len;
@@ -814,9 +859,6 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
     return fail(RPA_EINVAL_SHAPE, "decode rows=%d exceed tokens=%d", p->num_seqs, p->num_tokens);
   const int64_t rows = token_rows ? p->num_tokens : p->num_seqs;
   if (rows <= 0) return RPA_OK;
-  if (rows > 65535)  // rows sit on the second grid dimension
-    return fail(RPA_EUNSUPPORTED, "MLA: at most 65535 rows (%s) per call, got %lld",
-                token_rows ? "query tokens" : "sequences", (long long)rows);
   const SplitPlan sp = mla_plan(p, rows);
   rpa::MlaDecodeArgs a;
   a.ql_nope = static_cast<const uint16_t*>(p->ql_nope);
@@ -850,9 +892,9 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   a.cu_tiles = nullptr;
   a.balanced = mla_use_balanced(p, sp, token_rows) ? 1 : 0;
   a.num_wgs = mla_wgs();
-  a.min_tiles_per_wg = std::max(1, env_int("RPA_MLA_MIN_CHUNK", 256) / 32);
+  a.min_tiles_per_wg = std::max(1, rpa::tuning().mla_min_chunk / 32);
   a.forced_tiles_per_wg = 0;
-  a.piece_pad = std::max(0, env_int("RPA_MLA_PIECE_PAD", 5));
+  a.piece_pad = std::max(0, rpa::tuning().mla_piece_pad);
   if (p->num_splits > 0) {
     const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                        p->cu_kv_lens != nullptr);

@@ -467,17 +467,19 @@ __device__ __forceinline__ void decode_segment(const DecodeArgs& a, int seq, int
   write_rows<MT>(a, acc, m, l, tq, hk, row0, dest, c, g);
 }
 
-// ---- fixed split plan: grid = (max_splits, decode rows, head groups * row groups); block = NW waves
+// ---- fixed split plan: grid = (max_splits * decode rows, 1, head groups * row groups), splits fastest (rows do
+// not sit on a grid dimension of their own: that one ends at 65535); block = NW waves
 template <int MT, bool FP8, bool UNIFORM_PAGE, bool CAP>
 __global__ __launch_bounds__(256, 2) void rpa_decode_splitkv_kernel(const DecodeArgs a_in) {
   DecodeArgs a = a_in;  // static-shape mode: the number of decode rows comes from the device
   if (a.dist) a.num_rows = min(a.num_rows, scalar_load_i32(a.dist));
-  if ((int)blockIdx.y >= a.num_rows) return;
+  const int nsp = max(a.max_splits, 1);
+  const int seq = (int)(blockIdx.x / (unsigned)nsp);
+  const int split = (int)blockIdx.x - seq * nsp;
+  if (seq >= a.num_rows) return;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
-  const int seq = blockIdx.y;
-  const int split = blockIdx.x;
   const int head_groups = (a.Hkv + nw - 1) / nw;
   const int hg = blockIdx.z % head_groups;
   const int rg = blockIdx.z / head_groups;
@@ -1113,13 +1115,13 @@ __device__ __forceinline__ void merge_rows(const DecodeArgs& a, int seq, int hea
   for (int e = 0; e < kDpl; e += 2) op[e / 2] = pack_bf16x2(acc[e] * inv, acc[e + 1] * inv);
 }
 
-// Merge the partial rows of the balanced plan.  grid = (Hq, decode rows); block = one wave.
+// Merge the partial rows of the balanced plan.  grid = (Hq * decode rows); block = one wave.
 __global__ __launch_bounds__(64) void rpa_combine_balanced_kernel(const DecodeArgs a_in) {
   DecodeArgs a = a_in;  // static-shape mode: the number of decode rows comes from the device
   if (a.dist) a.num_rows = min(a.num_rows, scalar_load_i32(a.dist));
-  if ((int)blockIdx.y >= a.num_rows) return;
-  const int head = blockIdx.x;
-  const int seq = blockIdx.y;
+  const int seq = (int)(blockIdx.x / (unsigned)a.Hq);  // grid.x = Hq * rows, heads fastest
+  const int head = (int)blockIdx.x - seq * a.Hq;
+  if (seq >= a.num_rows) return;
   const int lane = threadIdx.x;
   const int nw = a.waves_per_wg;
   const int row_groups = (a.G + 15) / 16;
@@ -1163,9 +1165,18 @@ __device__ __forceinline__ int owner_of_token(const int32_t* cu_q_lens, int num_
   return lo;
 }
 
-// grid = (token rows, Hkv, row groups of 16 query heads); block = one wave
+// grid = (token rows, Hkv, row groups of 16 query heads); block = one wave.
+// With the composition on the device (a.dist) seq_end is only a bound: dist_role 1 = the decode partition
+// [0, dist[0]), 2 = everything behind it [dist[0], dist[2]) (custom-mask calls: [0, dist[2])).
 template <bool FP8, bool UNIFORM_PAGE>
-__global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int seq_begin, int seq_end) {
+__global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int seq_begin, int seq_end, int dist_role) {
+  if (a.dist && dist_role == 1) {
+    seq_end = min(seq_end, scalar_load_i32(a.dist));
+  } else if (a.dist && dist_role == 2) {
+    seq_begin = (a.sm.mask_mode == 1) ? 0 : min(seq_end, scalar_load_i32(a.dist));
+    seq_end = min(seq_end, scalar_load_i32(a.dist + 2));
+  }
+  if (seq_end <= seq_begin) return;
   const int lane = threadIdx.x;
   const int c = lane & 15, g = lane >> 4;
   const int rg = blockIdx.z, hk = blockIdx.y;
@@ -1345,7 +1356,7 @@ __global__ __launch_bounds__(64) void rpa_rows256_kernel(const DecodeArgs a, int
 }
 
 // Merge the split partials: out = sum_j o_j 2^(m_j - m*) / sum_j l_j 2^(m_j - m*).
-// grid = (Hq, decode rows); block = one wave, 2 dims per lane (D = 128).  Lane j
+// grid = (Hq * decode rows); block = one wave, 2 dims per lane (D = 128).  Lane j
 // first fetches (m_j, l_j) of split j, the wave reduces m* and the denominator
 // with shuffles, then the weights are broadcast lane by lane while the partial
 // rows stream in with independent loads.
@@ -1353,9 +1364,9 @@ template <int HD>
 __global__ __launch_bounds__(64) void rpa_combine_kernel(const DecodeArgs a_in) {
   DecodeArgs a = a_in;  // static-shape mode: the number of decode rows comes from the device
   if (a.dist) a.num_rows = min(a.num_rows, scalar_load_i32(a.dist));
-  if ((int)blockIdx.y >= a.num_rows) return;
-  const int head = blockIdx.x;
-  const int seq = blockIdx.y;
+  const int seq = (int)(blockIdx.x / (unsigned)a.Hq);  // grid.x = Hq * rows, heads fastest
+  const int head = (int)blockIdx.x - seq * a.Hq;
+  if (seq >= a.num_rows) return;
   const int lane = threadIdx.x;
   const int kv_len = a.pt.kv_lens[seq];
   const int t0 = first_block_token(kv_len, a.sm.window);
@@ -1459,15 +1470,17 @@ hipError_t launch_decode(const DecodeArgs& a, hipStream_t stream) {
     hipError_t e = launch_decode_mt(a, dim3(a.num_wgs), dim3(a.waves_per_wg * 64), uniform, stream);
     if (e != hipSuccess) return e;
     if (!a.merge_counters)
-      hipLaunchKernelGGL(rpa_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
+      hipLaunchKernelGGL(rpa_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(64), 0, stream, a);
     return hipGetLastError();
   }
-  dim3 grid(a.max_splits, a.num_rows, head_groups * row_groups);
+  if ((int64_t)a.max_splits * a.num_rows > 0x7fffffffLL || (int64_t)a.Hq * a.num_rows > 0x7fffffffLL)
+    return hipErrorInvalidValue;
+  dim3 grid((unsigned)max(a.max_splits, 1) * (unsigned)a.num_rows, 1, head_groups * row_groups);
   dim3 block(nw * 64);
   hipError_t e = launch_decode_mt(a, grid, block, uniform, stream);
   if (e != hipSuccess) return e;
   if (a.max_splits > 1) {
-    hipLaunchKernelGGL(rpa_combine_kernel<128>, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
+    hipLaunchKernelGGL(rpa_combine_kernel<128>, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(64), 0, stream, a);
     e = hipGetLastError();
   }
   return e;
@@ -1481,7 +1494,8 @@ hipError_t launch_gather(const GatherArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int max_token_rows, hipStream_t stream) {
+hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int max_token_rows, int dist_role,
+                          hipStream_t stream) {
   if (seq_end <= seq_begin || max_token_rows <= 0) return hipSuccess;
   if (a.Hkv > 65535) return hipErrorInvalidValue;  // grid.y
   const int nsplit = a.max_splits > 1 ? a.max_splits : 1;
@@ -1489,16 +1503,16 @@ hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int m
   const dim3 grid(max_token_rows * nsplit, a.Hkv, (a.G + 15) / 16), block(64);
   const bool uniform = (a.pt.page_size % kBlk) == 0;
   if (a.fp8) {
-    if (uniform) hipLaunchKernelGGL((rpa_rows256_kernel<true, true>), grid, block, 0, stream, a, seq_begin, seq_end);
-    else hipLaunchKernelGGL((rpa_rows256_kernel<true, false>), grid, block, 0, stream, a, seq_begin, seq_end);
+    if (uniform) hipLaunchKernelGGL((rpa_rows256_kernel<true, true>), grid, block, 0, stream, a, seq_begin, seq_end, dist_role);
+    else hipLaunchKernelGGL((rpa_rows256_kernel<true, false>), grid, block, 0, stream, a, seq_begin, seq_end, dist_role);
   } else {
-    if (uniform) hipLaunchKernelGGL((rpa_rows256_kernel<false, true>), grid, block, 0, stream, a, seq_begin, seq_end);
-    else hipLaunchKernelGGL((rpa_rows256_kernel<false, false>), grid, block, 0, stream, a, seq_begin, seq_end);
+    if (uniform) hipLaunchKernelGGL((rpa_rows256_kernel<false, true>), grid, block, 0, stream, a, seq_begin, seq_end, dist_role);
+    else hipLaunchKernelGGL((rpa_rows256_kernel<false, false>), grid, block, 0, stream, a, seq_begin, seq_end, dist_role);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || nsplit == 1) return e;
-  if (a.num_rows > 65535) return hipErrorInvalidValue;  // rows sit on the second grid dimension
-  hipLaunchKernelGGL(rpa_combine_kernel<256>, dim3(a.Hq, a.num_rows), dim3(64), 0, stream, a);
+  if ((int64_t)a.Hq * a.num_rows > 0x7fffffffLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(rpa_combine_kernel<256>, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(64), 0, stream, a);
   return hipGetLastError();
 }
 

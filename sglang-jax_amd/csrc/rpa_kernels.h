@@ -180,8 +180,10 @@ int prefill_kv_splits(const PrefillArgs& a);
 size_t prefill_split_workspace_bytes(const PrefillArgs& a, int splits);
 hipError_t launch_gather(const GatherArgs& a, hipStream_t stream);
 // head_dim 256: every query token of sequences [seq_begin, seq_end) as a row of its own; at most
-// max_token_rows tokens (a host bound) are covered
-hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int max_token_rows, hipStream_t stream);
+// max_token_rows tokens (a host bound) are covered.  With a.dist set, seq_end is a bound and dist_role says
+// which partition the kernel takes from the device: 1 = decode rows, 2 = everything behind them
+hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int max_token_rows, int dist_role,
+                          hipStream_t stream);
 hipError_t launch_kv_write(const KvWriteArgs& a, hipStream_t stream);
 hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream);
 hipError_t launch_mla_kv_write(const MlaWriteArgs& a, hipStream_t stream);

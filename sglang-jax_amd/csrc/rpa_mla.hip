@@ -28,6 +28,7 @@
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
+#include "rpa_tuning.h"
 #include "rpa_mla_pipe_loop.inc"
 #include "rpa_mla_wide_loop.inc"
 #include "rpa_mla_wide32_loop.inc"
@@ -689,7 +690,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   }
 }
 
-// ---- fixed split plan: grid = (max_splits, rows, head groups of 128); block = 512 threads
+// ---- fixed split plan: grid = (max_splits * rows, 1, head groups of 128); block = 512 threads
 template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false, int DS = 1>
 __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeArgs a) {
   // three separate arrays: lets the compiler see that a copy into one slot does not alias the
@@ -698,8 +699,9 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_decode_kernel(const MlaDecodeA
   __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot3[kSlotB];
-  const int row_id = blockIdx.y;
-  const int split = blockIdx.x;
+  const int nsp = max(a.max_splits, 1);  // grid.x = max_splits * rows, splits fastest
+  const int row_id = (int)(blockIdx.x / (unsigned)nsp);
+  const int split = (int)blockIdx.x - row_id * nsp;
   const MlaRow mr = mla_row(a, row_id);
   if (!mr.valid) return;
   const int kv_len = mr.kv_len;
@@ -982,12 +984,13 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   __syncthreads();
 }
 
-// ---- fixed split plan, wide workgroups: grid = (max_splits, rows, head groups of 128); block = 256 threads
+// ---- fixed split plan, wide workgroups: grid = (max_splits * rows, 1, head groups of 128); block = 256 threads
 template <bool M32>
 __global__ __launch_bounds__(256, 1) void rpa_mla_decode_wide_kernel(const MlaDecodeArgs a) {
   __shared__ __attribute__((aligned(1024))) char ring[4 * kSlotB];
-  const int row_id = blockIdx.y;
-  const int split = blockIdx.x;
+  const int nsp = max(a.max_splits, 1);  // grid.x = max_splits * rows, splits fastest
+  const int row_id = (int)(blockIdx.x / (unsigned)nsp);
+  const int split = (int)blockIdx.x - row_id * nsp;
   const MlaRow mr = mla_row(a, row_id);
   if (!mr.valid) return;
   const int kv_len = mr.kv_len;
@@ -1195,9 +1198,10 @@ __device__ __forceinline__ void mla_merge(const MlaDecodeArgs& a, int n, SlotOf 
   *reinterpret_cast<u32x2_t*>(a.out + ((int64_t)tq * a.Hq + head) * 512 + d) = w;
 }
 
-// Merge of the balanced plan.  grid = (Hq, rows); block = 128 threads, 4 dims each.
+// Merge of the balanced plan.  grid = (Hq * rows); block = 128 threads, 4 dims each.
 __global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const MlaDecodeArgs a) {
-  const int head = blockIdx.x, seq = blockIdx.y;
+  const int seq = (int)(blockIdx.x / (unsigned)a.Hq);  // grid.x = Hq * rows, heads fastest
+  const int head = (int)blockIdx.x - seq * a.Hq;
   const int nt = mla_tiles(a.pt.kv_lens[seq], a.sm.window);
   if (nt == 0) return;
   const int units = (a.Hq + 127) / 128;
@@ -1219,9 +1223,10 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const Mla
   mla_merge(a, w_last - w_first + 1, [&](int j) { return slot_of(w_first + j); }, head, tq);
 }
 
-// grid = (Hq, rows); block = 128 threads, 4 dims each.
+// grid = (Hq * rows); block = 128 threads, 4 dims each.
 __global__ __launch_bounds__(128) void rpa_mla_combine_kernel(const MlaDecodeArgs a) {
-  const int head = blockIdx.x, row_id = blockIdx.y;
+  const int row_id = (int)(blockIdx.x / (unsigned)a.Hq);  // grid.x = Hq * rows, heads fastest
+  const int head = (int)blockIdx.x - row_id * a.Hq;
   const MlaRow mr = mla_row(a, row_id);
   if (!mr.valid || mr.kv_len <= 0) return;
   const int kv_len = mr.kv_len;
@@ -1269,20 +1274,21 @@ hipError_t launch_mla_kv_write(const MlaWriteArgs& a, hipStream_t stream) {
 hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   if (a.num_rows <= 0) return hipSuccess;
   const int head_groups = (a.Hq + 127) / 128;
-  const dim3 grid(a.max_splits, a.num_rows, head_groups), block(512);
+  if ((int64_t)a.max_splits * a.num_rows > 0x7fffffffLL || (int64_t)a.Hq * a.num_rows > 0x7fffffffLL)
+    return hipErrorInvalidValue;
+  const dim3 grid((unsigned)max(a.max_splits, 1) * (unsigned)a.num_rows, 1, head_groups), block(512);
   const bool uniform = (a.pt.page_size % kTok) == 0;
   const bool cap = a.sm.soft_cap != 0.f;
   // the assembly tile loop: whole tiles inside one page, every wave of a workgroup at work
-  const char* pipe_env = getenv("RPA_MLA_PIPE");  // read per call: tests switch it
-  const bool use_pipe = !(pipe_env && *pipe_env == '0');
+  const Tuning& tune = tuning();
+  const bool use_pipe = tune.mla_pipe != 0;
   const int P = a.pt.page_size;
   const bool pipe = use_pipe && uniform && !cap && (P & (P - 1)) == 0 && (a.Hq % 128) == 0 &&
                     (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);
   // at most 64 heads (a tensor-parallel share): the waves of a workgroup share each tile of a block of 16 heads
   // (mla_segment, DS) instead of leaving most of them without heads.  RPA_MLA_SHARED_TILES=0: one wave per block,
-  // as with 128 heads (read per call).
-  const char* ds_env = getenv("RPA_MLA_SHARED_TILES");
-  const int ds = (uniform && !cap && a.Hq <= 64 && !(ds_env && *ds_env == '0')) ? (a.Hq <= 16 ? 8 : (a.Hq <= 32 ? 4 : 2)) : 1;
+  // as with 128 heads.
+  const int ds = (uniform && !cap && a.Hq <= 64 && tune.mla_shared_tiles != 0) ? (a.Hq <= 16 ? 8 : (a.Hq <= 32 ? 4 : 2)) : 1;
   if (ds != 1) {
 #define RPA_MLA_DS(KERNEL, GRID, F8)                                                                                  \
   do {                                                                                                                \
@@ -1296,7 +1302,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
       else RPA_MLA_DS(rpa_mla_balanced_kernel, bgrid, false);
       hipError_t eb = hipGetLastError();
       if (eb != hipSuccess) return eb;
-      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
       return hipGetLastError();
     }
     if (a.fp8) RPA_MLA_DS(rpa_mla_decode_kernel, grid, true);
@@ -1305,7 +1311,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     hipError_t es = hipGetLastError();
     if (es != hipSuccess) return es;
     if (a.max_splits > 1) {
-      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
       es = hipGetLastError();
     }
     return es;
@@ -1324,7 +1330,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
       }
       hipError_t eb = hipGetLastError();
       if (eb != hipSuccess) return eb;
-      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
       return hipGetLastError();
     }
     if (pipe) {
@@ -1339,26 +1345,25 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     hipError_t ef = hipGetLastError();
     if (ef != hipSuccess) return ef;
     if (a.max_splits > 1) {
-      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
       ef = hipGetLastError();
     }
     return ef;
   }
   // wide workgroups (four waves of 32 heads) wherever the assembly loop applies; RPA_MLA_WIDE=0 keeps the
-  // eight-wave kernels (read per call: tests switch it)
-  const char* wide_env = getenv("RPA_MLA_WIDE");
-  const bool wide = !(wide_env && *wide_env == '0') && pipe;
+  // eight-wave kernels
+  const bool wide = tune.mla_wide != 0 && pipe;
   // RPA_MLA_WIDE=32: the wide loop on 32x32x16 matrix instructions (one head per lane and half).  Half the matrix
   // instructions, and 8 % faster than the default loop when neither reads its operands -- but its 32-row LDS
   // reads collide on the 1184-byte row pitch that suits the 16-row reads (7 % slower as a whole): opt-in until
   // it has a row layout of its own
-  const bool m32 = wide_env && wide_env[0] == '3' && wide_env[1] == '2';
+  const bool m32 = tune.mla_wide == 32;
   if (wide && a.balanced) {
     if (m32) hipLaunchKernelGGL(rpa_mla_balanced_wide_kernel<true>, dim3(a.num_wgs), dim3(256), 0, stream, a);
     else hipLaunchKernelGGL(rpa_mla_balanced_wide_kernel<false>, dim3(a.num_wgs), dim3(256), 0, stream, a);
     hipError_t eb = hipGetLastError();
     if (eb != hipSuccess) return eb;
-    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
     return hipGetLastError();
   }
   if (wide) {
@@ -1367,7 +1372,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     hipError_t ew = hipGetLastError();
     if (ew != hipSuccess) return ew;
     if (a.max_splits > 1) {
-      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
       ew = hipGetLastError();
     }
     return ew;
@@ -1385,7 +1390,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     }
     hipError_t eb = hipGetLastError();
     if (eb != hipSuccess) return eb;
-    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
     return hipGetLastError();
   }
   if (pipe) {
@@ -1400,7 +1405,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (a.max_splits > 1) {
-    hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3(a.Hq, a.num_rows), dim3(128), 0, stream, a);
+    hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
     e = hipGetLastError();
   }
   return e;

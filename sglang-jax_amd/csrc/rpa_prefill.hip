@@ -581,20 +581,18 @@ hipError_t launch_mask_bits(const PrefillArgs& a, hipStream_t stream) {
 }
 
 bool takes_pipe_kernel(const PrefillArgs& a) {
-  static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
-  static const bool use_pipe = [] { const char* v = getenv("RPA_PREFILL_PIPE"); return !(v && *v == '0'); }();
-  return use_pipe && !force_staged && prefill_pipe_applies(a);
+  const Tuning& tune = tuning();
+  return tune.prefill_pipe != 0 && tune.prefill_staged != 1 && prefill_pipe_applies(a);
 }
 }  // namespace
 
 namespace {
 // The compiled flash kernel's short-chunk tile: 32 positions x 4 heads per workgroup for chunks of at most 64
-// tokens (128-wide heads, heads in fours; RPA_PREFILL_PIPE_TILE=32|128 forces either, read per call).
+// tokens (128-wide heads, heads in fours; RPA_PREFILL_PIPE_TILE=32|128 forces either).
 bool compiled_short_chunk_tile(const PrefillArgs& a) {
-  static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
+  const bool force_staged = tuning().prefill_staged == 1;
   if ((force_staged && !a.fp8) || a.head_dim != 128 || (a.G % 4) != 0) return false;
-  const char* tile_env = getenv("RPA_PREFILL_PIPE_TILE");
-  const int force_tile = tile_env ? atoi(tile_env) : 0;
+  const int force_tile = tuning().prefill_pipe_tile;
   return force_tile ? force_tile == 32 : a.max_q_len <= 64;
 }
 }  // namespace
@@ -615,15 +613,14 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const int nseq = a.seq_end - a.seq_begin;
   if (nseq <= 0 || a.max_q_len <= 0) return hipSuccess;
   if (takes_pipe_kernel(a)) {
-    static const bool lo = [] { const char* v = getenv("RPA_PREFILL_LEVEL_ORDER"); return !(v && *v == '0'); }();
-    return launch_prefill_pipe(a, nseq, lo, stream);
+    return launch_prefill_pipe(a, nseq, tuning().prefill_level_order != 0, stream);
   }
   const bool heads4 = compiled_short_chunk_tile(a);
   const int bm = heads4 ? 32 : kBM;
   int tiles = (a.max_q_len + bm - 1) / bm;
   // levels 0 .. ceil(max_kv_len / rows): only worth their empty workgroups when prefixes are
   // not much longer than the chunks (else every tile of a sequence costs about the same anyway)
-  static const bool level_order = [] { const char* v = getenv("RPA_PREFILL_LEVEL_ORDER"); return !(v && *v == '0'); }();
+  const bool level_order = tuning().prefill_level_order != 0;
   const int levels = a.max_kv_len > 0 ? (a.max_kv_len + bm - 1) / bm + 1 : 0;
   const bool by_level = level_order && a.sm.mask_mode == 0 && levels > tiles && levels <= 2 * tiles + 2;
   if (by_level) tiles = levels;
@@ -633,8 +630,7 @@ hipError_t launch_prefill(const PrefillArgs& a, hipStream_t stream) {
   const bool uniform = (a.pt.page_size % kBN) == 0;
   // soft cap and logit rounding share the general score path
   const bool cap = a.sm.soft_cap != 0.f || a.sm.round_logits != 0;
-  static const bool force_staged = [] { const char* v = getenv("RPA_PREFILL_STAGED"); return v && *v == '1'; }();
-  const bool staged = a.fp8 || force_staged;
+  const bool staged = a.fp8 || tuning().prefill_staged == 1;
   if (a.sm.mask_mode == 1) {
     hipError_t e = launch_mask_bits(a, stream);
     if (e != hipSuccess) return e;

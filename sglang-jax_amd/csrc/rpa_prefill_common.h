@@ -5,6 +5,7 @@
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
+#include "rpa_tuning.h"
 
 namespace rpa {
 namespace pf {
@@ -454,13 +455,12 @@ inline hipError_t launch_prefill_combine(const PrefillArgs& a, hipStream_t strea
 // launch runs in rounds of 512 workgroups beyond; the merge costs a launch (~1.5 us) plus the partial rows'
 // way to memory and back (~0.29 ns per (token, head, piece) of 128 dims).  A cut must save at least 2 us,
 // leaves no piece under four tiles and makes at most 64 pieces.  bm / heads: query positions and query heads
-// per workgroup.  RPA_PREFILL_SPLITS: 0 / 1 never, n forces n (read per call).
+// per workgroup.  RPA_PREFILL_SPLITS: 0 / 1 never, n forces n.
 inline int kv_pieces(const PrefillArgs& a, int nseq, int bm, int heads, double tile_us) {
   // (with the composition on the device nseq, max_q_len, max_kv_len and num_tokens are bounds: a launch that is
   // under-filled even by its bounds is cut, and every workgroup fits the piece count to its own range)
   if (nseq <= 0 || a.max_q_len <= 0 || a.max_kv_len <= 0 || a.num_tokens <= 0) return 1;
-  const char* env = getenv("RPA_PREFILL_SPLITS");
-  const int forced = env ? atoi(env) : -1;
+  const int forced = tuning().prefill_splits;
   if (forced == 0 || forced == 1) return 1;
   if (forced > 1) return std::min(forced, 64);
   const int64_t tokens = std::max<int64_t>(1, (int64_t)a.num_tokens - a.seq_begin);

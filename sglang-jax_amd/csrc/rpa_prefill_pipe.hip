@@ -488,14 +488,10 @@ bool prefill_pipe_applies(const PrefillArgs& a) {
 }
 
 namespace {
-int forced_nq() {
-  static const int v = [] { const char* e = getenv("RPA_PREFILL_PIPE_NQ"); return e ? atoi(e) : 0; }();
-  return v;
-}
-// 32 positions x 4 heads per workgroup instead of 128 x 1 (read per call: tests switch it)
+int forced_nq() { return tuning().prefill_pipe_nq; }
+// 32 positions x 4 heads per workgroup instead of 128 x 1
 bool short_chunk_tile(const PrefillArgs& a, int nq) {
-  const char* tile_env = getenv("RPA_PREFILL_PIPE_TILE");
-  const int force_tile = tile_env ? atoi(tile_env) : 0;
+  const int force_tile = tuning().prefill_pipe_tile;
   return nq == 1 && (a.G % 4) == 0 && (force_tile ? force_tile == 32 : a.max_q_len <= 64);
 }
 }  // namespace
@@ -510,7 +506,7 @@ int prefill_pipe_kv_splits(const PrefillArgs& a, int nseq) {
 hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order, hipStream_t stream) {
   const int force_nq = forced_nq();
   // a half's row sum above the limit sends a wave through the rescaling path (testing knob: -1 = always)
-  static const float limit = [] { const char* v = getenv("RPA_PREFILL_PIPE_LIMIT"); return v ? (float)atof(v) : kRowSumLimit; }();
+  const float limit = tuning().prefill_pipe_limit != 0.f ? tuning().prefill_pipe_limit : kRowSumLimit;
   const int nq = force_nq ? force_nq : 1;
   // Tile by shape (the reference's per-shape block sizes, tuned_block_sizes.py, have this one counterpart
   // here): chunks of at most 64 tokens take 32 positions x 4 heads per workgroup when the heads come in fours

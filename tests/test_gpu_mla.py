@@ -292,6 +292,29 @@ def test_c5_full_size_page_permutation_invariance(pkg, wl, gpu, f8):
     assert_parity(a.float(), one.float(), **TOL)  # element-wise and every row relative to its own norm
 
 
+def test_mla_more_rows_than_a_grid_dimension_holds(pkg, wl, gpu):
+    """A prefill call of 66000 query tokens (one kernel row each; the reference loops over any number,
+    kernels/mla/v2/kernel.py:1722-1739): rows are folded onto the first grid dimension.  16 heads, short prefixes;
+    a sample of sequences against the oracle."""
+    q_lens = [3000] * 22
+    kv_lens = [3000 + 64 * i for i in range(22)]
+    b = wl.make_mla_batch("mla_many_rows", q_lens, kv_lens, num_q_heads=16, lkv_dim=512, rope_dim=64, page_size=64,
+                          seed=93, sm_scale=192 ** -0.5, device=gpu)
+    g = b
+    out, _ = pkg.mla_ragged_paged_attention(
+        g.ql_nope, g.q_pe, None, None, g.cache_kv, g.kv_lens, g.page_indices, g.cu_q_lens, g.cu_kv_lens,
+        b.distribution.cpu().numpy(), sm_scale=b.sm_scale, max_kv_len=max(kv_lens))
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    sample = wl.mla_sub_batch(b, [21])
+    # the last 64 tokens of the last sequence hold the highest row numbers (65936 ..)
+    want = oracle(sample)
+    got = out[torch.tensor(sample.meta["rows"], device=gpu)].cpu()
+    assert_parity(got[-64:].float(), want[-64:].float(), **TOL)
+    first = wl.mla_sub_batch(b, [0])
+    assert_parity(out[torch.tensor(first.meta["rows"][:64], device=gpu)].cpu().float(), oracle(first)[:64].float(), **TOL)
+
+
 @pytest.mark.parametrize("seed", list(range(8)))
 def test_random_mla_batches_against_oracle(pkg, wl, gpu, seed):
     """Seeded random decode and mixed batches, head counts, page sizes, window and soft cap."""

@@ -1212,6 +1212,78 @@ def test_device_side_distribution_matches_host_integers(pkg, wl, gpu, kv_dtype):
         assert_parity(out[: sum(sub_q)].cpu().float(), oracle_out(c).float(), **tol)
 
 
+@pytest.mark.parametrize("kv_dtype", [torch.bfloat16, torch.float8_e4m3fn])
+@pytest.mark.parametrize("rows_kernel", [False, True])
+def test_device_side_distribution_with_256_wide_heads(pkg, wl, gpu, monkeypatch, kv_dtype, rows_kernel):
+    """The jitted reference call always holds the composition on the device (rpa_v3:1676, 2060-2090), 256-wide
+    heads included (test_flashattention_misc.py:10-58): bit for bit the host-integer results when both modes cut
+    the decode rows alike, on a bucket padded with empty sequences and spare tokens; chunks through the flash
+    kernel and through the row kernel."""
+    tol = BF16_TOL if kv_dtype == torch.bfloat16 else FP8_TOL
+    if rows_kernel:
+        monkeypatch.setenv("RPA_PREFILL_ROWS256", "1")
+    q_lens = [1] * 4 + [70, 200, 33]
+    kv_lens = [700, 33, 3000, 1] + [70, 900, 640]
+    b = wl.make_batch("static256", q_lens, kv_lens, num_q_heads=8, num_kv_heads=2, head_dim=256, page_size=32, seed=8411,
+                      kv_dtype=kv_dtype, pad_tokens=21, pad_seqs=6)
+    wl.plant_needles(b, seed=6, logit=10.0)
+    want = oracle_out(b)
+    g = b.to(gpu)
+    T = sum(q_lens)
+    kw = dict(sm_scale=b.sm_scale, k_scale=g.k_scale, v_scale=g.v_scale)
+
+    def run(dist, **extra):
+        out, _ = pkg.ragged_paged_attention(g.q, None, None, g.kv_cache, g.kv_lens, g.page_indices, g.cu_q_lens,
+                                            g.cu_kv_lens, dist, None, **kw, **extra)
+        torch.cuda.synchronize()
+        return out[:T].cpu()
+
+    # whole rows and whole K/V ranges in both modes (few heads: a launch this small would otherwise cut its K/V
+    # ranges into a number of pieces that depends on the bounds each mode knows)
+    monkeypatch.setenv("RPA_PREFILL_SPLITS", "0")
+    host_whole = run(b.distribution.cpu().numpy(), num_splits=1, max_kv_len=max(kv_lens), max_q_len=max(q_lens))
+    assert_parity(host_whole.float(), want.float(), **tol)
+    dev_whole = run(g.distribution, num_splits=1)
+    assert torch.equal(dev_whole.view(torch.int16), host_whole.view(torch.int16))
+    monkeypatch.delenv("RPA_PREFILL_SPLITS")
+    dev_auto = run(g.distribution)  # the plan for the bounds: every sequence a possible decode row, rows and ranges cut
+    assert_parity(dev_auto.float(), want.float(), **tol)
+    # the same bucket holding only decode rows / only chunks
+    for dist in ([4, 4, 4], [0, 0, 3]):
+        sub_q = [1] * 4 if dist[2] == 4 else [70, 200, 33]
+        sub_kv = kv_lens[:4] if dist[2] == 4 else [70, 900, 640]
+        c = wl.make_batch("static256b", sub_q, sub_kv, num_q_heads=8, num_kv_heads=2, head_dim=256, page_size=32,
+                          seed=8412, kv_dtype=kv_dtype, pad_seqs=11 - len(sub_q), pad_tokens=5)
+        gc = c.to(gpu)
+        out, _ = pkg.ragged_paged_attention(gc.q, None, None, gc.kv_cache, gc.kv_lens, gc.page_indices, gc.cu_q_lens,
+                                            gc.cu_kv_lens, torch.tensor(dist, dtype=torch.int32, device=gpu), None,
+                                            sm_scale=c.sm_scale, k_scale=gc.k_scale, v_scale=gc.v_scale)
+        torch.cuda.synchronize()
+        assert_parity(out[: sum(sub_q)].cpu().float(), oracle_out(c).float(), **tol)
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+def test_more_decode_rows_than_a_grid_dimension_holds(pkg, wl, gpu, head_dim):
+    """70000 decode rows in one call (the reference loops over any number of sequences, rpa_v3:1126-1135): rows
+    are folded onto the first grid dimension, which has the room.  Short rows; a sample against the oracle, and
+    the rows past 65000 against the same rows run as a batch of their own."""
+    n = 70000
+    rng = np.random.default_rng(5)
+    kv_lens = rng.integers(1, 40, size=n)
+    b = wl.make_batch("many_rows", [1] * n, kv_lens, num_q_heads=4, num_kv_heads=2, head_dim=head_dim, page_size=16,
+                      seed=91, device=gpu)
+    got = gpu_out(pkg, b, gpu)
+    assert torch.isfinite(got.float()).all()
+    picks = [0, 1, 65534, 65535, 65536, n - 1] + [int(x) for x in rng.integers(0, n, size=20)]
+    sample = wl.sub_batch(b, picks)
+    want = oracle_out(sample)
+    assert_parity(got[torch.tensor(sample.meta["rows"])].float(), want.float(), **BF16_TOL)
+    # (to rounding: the large batch deals its rows out evenly and cuts some, the small one runs whole rows)
+    tail = wl.sub_batch(b, list(range(65000, n)))
+    again = gpu_out(pkg, tail, gpu)
+    assert_parity(got[65000:].float(), again.float(), **BF16_TOL)
+
+
 # ---- prefill launches that would leave most of the GPU idle: K/V ranges cut into pieces + merge ----
 KV_PIECE_CASES = [
     # name, q_lens, kv_lens, Hq, Hkv, P, window, sink, whether the automatic plan cuts the launch
