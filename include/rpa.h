@@ -117,11 +117,16 @@ typedef struct RpaParams {
   int32_t decode_end;
   /* ---- host-side bounds used only to size grids (never to index memory) ---- */
   int32_t max_kv_len;         /* upper bound of kv_lens[0:num_seqs]; 0 => pages_per_seq*P or total_pages*P */
-  int32_t max_q_len;          /* upper bound of q_len over [decode_end, num_seqs); 0 => T */
+  int32_t max_q_len;          /* upper bound of q_len over [decode_end, num_seqs); 0 => T.  A promise: rows of a
+                                 longer sequence past the bound are not computed */
   int32_t num_splits;         /* decode split-KV count per sequence; 0 => automatic */
   /* ---- options ---- */
   int32_t sliding_window;     /* 0 => off */
-  float sm_scale;
+  float sm_scale;             /* the pipelined prefill kernel (bf16 cache, 128-wide heads, causal, no option)
+                                 multiplies the bf16 queries by sm_scale * log2(e) and rounds them to bf16 once,
+                                 where the reference scales the f32 scores (:149): element-wise inside the
+                                 reference's rtol = atol = 2e-2, and at most 1.5e-2 of a row's norm on rows whose
+                                 weight sits on one or two keys (1e-2 for every other path) */
   float soft_cap;             /* 0 => off */
   float mask_value;           /* 0 => default -0.7 * FLT_MAX */
   /* sum of kv_lens over the decode rows (host-side, balances the split plan); 0 => unknown */
@@ -154,7 +159,9 @@ typedef struct RpaParams {
    * decode_end and sum_decode_kv_len are ignored and num_seqs is only the static bound S (the length of
    * kv_lens): grids are sized from T, S and the page-table bound, every workgroup reads the
    * composition itself and the ones with nothing to do leave at once, so one compiled call serves
-   * every batch of a bucket and nothing is read back to the host.  head_dim 128 only. */
+   * every batch of a bucket and nothing is read back to the host.  128- and 256-wide heads alike.
+   * Neither mode limits the sequences or tokens of a call beyond int32: rows are folded onto the first
+   * grid dimension. */
   const int32_t* distribution;
 } RpaParams;
 
