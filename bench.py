@@ -25,6 +25,8 @@ One JSON line is printed:
               frac_of_achievable (of these)
   settle_ms   untimed steps of the same workload run before the warm-up so that the device's clocks have
               left their idle state when the W warm-up and K timed steps start (--settle-ms 0 switches it off)
+  host_path   host microseconds per rpa_attention call and per plan-only call, and C1's device time per call
+              inside one HIP graph (its latency figure: C1 is bound by launches, not by bytes)
   cpu_baseline  the CPU oracle timed on this box's host cores on a bounded sample
 
 The reference's published perf-guard workloads (32 rows) go to stderr as a JSON line of their own; the line on
@@ -428,6 +430,57 @@ def measure_ceilings(dev, nbytes=2 << 30, reps=5):
     }
 
 
+def host_path(pkg, wl, dev, calls=2000, reps=50):
+    """What the host side of a call costs, on the latency-bound configuration (C1: 8 decode rows, 14 us of GPU
+    work): microseconds of host time per rpa_attention through the C ABI (ctypes included; the queue is drained
+    first and the loop is short enough not to fill it), the same for the plan arithmetic alone
+    (rpa_workspace_bytes: shape table, split plan, no launch), and the device time per call when `reps` calls
+    are replayed as one HIP graph (kernels back to back, no host in between)."""
+    import ctypes
+
+    import torch
+
+    b = wl.config_c1(dev)
+    call = make_call(pkg, b)
+    lib = pkg._lib.load()
+    for _ in range(20):
+        call.attention()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        call.attention()
+    t1 = time.perf_counter()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    pp = ctypes.byref(call.params)
+    t3 = time.perf_counter()
+    for _ in range(calls):
+        lib.rpa_workspace_bytes(pp)
+    t4 = time.perf_counter()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            call.attention()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(reps):
+            call.attention()
+    graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = _events(2)
+    e0.record()
+    graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return {"workload": b.name, "host_us_per_rpa_attention": (t1 - t0) * 1e6 / calls,
+            "wall_us_per_call_drained": (t2 - t0) * 1e6 / calls,
+            "host_us_per_plan_only_call": (t4 - t3) * 1e6 / calls,
+            "device_us_per_call_in_one_graph": e0.elapsed_time(e1) * 1e3 / reps, "calls": calls, "graph_calls": reps}
+
+
 def cpu_baseline(wl, budget_s=10.0, prefill_budget_s=8.0):
     """CPU oracle on a bounded sample of the default workload: its first decode rows
     (same seeded lengths and layout, values drawn on the host), and -- reported under `prefill` -- one
@@ -673,6 +726,8 @@ def main():
             "what": what + "; the rows are on stderr", "workloads": len(rows),
             "speedup_vs_v6e_min_max": [min(v6), max(v6)], "speedup_vs_v7_min_max": [min(v7), max(v7)],
             "ahead_of_v6e": sum(x > 1 for x in v6), "ahead_of_v7": sum(x > 1 for x in v7)}
+    if not args.main_only:
+        line["host_path"] = host_path(pkg, wl, dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(line))

@@ -279,6 +279,17 @@ RPA_API int rpa_prefill(const RpaParams* p, void* stream);
 RPA_API int rpa_attention(const RpaParams* p, void* stream);
 
 /*
+ * Which launch shape a call would take, as text: the row of the library's shape table (kernel family, query
+ * positions x query heads x K/V tokens per workgroup, waves walked together, resident waves), the split plan
+ * of the decode rows and the workspace behind it.  The counterpart of the reference's get_tuned_block_sizes /
+ * get_default_block_sizes, which answer the same question for its tile table
+ * (kernels/ragged_paged_attention/tuned_block_sizes_v3.py:2163-2229, ragged_paged_attention_v3.py:1490-1638).
+ * Host arithmetic only (no launch, no device read).  Writes at most len - 1 characters plus a NUL into buf and
+ * returns the length of the whole text (as snprintf does), or a negative RpaStatus.
+ */
+RPA_API int rpa_describe_plan(const RpaParams* p, char* buf, size_t len);
+
+/*
  * rpa_attention for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid it).  No counterpart in the reference, where XLA owns
  * every buffer.  Same arguments and results as rpa_attention, except that p->workspace and
@@ -314,6 +325,9 @@ RPA_API int rpa_mla_decode(const RpaMlaParams* p, void* stream);
  */
 RPA_API size_t rpa_mla_attention_workspace_bytes(const RpaMlaParams* p);
 RPA_API int rpa_mla_attention(const RpaMlaParams* p, void* stream);
+
+/* rpa_describe_plan for the absorbed-MLA entry points: token_rows = 0 describes rpa_mla_decode, 1 rpa_mla_attention. */
+RPA_API int rpa_mla_describe_plan(const RpaMlaParams* p, int token_rows, char* buf, size_t len);
 
 /*
  * Write the new latent rows into the paged cache: update_kv_cache of kernels/mla/v1/ref.py:56-105

@@ -45,6 +45,7 @@ EXPORTED_SYMBOLS = (
     "rpa_decode",
     "rpa_prefill",
     "rpa_attention",
+    "rpa_describe_plan",
     "rpa_noalloc_max_workspace_bytes",
     "rpa_attention_noalloc",
     "rpa_kv_write",
@@ -52,6 +53,7 @@ EXPORTED_SYMBOLS = (
     "rpa_mla_attention_workspace_bytes",
     "rpa_mla_attention",
     "rpa_mla_kv_write",
+    "rpa_mla_describe_plan",
 )
 
 
@@ -193,6 +195,10 @@ def load() -> ctypes.CDLL:
     lib.rpa_mla_attention.argtypes = [P(RpaMlaParams), ctypes.c_void_p]
     lib.rpa_mla_kv_write.restype = ctypes.c_int
     lib.rpa_mla_kv_write.argtypes = [P(RpaMlaParams), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    lib.rpa_describe_plan.restype = ctypes.c_int
+    lib.rpa_describe_plan.argtypes = [P(RpaParams), ctypes.c_char_p, ctypes.c_size_t]
+    lib.rpa_mla_describe_plan.restype = ctypes.c_int
+    lib.rpa_mla_describe_plan.argtypes = [P(RpaMlaParams), ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
     _lib = lib
     return lib
 
@@ -209,3 +215,24 @@ class RpaError(ValueError):
 def check(code: int):
     if code != 0:
         raise RpaError(code, load().rpa_last_error().decode("utf-8", "replace"))
+
+
+def describe_plan(params) -> str:
+    """``rpa_describe_plan`` / ``rpa_mla_describe_plan``: the launch shape a call would take, as text."""
+    lib = load()
+    buf = ctypes.create_string_buffer(2048)
+    if isinstance(params, RpaMlaParams):
+        raise TypeError("use describe_mla_plan(params, token_rows)")
+    n = lib.rpa_describe_plan(ctypes.byref(params), buf, len(buf))
+    if n < 0:
+        check(n)
+    return buf.value.decode()
+
+
+def describe_mla_plan(params, token_rows: bool) -> str:
+    lib = load()
+    buf = ctypes.create_string_buffer(1024)
+    n = lib.rpa_mla_describe_plan(ctypes.byref(params), 1 if token_rows else 0, buf, len(buf))
+    if n < 0:
+        check(n)
+    return buf.value.decode()

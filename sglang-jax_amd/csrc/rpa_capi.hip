@@ -262,32 +262,32 @@ int64_t decode_kv_bytes(const RpaParams* p) {
   return tokens * 2 * p->num_kv_heads * p->head_dim * esize_of(p->kv_dtype);
 }
 
-// Waves of a workgroup = neighbouring kv heads walked together (their rows are adjacent in the
-// cache).  Four on batches that stream tens of megabytes (C2 109 -> 105 us, C4 243 -> 238 us
-// against two); two on small, latency-bound batches, which want their few waves spread over
-// more CUs (C1 14.0 against 15.9 us).
+// The decode rows' row of the shape table (rpa_shapes.h): waves of a workgroup = neighbouring kv heads walked
+// together (their rows are adjacent in the cache), and the waves resident at once = bytes in flight.
+const rpa::ShapeRule& decode_shape(const RpaParams* p) {
+  rpa::ShapeKey k = {};
+  k.stage = rpa::kStageDecode;
+  k.kv_bits = 8 * esize_of(p->kv_dtype);
+  k.head_dim = p->head_dim;
+  k.heads = p->num_q_heads / p->num_kv_heads;
+  k.kv_bytes = decode_kv_bytes(p);
+  return rpa::select_shape(k);
+}
+
 int decode_waves_per_wg(const RpaParams* p) {
-  const int dflt = decode_kv_bytes(p) >= (32ll << 20) ? 4 : 2;
   const int forced = rpa::tuning().decode_waves_per_wg;
-  const int nw = forced > 0 ? forced : dflt;
+  const int nw = forced > 0 ? forced : decode_shape(p).waves_per_wg;
   return std::max(1, std::min(std::min(nw, 4), p->num_kv_heads));
 }
 
-// Decode waves resident at once.  A wave keeps one 32-token block of one head in flight: 16 KiB
-// of a 16-bit cache, 8 KiB of an fp8 one.  About 14 MB in flight saturate HBM; beyond that the
-// queues only get longer and DRAM locality worse (measured, C2 / C3 decode: 896 waves
-// 104.1 / 356 us, 1024: 105.2 / 362, 2048: 108.5 / 367; fp8 C4: 2048 best, 1536 equal, 1024
-// -25 %).  So four waves per CU for a 16-bit cache, less an eighth (the same 85 % the fixed plan
-// aims at on ragged rows), eight per CU for fp8 -- always a whole number of workgroups, and
-// never a workgroup count between one and two per CU, which the dispatcher spreads unevenly
-// (1152 waves in 4-wave workgroups: 133 us on C2).
+// Always a whole number of workgroups, and never a workgroup count between one and two per CU, which the
+// dispatcher spreads unevenly (1152 waves in 4-wave workgroups: 133 us on C2).
 int decode_wave_capacity(const RpaParams* p) {
   const int env = rpa::tuning().decode_wave_capacity;
   if (env > 0) return env;
   const int cus = wave_capacity() / 8;
-  if (esize_of(p->kv_dtype) == 1) return cus * 8;
   const int nw = decode_waves_per_wg(p);
-  return std::max(nw, cus * 4 * 7 / 8 / nw * nw);
+  return std::max(nw, cus * decode_shape(p).resident_x8 / 8 / nw * nw);
 }
 
 int decode_wgs(const RpaParams* p) { return std::max(1, decode_wave_capacity(p) / decode_waves_per_wg(p)); }
@@ -729,6 +729,53 @@ int rpa_attention(const RpaParams* p, void* stream) {
   return rpa_prefill(p, stream);
 }
 
+int rpa_describe_plan(const RpaParams* p_in, char* buf, size_t len) {
+  int rc = rpa_validate(p_in);
+  if (rc != RPA_OK) return rc;
+  if (!buf || len == 0) return fail(RPA_EINVAL_NULL, "buf is NULL or empty");
+  const RpaParams pv = planning_view(p_in);
+  const RpaParams* p = &pv;
+  size_t at = 0;
+  auto put = [&](const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    const size_t from = std::min(at, len - 1);
+    const int n = vsnprintf(buf + from, len - from, fmt, ap);
+    va_end(ap);
+    if (n > 0) at += (size_t)n;
+  };
+  buf[0] = 0;
+  if (p->decode_end > 0 && p->mask_mode != RPA_MASK_CUSTOM) {
+    const rpa::ShapeRule& r = decode_shape(p);
+    if (p->head_dim == 256) {
+      const SplitPlan sp = rows256_plan(p);
+      put("decode: shape=%s kernel=rpa_rows256_kernel rows=%d pieces_per_row=%d", r.name, p->decode_end, sp.splits);
+    } else {
+      const SplitPlan sp = decode_plan(p);
+      const bool bal = use_balanced(p, sp);
+      put("decode: shape=%s kernel=%s rows=%d waves_per_wg=%d", r.name,
+          bal ? "rpa_decode_balanced_kernel" : "rpa_decode_splitkv_kernel", p->decode_end, decode_waves_per_wg(p));
+      if (bal) put(" resident_waves=%d merge=rpa_combine_balanced_kernel", decode_wave_capacity(p));
+      else put(" pieces_per_row=%d chunk=%d merge=%s", sp.splits, sp.chunk, sp.splits > 1 ? "rpa_combine_kernel" : "none");
+    }
+    put(" workspace=%zu\n", required_workspace_bytes(p_in));
+  }
+  rpa::PrefillArgs a;
+  if (prefill_args(p_in, a)) {
+    if (p->head_dim == 256 && rpa::tuning().prefill_rows256 != 0) {
+      put("prefill: kernel=rpa_rows256_kernel (RPA_PREFILL_ROWS256)\n");
+    } else {
+      const rpa::ShapeRule& r = rpa::prefill_shape_of(a);
+      const char* kernel = r.kernel == rpa::kKernelPrefillPipe ? "rpa_prefill_pipe_kernel"
+                           : (r.kernel == rpa::kKernelPrefillStaged ? "rpa_prefill_staged_kernel" : "rpa_prefill_async_kernel");
+      const PrefillWorkspace w = prefill_workspace(p_in, a);
+      put("prefill: shape=%s kernel=%s tile=%dx%dx%d kv_pieces_with_workspace=%d mask_bits=%s optional_workspace=%zu\n",
+          r.name, kernel, r.tile_q, r.tile_heads, r.tile_kv, w.splits, w.bits_bytes ? "yes" : "no", w.total);
+    }
+  }
+  return (int)std::min<size_t>(at, 0x7fffffff);
+}
+
 size_t rpa_noalloc_max_workspace_bytes(void) { return kNoAllocScratchBytes; }
 
 int rpa_attention_noalloc(const RpaParams* p, void* stream) {
@@ -917,6 +964,26 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   }
   return check_hip(rpa::launch_mla_decode(a, static_cast<hipStream_t>(stream)),
                    token_rows ? "rpa_mla_attention" : "rpa_mla_decode");
+}
+
+int rpa_mla_describe_plan(const RpaMlaParams* p, int token_rows, char* buf, size_t len) {
+  int rc = mla_validate(p);
+  if (rc != RPA_OK) return rc;
+  if (!buf || len == 0) return fail(RPA_EINVAL_NULL, "buf is NULL or empty");
+  const int64_t rows = token_rows ? p->num_tokens : p->num_seqs;
+  rpa::MlaDecodeArgs a = {};
+  a.pt.page_size = p->page_size;
+  a.sm.soft_cap = p->soft_cap;
+  a.fp8 = p->cache_dtype == RPA_KV_FP8_E4M3 ? 1 : 0;
+  a.Hq = p->num_q_heads;
+  a.row_stride = p->row_stride;
+  const rpa::ShapeRule& r = rpa::select_shape(rpa::mla_shape_key(a), rpa::mla_shape_skip(rpa::tuning()));
+  const SplitPlan sp = mla_plan(p, std::max<int64_t>(rows, 1));
+  const bool bal = rows > 0 && mla_use_balanced(p, sp, token_rows != 0);
+  return snprintf(buf, len, "mla: shape=%s rows=%lld waves_per_wg=%d heads_per_wg=%d share=%d plan=%s pieces_per_row=%d "
+                  "workgroups=%d workspace=%zu\n",
+                  r.name, (long long)rows, r.waves_per_wg, r.tile_heads, r.share, bal ? "balanced" : "fixed",
+                  bal ? 0 : sp.splits, bal ? mla_wgs() : 0, mla_workspace(p, rows, token_rows != 0));
 }
 
 int rpa_mla_decode(const RpaMlaParams* p, void* stream) { return mla_run(p, stream, false); }

@@ -5,6 +5,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "rpa_shapes.h"
+#include "rpa_tuning.h"
+
 namespace rpa {
 
 // How K and V rows of one (page, token, kv head) are addressed, in bytes.
@@ -186,6 +189,10 @@ hipError_t launch_rows256(const DecodeArgs& a, int seq_begin, int seq_end, int m
                           hipStream_t stream);
 hipError_t launch_kv_write(const KvWriteArgs& a, hipStream_t stream);
 hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream);
+// The rows of the shape table (rpa_shapes.h) these launchers select for a call, RPA_* overrides applied.
+const ShapeRule& prefill_shape_of(const PrefillArgs& a);
+ShapeKey mla_shape_key(const MlaDecodeArgs& a);
+unsigned mla_shape_skip(const Tuning& tune);
 hipError_t launch_mla_kv_write(const MlaWriteArgs& a, hipStream_t stream);
 
 }  // namespace rpa

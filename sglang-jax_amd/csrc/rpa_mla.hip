@@ -28,6 +28,7 @@
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
+#include "rpa_shapes.h"
 #include "rpa_tuning.h"
 #include "rpa_mla_pipe_loop.inc"
 #include "rpa_mla_wide_loop.inc"
@@ -1271,6 +1272,24 @@ hipError_t launch_mla_kv_write(const MlaWriteArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+ShapeKey mla_shape_key(const MlaDecodeArgs& a) {
+  const int P = a.pt.page_size;
+  ShapeKey k = {};
+  k.stage = kStageMla;
+  k.kv_bits = a.fp8 ? 8 : 16;
+  k.head_dim = 576;
+  k.heads = a.Hq;
+  k.options = (a.sm.soft_cap != 0.f ? kOptSoftCap : 0u) | ((P % kTok) != 0 ? kOptOddPages : 0u) |
+              ((P & (P - 1)) != 0 ? kOptNotPow2Pages : 0u) |
+              ((int64_t)a.row_stride * 2 * P >= (int64_t(1) << 32) ? kOptWidePages : 0u);
+  return k;
+}
+
+unsigned mla_shape_skip(const Tuning& tune) {
+  return (tune.mla_pipe == 0 ? (1u << kKernelMlaWide) | (1u << kKernelMlaPipe) : 0u) |
+         (tune.mla_wide == 0 ? (1u << kKernelMlaWide) : 0u) | (tune.mla_shared_tiles == 0 ? (1u << kKernelMlaShared) : 0u);
+}
+
 hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   if (a.num_rows <= 0) return hipSuccess;
   const int head_groups = (a.Hq + 127) / 128;
@@ -1279,16 +1298,14 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   const dim3 grid((unsigned)max(a.max_splits, 1) * (unsigned)a.num_rows, 1, head_groups), block(512);
   const bool uniform = (a.pt.page_size % kTok) == 0;
   const bool cap = a.sm.soft_cap != 0.f;
-  // the assembly tile loop: whole tiles inside one page, every wave of a workgroup at work
+  // the kernel family by shape (rpa_shapes.h): wide workgroups and the assembly tile loops need whole tiles inside
+  // power-of-two pages, no soft cap and head counts in multiples of 128; with at most 64 heads (a tensor-parallel
+  // share) the waves of a workgroup share each tile of a block of 16 heads; everything else runs the compiled
+  // loop.  RPA_MLA_PIPE=0, RPA_MLA_WIDE=0 and RPA_MLA_SHARED_TILES=0 take a family out of the selection.
   const Tuning& tune = tuning();
-  const bool use_pipe = tune.mla_pipe != 0;
-  const int P = a.pt.page_size;
-  const bool pipe = use_pipe && uniform && !cap && (P & (P - 1)) == 0 && (a.Hq % 128) == 0 &&
-                    (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);
-  // at most 64 heads (a tensor-parallel share): the waves of a workgroup share each tile of a block of 16 heads
-  // (mla_segment, DS) instead of leaving most of them without heads.  RPA_MLA_SHARED_TILES=0: one wave per block,
-  // as with 128 heads.
-  const int ds = (uniform && !cap && a.Hq <= 64 && tune.mla_shared_tiles != 0) ? (a.Hq <= 16 ? 8 : (a.Hq <= 32 ? 4 : 2)) : 1;
+  const ShapeRule& shape = select_shape(mla_shape_key(a), mla_shape_skip(tune));
+  const bool pipe = shape.kernel == kKernelMlaWide || shape.kernel == kKernelMlaPipe;
+  const int ds = shape.kernel == kKernelMlaShared ? shape.share : 1;
   if (ds != 1) {
 #define RPA_MLA_DS(KERNEL, GRID, F8)                                                                                  \
   do {                                                                                                                \
@@ -1352,7 +1369,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   }
   // wide workgroups (four waves of 32 heads) wherever the assembly loop applies; RPA_MLA_WIDE=0 keeps the
   // eight-wave kernels
-  const bool wide = tune.mla_wide != 0 && pipe;
+  const bool wide = shape.kernel == kKernelMlaWide;
   // RPA_MLA_WIDE=32: the wide loop on 32x32x16 matrix instructions (one head per lane and half).  Half the matrix
   // instructions, and 8 % faster than the default loop when neither reads its operands -- but its 32-row LDS
   // reads collide on the 1184-byte row pitch that suits the 16-row reads (7 % slower as a whole): opt-in until

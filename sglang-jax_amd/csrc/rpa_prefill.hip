@@ -580,22 +580,24 @@ hipError_t launch_mask_bits(const PrefillArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-bool takes_pipe_kernel(const PrefillArgs& a) {
-  const Tuning& tune = tuning();
-  return tune.prefill_pipe != 0 && tune.prefill_staged != 1 && prefill_pipe_applies(a);
-}
+bool takes_pipe_kernel(const PrefillArgs& a) { return prefill_shape(a).kernel == kKernelPrefillPipe; }
 }  // namespace
 
 namespace {
-// The compiled flash kernel's short-chunk tile: 32 positions x 4 heads per workgroup for chunks of at most 64
-// tokens (128-wide heads, heads in fours; RPA_PREFILL_PIPE_TILE=32|128 forces either).
+// The compiled flash kernels' short-chunk tile: 32 positions x 4 heads per workgroup (rows "prefill_options_short"
+// and "prefill_fp8_short" of the shape table).  RPA_PREFILL_STAGED=1 (bf16 rows through the register-staged
+// kernel, a testing path) has no such tile.
 bool compiled_short_chunk_tile(const PrefillArgs& a) {
-  const bool force_staged = tuning().prefill_staged == 1;
-  if ((force_staged && !a.fp8) || a.head_dim != 128 || (a.G % 4) != 0) return false;
-  const int force_tile = tuning().prefill_pipe_tile;
-  return force_tile ? force_tile == 32 : a.max_q_len <= 64;
+  if (tuning().prefill_staged == 1 && !a.fp8) return false;
+  const ShapeRule& r = prefill_shape(a);
+  return r.kernel != kKernelPrefillPipe && r.tile_q == 32;
 }
 }  // namespace
+
+const ShapeRule& prefill_shape_of(const PrefillArgs& a) {
+  // RPA_PREFILL_STAGED=1 on a bf16 cache is a testing path outside the table: the fp8 kernel's rows
+  return prefill_shape(a);
+}
 
 int prefill_kv_splits(const PrefillArgs& a) {
   const int nseq = a.seq_end - a.seq_begin;

@@ -5,6 +5,7 @@
 
 #include "rpa_common.h"
 #include "rpa_kernels.h"
+#include "rpa_shapes.h"
 #include "rpa_tuning.h"
 
 namespace rpa {
@@ -330,6 +331,34 @@ __device__ __forceinline__ void write_rows(const PrefillArgs& a, const Work& w, 
                    pack_bf16x2(O[d][4 * vq + 2] * inv, O[d][4 * vq + 3] * inv)};
       *reinterpret_cast<u32x2_t*>(op + d * 32 + vq * 8) = o;
     }
+}
+
+// -------------------------------------------------- the launch shape of a prefill call (rpa_shapes.h)
+// RPA_PREFILL_PIPE=0 / RPA_PREFILL_STAGED=1 take the assembly kernel out of the selection, RPA_PREFILL_PIPE_TILE
+// = 32 | 128 and RPA_PREFILL_PIPE_NQ=2 decide the short-chunk question by hand.
+inline ShapeKey prefill_shape_key(const PrefillArgs& a) {
+  const Tuning& tune = tuning();
+  const int P = a.pt.page_size;
+  ShapeKey k = {};
+  k.stage = kStagePrefill;
+  k.kv_bits = a.fp8 ? 8 : 16;
+  k.head_dim = a.head_dim;
+  k.heads = a.G;
+  k.max_q_len = a.max_q_len;
+  if (tune.prefill_pipe_tile == 32) k.max_q_len = 1;
+  else if (tune.prefill_pipe_tile != 0 || tune.prefill_pipe_nq == 2) k.max_q_len = 0;
+  k.options = ((a.sm.soft_cap != 0.f || a.sm.round_logits != 0) ? kOptSoftCap : 0u) |
+              (a.sm.mask_mode != 0 ? kOptMaskOther : 0u) | (a.sm.xai_len > 0.f ? kOptTemperature : 0u) |
+              (a.sm.q_scale > 0.f ? kOptQScale : 0u) | ((P % kBN) != 0 ? kOptOddPages : 0u) |
+              ((P & (P - 1)) != 0 ? kOptNotPow2Pages : 0u) |
+              (a.kv.page_stride >= (int64_t(1) << 32) ? kOptWidePages : 0u);
+  return k;
+}
+
+inline const ShapeRule& prefill_shape(const PrefillArgs& a) {
+  const Tuning& tune = tuning();
+  const unsigned skip = (tune.prefill_pipe == 0 || tune.prefill_staged == 1) ? (1u << kKernelPrefillPipe) : 0u;
+  return select_shape(prefill_shape_key(a), skip);
 }
 
 // -------------------------------------------------- K/V ranges cut into pieces (under-filled launches)

@@ -480,19 +480,16 @@ __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kerne
 
 }  // namespace
 
+// (what the assembly kernel can run is written down once, as the conditions of its rows in the shape table)
 bool prefill_pipe_applies(const PrefillArgs& a) {
-  const int P = a.pt.page_size;
-  return !a.fp8 && a.head_dim == 128 && P >= kBN && (P & (P - 1)) == 0 && a.kv.page_stride < (int64_t(1) << 32) &&
-         a.sm.mask_mode == 0 && a.sm.soft_cap == 0.f && a.sm.round_logits == 0 && !(a.sm.xai_len > 0.f) &&
-         !(a.sm.q_scale > 0.f);
+  return select_shape(prefill_shape_key(a)).kernel == kKernelPrefillPipe;
 }
 
 namespace {
 int forced_nq() { return tuning().prefill_pipe_nq; }
-// 32 positions x 4 heads per workgroup instead of 128 x 1
+// 32 positions x 4 heads per workgroup instead of 128 x 1: row "prefill_pipe_short" of the shape table
 bool short_chunk_tile(const PrefillArgs& a, int nq) {
-  const int force_tile = tuning().prefill_pipe_tile;
-  return nq == 1 && (a.G % 4) == 0 && (force_tile ? force_tile == 32 : a.max_q_len <= 64);
+  return nq == 1 && select_shape(prefill_shape_key(a)).tile_q == 32;
 }
 }  // namespace
 

@@ -340,3 +340,88 @@ def test_generated_assembly_is_up_to_date(tmp_path):
         subprocess.run([sys.executable, str(work / gen)], check=True, env=env, stdout=subprocess.DEVNULL)
         with open(work / inc) as f, open(os.path.join(csrc, inc)) as g:
             assert f.read() == g.read(), f"{inc} is stale: run {gen}"
+
+
+# ------------------------------------------------------------------ the shape table (csrc/rpa_shapes.h)
+def _shape_params(pkg, *, S, decode_end, T, Hq, Hkv, D=128, P=64, fp8=False, max_q=0, max_kv=0, sum_dec=0, **opts):
+    p = base_params(pkg)
+    p.num_tokens, p.num_seqs, p.num_q_heads, p.num_kv_heads = T, S, Hq, Hkv
+    p.head_dim, p.page_size, p.total_pages = D, P, 1 << 20
+    p.decode_end, p.max_q_len, p.max_kv_len, p.sum_decode_kv_len = decode_end, max_q, max_kv, sum_dec
+    p.kv_dtype = pkg._lib.RPA_KV_FP8_E4M3 if fp8 else pkg._lib.RPA_KV_BF16
+    for k, v in opts.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_shape_table_rows_of_the_benchmark_configurations(pkg):
+    """rpa_describe_plan: which row of the shape table, which kernel and which split plan a call takes (the
+    reference answers the same question with get_tuned_block_sizes, tuned_block_sizes_v3.py:2163-2229).
+    The five benchmark shapes and the option / head-width / chunk-length branches of the table."""
+    d = pkg._lib.describe_plan
+    c1 = d(_shape_params(pkg, S=8, decode_end=8, T=8, Hq=16, Hkv=8, P=16, max_kv=512, sum_dec=2300))
+    assert "shape=decode_bf16_small" in c1 and "rpa_decode_splitkv_kernel" in c1 and "waves_per_wg=2" in c1
+    assert "prefill" not in c1
+    c2 = d(_shape_params(pkg, S=64, decode_end=56, T=8760, Hq=32, Hkv=8, max_q=2048, max_kv=4096, sum_dec=130000))
+    assert "shape=decode_bf16_stream kernel=rpa_decode_balanced_kernel rows=56 waves_per_wg=4 resident_waves=896" in c2
+    assert "shape=prefill_pipe kernel=rpa_prefill_pipe_kernel tile=128x1x64 kv_pieces_with_workspace=1" in c2
+    c3 = d(_shape_params(pkg, S=16, decode_end=16, T=16, Hq=32, Hkv=8, max_kv=32768, sum_dec=16 * 32768))
+    assert "shape=decode_bf16_stream kernel=rpa_decode_splitkv_kernel" in c3 and "merge=rpa_combine_kernel" in c3
+    c4 = d(_shape_params(pkg, S=128, decode_end=128, T=128, Hq=64, Hkv=8, fp8=True, max_kv=8192, sum_dec=590000))
+    assert "shape=decode_fp8_stream kernel=rpa_decode_balanced_kernel" in c4 and "resident_waves=2048" in c4
+    # chunks of at most 64 tokens with heads in fours: the short-chunk tile; a long prompt on few heads is cut
+    short = d(_shape_params(pkg, S=64, decode_end=0, T=1024, Hq=32, Hkv=8, max_q=16, max_kv=4096))
+    assert "shape=prefill_pipe_short" in short and "tile=32x4x64" in short
+    one = d(_shape_params(pkg, S=1, decode_end=0, T=16, Hq=8, Hkv=2, max_q=16, max_kv=32768))
+    assert "kv_pieces_with_workspace=1 " not in one  # an under-filled launch cuts its K/V range
+    # options and cache types leave the assembly kernel
+    assert "shape=prefill_options kernel=rpa_prefill_async_kernel" in d(_shape_params(
+        pkg, S=2, decode_end=0, T=600, Hq=32, Hkv=8, max_q=300, max_kv=600, soft_cap=30.0))
+    assert "shape=prefill_fp8 kernel=rpa_prefill_staged_kernel" in d(_shape_params(
+        pkg, S=2, decode_end=0, T=600, Hq=32, Hkv=8, max_q=300, max_kv=600, fp8=True))
+    assert "shape=prefill_pipe " not in d(_shape_params(pkg, S=2, decode_end=0, T=600, Hq=32, Hkv=8, P=48, max_q=300, max_kv=600))
+    wide = d(_shape_params(pkg, S=6, decode_end=4, T=304, Hq=16, Hkv=4, D=256, max_q=200, max_kv=900, sum_dec=3000))
+    assert "shape=decode_256 kernel=rpa_rows256_kernel" in wide and "shape=prefill_256 kernel=rpa_prefill_async_kernel" in wide
+
+
+def test_shape_table_environment_overrides(pkg, monkeypatch):
+    d = pkg._lib.describe_plan
+    p = _shape_params(pkg, S=64, decode_end=56, T=8760, Hq=32, Hkv=8, max_q=2048, max_kv=4096, sum_dec=130000)
+    assert "rpa_prefill_pipe_kernel" in d(p)
+    monkeypatch.setenv("RPA_PREFILL_PIPE", "0")  # the switches are read again whenever the environment changes
+    assert "shape=prefill_options kernel=rpa_prefill_async_kernel" in d(p)
+    monkeypatch.delenv("RPA_PREFILL_PIPE")
+    monkeypatch.setenv("RPA_DECODE_BALANCED", "0")
+    monkeypatch.setenv("RPA_DECODE_WAVES_PER_WG", "2")
+    text = d(p)
+    assert "rpa_decode_splitkv_kernel" in text and "waves_per_wg=2" in text and "rpa_prefill_pipe_kernel" in text
+    monkeypatch.delenv("RPA_DECODE_BALANCED")
+    monkeypatch.delenv("RPA_DECODE_WAVES_PER_WG")
+    assert "rpa_decode_balanced_kernel" in d(p)
+
+
+def test_mla_shape_table_rows(pkg, monkeypatch):
+    def params(Hq, P=64, fp8=False, S=64, T=64, max_kv=16384, sum_kv=590000, soft_cap=0.0):
+        p = pkg._lib.RpaMlaParams()
+        for f in ("ql_nope", "q_pe", "out", "cache_kv", "kv_lens", "page_indices", "cu_q_lens", "cu_kv_lens"):
+            setattr(p, f, 0x1000)
+        p.num_tokens, p.num_seqs, p.num_q_heads = T, S, Hq
+        p.lkv_dim, p.rope_dim, p.page_size, p.total_pages = 512, 64, P, 1 << 16
+        p.row_stride, p.rope_offset = 576, 512
+        p.max_kv_len, p.sum_kv_len, p.sm_scale, p.soft_cap = max_kv, sum_kv, 0.07, soft_cap
+        p.cache_dtype = pkg._lib.RPA_KV_FP8_E4M3 if fp8 else pkg._lib.RPA_KV_BF16
+        return p
+
+    d = pkg._lib.describe_mla_plan
+    c5 = d(params(128), False)
+    assert "shape=mla_wide" in c5 and "waves_per_wg=4" in c5 and "plan=balanced" in c5 and "workgroups=256" in c5
+    assert "shape=mla_pipe" in d(params(128, fp8=True), False)
+    assert "shape=mla_shared_16" in d(params(16), False) and "share=8" in d(params(16), False)
+    assert "shape=mla_shared_64" in d(params(48), False)
+    assert "shape=mla_compiled" in d(params(128, P=16), False)
+    assert "shape=mla_compiled" in d(params(128, soft_cap=30.0), False)
+    assert "shape=mla_compiled" in d(params(160), False)
+    monkeypatch.setenv("RPA_MLA_WIDE", "0")
+    assert "shape=mla_pipe" in d(params(128), False)
+    monkeypatch.setenv("RPA_MLA_PIPE", "0")
+    assert "shape=mla_compiled" in d(params(128), False)
