@@ -941,7 +941,9 @@ static int mla_run(const RpaMlaParams* p, void* stream, bool token_rows) {
   a.num_wgs = mla_wgs();
   a.min_tiles_per_wg = std::max(1, rpa::tuning().mla_min_chunk / 32);
   a.forced_tiles_per_wg = 0;
-  a.piece_pad = std::max(0, rpa::tuning().mla_piece_pad);
+  a.piece_pad = rpa::tuning().mla_piece_pad >= 0
+                    ? rpa::tuning().mla_piece_pad
+                    : rpa::select_shape(rpa::mla_shape_key(a), rpa::mla_shape_skip(rpa::tuning())).piece_pad;
   if (p->num_splits > 0) {
     const int64_t bound = kv_len_bound(p->max_kv_len, p->pages_per_seq, p->page_size, p->total_pages,
                                        p->cu_kv_lens != nullptr);

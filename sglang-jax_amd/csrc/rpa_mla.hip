@@ -36,6 +36,19 @@
 
 namespace rpa {
 
+// Per-workgroup timestamps of the wide balanced kernel, compiled in with -DRPA_MLA_TRACE only (build.py passes
+// extra flags through): for up to four pieces per workgroup the 100 MHz clock at piece entry, first tiles and
+// queries landed, tile loop entered, tile loop left, rows written.  rpa_debug_mla_trace() copies them out.
+#ifdef RPA_MLA_TRACE
+__device__ unsigned long long rpa_mla_trace_buf[1024][4][8];
+#define RPA_MLA_STAMP(slot)                                                                              \
+  do {                                                                                                   \
+    if (threadIdx.x == 0 && trace_piece < 4) rpa_mla_trace_buf[blockIdx.x & 1023][trace_piece][slot] = wall_clock64(); \
+  } while (0)
+#else
+#define RPA_MLA_STAMP(slot) do { } while (0)
+#endif
+
 namespace {
 
 constexpr int kTok = 32;                 // tokens per tile
@@ -733,7 +746,10 @@ constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 // 16 heads on 16x16x32 instructions.
 template <bool M32>
 __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
-                                                 int t_begin, int t_end, const MlaDest dest, char* ring) {
+                                                 int t_begin, int t_end, const MlaDest dest, char* ring,
+                                                 int trace_piece = 0) {
+  (void)trace_piece;
+  RPA_MLA_STAMP(0);
   constexpr int CPW = 2 * kCopiesPerWave;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -795,6 +811,7 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   static_assert(RPA_MLA_WIDE_COPIES_AHEAD == RPA_MLA_WIDE32_COPIES_AHEAD, "one prologue for both loops");
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(RPA_MLA_WIDE_COPIES_AHEAD));
   __syncthreads();
+  RPA_MLA_STAMP(1);
 
   // ---- the reference of the probabilities: per head, the maximum of the first tile's visible scores ----
   float m_init[2];
@@ -900,6 +917,7 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   // `t` and `pg` change inside the block while the inputs are still being read: early-clobber, or the compiler
   // may give an input that happens to hold the same value on entry (the LDS base, 0, and t = 0) the same register
   int k = 0;
+  RPA_MLA_STAMP(2);
   // both loops bind their operands to the same registers
 #define C(n) RPA_MLA_WIDE_C_##n
 #define RPA_WIDE_OPERANDS                                                                                              \
@@ -917,6 +935,7 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
 #undef RPA_WIDE_OPERANDS
 #undef C
   __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the copies issued past the end
+  RPA_MLA_STAMP(3);
 
   // ---- epilogue ----
   const int lo_ = fresh_lane();
@@ -983,6 +1002,13 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   // every wave has left the loop behind its last barrier; the next segment's first copies overwrite slots
   // 0 .. 2, whose last readers (this segment's last steps) may still be running in another wave
   __syncthreads();
+  RPA_MLA_STAMP(4);
+#ifdef RPA_MLA_TRACE
+  if (threadIdx.x == 0 && trace_piece < 4) {
+    rpa_mla_trace_buf[blockIdx.x & 1023][trace_piece][5] = (unsigned long long)((t_end - t_begin + kTok - 1) / kTok);
+    rpa_mla_trace_buf[blockIdx.x & 1023][trace_piece][6] = (unsigned long long)dest.final_rows;
+  }
+#endif
 }
 
 // ---- fixed split plan, wide workgroups: grid = (max_splits * rows, 1, head groups of 128); block = 256 threads
@@ -1043,6 +1069,9 @@ __device__ __forceinline__ void mla_balanced_body(const MlaDecodeArgs& a, Segmen
   const int lane = threadIdx.x & 63;
   const int wg = blockIdx.x;
   const int units = (a.Hq + 127) / 128;
+#ifdef RPA_MLA_TRACE
+  if (threadIdx.x == 0) rpa_mla_trace_buf[blockIdx.x & 1023][0][7] = wall_clock64();  // kernel entry
+#endif
   // prefix sums of tiles over the sequences: every wave scans (the result is wave-uniform)
   int total = 0, seq = -1, seq_first = 0;
   {
@@ -1102,6 +1131,7 @@ __device__ __forceinline__ void mla_balanced_body(const MlaDecodeArgs& a, Segmen
   int nt = mla_tiles(kv_len, a.sm.window);
   const int pad = a.piece_pad;
   bool first_piece = true;
+  int piece_no = 0;  // (only the optional timestamps use it)
   while (x < x_end) {
     const int r = x - seq_first;  // position inside the row's padded extents
     const int unit = r / (nt + pad);
@@ -1124,7 +1154,7 @@ __device__ __forceinline__ void mla_balanced_body(const MlaDecodeArgs& a, Segmen
     dest.final_rows = (tile == 0) && (take == nt);
     dest.base = ((int64_t)wg * 2 + (first_piece ? 0 : 1)) * 128 - unit * 128;  // + head
     first_piece = false;
-    segment(mr, unit * 128, t_lo, t0 + tile * kTok, min(kv_len, t0 + (tile + take) * kTok), dest);
+    segment(mr, unit * 128, t_lo, t0 + tile * kTok, min(kv_len, t0 + (tile + take) * kTok), dest, piece_no++);
     x += take;
     if (x < x_end && tile + take == nt && unit == units - 1) {
       seq_first += (nt + pad) * units;
@@ -1144,7 +1174,7 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
   __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
   __shared__ __attribute__((aligned(1024))) char slot3[kSlotB];
-  mla_balanced_body(a, [&](const MlaRow& mr, int head_base, int t_lo, int t_begin, int t_end, const MlaDest& dest)
+  mla_balanced_body(a, [&](const MlaRow& mr, int head_base, int t_lo, int t_begin, int t_end, const MlaDest& dest, int)
                         __attribute__((always_inline)) {
     mla_segment<UNIFORM, CAP, PIPE, FP8, DS>(a, mr, head_base, t_lo, t_begin, t_end, dest, slot0, slot1, slot2, slot3);
   });
@@ -1154,9 +1184,9 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_balanced_kernel(const MlaDecod
 template <bool M32>
 __global__ __launch_bounds__(256, 1) void rpa_mla_balanced_wide_kernel(const MlaDecodeArgs a) {
   __shared__ __attribute__((aligned(1024))) char ring[4 * kSlotB];
-  mla_balanced_body(a, [&](const MlaRow& mr, int head_base, int t_lo, int t_begin, int t_end, const MlaDest& dest)
-                        __attribute__((always_inline)) {
-    mla_segment_wide<M32>(a, mr, head_base, t_lo, t_begin, t_end, dest, ring);
+  mla_balanced_body(a, [&](const MlaRow& mr, int head_base, int t_lo, int t_begin, int t_end, const MlaDest& dest,
+                           int piece) __attribute__((always_inline)) {
+    mla_segment_wide<M32>(a, mr, head_base, t_lo, t_begin, t_end, dest, ring, piece);
   });
 }
 
@@ -1429,3 +1459,9 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
 }
 
 }  // namespace rpa
+
+#ifdef RPA_MLA_TRACE
+extern "C" __attribute__((visibility("default"))) int rpa_debug_mla_trace(void* host, size_t bytes) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(rpa::rpa_mla_trace_buf), std::min(bytes, sizeof(rpa::rpa_mla_trace_buf)));
+}
+#endif

@@ -69,6 +69,7 @@ struct ShapeRule {
   int waves_per_wg;        // decode: neighbouring kv heads walked together; others: waves of a workgroup
   int resident_x8;         // decode: resident waves per CU in eighths (28 = 3.5); MLA: workgroups per CU x 8
   int share;               // MLA shared tiles: waves that share a block of 16 heads
+  int piece_pad;           // MLA balanced plan: what starting one more row costs a workgroup, in 32-token tiles
   const char* why;         // the measurement behind the row
 };
 
@@ -79,45 +80,45 @@ constexpr unsigned kOptPlainOnly = kOptSoftCap | kOptMaskOther | kOptTemperature
 constexpr ShapeRule kShapeRules[] = {
   // ---------------- decode rows (HBM bound: bytes in flight and launch overhead decide)
   {"decode_256", kStageDecode, 0, 256, 0, 0, 0, 0, 0, 0,
-   kKernelRows256, 1, 16, 32, 1, 64, 1, "one wave per (token, kv head, 16 query heads); 5.6-5.75 TB/s on long rows"},
+   kKernelRows256, 1, 16, 32, 1, 64, 1, 0, "one wave per (token, kv head, 16 query heads); 5.6-5.75 TB/s on long rows"},
   {"decode_fp8_stream", kStageDecode, 8, 128, 0, 0, 0, 0, 32ll << 20, 0,
-   kKernelDecode, 1, 16, 32, 4, 64, 1, "8 KiB per wave in flight: every wave slot; C4 1024 waves 254 us, 1536 240.5, 2048 238.5"},
+   kKernelDecode, 1, 16, 32, 4, 64, 1, 0, "8 KiB per wave in flight: every wave slot; C4 1024 waves 254 us, 1536 240.5, 2048 238.5"},
   {"decode_fp8_small", kStageDecode, 8, 128, 0, 0, 0, 0, 0, 0,
-   kKernelDecode, 1, 16, 32, 2, 64, 1, "latency bound: few waves spread over more CUs"},
+   kKernelDecode, 1, 16, 32, 2, 64, 1, 0, "latency bound: few waves spread over more CUs"},
   {"decode_bf16_stream", kStageDecode, 16, 128, 0, 0, 0, 0, 32ll << 20, 0,
-   kKernelDecode, 1, 16, 32, 4, 28, 1, "14 MB in flight saturate HBM: C2 / C3 896 waves 104.1 / 356 us, 1024 105.2 / 362, 2048 108.5 / 367"},
+   kKernelDecode, 1, 16, 32, 4, 28, 1, 0, "14 MB in flight saturate HBM: C2 / C3 896 waves 104.1 / 356 us, 1024 105.2 / 362, 2048 108.5 / 367"},
   {"decode_bf16_small", kStageDecode, 16, 128, 0, 0, 0, 0, 0, 0,
-   kKernelDecode, 1, 16, 32, 2, 28, 1, "C1 14.0 us with two waves per workgroup against 15.9 with four"},
+   kKernelDecode, 1, 16, 32, 2, 28, 1, 0, "C1 14.0 us with two waves per workgroup against 15.9 with four"},
   // ---------------- prefill / mixed rows (MFMA bound)
   {"prefill_pipe_short", kStagePrefill, 16, 128, 0, 0, 4, 64, 0, kOptPlainOnly,
-   kKernelPrefillPipe, 32, 4, 64, 4, 16, 1, "chunks of <= 64 tokens fill a 32 x 4-head tile: 64 x 16 tokens on 4 k prefixes 362 -> 196 us"},
+   kKernelPrefillPipe, 32, 4, 64, 4, 16, 1, 0, "chunks of <= 64 tokens fill a 32 x 4-head tile: 64 x 16 tokens on 4 k prefixes 362 -> 196 us"},
   {"prefill_pipe", kStagePrefill, 16, 128, 0, 0, 0, 0, 0, kOptPlainOnly,
-   kKernelPrefillPipe, 128, 1, 64, 4, 16, 1, "assembly steady state: C2 295 -> 236 us"},
+   kKernelPrefillPipe, 128, 1, 64, 4, 16, 1, 0, "assembly steady state: C2 295 -> 236 us"},
   {"prefill_256_fp8", kStagePrefill, 8, 256, 0, 0, 0, 0, 0, 0,
-   kKernelPrefillAsync, 128, 1, 64, 4, 8, 1, "e4m3 rows widened on their way into the bf16 LDS tiles: 582-639 TFLOP/s"},
+   kKernelPrefillAsync, 128, 1, 64, 4, 8, 1, 0, "e4m3 rows widened on their way into the bf16 LDS tiles: 582-639 TFLOP/s"},
   {"prefill_256", kStagePrefill, 16, 256, 0, 0, 0, 0, 0, 0,
-   kKernelPrefillAsync, 128, 1, 64, 4, 8, 1, "two 64 KiB ring slots, one workgroup per CU: 666-725 TFLOP/s"},
+   kKernelPrefillAsync, 128, 1, 64, 4, 8, 1, 0, "two 64 KiB ring slots, one workgroup per CU: 666-725 TFLOP/s"},
   {"prefill_fp8_short", kStagePrefill, 8, 128, 0, 0, 4, 64, 0, 0,
-   kKernelPrefillStaged, 32, 4, 64, 4, 16, 1, "short-chunk tile of the register-staged kernel"},
+   kKernelPrefillStaged, 32, 4, 64, 4, 16, 1, 0, "short-chunk tile of the register-staged kernel"},
   {"prefill_fp8", kStagePrefill, 8, 128, 0, 0, 0, 0, 0, 0,
-   kKernelPrefillStaged, 128, 1, 64, 4, 16, 1, "rows dequantised once per tile on their way to LDS"},
+   kKernelPrefillStaged, 128, 1, 64, 4, 16, 1, 0, "rows dequantised once per tile on their way to LDS"},
   {"prefill_options_short", kStagePrefill, 16, 128, 0, 0, 4, 64, 0, 0,
-   kKernelPrefillAsync, 32, 4, 64, 4, 16, 1, "masked / capped verify steps: 16 draft tokens on 4 k prefixes 2329 -> 261 us with the bit mask"},
+   kKernelPrefillAsync, 32, 4, 64, 4, 16, 1, 0, "masked / capped verify steps: 16 draft tokens on 4 k prefixes 2329 -> 261 us with the bit mask"},
   {"prefill_options", kStagePrefill, 16, 128, 0, 0, 0, 0, 0, 0,
-   kKernelPrefillAsync, 128, 1, 64, 4, 16, 1, "compiled flash kernel: every option"},
+   kKernelPrefillAsync, 128, 1, 64, 4, 16, 1, 0, "compiled flash kernel: every option"},
   // ---------------- absorbed MLA (near the ridge: LDS operand reads and piece starts decide)
   {"mla_wide", kStageMla, 16, 576, 128, 0, 128, 0, 0, kOptSoftCap | kOptAsmPages,
-   kKernelMlaWide, 1, 128, 32, 4, 8, 1, "every operand fragment feeds two matrix instructions: C5 226 -> 205 us, prefill chunks 48 -> 55 % of peak"},
+   kKernelMlaWide, 1, 128, 32, 4, 8, 1, 12, "every operand fragment feeds two matrix instructions: C5 226 -> 205 us, prefill chunks 48 -> 55 % of peak; a row switch costs 22 us = 12 tiles (C5 197 -> 191 us against 5)"},
   {"mla_pipe", kStageMla, 0, 576, 128, 0, 128, 0, 0, kOptSoftCap | kOptAsmPages,
-   kKernelMlaPipe, 1, 128, 32, 8, 8, 1, "e4m3 latents (bytes staged and expanded once per tile) and RPA_MLA_WIDE=0"},
+   kKernelMlaPipe, 1, 128, 32, 8, 8, 1, 12, "e4m3 latents (bytes staged and expanded once per tile) and RPA_MLA_WIDE=0"},
   {"mla_shared_16", kStageMla, 0, 576, 1, 16, 0, 0, 0, kOptSoftCap | kOptOddPages,
-   kKernelMlaShared, 1, 16, 32, 8, 8, 8, "a tensor-parallel share of the heads: 64 rows x 8192 tokens 146 -> 120 us"},
+   kKernelMlaShared, 1, 16, 32, 8, 8, 8, 8, "a tensor-parallel share of the heads: 64 rows x 8192 tokens 146 -> 120 us"},
   {"mla_shared_32", kStageMla, 0, 576, 17, 32, 0, 0, 0, kOptSoftCap | kOptOddPages,
-   kKernelMlaShared, 1, 32, 32, 8, 8, 4, "144 -> 126 us"},
+   kKernelMlaShared, 1, 32, 32, 8, 8, 4, 8, "144 -> 126 us"},
   {"mla_shared_64", kStageMla, 0, 576, 33, 64, 0, 0, 0, kOptSoftCap | kOptOddPages,
-   kKernelMlaShared, 1, 64, 32, 8, 8, 2, "159 -> 147 us"},
+   kKernelMlaShared, 1, 64, 32, 8, 8, 2, 8, "159 -> 147 us"},
   {"mla_compiled", kStageMla, 0, 576, 0, 0, 0, 0, 0, 0,
-   kKernelMlaCompiled, 1, 128, 32, 8, 8, 1, "soft cap, pages under 32 tokens, head counts that are no multiple of 128"},
+   kKernelMlaCompiled, 1, 128, 32, 8, 8, 1, 5, "soft cap, pages under 32 tokens, head counts that are no multiple of 128"},
 };
 // clang-format on
 

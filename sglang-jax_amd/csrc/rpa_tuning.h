@@ -30,7 +30,7 @@ struct Tuning {
   int mla_min_chunk = 256;          // RPA_MLA_MIN_CHUNK
   int mla_wg_capacity = 0;          // RPA_MLA_WG_CAPACITY        0: one workgroup per CU
   int mla_balanced = 1;             // RPA_MLA_BALANCED
-  int mla_piece_pad = 5;            // RPA_MLA_PIECE_PAD          tiles a workgroup pays for starting another row
+  int mla_piece_pad = -1;           // RPA_MLA_PIECE_PAD          -1: the shape table's; tiles a workgroup pays for starting another row
   int mla_pipe = 1;                 // RPA_MLA_PIPE               0: compiled tile loop
   int mla_shared_tiles = 1;         // RPA_MLA_SHARED_TILES       0: one wave per block of 16 heads, always
   int mla_wide = 1;                 // RPA_MLA_WIDE               0: eight-wave kernels; 32: wide loop on 32x32x16
