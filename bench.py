@@ -536,9 +536,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5", "c5fp8", "c5tp8", "c5p"],
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c4swa", "c5", "c5fp8", "c5tp8", "c5p", "c5p16"],
                     help="c5p: absorbed-MLA prefill chunks (512 tokens on 4096-token prefixes), DeepSeek-V3 shape; "
-                         "c5fp8: C5 on an e4m3 latent cache; c5tp8: C5 with 16 of the 128 heads (one GPU's share at tensor-parallel 8)")
+                         "c5fp8: C5 on an e4m3 latent cache; c5tp8: C5 with 16 of the 128 heads (one GPU's share at tensor-parallel 8); "
+                         "c5p16: the c5p chunks with 16 heads, the head count of the reference's own MLA tests")
     ap.add_argument("--all", action="store_true", help="(default) also time the other configurations")
     ap.add_argument("--main-only", action="store_true", help="skip the other configurations")
     ap.add_argument("--reference-suite", action="store_true",
@@ -605,11 +606,12 @@ def main():
                 "c4": lambda: wl.config_c4(dev), "c4swa": lambda: wl.config_c4(dev, window=True),
                 "c5": lambda: wl.config_c5(dev), "c5p": lambda: wl.config_c5_prefill(dev),
                 "c5fp8": lambda: wl.config_c5(dev, kv_dtype=torch.float8_e4m3fn),
-                "c5tp8": lambda: wl.config_c5(dev, num_q_heads=16)}[name]()
+                "c5tp8": lambda: wl.config_c5(dev, num_q_heads=16),
+                "c5p16": lambda: wl.config_c5_prefill(dev, num_q_heads=16)}[name]()
 
     def run(name, keep=False):
         b = build(name)
-        if name in ("c5", "c5p", "c5fp8", "c5tp8"):
+        if name in ("c5", "c5p", "c5fp8", "c5tp8", "c5p16"):
             r = run_mla_config(pkg, wl, b, args.steps, args.warmup, settle_ms=args.settle_ms)
         elif keep:
             r, call = run_rpa_config(pkg, wl, b, args.steps, args.warmup, keep_call=True,
@@ -633,7 +635,7 @@ def main():
                 "frac_back_to_back": (res["decode_gbps_back_to_back"] / HBM_PEAK_GBPS
                                       if "decode_gbps_back_to_back" in res else None)}
 
-    if args.config in ("c5", "c5p", "c5fp8", "c5tp8"):
+    if args.config in ("c5", "c5p", "c5fp8", "c5tp8", "c5p16"):
         main_res, sample = run(args.config), None
     else:
         main_res, sample = run(args.config, keep=True)
@@ -641,7 +643,8 @@ def main():
     pre_tflops = main_res.get("prefill_tflops")
     # dominant kernel of the workload (largest average launch time inside the timed region)
     roofline_decode = with_achievable(decode_roofline(args.config, main_res)) if dec_gbps is not None else None
-    prefill_kernel = "rpa_mla_decode_wide_kernel (one row per query token)" if args.config == "c5p" else PREFILL_KERNEL
+    prefill_kernel = {"c5p": "rpa_mla_decode_wide_kernel (one row per query token)",
+                      "c5p16": "rpa_mla_token_group_kernel (8 query tokens per workgroup)"}.get(args.config, PREFILL_KERNEL)
 
     def prefill_roofline(name, res, kernel):
         return with_achievable({
@@ -690,13 +693,14 @@ def main():
         configs[args.config + (" prefill rows" if roofline_decode is not None else "")] = compact(roofline_prefill)
     if not args.main_only:
         others = {}
-        for name in ("c1", "c2", "c3", "c4", "c4swa", "c5", "c5fp8", "c5tp8", "c5p"):
+        for name in ("c1", "c2", "c3", "c4", "c4swa", "c5", "c5fp8", "c5tp8", "c5p", "c5p16"):
             if name == args.config:
                 continue
             r = run(name)
-            if name == "c5p":
+            if name in ("c5p", "c5p16"):
                 r["roofline"] = with_achievable({
-                    "kernel": "rpa_mla_decode_wide_kernel (one row per query token)", "bound": "mfma",
+                    "kernel": "rpa_mla_decode_wide_kernel (one row per query token)" if name == "c5p"
+                              else "rpa_mla_token_group_kernel (8 query tokens per workgroup)", "bound": "mfma",
                     "achieved": r["prefill_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": r["prefill_tflops"] / MFMA_BF16_PEAK_TFLOPS, "avg_launch_ms": r["prefill_ms"],
                     "flops_per_launch": r["prefill_flops"]})

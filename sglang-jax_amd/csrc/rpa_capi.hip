@@ -54,6 +54,7 @@ const Tuning& tuning() {
   geti("RPA_MLA_PIPE", t.mla_pipe);
   geti("RPA_MLA_SHARED_TILES", t.mla_shared_tiles);
   geti("RPA_MLA_WIDE", t.mla_wide);
+  geti("RPA_MLA_TOKEN_GROUPS", t.mla_token_groups);
   if (const char* v = getenv("RPA_PREFILL_PIPE_LIMIT")) {
     if (*v) t.prefill_pipe_limit = (float)atof(v);
   }

@@ -301,18 +301,33 @@ struct MlaDest {
 // block of 16 heads share its tile instead: wave `sub` of the block takes token half sub & 1 and k-step group
 // sub >> 1 of the first product, leaves its partial scores in LDS, every wave of the block sums them and takes
 // the (same) probabilities, and the second product's 32 output chunks are dealt out 32 / DS per wave.
-template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false, int DS = 1>
+// TG (token group): with 16 / 32 / 64 heads, the eight waves hold 8 / 4 / 2 CONSECUTIVE QUERY TOKENS of one
+// sequence instead of one token's heads, `group_tokens` of them real (a chunk's tail may leave fewer): wave w
+// owns token (16 w) / Hq of the group and the block of 16 heads (16 w) % Hq.  mr.tq is the group's first token,
+// mr.kv_len what its LAST token sees; a wave's own token sees kv_len - (group_tokens - 1) + its place, and
+// masks with that.  Tokens of one sequence follow each other in q and out, so (token, head) of the group is
+// "head" 16 w + c of a 128-head row at mr.tq: every address below stays what it was.  The reference's
+// kernel shares each latent tile among 16 query tokens the same way (kernels/mla/v2/kernel.py:1448-1459).
+template <bool UNIFORM, bool CAP, bool PIPE = false, bool FP8 = false, int DS = 1, bool TG = false>
 __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
                                             int t_begin, int t_end, const MlaDest dest, char* slot0, char* slot1,
-                                            char* slot2, char* slot3) {
+                                            char* slot2, char* slot3, int group_tokens = 1) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, g = lane >> 4;
   static_assert(DS == 1 || (UNIFORM && !PIPE), "shared tiles: compiled loop, whole tiles per page (LDS for the partial scores)");
+  static_assert(!TG || DS == 1, "token groups: one wave per (token, block of 16 heads)");
   const int sub = wave % DS;                       // this wave's place among the DS waves of its block of heads
-  const int head0 = head_base + (wave / DS) * 16;
-  const bool wave_on = head0 < a.Hq;
+  // token groups: a wave past the group's last real token repeats that token's work and writes nothing
+  const int tg_place = TG ? min((wave * 16) / a.Hq, group_tokens - 1) : 0;
+  const bool tg_real = !TG || (wave * 16) / a.Hq < group_tokens;
+  const int head0 = TG ? tg_place * a.Hq + (wave * 16) % a.Hq : head_base + (wave / DS) * 16;
+  const bool wave_on = TG || head0 < a.Hq;
+  // what this wave's token sees (all waves alike unless TG)
+  const int kv_len_w = TG ? mr.kv_len - (group_tokens - 1) + tg_place : mr.kv_len;
+  const int t_lo_w = (TG && a.sm.window > 0) ? max(0, kv_len_w - a.sm.window) : t_lo;
+  const int t_lo_last = (TG && a.sm.window > 0) ? max(0, mr.kv_len - a.sm.window) : t_lo;  // the largest of the group
   constexpr int kChunksPerWave = 32 / DS;          // output chunks of 16 dims per wave
   __shared__ __attribute__((aligned(16))) float partial_scores[DS == 1 ? 1 : 8][DS == 1 ? 4 : 256];  // [wave][lane x 4]
   const int seq = mr.seq;
@@ -354,7 +369,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   const int tq = mr.tq;
   u32x4_t qB[18];
   {
-    const int head = min(head0 + c, a.Hq - 1);
+    const int head = TG ? head0 + c : min(head0 + c, a.Hq - 1);
     const uint16_t* qn = a.ql_nope + ((int64_t)tq * a.Hq + head) * 512 + g * 8;
     const uint16_t* qr = a.q_pe + ((int64_t)tq * a.Hq + head) * 64 + g * 8;
 #pragma unroll
@@ -490,11 +505,11 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
         else v = v * scale2;
         x[i] = v;
       }
-      if ((tb + kTok > kv_len) || (tb < t_lo)) {
+      if ((tb + kTok > kv_len_w) || (tb < t_lo_w)) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const int tok = tb + tok_of(g_t, i);
-          if (tok >= kv_len || tok < t_lo) x[i] = mask2;
+          if (tok >= kv_len_w || tok < t_lo_w) x[i] = mask2;
         }
       }
       float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
@@ -567,7 +582,9 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
     // probabilities are taken against) and past the window's edge; the loop copies tile k + 3 without
     // clamping rows, so that one has to be a whole tile of the row
     int k0 = 1;
-    if (t_begin < t_lo) k0 = max(k0, (t_lo - t_begin + kTok - 1) / kTok);
+    // (every wave must have met a token it sees, and with it a real reference, before the loop: with token
+    // groups the last token's window may open a tile later than the first one's)
+    if (t_begin < t_lo_last) k0 = max(k0, TG ? (t_lo_last - t_begin) / kTok + 1 : (t_lo_last - t_begin + kTok - 1) / kTok);
     const int k1 = min(nT, (kv_len - t_begin) / kTok - 3);
     typedef __attribute__((address_space(3))) char* lds_ptr_t;
     int k = 0;
@@ -677,7 +694,7 @@ __device__ __forceinline__ void mla_segment(const MlaDecodeArgs& a, const MlaRow
   }
   asm volatile("" : "+v"(c_out), "+v"(g_out));
   const int head = head0 + c_out;
-  if (!wave_on || head >= a.Hq) return;
+  if (TG ? !tg_real : (!wave_on || head >= a.Hq)) return;
   const int chunk0 = DS > 1 ? sub * kChunksPerWave : 0;  // shared tiles: this wave's output chunks
   if (dest.final_rows) {
     const float inv = a.out_scale / l;
@@ -1011,6 +1028,54 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
 #endif
 }
 
+// ---- token groups (see mla_segment, TG): 16 / 32 / 64 heads, every query token a row, whole rows (no pieces).
+// grid = windows of 128 / Hq consecutive query tokens of the call.  A window that lies inside one sequence is one
+// group; one that spans a border between sequences (the end of a chunk, decode rows of one token each) runs one
+// group per sequence, one after the other.
+template <bool PIPE, bool FP8>
+__global__ __launch_bounds__(512, 2) void rpa_mla_token_group_kernel(const MlaDecodeArgs a) {
+  __shared__ __attribute__((aligned(1024))) char slot0[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot1[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot2[kSlotB];
+  __shared__ __attribute__((aligned(1024))) char slot3[kSlotB];
+  const int num_seqs = a.dist ? min(a.num_seqs, scalar_load_i32(a.dist + 2)) : a.num_seqs;
+  const int total = min(a.num_rows, scalar_load_i32(a.pt.cu_q_lens + num_seqs));
+  const int per = 128 / a.Hq;
+  int t = (int)blockIdx.x * per;
+  if (t >= total) return;
+  const int t_stop = min(t + per, total);
+  int seq = owner_of_token(a.pt.cu_q_lens, num_seqs, t);
+  while (t < t_stop) {
+    // (everything here is the same in every lane; said so explicitly, the assembly loop takes scalars)
+    seq = __builtin_amdgcn_readfirstlane(seq);
+    t = __builtin_amdgcn_readfirstlane(t);
+    const int q0 = scalar_load_i32(a.pt.cu_q_lens + seq);
+    const int q1 = scalar_load_i32(a.pt.cu_q_lens + seq + 1);
+    if (q1 <= t) {  // (a sequence without tokens)
+      ++seq;
+      continue;
+    }
+    const int n = __builtin_amdgcn_readfirstlane(min(t_stop, q1) - t);  // tokens of this sequence in the window
+    MlaRow mr;
+    mr.seq = seq;
+    mr.tq = t;
+    mr.valid = true;
+    // what the group's last token sees
+    mr.kv_len = __builtin_amdgcn_readfirstlane(scalar_load_i32(a.pt.kv_lens + seq) - (q1 - q0) + (t + n - 1 - q0) + 1);
+    const int first_len = mr.kv_len - (n - 1);
+    if (mr.kv_len > 0 && first_len > 0) {
+      const int t_lo = (a.sm.window > 0) ? max(0, first_len - a.sm.window) : 0;
+      MlaDest dest;
+      dest.final_rows = true;
+      dest.base = 0;
+      mla_segment<true, false, PIPE, FP8, 1, true>(a, mr, 0, t_lo, t_lo & ~(kTok - 1), mr.kv_len, dest, slot0, slot1, slot2,
+                                                   slot3, n);
+    }
+    t += n;
+    if (t >= q1) ++seq;
+  }
+}
+
 // ---- fixed split plan, wide workgroups: grid = (max_splits * rows, 1, head groups of 128); block = 256 threads
 template <bool M32>
 __global__ __launch_bounds__(256, 1) void rpa_mla_decode_wide_kernel(const MlaDecodeArgs a) {
@@ -1336,6 +1401,25 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   const ShapeRule& shape = select_shape(mla_shape_key(a), mla_shape_skip(tune));
   const bool pipe = shape.kernel == kKernelMlaWide || shape.kernel == kKernelMlaPipe;
   const int ds = shape.kernel == kKernelMlaShared ? shape.share : 1;
+  // Prefill / mixed rows with few heads: a workgroup holds 128 / Hq consecutive query tokens of a sequence over
+  // shared tiles instead of one token whose heads leave most of it idle (rows_are_tokens, whole rows, a head count
+  // that divides 128, whole tiles in power-of-two pages, no soft cap; RPA_MLA_TOKEN_GROUPS=0 keeps one token per
+  // workgroup).  Decode batches (one token per sequence) have nothing to group and keep the shared tiles.
+  if (ds != 1 && a.rows_are_tokens && a.max_splits <= 1 && !a.balanced && tune.mla_token_groups != 0 &&
+      (128 % a.Hq) == 0 && a.Hq >= 16 && a.num_rows >= 4 * a.num_seqs) {
+    const int P = a.pt.page_size;
+    const bool pipe_ok = tune.mla_pipe != 0 && (P & (P - 1)) == 0 && (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);
+    const int per = 128 / a.Hq;
+    const dim3 tg_grid((unsigned)((a.num_rows + per - 1) / per));
+    if (a.fp8) {
+      if (pipe_ok) hipLaunchKernelGGL((rpa_mla_token_group_kernel<true, true>), tg_grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((rpa_mla_token_group_kernel<false, true>), tg_grid, block, 0, stream, a);
+    } else {
+      if (pipe_ok) hipLaunchKernelGGL((rpa_mla_token_group_kernel<true, false>), tg_grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((rpa_mla_token_group_kernel<false, false>), tg_grid, block, 0, stream, a);
+    }
+    return hipGetLastError();
+  }
   if (ds != 1) {
 #define RPA_MLA_DS(KERNEL, GRID, F8)                                                                                  \
   do {                                                                                                                \

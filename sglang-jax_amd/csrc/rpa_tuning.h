@@ -34,6 +34,7 @@ struct Tuning {
   int mla_pipe = 1;                 // RPA_MLA_PIPE               0: compiled tile loop
   int mla_shared_tiles = 1;         // RPA_MLA_SHARED_TILES       0: one wave per block of 16 heads, always
   int mla_wide = 1;                 // RPA_MLA_WIDE               0: eight-wave kernels; 32: wide loop on 32x32x16
+  int mla_token_groups = 1;         // RPA_MLA_TOKEN_GROUPS       0: prefill rows with few heads one token per workgroup
 };
 
 const Tuning& tuning();

@@ -324,7 +324,8 @@ def config_c5_prefill(device="cpu", scale: float = 1.0, num_q_heads: int = 128, 
     seed = 1006
     q = _scaled(512, scale)
     kv = _scaled(4096, scale) + q
-    return make_mla_batch("c5p_deepseek_v3_mla_prefill", np.full(num_seqs, q), np.full(num_seqs, kv),
+    name = "c5p_deepseek_v3_mla_prefill" + ("" if num_q_heads == 128 else f"_{num_q_heads}_heads")
+    return make_mla_batch(name, np.full(num_seqs, q), np.full(num_seqs, kv),
                           num_q_heads=num_q_heads, lkv_dim=512, rope_dim=64, page_size=64, seed=seed, device=device,
                           sm_scale=1.0 / math.sqrt(192.0))
 

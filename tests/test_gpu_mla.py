@@ -102,6 +102,42 @@ def test_mla_waves_share_tiles_when_heads_are_few(pkg, wl, gpu, monkeypatch, Hq,
         assert torch.equal(shared, run_gpu(pkg, b, gpu)[:T])
 
 
+@pytest.mark.parametrize("Hq", [16, 32, 64])
+@pytest.mark.parametrize("f8", [False, True])
+def test_mla_prefill_rows_share_tiles_among_query_tokens_when_heads_are_few(pkg, wl, gpu, monkeypatch, Hq, f8):
+    """Prefill / mixed batches with 16 / 32 / 64 heads (the reference's own MLA test shape has 16,
+    test_mla_attention.py:346): a workgroup holds 8 / 4 / 2 consecutive query tokens of a sequence over shared
+    latent tiles, each wave masking with its own token's length (the reference's kernel shares a tile among 16
+    query tokens, kernels/mla/v2/kernel.py:1448-1459).  Against the oracle and against one token per workgroup
+    (RPA_MLA_TOKEN_GROUPS=0): chunk lengths that leave partial groups, windows of tokens that span the border
+    between two sequences, decode rows in front, a chunk with no prefix, a sliding window shorter than the chunk,
+    pages of 32 and 128 tokens, planted keys."""
+    ref = fp8_oracle if f8 else oracle
+    cases = (("chunks", [300, 77, 130], [1500, 77, 4230], None, 64),
+             ("mixed", [1, 1, 1, 259, 64], [900, 33, 2000, 1259, 3064], None, 32),
+             ("window", [200, 45], [3000, 700], 150, 128),
+             ("long_chunk", [1024], [1024 + 4096], None, 64))
+    for name, q_lens, kv_lens, window, P in cases:
+        say(f"mla token groups Hq={Hq} f8={f8} {name}")
+        b = wl.make_mla_batch("mla_tg_" + name, q_lens, kv_lens, num_q_heads=Hq, lkv_dim=512, rope_dim=64, page_size=P,
+                              seed=470 + Hq, sm_scale=192 ** -0.5, sliding_window=window,
+                              kv_dtype=torch.float8_e4m3fn if f8 else torch.bfloat16)
+        wl.plant_mla_needles(b, seed=7)
+        want = ref(b)
+        T = sum(q_lens)
+        grouped = run_gpu(pkg, b, gpu)[:T]
+        assert_parity(grouped.float(), want.float(), **TOL)
+        monkeypatch.setenv("RPA_MLA_TOKEN_GROUPS", "0")
+        single = run_gpu(pkg, b, gpu)[:T]
+        monkeypatch.delenv("RPA_MLA_TOKEN_GROUPS")
+        assert_parity(single.float(), want.float(), **TOL)
+        assert_parity(grouped.float(), single.float(), **TOL)
+        monkeypatch.setenv("RPA_MLA_PIPE", "0")  # the compiled tile loop under the same grouping
+        compiled = run_gpu(pkg, b, gpu)[:T]
+        monkeypatch.delenv("RPA_MLA_PIPE")
+        assert_parity(compiled.float(), want.float(), **TOL)
+
+
 @pytest.mark.parametrize("window,cap", [(128, None), (None, 30.0), (128, 30.0)])
 def test_mla_window_and_soft_cap(pkg, wl, gpu, window, cap):
     kv_lens = [100, 128, 129, 700]
