@@ -22,6 +22,11 @@ maximum known before it; if some row sum of the half exceeds 2^8 (a score beat t
 by more than 4) the wave takes the rare path: the true maximum is taken, accumulators, row sums,
 the splat and the scores in flight are moved to it and the half's probabilities redone.
 
+A second variant of the loop (masked = True, one block of rows per wave only) applies the causal mask to every
+half before its exponentials: one compare of the register's token offset against a per-lane threshold
+(query position - first token of the half - 4 * lane half) and one select of -1e30 per score.  It runs the
+steps that touch the causal diagonal, which would otherwise fall back to the compiled general step.
+
 The whole loop is one block because the register allocator will not keep hundreds of registers in
 place around a block that is only a loop body: here they are moved in and out once per loop.
 
@@ -52,6 +57,8 @@ KB, VB = 60, 62                           # s[60:61], s[62:63]: global base of t
 ST = [64, 65, 66, 67]                     # temporaries
 PGC = 68                                  # page id of tile t + 2
 WV = 69                                   # this wave's index in its workgroup (staggered copies)
+MASK_SGPR = [70, 72, 74, 76]              # s[70:71] .. s[76:77]: lane masks of the masked variant
+SGPR_BASE = 5000                          # register ids >= SGPR_BASE name scalar registers in the hazard bookkeeping
 SGPR_CLOBBERS = list(range(60, 70 if "stagger" in X else 69))
 
 K_SLOT = [0, 16384]                       # byte offsets of the ring slots from the LDS array's start
@@ -64,13 +71,15 @@ VALU_TO_MFMA = 2
 TRANS_TO_VALU = 1
 VALU_TO_SWAP = 2
 DOT_TO_VALU = 3
+VALU_SGPR_TO_VALU = 2                     # a vector instruction's scalar result read by a vector instruction
 
 
 class Table:
     """Register table of one NQ variant."""
 
-    def __init__(self, nq):
+    def __init__(self, nq, masked=False):
         self.nq = nq
+        self.masked = masked
         self._v, self._a = 0, ACC
 
         def v(n):
@@ -100,6 +109,9 @@ class Table:
         self.VOFF = v(4)                                           # ... of the V^T operand reads
         self.OFSK = v(4)                                           # per-lane global byte offsets of this wave's K copies
         self.OFSV = v(4)
+        if masked:
+            self.THR = v(1)                                        # query position - first token of the half - 4 * lane half
+            self.NINF = v(1)                                       # -1e30
         self.first_scratch = self._v
         self.PS = [[v(1), v(1)] for q in range(nq)]                # row-sum accumulators of the half
         self.MX, self.T0, self.T1 = v(1), v(1), v(1)
@@ -166,6 +178,9 @@ class Emitter:
             self.lds_queue = self.lds_queue[pos + 1:]
         r, w = ins.reads, ins.writes
         if ins.kind in ("valu", "trans", "swap", "dot"):
+            sr = {x for x in r if x >= SGPR_BASE}
+            if sr:
+                self._pad(VALU_SGPR_TO_VALU, lambda p: p.kind in ("valu", "trans", "swap", "dot") and (p.writes & sr))
             self._pad(MFMA_TO_VALU, lambda p: p.kind == "mfma" and (p.writes & (r | w)))
             self._pad(TRANS_TO_VALU, lambda p: p.kind == "trans" and (p.writes & r))
             if ins.kind == "swap":
@@ -193,9 +208,11 @@ def valu(text, reads, writes, kind="valu"):
 
 
 class Gen:
-    def __init__(self, nq):
+    def __init__(self, nq, masked=False):
+        assert not (masked and nq != 1)
         self.nq = nq
-        self.t = Table(nq)
+        self.masked = masked
+        self.t = Table(nq, masked)
 
     # ---------------------------------------------------------------- instruction builders
     def mfma(self, dst, a, b, c):
@@ -259,7 +276,34 @@ class Gen:
 
         return exps, cvt, dot
 
-    def softmax_stream(self, sc, check=True):
+    def mask_ops(self, q, sc):
+        """Causal mask of the 16 scores of S[q][sc], per score pair j: the two compares (token offset of the
+        register inside the half against the lane's threshold) into a pair of scalar registers each, and the two
+        selects.  The compares of a pair are issued one pair ahead of its selects."""
+        t = self.t
+
+        def cmps(j):
+            out = []
+            for e in (0, 1):
+                v = 2 * j + e
+                k = 8 * (v >> 2) + (v & 3)
+                sg = MASK_SGPR[2 * (j & 1) + e]
+                out.append(valu(f"v_cmp_gt_i32_e64 s[{sg}:{sg + 1}], {k}, {vr(t.THR)}", [t.THR], [SGPR_BASE + sg]))
+            return out
+
+        def sels(j):
+            out = []
+            for e in (0, 1):
+                v = 2 * j + e
+                sg = MASK_SGPR[2 * (j & 1) + e]
+                r = t.S[q][sc] + v
+                out.append(valu(f"v_cndmask_b32_e64 {vr(r)}, {vr(r)}, {vr(t.NINF)}, s[{sg}:{sg + 1}]",
+                                [r, t.NINF, SGPR_BASE + sg], [r]))
+            return out
+
+        return cmps, sels
+
+    def softmax_stream(self, sc, check=True, masked=False):
         """All row blocks' softmax work in issue order.  The stages of a pair are spread out (packing
         `lag` pairs behind the exponentials, the row sum one pair behind the packing) and the row blocks
         are interleaved, so no instruction needs the result of the few in front of it: a wave issues in
@@ -270,7 +314,16 @@ class Gen:
         ops = [self.softmax_ops(q, sc) for q in range(nq)]
         for q in range(nq):
             out += [valu(f"v_mov_b32 {vr(t.PS[q][0])}, 0", [], [t.PS[q][0]]), valu(f"v_mov_b32 {vr(t.PS[q][1])}, 0", [], [t.PS[q][1]])]
+        if masked:
+            cmps, sels = self.mask_ops(0, sc)
+            out = cmps(0) + out
         for step in range(8 + lag + 1):
+            if masked and step < 8:
+                if step + 1 < 8:
+                    out += cmps(step + 1)
+                else:  # the last compares of the half are out: the threshold moves on to the next half
+                    out.append(valu(f"v_subrev_u32_e32 {vr(t.THR)}, 32, {vr(t.THR)}", [t.THR], [t.THR]))
+                out += sels(step)
             for q in range(nq):
                 if step < 8:
                     out += ops[q][0](step)
@@ -315,7 +368,7 @@ class Gen:
         nq = self.nq
         sc = 1 - it
         sn, pp = 1 - sc, 1 - sc
-        stream = self.softmax_stream(sc)
+        stream = self.softmax_stream(sc, masked=self.masked)
         pos = 0
 
         def deal(n):
@@ -334,7 +387,7 @@ class Gen:
 
         # the first iteration's scores were finished in the previous step: a first chunk of vector work
         # runs while the step's first fragments travel; the rest is dealt out behind the matrix instructions
-        lead = 6 if it == 0 else 0
+        lead = (12 if self.masked else 6) if it == 0 else 0
         deal(lead)
         slots = 16 * nq
         rest = len(stream) - lead
@@ -500,9 +553,9 @@ class Gen:
         em = self.generate()
         n_mfma = sum(1 for i in em.out if i.kind == "mfma")
         n_valu = sum(1 for i in em.out if i.kind in ("valu", "trans", "swap", "dot"))
-        sfx = f"_NQ{nq}"
+        sfx = f"_NQ{nq}" + ("M" if self.masked else "")
         text = (
-            f"// ---- NQ = {nq}: {len(em.out)} lines, {n_mfma} matrix and {n_valu} vector instructions (rare paths "
+            f"// ---- NQ = {nq}{' with the causal mask' if self.masked else ''}: {len(em.out)} lines, {n_mfma} matrix and {n_valu} vector instructions (rare paths "
             f"included), {em.nops} padding wait states; {t.num_vgpr} vector + {t.num_agpr} accumulation registers\n"
         )
         binds = {}
@@ -515,6 +568,8 @@ class Gen:
             binds[f"NM{q}"] = (t.NM[q], 16)
             binds[f"M{q}"], binds[f"L{q}"] = (t.M[q], 1), (t.L[q], 1)
         binds.update({"KOFF": (t.KOFF, 8), "VOFF": (t.VOFF, 4), "OFSK": (t.OFSK, 4), "OFSV": (t.OFSV, 4)})
+        if self.masked:
+            binds.update({"THR": (t.THR, 1), "NINF": (t.NINF, 1)})
         for name, (lo, n) in binds.items():
             text += f'#define RPA_PIPE{sfx}_C_{name} "{{{vr(lo, n)}}}"\n'
         lines = ['    "%s\\n"' % ins.text for ins in em.out]
@@ -522,8 +577,10 @@ class Gen:
         clob = ['"v%d"' % r for r in range(t.first_scratch, t.num_vgpr)]
         clob += ['"%s"' % vr(r) for r in list(rng(t.KF, 4 * NBUF)) + list(rng(t.VF, 4 * NBUF))]
         clob += ['"s%d"' % r for r in SGPR_CLOBBERS]
+        if self.masked:
+            clob += ['"s%d"' % r for sg in MASK_SGPR for r in (sg, sg + 1)]
         text += f"#define RPA_PIPE{sfx}_CLOBBERS " + ", ".join(clob) + ', "vcc", "scc", "m0", "memory"\n'
-        print(f"NQ={nq}: {len(em.out)} lines, {n_mfma} MFMAs, {n_valu} vector, {em.nops} padding wait states, "
+        print(f"NQ={nq}{'M' if self.masked else ''}: {len(em.out)} lines, {n_mfma} MFMAs, {n_valu} vector, {em.nops} padding wait states, "
               f"{t.num_vgpr} VGPRs + {t.num_agpr} AGPRs")
         return text
 
@@ -536,6 +593,7 @@ def main():
             "// that bind the kernel's variables to the registers the assembly uses.\n")
     for nq in (1, 2):
         text += Gen(nq).emit_text()
+    text += Gen(1, masked=True).emit_text()
     with open(os.path.join(here, "rpa_prefill_pipe_loop.inc"), "w") as f:
         f.write(text)
 

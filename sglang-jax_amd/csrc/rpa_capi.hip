@@ -46,6 +46,7 @@ const Tuning& tuning() {
   geti("RPA_PREFILL_PIPE_TILE", t.prefill_pipe_tile);
   geti("RPA_PREFILL_LEVEL_ORDER", t.prefill_level_order);
   geti("RPA_PREFILL_PIPE_NQ", t.prefill_pipe_nq);
+  geti("RPA_PREFILL_PIPE_MASKED", t.prefill_pipe_masked);
   geti("RPA_PREFILL_SPLITS", t.prefill_splits);
   geti("RPA_MLA_MIN_CHUNK", t.mla_min_chunk);
   geti("RPA_MLA_WG_CAPACITY", t.mla_wg_capacity);

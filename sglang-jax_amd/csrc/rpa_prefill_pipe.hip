@@ -248,6 +248,25 @@ __device__ __forceinline__ void pipe_loop(RowBlock (&b)[1], const Shared& sh, in
 #undef C
 }
 
+// The same steps with the causal mask applied to every half before its exponentials (the steps on the
+// diagonal).  thr: query position - first token of the half whose probabilities the block's first iteration
+// takes (half 2t - 1) - 4 * (lane / 32); the block moves it on by 32 per half.
+__device__ __forceinline__ void pipe_loop_masked(RowBlock (&b)[1], const Shared& sh, int& t, int& pg_a, int& pg_b,
+                                                 const LoopScalars& sc, int thr) {
+#define C(n) RPA_PIPE_NQ1M_C_##n
+  const float ninf = -1.0e30f;
+  asm volatile(RPA_PIPE_NQ1M_ASM
+               : "+" C(O00)(b[0].O[0]), "+" C(O01)(b[0].O[1]), "+" C(O02)(b[0].O[2]), "+" C(O03)(b[0].O[3]),
+                 "+" C(S00)(b[0].S[0]), "+" C(S01)(b[0].S[1]), "+" C(P00)(b[0].P[0]), "+" C(P01)(b[0].P[1]),
+                 "+" C(NM0)(b[0].NM), "+" C(M0)(b[0].m), "+" C(L0)(b[0].l), "+" C(THR)(thr),
+                 [t] "+&s"(t), [pg_a] "+&s"(pg_a), [pg_b] "+&s"(pg_b)
+               : C(Q0)(b[0].Q), C(KOFF)(sh.koff), C(VOFF)(sh.voff), C(OFSK)(sh.ofs_k), C(OFSV)(sh.ofs_v), C(NINF)(ninf),
+                 RPA_PIPE_SCALARS(sc)
+               : RPA_PIPE_NQ1M_CLOBBERS);
+#undef C
+}
+__device__ __forceinline__ void pipe_loop_masked(RowBlock (&)[2], const Shared&, int&, int&, int&, const LoopScalars&, int) {}
+
 __device__ __forceinline__ void pipe_loop(RowBlock (&b)[2], const Shared& sh, int& t, int& pg_a, int& pg_b,
                                           const LoopScalars& sc) {
 #define C(n) RPA_PIPE_NQ2_C_##n
@@ -275,7 +294,8 @@ __device__ __forceinline__ void pipe_loop(RowBlock (&b)[2], const Shared& sh, in
 // rpa_prefill_combine_kernel instead of finished rows.
 template <bool WIN, int NQ, bool HEADS4 = false, bool SPLIT = false>
 __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kernel(const PrefillArgs a_in, int tiles, int nseq,
-                                                                                 bool by_level, float row_sum_limit) {
+                                                                                 bool by_level, float row_sum_limit,
+                                                                                 bool masked_steps) {
   PrefillArgs a = a_in;  // static-shape mode: the sequences to process come from the device
   if (a.dist) {
     a.seq_begin = (a.sm.mask_mode == 1) ? 0 : scalar_load_i32(a.dist);
@@ -456,13 +476,39 @@ __global__ __launch_bounds__(256, (NQ == 1 ? 2 : 1)) void rpa_prefill_pipe_kerne
   // general step would move the whole register state to a common place on every trip): general steps
   // up to the first steady-state step, the assembly loop, general steps to the end.
   const bool has_fast = t_fb < t_fe && row_sum_limit > -1.5f;  // (limit -2: a probe that keeps every step general)
-  const int t_first = has_fast ? t_fb : nT + 1;
+  // Steps [t_mb, t_me): the ones behind the steady state that touch the causal diagonal, up to the wave's last
+  // half, in the masked assembly loop (no window, or one far wider than a tile: the loop masks the diagonal only).
+  // Every row has met a token it sees by then (half 0 at the latest, which step 0 takes), the tiles the steps copy
+  // are whole, and halves past the wave's rows come out with every score masked, so they add nothing.
+  int t_mb = nT + 1, t_me = nT + 1;
+  if constexpr (NQ == 1) {
+    // (without steady-state steps in front: only if the range starts at or before the wave's first row, so that
+    // step 0 has shown every row a token and with it a real reference for its probabilities)
+    const bool seen_early = W_ == 0 && t_lo <= w.prefix + r_lo;
+    if (masked_steps && active && row_sum_limit > -1.5f && (W_ == 0 || W_ >= 4 * kBN) && (has_fast || seen_early)) {
+      t_mb = has_fast ? t_fe : max(t_fb, 1);
+      t_me = min(min(((n_w + 1) >> 1) + 1, n_full - 1), nT + 1);
+    }
+  }
+  t_mb = __builtin_amdgcn_readfirstlane(t_mb);
+  t_me = __builtin_amdgcn_readfirstlane(t_me);
+  const bool has_masked = t_mb < t_me;
+  const int t_first = has_fast ? t_fb : (has_masked ? t_mb : nT + 1);
   int t = 0;
   for (; t < t_first; ++t) general_step(t);
   if (has_fast) {
     pipe_loop(b, sh, t, pg_a, pg_b, sc);  // leaves t == t_fe
 #pragma unroll
     for (int q = 0; q < NQ; ++q) b[q].seen = 1.0f;  // a steady-state half hides nothing from any row
+  }
+  if (has_masked) {
+    sc.t_end = t_me;
+    // (a piece of a K/V range may end in front of the diagonal: its end masks like a row's own position)
+    pipe_loop_masked(b, sh, t, pg_a, pg_b, sc, min(b[0].qpos, t_hi - 1) - t_lo - 32 * (2 * t - 1) - 4 * h);  // leaves t == t_me
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) b[q].seen = 1.0f;
+  }
+  if (has_fast || has_masked) {
     for (; t <= nT; ++t) general_step(t);
   }
 #pragma unroll
@@ -504,6 +550,7 @@ hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order,
   const int force_nq = forced_nq();
   // a half's row sum above the limit sends a wave through the rescaling path (testing knob: -1 = always)
   const float limit = tuning().prefill_pipe_limit != 0.f ? tuning().prefill_pipe_limit : kRowSumLimit;
+  const bool masked = tuning().prefill_pipe_masked != 0;  // the steps on the causal diagonal in assembly too
   const int nq = force_nq ? force_nq : 1;
   // Tile by shape (the reference's per-shape block sizes, tuned_block_sizes.py, have this one counterpart
   // here): chunks of at most 64 tokens take 32 positions x 4 heads per workgroup when the heads come in fours
@@ -522,7 +569,7 @@ hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order,
     if (!a.ws_o || !a.ws_ml || a.kv_splits > 64) return hipErrorInvalidValue;
     const dim3 gs((unsigned)grid, (unsigned)a.kv_splits);
 #define RPA_LAUNCH_SPLIT(W, H4) \
-  hipLaunchKernelGGL((rpa_prefill_pipe_kernel<W, 1, H4, true>), gs, blk, 0, stream, a, tiles, nseq, by_level, limit)
+  hipLaunchKernelGGL((rpa_prefill_pipe_kernel<W, 1, H4, true>), gs, blk, 0, stream, a, tiles, nseq, by_level, limit, masked)
     if (heads4) {
       if (win) RPA_LAUNCH_SPLIT(true, true);
       else RPA_LAUNCH_SPLIT(false, true);
@@ -534,10 +581,10 @@ hipError_t launch_prefill_pipe(const PrefillArgs& a, int nseq, bool level_order,
     return launch_prefill_combine(a, stream);
   }
 #define RPA_LAUNCH(W, N) \
-  hipLaunchKernelGGL((rpa_prefill_pipe_kernel<W, N>), g, blk, 0, stream, a, tiles, nseq, by_level, limit)
+  hipLaunchKernelGGL((rpa_prefill_pipe_kernel<W, N>), g, blk, 0, stream, a, tiles, nseq, by_level, limit, masked)
   if (heads4) {
-    if (win) hipLaunchKernelGGL((rpa_prefill_pipe_kernel<true, 1, true>), g, blk, 0, stream, a, tiles, nseq, by_level, limit);
-    else hipLaunchKernelGGL((rpa_prefill_pipe_kernel<false, 1, true>), g, blk, 0, stream, a, tiles, nseq, by_level, limit);
+    if (win) hipLaunchKernelGGL((rpa_prefill_pipe_kernel<true, 1, true>), g, blk, 0, stream, a, tiles, nseq, by_level, limit, masked);
+    else hipLaunchKernelGGL((rpa_prefill_pipe_kernel<false, 1, true>), g, blk, 0, stream, a, tiles, nseq, by_level, limit, masked);
   } else if (nq == 1) {
     if (win) RPA_LAUNCH(true, 1);
     else RPA_LAUNCH(false, 1);

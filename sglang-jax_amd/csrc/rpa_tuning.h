@@ -25,6 +25,7 @@ struct Tuning {
   int prefill_level_order = 1;      // RPA_PREFILL_LEVEL_ORDER    0: query tiles in sequence order
   int prefill_pipe_nq = 0;          // RPA_PREFILL_PIPE_NQ        2: 64 query rows per wave
   float prefill_pipe_limit = 0.f;   // RPA_PREFILL_PIPE_LIMIT     0: the kernel's own row-sum limit
+  int prefill_pipe_masked = 1;      // RPA_PREFILL_PIPE_MASKED    0: the steps on the causal diagonal through compiled code
   int prefill_splits = -1;          // RPA_PREFILL_SPLITS         -1: cost model; 0 | 1 never; n forces n pieces
   // ---- absorbed MLA (rpa_mla.hip)
   int mla_min_chunk = 256;          // RPA_MLA_MIN_CHUNK
