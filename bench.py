@@ -49,9 +49,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
-# HBM bytes per launch (read + write) of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE scaled by a 1 GiB device copy (profiles/hbm_traffic_pmc.txt).  Counter runs cannot be
-# taken inside this process, so these are the figures of the committed profile, not live ones.
+# HBM bytes per launch (read + write) of the dominant kernels, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE scaled
+# by a 1 GiB device copy (profiles/hbm_traffic_pmc.txt).  Counter runs cannot be taken inside this process, so the
+# figures come from sglang-jax_amd/measured_traffic.json, written next to that profile together with the hash of
+# the kernel sources they were measured on: when the sources have changed since, `traffic` is null rather than stale.
 # kernel that streams the KV bytes of each workload's decode rows: ragged batches that need
 # splitting take the balanced plan, equal-length and tiny ones the fixed split plan
 DECODE_KERNEL = {
@@ -68,13 +69,22 @@ DECODE_KERNEL = {
 
 PREFILL_KERNEL = "rpa_prefill_pipe_kernel"
 
-MEASURED_TRAFFIC_BYTES = {
-    ("c2", PREFILL_KERNEL): 326.5e6 + 77.2e6,
-    ("c2", "rpa_decode_balanced_kernel"): 501.0e6 + 2.7e6,
-    ("c3", "rpa_decode_splitkv_kernel"): 2148.6e6 + 1.9e6,
-    ("c5", "rpa_mla_balanced_wide_kernel"): 820.3e6 + 44.8e6,
-    ("c5p", "rpa_mla_decode_wide_kernel (one row per query token)"): 633.0e6 + 268.4e6,
-}
+
+def _load_measured_traffic():
+    path = os.path.join(ROOT, "sglang-jax_amd", "measured_traffic.json")
+    try:
+        with open(path) as f:
+            rec = json.load(f)
+        import __graft_entry__ as graft
+
+        if rec.get("source_hash") != graft._load_build_module().source_hash():
+            return {}, "the kernel sources changed since profiles/hbm_traffic_pmc.txt was taken"
+        return {tuple(k.split("|")): v for k, v in rec["bytes"].items()}, None
+    except (OSError, ValueError, KeyError) as e:
+        return {}, f"no counter record ({e.__class__.__name__})"
+
+
+MEASURED_TRAFFIC_BYTES, TRAFFIC_NOTE = _load_measured_traffic()
 
 
 def _events(n):
@@ -596,6 +606,8 @@ def main():
     def with_achievable(r):
         """frac_of_achievable next to frac: the same figure against what a plain kernel reaches on this device"""
         top = achievable(r["bound"])
+        if TRAFFIC_NOTE and "traffic" in r:
+            r["traffic_note"] = TRAFFIC_NOTE
         r["frac_of_achievable"] = None if top is None else r["achieved"] / top
         if r.get("frac_back_to_back") is not None and top is not None:
             r["frac_of_achievable_back_to_back"] = r["frac_back_to_back"] * r["peak"] / top
