@@ -141,8 +141,10 @@ inline bool shape_rule_matches(const ShapeRule& r, const ShapeKey& k) {
 inline const ShapeRule& select_shape(const ShapeKey& k, unsigned skip = 0) {
   for (int i = 0; i < kNumShapeRules; ++i)
     if (!(skip & (1u << kShapeRules[i].kernel)) && shape_rule_matches(kShapeRules[i], k)) return kShapeRules[i];
-  // every stage ends in a row without conditions; a key of no stage is a programming error
-  return kShapeRules[k.stage == kStageDecode ? 4 : (k.stage == kStagePrefill ? 12 : kNumShapeRules - 1)];
+  // every stage ends in a row with the fewest conditions: the last row of the key's stage
+  for (int i = kNumShapeRules - 1; i > 0; --i)
+    if (kShapeRules[i].stage == k.stage) return kShapeRules[i];
+  return kShapeRules[0];
 }
 
 }  // namespace rpa

@@ -690,3 +690,31 @@ def test_mla_device_side_distribution(pkg, wl, gpu):
     assert_parity(auto[:T].cpu().float(), want.float(), **TOL)
     # whole rows in both modes: the same arithmetic, bit for bit
     assert torch.equal(dev[:T].view(torch.int16), host[:T].view(torch.int16))
+
+
+def test_mla_token_groups_with_the_composition_on_the_device(pkg, wl, gpu):
+    """16 heads, chunks whose tokens run eight to a workgroup, in static-shape mode: the token total and the number of
+    sequences are bounds (a bucket padded with empty sequences and spare tokens), windows of tokens past the real
+    total leave at once."""
+    q_lens = [1, 300, 77]
+    kv_lens = [900, 1500, 77]
+    b = wl.make_mla_batch("mla_tg_static", q_lens, kv_lens, num_q_heads=16, lkv_dim=512, rope_dim=64, page_size=64, seed=8307,
+                          sm_scale=192 ** -0.5)
+    wl.plant_mla_needles(b, seed=8)
+    T = sum(q_lens)
+    pad_s, pad_t = 5, 130
+    g = b.to(gpu)
+    kv_pad = torch.cat([g.kv_lens, torch.zeros(pad_s, dtype=torch.int32, device=gpu)])
+    cu_q_pad = torch.cat([g.cu_q_lens, torch.full((pad_s,), T, dtype=torch.int32, device=gpu)])
+    cu_kv_pad = torch.cat([g.cu_kv_lens, g.cu_kv_lens[-1:].expand(pad_s)])
+    qn = torch.cat([g.ql_nope, torch.zeros(pad_t, 16, 512, dtype=torch.bfloat16, device=gpu)])
+    qp = torch.cat([g.q_pe, torch.zeros(pad_t, 16, 64, dtype=torch.bfloat16, device=gpu)])
+    want = oracle(b)
+    dev, _ = pkg.mla_ragged_paged_attention(qn, qp, None, None, g.cache_kv, kv_pad, g.page_indices, cu_q_pad, cu_kv_pad,
+                                            g.distribution, sm_scale=b.sm_scale)
+    host, _ = pkg.mla_ragged_paged_attention(qn, qp, None, None, g.cache_kv, kv_pad, g.page_indices, cu_q_pad, cu_kv_pad,
+                                             b.distribution.cpu().numpy(), sm_scale=b.sm_scale, max_kv_len=max(kv_lens))
+    torch.cuda.synchronize()
+    assert_parity(dev[:T].cpu().float(), want.float(), **TOL)
+    assert torch.equal(dev[:T].view(torch.int16), host[:T].view(torch.int16))
+
