@@ -25,7 +25,10 @@ The loop runs EVERY tile of a segment, so no compiled code ever holds the accumu
     tile's scores, worked out before any accumulator exists) and only ever rises (rare path, as in
     gen_mla_pipe_loop.py: +16, +32, +64 ... for the heads whose row sum passed 2^8);
   * the first tile and the row's last tile take a masking detour after their scores: tokens before the
-    window's edge or past the row's end get -1e30 (per-lane limits come in with the caller's operands);
+    window's edge or past the row's end get -1e30 (per-lane limits come in with the caller's operands).  Token
+    groups (a wave's two blocks of heads belong to neighbouring query tokens of a chunk, whose rows end up to
+    seven tokens before the group's last) also take it on the tile before the last (%[mask_early] = 1), and the
+    second block's row ends %[hi_step] tokens after the first's;
   * from the moment the tile being copied (three ahead) is the row's last, the copies use a second set of
     per-lane offsets whose rows are clamped to the last valid token, so no bytes from beyond the row ever
     reach LDS.
@@ -89,7 +92,7 @@ ST = [62, 63, 64, 65]        # temporaries
 PGN = 66                     # page id of tile t + 4
 ONES, LIMIT, DELTA, PASS = 67, 68, 69, 70
 PMASK, PSTR = 71, 72         # page_size - 1, bytes per page
-LASTK = 73                   # index of the row's last tile inside the segment
+LASTK = 73                   # first tile, counted from the segment's first, of the masked tail (the row's last, or the one before)
 CPB, CPL = 74, 75            # LDS addresses for the step's copies (see copy_group)
 SGPR_CLOBBERS = list(range(60, 76))
 
@@ -225,6 +228,8 @@ def mask_block(em, k, sc, tag):
     em.emit(valu(f"v_subrev_u32 {vr(T1)}, {a}, {vr(HI)}", [HI], [T1]))       # HI - 32 t
     em.emit(valu(f"v_mov_b32 {vr(A)}, {NEG_BIG}", [], [A]))
     for hb in range(2):
+        if hb == 1:
+            em.emit(valu(f"v_add_u32 {vr(T1)}, %[hi_step], {vr(T1)}", [T1], [T1]))   # the second block's own row end
         for b in range(2):
             for r in range(4):
                 reg = sc[hb][b] + r
@@ -237,10 +242,10 @@ def mask_block(em, k, sc, tag):
 
 
 def mask_check(em, tag):
-    """detour for the segment's first tile (t == 0) and the row's last (t == LASTK)"""
+    """detour for the segment's first tile (t == 0) and the masked tail (t >= LASTK)"""
     em.raw("s_cmp_eq_u32 %[t], 0")
     em.raw(f"s_cbranch_scc1 L_mask_{tag}_%=")
-    em.raw(f"s_cmp_eq_u32 %[t], s{LASTK}")
+    em.raw(f"s_cmp_ge_i32 %[t], s{LASTK}")
     em.raw(f"s_cbranch_scc1 L_mask_{tag}_%=")
     em.label(f"L_mask_back_{tag}_%=")
 
@@ -431,6 +436,7 @@ def generate():
     em.raw(f"s_lshl_b32 s{PSTR}, %[row_bytes], %[pshift]")
     em.raw(f"s_sub_u32 s{LASTK}, %[last_tile_tok], %[t_begin]")
     em.raw(f"s_ashr_i32 s{LASTK}, s{LASTK}, 5")                 # the row's last tile, counted from the segment's first
+    em.raw(f"s_sub_u32 s{LASTK}, s{LASTK}, %[mask_early]")
     for hb in range(2):
         em.emit(valu(f"v_mul_f32 {vr(NEGM[hb])}, -1.0, {vr(M[hb])}", [M[hb]], [NEGM[hb]]))
     if PIPELINED:

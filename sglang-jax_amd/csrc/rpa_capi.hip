@@ -984,10 +984,19 @@ int rpa_mla_describe_plan(const RpaMlaParams* p, int token_rows, char* buf, size
   const rpa::ShapeRule& r = rpa::select_shape(rpa::mla_shape_key(a), rpa::mla_shape_skip(rpa::tuning()));
   const SplitPlan sp = mla_plan(p, std::max<int64_t>(rows, 1));
   const bool bal = rows > 0 && mla_use_balanced(p, sp, token_rows != 0);
-  return snprintf(buf, len, "mla: shape=%s rows=%lld waves_per_wg=%d heads_per_wg=%d share=%d plan=%s pieces_per_row=%d "
-                  "workgroups=%d workspace=%zu\n",
-                  r.name, (long long)rows, r.waves_per_wg, r.tile_heads, r.share, bal ? "balanced" : "fixed",
-                  bal ? 0 : sp.splits, bal ? mla_wgs() : 0, mla_workspace(p, rows, token_rows != 0));
+  a.sm.window = p->sliding_window;
+  a.num_rows = (int32_t)rows;
+  a.num_seqs = p->num_seqs;
+  a.rows_are_tokens = token_rows ? 1 : 0;
+  a.max_splits = sp.splits;
+  a.balanced = bal ? 1 : 0;
+  static const char* const kGroups[] = {"off", "eight_waves_compiled", "eight_waves", "wide"};
+  const int tg = rpa::mla_token_group_mode(a, rpa::tuning(), r);
+  return snprintf(buf, len, "mla: shape=%s rows=%lld waves_per_wg=%d heads_per_wg=%d share=%d token_groups=%s plan=%s "
+                  "pieces_per_row=%d workgroups=%d workspace=%zu\n",
+                  r.name, (long long)rows, tg == 3 ? 4 : r.waves_per_wg, tg ? 128 : r.tile_heads, tg ? 1 : r.share, kGroups[tg],
+                  bal ? "balanced" : "fixed", bal ? 0 : sp.splits, bal ? mla_wgs() : 0,
+                  mla_workspace(p, rows, token_rows != 0));
 }
 
 int rpa_mla_decode(const RpaMlaParams* p, void* stream) { return mla_run(p, stream, false); }

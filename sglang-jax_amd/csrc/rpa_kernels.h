@@ -193,6 +193,8 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream);
 const ShapeRule& prefill_shape_of(const PrefillArgs& a);
 ShapeKey mla_shape_key(const MlaDecodeArgs& a);
 unsigned mla_shape_skip(const Tuning& tune);
+// how query tokens of a chunk share a workgroup (0: they do not; 1, 2: eight waves; 3: wide workgroups)
+int mla_token_group_mode(const MlaDecodeArgs& a, const Tuning& tune, const ShapeRule& shape);
 hipError_t launch_mla_kv_write(const MlaWriteArgs& a, hipStream_t stream);
 
 }  // namespace rpa

@@ -761,10 +761,16 @@ constexpr int vmcnt_imm(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 // M32: the loop of rpa_mla_wide32_loop.inc (32x32x16 matrix instructions, one head per lane and half: lane c of
 // half h = lane / 32 owns head head0 + c and the tokens 8 (i / 4) + 4 h + i % 4 of a tile) instead of two blocks of
 // 16 heads on 16x16x32 instructions.
-template <bool M32>
+// TG (token group, see mla_segment; 16 / 32 / 64 heads, no window): the workgroup's eight blocks of 16 heads are the
+// heads of 8 / 4 / 2 consecutive query tokens of one sequence, `group_tokens` of them real.  Block hb of wave w
+// is "head" 32 w + 16 hb .. of a 128-head row at mr.tq, i.e. token (32 w + 16 hb) / Hq of the group; mr.kv_len is what
+// the group's LAST token sees, a block's own token sees up to group_tokens - 1 fewer, so the loop masks the
+// tile before the last too and takes the second block's row end relative to the first's.
+template <bool M32, bool TG = false>
 __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const MlaRow mr, int head_base, int t_lo,
                                                  int t_begin, int t_end, const MlaDest dest, char* ring,
-                                                 int trace_piece = 0) {
+                                                 int trace_piece = 0, int group_tokens = 1) {
+  static_assert(!(M32 && TG), "token groups run on the loop of two 16-head blocks");
   (void)trace_piece;
   RPA_MLA_STAMP(0);
   constexpr int CPW = 2 * kCopiesPerWave;
@@ -776,6 +782,25 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   const int seq = mr.seq;
   const int kv_len = mr.kv_len;
   const int tq = mr.tq;
+  // per block of 16 heads: its first head in the row at tq, whether it writes, and the length its token sees
+  int blk_head[2], blk_len[2];
+  bool blk_real[2];
+#pragma unroll
+  for (int hb = 0; hb < 2; ++hb) {
+    if constexpr (TG) {
+      // (16, 32 or 64 heads: shifts, and every value the same in all lanes)
+      const int hq_shift = __builtin_amdgcn_readfirstlane(31 - __builtin_clz(a.Hq));
+      const int h = wave * 32 + 16 * hb;
+      const int place = min(h >> hq_shift, group_tokens - 1);  // a block past the group's last real token repeats that token
+      blk_real[hb] = (h >> hq_shift) < group_tokens;
+      blk_head[hb] = __builtin_amdgcn_readfirstlane((place << hq_shift) + (h & (a.Hq - 1)));
+      blk_len[hb] = __builtin_amdgcn_readfirstlane(kv_len - (group_tokens - 1) + place);
+    } else {
+      blk_real[hb] = true;
+      blk_head[hb] = head0 + 16 * hb;
+      blk_len[hb] = kv_len;
+    }
+  }
 
   Src src;
   src.page_size = a.pt.page_size;
@@ -804,7 +829,7 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   } else {
 #pragma unroll
     for (int hb = 0; hb < 2; ++hb) {
-      const int head = min(head0 + 16 * hb + c, a.Hq - 1);
+      const int head = TG ? blk_head[hb] + c : min(head0 + 16 * hb + c, a.Hq - 1);
       const uint16_t* qn = a.ql_nope + ((int64_t)tq * a.Hq + head) * 512 + g * 8;
       const uint16_t* qr = a.q_pe + ((int64_t)tq * a.Hq + head) * 64 + g * 8;
 #pragma unroll
@@ -866,7 +891,7 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int tok = t_begin + tok_of(g, i);
-        if (tok < kv_len && tok >= t_lo) mx = fmaxf(mx, s[hb][i >> 2][i & 3] * scale2);
+        if (tok < blk_len[hb] && tok >= t_lo) mx = fmaxf(mx, s[hb][i >> 2][i & 3] * scale2);
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16));
       mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -913,8 +938,10 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
     ml = u32x8_t{__float_as_uint(m_init[0]), 0u, __float_as_uint(m_init[1]), 0u,
                  lds_base + (uint32_t)(cc * kRowB + gg * 16),
                  lds_base + (uint32_t)((4 * gg + (cc >> 2)) * kRowB + (cc & 3) * 8),
-                 (uint32_t)(t_lo - t_begin - 4 * gg), (uint32_t)(kv_len - t_begin - 4 * gg)};
+                 (uint32_t)(t_lo - t_begin - 4 * gg), (uint32_t)(blk_len[0] - t_begin - 4 * gg)};
   }
+  const int hi_step = blk_len[1] - blk_len[0];
+  const int mask_early = TG ? 1 : 0;
   u32x16_t ofs, ofsl;
 #pragma unroll
   for (int n = 0; n < 16; ++n) ofs[n] = ofsl[n] = 0;
@@ -943,7 +970,7 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   : C(Q0)(q0), C(Q1)(q1), C(Q2)(q2), C(Q3)(q3), C(Q4)(q4), C(OFSL)(ofsl), [t_end] "s"(nT), [t_begin] "s"(t_begin),     \
     [last_tile_tok] "s"(last_tile_tok), [row_bytes] "s"(src.row_bytes), [pshift] "s"(src.page_shift),                  \
     [cache_lo] "s"(cache_lo), [cache_hi] "s"(cache_hi), [pages] "s"(src.pages), [scale2] "s"(scale2_bits),             \
-    [wave_blk] "s"(wave_blk), [slot0] "s"(lds_base)
+    [wave_blk] "s"(wave_blk), [slot0] "s"(lds_base), [hi_step] "s"(hi_step), [mask_early] "s"(mask_early)
   if constexpr (M32) {
     asm volatile(RPA_MLA_WIDE32_ASM RPA_WIDE_OPERANDS : RPA_MLA_WIDE32_CLOBBERS);
   } else {
@@ -989,8 +1016,8 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
     float l = __uint_as_float(ml[2 * hb + 1]);
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
-    const int head = head0 + 16 * hb + c_out;
-    if (head >= a.Hq) continue;
+    const int head = blk_head[hb] + c_out;
+    if (TG ? !blk_real[hb] : head >= a.Hq) continue;
     if (dest.final_rows) {
       const float inv = a.out_scale / l;
       uint16_t* op = a.out + ((int64_t)tq * a.Hq + head) * 512 + g_out * 4;
@@ -1070,6 +1097,43 @@ __global__ __launch_bounds__(512, 2) void rpa_mla_token_group_kernel(const MlaDe
       dest.base = 0;
       mla_segment<true, false, PIPE, FP8, 1, true>(a, mr, 0, t_lo, t_lo & ~(kTok - 1), mr.kv_len, dest, slot0, slot1, slot2,
                                                    slot3, n);
+    }
+    t += n;
+    if (t >= q1) ++seq;
+  }
+}
+
+// ---- token groups on wide workgroups (see mla_segment_wide, TG): bf16 latents, no window.  Same grid and the same
+// walk over a window of 128 / Hq query tokens as rpa_mla_token_group_kernel.
+__global__ __launch_bounds__(256, 1) void rpa_mla_token_group_wide_kernel(const MlaDecodeArgs a) {
+  __shared__ __attribute__((aligned(1024))) char ring[4 * kSlotB];
+  const int num_seqs = a.dist ? min(a.num_seqs, scalar_load_i32(a.dist + 2)) : a.num_seqs;
+  const int total = min(a.num_rows, scalar_load_i32(a.pt.cu_q_lens + num_seqs));
+  const int per = 128 / a.Hq;
+  int t = (int)blockIdx.x * per;
+  if (t >= total) return;
+  const int t_stop = min(t + per, total);
+  int seq = owner_of_token(a.pt.cu_q_lens, num_seqs, t);
+  while (t < t_stop) {
+    seq = __builtin_amdgcn_readfirstlane(seq);
+    t = __builtin_amdgcn_readfirstlane(t);
+    const int q0 = scalar_load_i32(a.pt.cu_q_lens + seq);
+    const int q1 = scalar_load_i32(a.pt.cu_q_lens + seq + 1);
+    if (q1 <= t) {  // (a sequence without tokens)
+      ++seq;
+      continue;
+    }
+    const int n = __builtin_amdgcn_readfirstlane(min(t_stop, q1) - t);  // tokens of this sequence in the window
+    MlaRow mr;
+    mr.seq = seq;
+    mr.tq = t;
+    mr.valid = true;
+    mr.kv_len = __builtin_amdgcn_readfirstlane(scalar_load_i32(a.pt.kv_lens + seq) - (q1 - q0) + (t + n - 1 - q0) + 1);
+    if (mr.kv_len > 0 && mr.kv_len - (n - 1) > 0) {
+      MlaDest dest;
+      dest.final_rows = true;
+      dest.base = 0;
+      mla_segment_wide<false, true>(a, mr, 0, 0, 0, mr.kv_len, dest, ring, 0, n);
     }
     t += n;
     if (t >= q1) ++seq;
@@ -1385,6 +1449,24 @@ unsigned mla_shape_skip(const Tuning& tune) {
          (tune.mla_wide == 0 ? (1u << kKernelMlaWide) : 0u) | (tune.mla_shared_tiles == 0 ? (1u << kKernelMlaShared) : 0u);
 }
 
+// Prefill / mixed rows with few heads: a workgroup holds 128 / Hq consecutive query tokens of a sequence over
+// shared tiles instead of one token whose heads leave most of it idle (rows_are_tokens, whole rows, a head count
+// that divides 128, whole tiles in pages, no soft cap; RPA_MLA_TOKEN_GROUPS=0 keeps one token per workgroup).
+// Decode batches (one token per sequence) have nothing to group and keep the shared tiles.
+// 0: no groups; 1: eight waves of one block of 16 heads (compiled tile loop); 2: the same around the assembly
+// steady state; 3: four waves of two blocks on the wide loop (every operand fragment feeds two matrix
+// instructions: bf16 latents, power-of-two pages, no window).
+int mla_token_group_mode(const MlaDecodeArgs& a, const Tuning& tune, const ShapeRule& shape) {
+  if (shape.kernel != kKernelMlaShared || !a.rows_are_tokens || a.max_splits > 1 || a.balanced ||
+      tune.mla_token_groups == 0 || (128 % a.Hq) != 0 || a.Hq < 16 || a.num_rows < 4 * a.num_seqs)
+    return 0;
+  const int P = a.pt.page_size;
+  const bool pipe_ok = tune.mla_pipe != 0 && (P & (P - 1)) == 0 && (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);
+  if (!pipe_ok) return 1;
+  if (!a.fp8 && a.sm.window <= 0 && tune.mla_wide != 0 && tune.mla_wide != 32) return 3;
+  return 2;
+}
+
 hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   if (a.num_rows <= 0) return hipSuccess;
   const int head_groups = (a.Hq + 127) / 128;
@@ -1401,16 +1483,14 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   const ShapeRule& shape = select_shape(mla_shape_key(a), mla_shape_skip(tune));
   const bool pipe = shape.kernel == kKernelMlaWide || shape.kernel == kKernelMlaPipe;
   const int ds = shape.kernel == kKernelMlaShared ? shape.share : 1;
-  // Prefill / mixed rows with few heads: a workgroup holds 128 / Hq consecutive query tokens of a sequence over
-  // shared tiles instead of one token whose heads leave most of it idle (rows_are_tokens, whole rows, a head count
-  // that divides 128, whole tiles in power-of-two pages, no soft cap; RPA_MLA_TOKEN_GROUPS=0 keeps one token per
-  // workgroup).  Decode batches (one token per sequence) have nothing to group and keep the shared tiles.
-  if (ds != 1 && a.rows_are_tokens && a.max_splits <= 1 && !a.balanced && tune.mla_token_groups != 0 &&
-      (128 % a.Hq) == 0 && a.Hq >= 16 && a.num_rows >= 4 * a.num_seqs) {
-    const int P = a.pt.page_size;
-    const bool pipe_ok = tune.mla_pipe != 0 && (P & (P - 1)) == 0 && (int64_t)a.row_stride * 2 * P < (int64_t(1) << 32);
+  if (const int tg = mla_token_group_mode(a, tune, shape)) {
+    const bool pipe_ok = tg >= 2;
     const int per = 128 / a.Hq;
     const dim3 tg_grid((unsigned)((a.num_rows + per - 1) / per));
+    if (tg == 3) {
+      hipLaunchKernelGGL(rpa_mla_token_group_wide_kernel, tg_grid, dim3(256), 0, stream, a);
+      return hipGetLastError();
+    }
     if (a.fp8) {
       if (pipe_ok) hipLaunchKernelGGL((rpa_mla_token_group_kernel<true, true>), tg_grid, block, 0, stream, a);
       else hipLaunchKernelGGL((rpa_mla_token_group_kernel<false, true>), tg_grid, block, 0, stream, a);

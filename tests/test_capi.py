@@ -421,7 +421,21 @@ def test_mla_shape_table_rows(pkg, monkeypatch):
     assert "shape=mla_compiled" in d(params(128, P=16), False)
     assert "shape=mla_compiled" in d(params(128, soft_cap=30.0), False)
     assert "shape=mla_compiled" in d(params(160), False)
+    # query tokens of a chunk with few heads share a workgroup: on the wide loop for bf16 latents without a window
+    chunk = dict(S=4, T=4096, max_kv=8192, sum_kv=20000)
+    assert "token_groups=off" in d(params(16), False) and "token_groups=off" in d(params(16), True)  # decode rows
+    assert "token_groups=wide" in d(params(16, **chunk), True) and "waves_per_wg=4" in d(params(16, **chunk), True)
+    assert "token_groups=eight_waves " in d(params(32, fp8=True, **chunk), True)
+    windowed = params(64, **chunk)
+    windowed.sliding_window = 512
+    assert "token_groups=eight_waves " in d(windowed, True)
+    assert "token_groups=off" in d(params(48, **chunk), True) and "token_groups=off" in d(params(128, **chunk), True)
+    monkeypatch.setenv("RPA_MLA_TOKEN_GROUPS", "0")
+    assert "token_groups=off" in d(params(16, **chunk), True)
+    monkeypatch.delenv("RPA_MLA_TOKEN_GROUPS")
     monkeypatch.setenv("RPA_MLA_WIDE", "0")
+    assert "token_groups=eight_waves " in d(params(16, **chunk), True)
     assert "shape=mla_pipe" in d(params(128), False)
     monkeypatch.setenv("RPA_MLA_PIPE", "0")
     assert "shape=mla_compiled" in d(params(128), False)
+    assert "token_groups=eight_waves_compiled" in d(params(16, **chunk), True)

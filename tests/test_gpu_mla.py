@@ -108,8 +108,10 @@ def test_mla_prefill_rows_share_tiles_among_query_tokens_when_heads_are_few(pkg,
     """Prefill / mixed batches with 16 / 32 / 64 heads (the reference's own MLA test shape has 16,
     test_mla_attention.py:346): a workgroup holds 8 / 4 / 2 consecutive query tokens of a sequence over shared
     latent tiles, each wave masking with its own token's length (the reference's kernel shares a tile among 16
-    query tokens, kernels/mla/v2/kernel.py:1448-1459).  Against the oracle and against one token per workgroup
-    (RPA_MLA_TOKEN_GROUPS=0): chunk lengths that leave partial groups, windows of tokens that span the border
+    query tokens, kernels/mla/v2/kernel.py:1448-1459).  bf16 latents without a window run the groups on wide
+    workgroups (four waves, each with two blocks of heads that may belong to two tokens), everything else on eight
+    waves.  Against the oracle, against one token per workgroup (RPA_MLA_TOKEN_GROUPS=0) and against the
+    eight-wave groups (RPA_MLA_WIDE=0): chunk lengths that leave partial groups, windows of tokens that span the border
     between two sequences, decode rows in front, a chunk with no prefix, a sliding window shorter than the chunk,
     pages of 32 and 128 tokens, planted keys."""
     ref = fp8_oracle if f8 else oracle
@@ -132,6 +134,11 @@ def test_mla_prefill_rows_share_tiles_among_query_tokens_when_heads_are_few(pkg,
         monkeypatch.delenv("RPA_MLA_TOKEN_GROUPS")
         assert_parity(single.float(), want.float(), **TOL)
         assert_parity(grouped.float(), single.float(), **TOL)
+        monkeypatch.setenv("RPA_MLA_WIDE", "0")
+        eight = run_gpu(pkg, b, gpu)[:T]
+        monkeypatch.delenv("RPA_MLA_WIDE")
+        assert_parity(eight.float(), want.float(), **TOL)
+        assert_parity(grouped.float(), eight.float(), **TOL)
         monkeypatch.setenv("RPA_MLA_PIPE", "0")  # the compiled tile loop under the same grouping
         compiled = run_gpu(pkg, b, gpu)[:T]
         monkeypatch.delenv("RPA_MLA_PIPE")
