@@ -168,7 +168,6 @@ def step(em, k):
     """tile t in slot k: scores, softmax, second product; tile t + 3 goes to slot (k + 3) & 3"""
     fill = (k + 3) & 3
     tile_scalars(em, k)
-    copy_bases(em, fill)
     em.emit(valu(f"v_add_u32 {vr(KADDR)}, {k * SLOT_B}, {vr(KBASE)}", [KBASE], [KADDR]))
     em.emit(valu(f"v_add_u32 {vr(VADDR)}, {k * SLOT_B}, {vr(VBASE)}", [VBASE], [VADDR]))
     copies = [] if "nocopy" in X else [copy_group(n, fill) for n in range(COPIES)]
@@ -219,6 +218,7 @@ def generate():
     em.raw(f"s_lshl_b32 s{PSTR}, %[row_bytes], %[pshift]")
     em.raw(f"s_sub_u32 s{LASTK}, %[last_tile_tok], %[t_begin]")
     em.raw(f"s_ashr_i32 s{LASTK}, s{LASTK}, 5")
+    copy_bases(em)
     em.emit(valu(f"v_mul_f32 {vr(NEGM)}, -1.0, {vr(M)}", [M], [NEGM]))
     em.raw(f"s_and_b32 {a}, %[t], 3")
     for k in range(1, 4):

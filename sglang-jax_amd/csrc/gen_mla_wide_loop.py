@@ -52,7 +52,8 @@ PIPELINED = "pipe" in X      # scores of tile t + 1 under the softmax of tile t 
 NBUF = 4 if PIPELINED else 8  # operand fragment buffers (the second set of score registers of the pipelined loop pays for four)
 AHEAD = int(os.environ.get("RPA_MLA_WIDE_AHEAD", 3 if PIPELINED else 6))
 assert AHEAD < NBUF
-PAIRWAIT = "nopairwait" not in X
+WAITGROUP = int(os.environ.get("RPA_MLA_WIDE_WAITGROUP", 4))  # fragments whose data one wait instruction covers
+assert 1 <= WAITGROUP <= AHEAD
 
 ROW_B = 1184                 # bytes of a latent row in LDS
 SLOT_B = 37 * 1024           # one ring slot
@@ -93,8 +94,8 @@ PGN = 66                     # page id of tile t + 4
 ONES, LIMIT, DELTA, PASS = 67, 68, 69, 70
 PMASK, PSTR = 71, 72         # page_size - 1, bytes per page
 LASTK = 73                   # first tile, counted from the segment's first, of the masked tail (the row's last, or the one before)
-CPB, CPL = 74, 75            # LDS addresses for the step's copies (see copy_group)
-SGPR_CLOBBERS = list(range(60, 76))
+CPB = 74                     # LDS address of this wave's first copy block in slot 0 (see copy_group)
+SGPR_CLOBBERS = list(range(60, 75))
 
 NEG_BIG = "0xf149f2ca"       # -1e30
 
@@ -132,9 +133,9 @@ def frag_tags(f):
 
 
 def frag_mfmas(f, sc):
-    """the two matrix instructions (one per block of heads) that consume fragment f; scores go to `sc`.  With
-    PAIRWAIT the first instruction of an even fragment also waits for the odd fragment behind it (requested long
-    before): one wait instruction per two fragments."""
+    """the two matrix instructions (one per block of heads) that consume fragment f; scores go to `sc`.  The first
+    instruction of every WAITGROUP-th fragment also waits for the fragments behind it in its group (requested long
+    before): one wait instruction per group -- a lone wave pays for every instruction it issues."""
     out = []
     for hb in range(2):
         if f < 36:
@@ -144,8 +145,9 @@ def frag_mfmas(f, sc):
             j = f - 36
             ins = mfma(O[hb] + 4 * j, ring(f), P[hb], O[hb] + 4 * j)
         ins.lds_need = None if "nolds" in X else list(frag_tags(f))
-        if PAIRWAIT and hb == 0 and f % 2 == 0 and ins.lds_need is not None and AHEAD >= 2:
-            ins.lds_need += frag_tags(f + 1)
+        if hb == 0 and f % WAITGROUP == 0 and ins.lds_need is not None:
+            for g in range(f + 1, min(f + WAITGROUP, 68)):
+                ins.lds_need += frag_tags(g)
         out.append(ins)
     return out
 
@@ -167,19 +169,26 @@ def softmax(hb, sc, check=True):
     return out
 
 
+def copy_dest(n, fill_slot):
+    """m0 = LDS address of copy n of this wave: block wave + 4 n of the slot for n < 9 (36 blocks), the 37th block for
+    every wave's last copy (the same bytes four times).  s[CPB] = slot 0 + 1024 * wave."""
+    if n < COPIES - 1:
+        return Ins(f"s_add_u32 m0, s{CPB}, {fill_slot * SLOT_B + n * 4096}", "salu")
+    return Ins(f"s_add_u32 m0, %[slot0], {fill_slot * SLOT_B + (BLOCKS - 1) * 1024}", "salu")
+
+
+def copy_load(n):
+    return Ins(f"global_load_lds_dwordx4 {vr(OFS + n)}, s[{SB}:{SB + 1}]", "vmem", [OFS + n], [])
+
+
 def copy_group(n, fill_slot):
-    """copy n of this wave: block 10 * wave + n of the slot (blocks past the 37th repeat the last one); s[CPB] is
-    the LDS address of the wave's first block in the slot being filled, s[CPL] that of the slot's last block"""
-    return [Ins(f"s_add_u32 m0, s{CPB}, {n * 1024}", "salu"),
-            Ins(f"s_min_u32 m0, m0, s{CPL}", "salu"),
-            Ins("s_nop 0", "nop"),
-            Ins(f"global_load_lds_dwordx4 {vr(OFS + n)}, s[{SB}:{SB + 1}]", "vmem", [OFS + n], [])]
+    """one copy as a self-contained group (a wait state between the write of m0 and its use)"""
+    return [copy_dest(n, fill_slot), Ins("s_nop 0", "nop"), copy_load(n)]
 
 
-def copy_bases(em, fill_slot):
-    em.raw(f"s_add_u32 s{CPL}, %[slot0], {fill_slot * SLOT_B + (BLOCKS - 1) * 1024}")
-    em.raw(f"s_add_u32 s{CPB}, %[slot0], {fill_slot * SLOT_B}")
-    em.raw(f"s_add_u32 s{CPB}, s{CPB}, %[wave_blk]")
+def copy_bases(em):
+    """once per loop"""
+    em.raw(f"s_add_u32 s{CPB}, %[slot0], %[wave_blk]")
 
 
 def tile_scalars(em, k):
@@ -321,14 +330,17 @@ def qk_phase(em, sc, kaddr, copies, extra=None, into_pv=False):
     for f in range(AHEAD):
         emit_all(em, frag_read(f, kaddr))
     for f in range(36):
+        cp = copies[copy_at[f]] if (f in copy_at and copies) else None
+        if cp:
+            em.emit(cp[0])       # m0; the matrix instructions behind it are the wait state its use needs
         for ins in frag_mfmas(f, sc):
             em.emit(ins)
             if extra:
                 em.emit(extra.pop(0))
         if f + AHEAD < (68 if into_pv else 36):
             emit_all(em, frag_read(f + AHEAD, kaddr))
-        if f in copy_at and copies:
-            emit_all(em, copies[copy_at[f]])
+        if cp:
+            em.emit(cp[1])
     emit_all(em, extra)
 
 
@@ -360,10 +372,9 @@ def step_plain(em, k):
     """tile t in slot k: scores, softmax, second product; tile t + 3 goes to slot (k + 3) & 3"""
     fill = (k + 3) & 3
     tile_scalars(em, k)
-    copy_bases(em, fill)
     em.emit(valu(f"v_add_u32 {vr(KADDR)}, {k * SLOT_B}, {vr(KBASE)}", [KBASE], [KADDR]))
     em.emit(valu(f"v_add_u32 {vr(VADDR)}, {k * SLOT_B}, {vr(VBASE)}", [VBASE], [VADDR]))
-    copies = [] if "nocopy" in X else [copy_group(n, fill) for n in range(COPIES)]
+    copies = [] if "nocopy" in X else [(copy_dest(n, fill), copy_load(n)) for n in range(COPIES)]
     qk_phase(em, SC, KADDR, copies, into_pv=True)
     mask_check(em, f"{k}")
     for hb in range(2):
@@ -378,7 +389,6 @@ def step_pipelined(em, k):
     fill = (k + 3) & 3
     cur, nxt = (SC, SC2) if k % 2 == 0 else (SC2, SC)
     tile_scalars(em, k)
-    copy_bases(em, fill)
     em.emit(valu(f"v_add_u32 {vr(KADDR2)}, {((k + 1) & 3) * SLOT_B}, {vr(KBASE)}", [KBASE], [KADDR2]))
     em.emit(valu(f"v_add_u32 {vr(VADDR)}, {k * SLOT_B}, {vr(VBASE)}", [VBASE], [VADDR]))
     copies = [] if "nocopy" in X else [copy_group(n, fill) for n in range(COPIES)]
@@ -437,6 +447,7 @@ def generate():
     em.raw(f"s_sub_u32 s{LASTK}, %[last_tile_tok], %[t_begin]")
     em.raw(f"s_ashr_i32 s{LASTK}, s{LASTK}, 5")                 # the row's last tile, counted from the segment's first
     em.raw(f"s_sub_u32 s{LASTK}, s{LASTK}, %[mask_early]")
+    copy_bases(em)
     for hb in range(2):
         em.emit(valu(f"v_mul_f32 {vr(NEGM[hb])}, -1.0, {vr(M[hb])}", [M[hb]], [NEGM[hb]]))
     if PIPELINED:

@@ -120,7 +120,9 @@ template <int CPW = kCopiesPerWave>
 __device__ __forceinline__ int copy_block(int wave, int n) {
   const int blk = wave * CPW + n;
   if constexpr (CPW == kCopiesPerWave) return blk < kUsedBlocks ? blk : 0;
-  else return min(blk, kUsedBlocks - 1);  // wide workgroups: the spare copies repeat the last block
+  // wide workgroups: copy n < 9 of wave w is block w + 4 n (the assembly loop then adds a constant to one base
+  // per copy), and every wave's last copy is the 37th block (the same bytes four times)
+  else return n < CPW - 1 ? wave + 4 * n : kUsedBlocks - 1;
 }
 
 template <int CPW = kCopiesPerWave>
@@ -957,7 +959,7 @@ __device__ __forceinline__ void mla_segment_wide(const MlaDecodeArgs& a, const M
   const uint32_t cache_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)a.cache >> 32));
   const int last_tile_tok = __builtin_amdgcn_readfirstlane(src.last_tok & ~(kTok - 1));
   const uint32_t scale2_bits = __builtin_amdgcn_readfirstlane(__float_as_uint(scale2));
-  const int wave_blk = wave * CPW * 1024;
+  const int wave_blk = wave * 1024;  // the wave's first copy block inside a slot (see copy_block)
   // `t` and `pg` change inside the block while the inputs are still being read: early-clobber, or the compiler
   // may give an input that happens to hold the same value on entry (the LDS base, 0, and t = 0) the same register
   int k = 0;
