@@ -656,7 +656,7 @@ def main():
     # dominant kernel of the workload (largest average launch time inside the timed region)
     roofline_decode = with_achievable(decode_roofline(args.config, main_res)) if dec_gbps is not None else None
     prefill_kernel = {"c5p": "rpa_mla_decode_wide_kernel (one row per query token)",
-                      "c5p16": "rpa_mla_token_group_kernel (8 query tokens per workgroup)"}.get(args.config, PREFILL_KERNEL)
+                      "c5p16": "rpa_mla_token_group_wide_kernel (8 query tokens per workgroup)"}.get(args.config, PREFILL_KERNEL)
 
     def prefill_roofline(name, res, kernel):
         return with_achievable({
@@ -712,7 +712,7 @@ def main():
             if name in ("c5p", "c5p16"):
                 r["roofline"] = with_achievable({
                     "kernel": "rpa_mla_decode_wide_kernel (one row per query token)" if name == "c5p"
-                              else "rpa_mla_token_group_kernel (8 query tokens per workgroup)", "bound": "mfma",
+                              else "rpa_mla_token_group_wide_kernel (8 query tokens per workgroup)", "bound": "mfma",
                     "achieved": r["prefill_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": r["prefill_tflops"] / MFMA_BF16_PEAK_TFLOPS, "avg_launch_ms": r["prefill_ms"],
                     "flops_per_launch": r["prefill_flops"]})
