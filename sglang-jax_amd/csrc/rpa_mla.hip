@@ -1321,47 +1321,60 @@ __global__ __launch_bounds__(256, 1) void rpa_mla_balanced_wide_kernel(const Mla
   });
 }
 
-// Merge the n partial rows of one (row, head): 128 threads, 4 dims each.  Partials are taken eight at
+// Merge the n partial rows of one (row, head): one wave, 8 dims (16 bytes) per lane.  Partials are taken eight at
 // a time with every load of a group (references, sums, rows) requested before any is used -- one
 // round trip to memory per group instead of one per partial -- and groups are chained like tiles of
-// an online softmax.
+// an online softmax.  Places of a group past the last partial load nothing.
+constexpr int kMergeThreads = 64;
 template <typename SlotOf>
 __device__ __forceinline__ void mla_merge(const MlaDecodeArgs& a, int n, SlotOf slot_of, int head, int tq) {
-  const int d = threadIdx.x * 4;
+  const int d = threadIdx.x * 8;
   float mstar = -INFINITY, den = 0.f;
-  f32x4_t o = {0.f, 0.f, 0.f, 0.f};
+  float o[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = 0.f;
   for (int j0 = 0; j0 < n; j0 += 8) {
     float mj[8], lj[8];
-    u32x2_t pr[8];
+    u32x4_t pr[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const int64_t slot = slot_of(min(j0 + u, n - 1));
-      mj[u] = a.ws_ml[slot * 2];
-      lj[u] = a.ws_ml[slot * 2 + 1];
-      pr[u] = *reinterpret_cast<const u32x2_t*>(a.ws_o + slot * 512 + d);
+      mj[u] = -INFINITY;
+      lj[u] = 0.f;
+      pr[u] = u32x4_t{0u, 0u, 0u, 0u};
+      if (j0 + u < n) {  // (the same in every lane)
+        const int64_t slot = slot_of(j0 + u);
+        mj[u] = a.ws_ml[slot * 2];
+        lj[u] = a.ws_ml[slot * 2 + 1];
+        pr[u] = ld16(a.ws_o + slot * 512 + d);
+      }
     }
     float mnew = mstar;
 #pragma unroll
-    for (int u = 0; u < 8; ++u) mnew = fmaxf(mnew, mj[u]);  // a repeated last partial changes nothing
+    for (int u = 0; u < 8; ++u) mnew = fmaxf(mnew, mj[u]);
     const float keep = fast_exp2(mstar - mnew);  // 0 for the first group
     den *= keep;
-    o *= keep;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] *= keep;
     mstar = mnew;
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const float w = (j0 + u < n) ? fast_exp2(mj[u] - mstar) : 0.f;
       den += lj[u] * w;
-      o += f32x4_t{bf16_lo_to_f32(pr[u][0]), bf16_hi_to_f32(pr[u][0]), bf16_lo_to_f32(pr[u][1]),
-                   bf16_hi_to_f32(pr[u][1])} * w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        o[2 * e] += bf16_lo_to_f32(pr[u][e]) * w;
+        o[2 * e + 1] += bf16_hi_to_f32(pr[u][e]) * w;
+      }
     }
   }
   const float inv = a.out_scale / den;
-  u32x2_t w = {pack_bf16x2(o[0] * inv, o[1] * inv), pack_bf16x2(o[2] * inv, o[3] * inv)};
-  *reinterpret_cast<u32x2_t*>(a.out + ((int64_t)tq * a.Hq + head) * 512 + d) = w;
+  const u32x4_t w = {pack_bf16x2(o[0] * inv, o[1] * inv), pack_bf16x2(o[2] * inv, o[3] * inv),
+                     pack_bf16x2(o[4] * inv, o[5] * inv), pack_bf16x2(o[6] * inv, o[7] * inv)};
+  st16(a.out + ((int64_t)tq * a.Hq + head) * 512 + d, w);
 }
 
-// Merge of the balanced plan.  grid = (Hq * rows); block = 128 threads, 4 dims each.
-__global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const MlaDecodeArgs a) {
+// Merge of the balanced plan.  grid = (Hq * rows); block = kMergeThreads.
+__global__ __launch_bounds__(kMergeThreads) void rpa_mla_combine_balanced_kernel(const MlaDecodeArgs a) {
   const int seq = (int)(blockIdx.x / (unsigned)a.Hq);  // grid.x = Hq * rows, heads fastest
   const int head = (int)blockIdx.x - seq * a.Hq;
   const int nt = mla_tiles(a.pt.kv_lens[seq], a.sm.window);
@@ -1385,8 +1398,8 @@ __global__ __launch_bounds__(128) void rpa_mla_combine_balanced_kernel(const Mla
   mla_merge(a, w_last - w_first + 1, [&](int j) { return slot_of(w_first + j); }, head, tq);
 }
 
-// grid = (Hq * rows); block = 128 threads, 4 dims each.
-__global__ __launch_bounds__(128) void rpa_mla_combine_kernel(const MlaDecodeArgs a) {
+// grid = (Hq * rows); block = kMergeThreads.
+__global__ __launch_bounds__(kMergeThreads) void rpa_mla_combine_kernel(const MlaDecodeArgs a) {
   const int row_id = (int)(blockIdx.x / (unsigned)a.Hq);  // grid.x = Hq * rows, heads fastest
   const int head = (int)blockIdx.x - row_id * a.Hq;
   const MlaRow mr = mla_row(a, row_id);
@@ -1515,7 +1528,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
       else RPA_MLA_DS(rpa_mla_balanced_kernel, bgrid, false);
       hipError_t eb = hipGetLastError();
       if (eb != hipSuccess) return eb;
-      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(kMergeThreads), 0, stream, a);
       return hipGetLastError();
     }
     if (a.fp8) RPA_MLA_DS(rpa_mla_decode_kernel, grid, true);
@@ -1524,7 +1537,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     hipError_t es = hipGetLastError();
     if (es != hipSuccess) return es;
     if (a.max_splits > 1) {
-      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(kMergeThreads), 0, stream, a);
       es = hipGetLastError();
     }
     return es;
@@ -1543,7 +1556,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
       }
       hipError_t eb = hipGetLastError();
       if (eb != hipSuccess) return eb;
-      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(kMergeThreads), 0, stream, a);
       return hipGetLastError();
     }
     if (pipe) {
@@ -1558,7 +1571,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     hipError_t ef = hipGetLastError();
     if (ef != hipSuccess) return ef;
     if (a.max_splits > 1) {
-      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(kMergeThreads), 0, stream, a);
       ef = hipGetLastError();
     }
     return ef;
@@ -1576,7 +1589,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     else hipLaunchKernelGGL(rpa_mla_balanced_wide_kernel<false>, dim3(a.num_wgs), dim3(256), 0, stream, a);
     hipError_t eb = hipGetLastError();
     if (eb != hipSuccess) return eb;
-    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
+    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(kMergeThreads), 0, stream, a);
     return hipGetLastError();
   }
   if (wide) {
@@ -1585,7 +1598,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     hipError_t ew = hipGetLastError();
     if (ew != hipSuccess) return ew;
     if (a.max_splits > 1) {
-      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
+      hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(kMergeThreads), 0, stream, a);
       ew = hipGetLastError();
     }
     return ew;
@@ -1603,7 +1616,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
     }
     hipError_t eb = hipGetLastError();
     if (eb != hipSuccess) return eb;
-    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
+    hipLaunchKernelGGL(rpa_mla_combine_balanced_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(kMergeThreads), 0, stream, a);
     return hipGetLastError();
   }
   if (pipe) {
@@ -1618,7 +1631,7 @@ hipError_t launch_mla_decode(const MlaDecodeArgs& a, hipStream_t stream) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (a.max_splits > 1) {
-    hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(128), 0, stream, a);
+    hipLaunchKernelGGL(rpa_mla_combine_kernel, dim3((unsigned)a.Hq * (unsigned)a.num_rows), dim3(kMergeThreads), 0, stream, a);
     e = hipGetLastError();
   }
   return e;
