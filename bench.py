@@ -369,9 +369,10 @@ def measure_ceilings(dev, nbytes=2 << 30, reps=5):
     """What this device delivers to the simplest kernels of the attention kernels' shape (csrc/rpa_ceilings.hip,
     lib/librpa_ceilings.so), event-timed on the current stream:
       * a streaming read of `nbytes` of random data, every wave sixteen 16-byte loads per lane in flight, over
-        wave counts from the decode plan's (3.5 per CU) to 32 per CU, contiguous and through a random table of
+        wave counts from 3.5 per CU (the decode plan's: 4) to 32 per CU, contiguous and through a random table of
         256 KiB pages (one page = 64 tokens of 8 kv heads x 128 dims, bf16 K and V), each wave on a contiguous
-        run of blocks or the waves interleaved block by block;
+        run of blocks or the waves interleaved block by block, with plain and with non-temporal loads (the
+        decode kernels' kind);
       * v_mfma_f32_32x32x16_bf16 into four independent accumulators, two waves per SIMD.
     `achievable` holds the best of each: the denominators of frac_of_achievable."""
     import ctypes
@@ -404,18 +405,19 @@ def measure_ceilings(dev, nbytes=2 << 30, reps=5):
         return a.elapsed_time(b) / n
 
     rows = []
-    plan_waves = cus * 4 - cus // 2  # the decode plan's resident waves on 16-bit caches
-    for waves in (plan_waves, cus * 4, cus * 8, cus * 16, cus * 32):
+    plan_waves = cus * 4  # the decode plan's resident waves on long rows (one per SIMD)
+    for waves in (cus * 4 - cus // 2, plan_waves, cus * 8, cus * 16, cus * 32):
         for order in (0, 1):
             for paged in (False, True):
-                def launch():
-                    rc = lib.rpa_ceiling_stream_read(src.data_ptr(), nbytes, table.data_ptr() if paged else None, page_bytes,
-                                                     waves, order, sink.data_ptr(), stream)
-                    if rc != 0:
-                        raise RuntimeError(f"rpa_ceiling_stream_read: hip error {rc}")
-                ms = timed(launch, reps)
-                rows.append({"waves": waves, "order": "contiguous runs" if order == 0 else "interleaved", "paged": paged,
-                             "ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9})
+                for nt in (False, True):
+                    def launch():
+                        rc = lib.rpa_ceiling_stream_read(src.data_ptr(), nbytes, table.data_ptr() if paged else None, page_bytes,
+                                                         waves, order + (4 if nt else 0), sink.data_ptr(), stream)
+                        if rc != 0:
+                            raise RuntimeError(f"rpa_ceiling_stream_read: hip error {rc}")
+                    ms = timed(launch, reps)
+                    rows.append({"waves": waves, "order": "contiguous runs" if order == 0 else "interleaved", "paged": paged,
+                                 "loads": "non-temporal" if nt else "plain", "ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9})
     iters = 2000
     wgs = 2 * cus
 
@@ -433,6 +435,8 @@ def measure_ceilings(dev, nbytes=2 << 30, reps=5):
                 "waves per SIMD, measured in this run" % (nbytes >> 20),
         "achievable": {"hbm_read_gbps_contiguous": best(False), "hbm_read_gbps_paged_256KiB": best(True),
                        "hbm_read_gbps_paged_at_decode_plan_waves": best(True, plan_waves),
+                       "hbm_read_gbps_plain_loads": max(r["gbps"] for r in rows if r["loads"] == "plain"),
+                       "hbm_read_gbps_non_temporal_loads": max(r["gbps"] for r in rows if r["loads"] == "non-temporal"),
                        "mfma_bf16_tflops": mfma_tflops},
         "frac_of_published_peak": {"hbm_contiguous": best(False) / HBM_PEAK_GBPS, "hbm_paged": best(True) / HBM_PEAK_GBPS,
                                    "mfma_bf16": mfma_tflops / MFMA_BF16_PEAK_TFLOPS},

@@ -5,7 +5,8 @@
 //
 //   rpa_ceiling_stream_read   every wave streams 16 KiB blocks (sixteen 16-byte loads per lane in flight, the
 //                             next block requested before the current one is consumed: the decode kernels'
-//                             block and pipeline), contiguous or through a page table, and folds them with xor
+//                             block and pipeline), contiguous or through a page table, with plain or with
+//                             non-temporal loads (what the decode kernels use), and folds them with xor
 //   rpa_ceiling_mfma          every wave issues v_mfma_f32_32x32x16_bf16 into four independent accumulators,
 //                             two waves per SIMD (two workgroups of four waves per CU, held there by LDS size)
 #include <hip/hip_runtime.h>
@@ -23,10 +24,13 @@ struct Block {
   u32x4 v[16];
 };
 
+template <bool NT>
 __device__ __forceinline__ void load_block(Block& b, const char* p, int lane) {
 #pragma unroll
-  for (int i = 0; i < 16; ++i)
-    b.v[i] = *reinterpret_cast<const u32x4*>(p + i * 1024 + lane * 16);
+  for (int i = 0; i < 16; ++i) {
+    const u32x4* q = reinterpret_cast<const u32x4*>(p + i * 1024 + lane * 16);
+    b.v[i] = NT ? __builtin_nontemporal_load(q) : *q;
+  }
 }
 
 __device__ __forceinline__ void fold_block(u32x4& acc, const Block& b) {
@@ -37,6 +41,8 @@ __device__ __forceinline__ void fold_block(u32x4& acc, const Block& b) {
 // order 0: wave w takes the contiguous run of blocks [w * per, (w + 1) * per)  (the balanced decode plan's shape)
 // order 1: wave w takes blocks w, w + waves, w + 2 * waves, ...               (neighbouring waves, neighbouring memory)
 // table != nullptr: block b lives in page table[b / blocks_per_page] at offset (b % blocks_per_page) * 16 KiB
+// NT: non-temporal loads
+template <bool NT>
 __global__ __launch_bounds__(256) void stream_read_kernel(const char* __restrict__ base, const int32_t* __restrict__ table,
                                                           int64_t num_blocks, int blocks_per_page, int64_t page_bytes,
                                                           int order, uint32_t* __restrict__ sink) {
@@ -58,9 +64,9 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const char* __restrict
   u32x4 acc = {0, 0, 0, 0};
   if (b < end) {
     Block cur, nxt;
-    load_block(cur, addr(b), lane);
+    load_block<NT>(cur, addr(b), lane);
     for (b += step; b < end; b += step) {
-      load_block(nxt, addr(b), lane);
+      load_block<NT>(nxt, addr(b), lane);
       fold_block(acc, cur);
       cur = nxt;
     }
@@ -100,14 +106,19 @@ __global__ __launch_bounds__(256) void mfma_issue_kernel(int iters, float* __res
 #define CEIL_API extern "C" __attribute__((visibility("default")))
 
 // Streams `bytes` (a multiple of 16 KiB) from `src` on `waves` wavefronts (a multiple of 4).  `table` (device,
-// nullable) maps page slots to pages of `page_bytes` (a multiple of 16 KiB).  Returns a hipError_t.
+// nullable) maps page slots to pages of `page_bytes` (a multiple of 16 KiB).  `order`: 0 / 1 as above, + 4 for
+// non-temporal loads.  Returns a hipError_t.
 CEIL_API int rpa_ceiling_stream_read(const void* src, int64_t bytes, const int32_t* table, int64_t page_bytes,
                                      int waves, int order, void* sink, void* stream) {
   if (bytes <= 0 || bytes % kBlockBytes || waves <= 0 || waves % 4) return (int)hipErrorInvalidValue;
   if (table != nullptr && (page_bytes <= 0 || page_bytes % kBlockBytes)) return (int)hipErrorInvalidValue;
   const int bpp = table ? (int)(page_bytes / kBlockBytes) : 1;
-  hipLaunchKernelGGL(stream_read_kernel, dim3(waves / 4), dim3(256), 0, (hipStream_t)stream, (const char*)src, table,
-                     bytes / kBlockBytes, bpp, page_bytes, order, (uint32_t*)sink);
+  if (order & 4)
+    hipLaunchKernelGGL(stream_read_kernel<true>, dim3(waves / 4), dim3(256), 0, (hipStream_t)stream, (const char*)src, table,
+                       bytes / kBlockBytes, bpp, page_bytes, order & 3, (uint32_t*)sink);
+  else
+    hipLaunchKernelGGL(stream_read_kernel<false>, dim3(waves / 4), dim3(256), 0, (hipStream_t)stream, (const char*)src, table,
+                       bytes / kBlockBytes, bpp, page_bytes, order & 3, (uint32_t*)sink);
   return (int)hipGetLastError();
 }
 

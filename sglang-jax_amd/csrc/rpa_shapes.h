@@ -82,11 +82,11 @@ constexpr ShapeRule kShapeRules[] = {
   {"decode_256", kStageDecode, 0, 256, 0, 0, 0, 0, 0, 0,
    kKernelRows256, 1, 16, 32, 1, 64, 1, 0, "one wave per (token, kv head, 16 query heads); 5.6-5.75 TB/s on long rows"},
   {"decode_fp8_stream", kStageDecode, 8, 128, 0, 0, 0, 0, 32ll << 20, 0,
-   kKernelDecode, 1, 16, 32, 4, 64, 1, 0, "8 KiB per wave in flight: every wave slot; C4 1024 waves 254 us, 1536 240.5, 2048 238.5"},
+   kKernelDecode, 1, 16, 32, 4, 32, 1, 0, "non-temporal loads: one wave per SIMD; C4 768 waves 226.7 us, 1024 208.7, 1536 245.9, 2048 213.3 (plain loads: 1024 254, 2048 238.5)"},
   {"decode_fp8_small", kStageDecode, 8, 128, 0, 0, 0, 0, 0, 0,
    kKernelDecode, 1, 16, 32, 2, 64, 1, 0, "latency bound: few waves spread over more CUs"},
   {"decode_bf16_stream", kStageDecode, 16, 128, 0, 0, 0, 0, 32ll << 20, 0,
-   kKernelDecode, 1, 16, 32, 4, 28, 1, 0, "14 MB in flight saturate HBM: C2 / C3 896 waves 104.1 / 356 us, 1024 105.2 / 362, 2048 108.5 / 367"},
+   kKernelDecode, 1, 16, 32, 4, 32, 1, 0, "non-temporal loads: one wave per SIMD; C2 / C3 768 waves 96.3 / 354.8 us, 896 90.5 / 326.2, 1024 89.3 / 316.0, 1280 117 / 431, 2048 95.1 / 332.1 (plain loads: 896 104.1 / 356)"},
   {"decode_bf16_small", kStageDecode, 16, 128, 0, 0, 0, 0, 0, 0,
    kKernelDecode, 1, 16, 32, 2, 28, 1, 0, "C1 14.0 us with two waves per workgroup against 15.9 with four"},
   // ---------------- prefill / mixed rows (MFMA bound)

@@ -363,12 +363,12 @@ def test_shape_table_rows_of_the_benchmark_configurations(pkg):
     assert "shape=decode_bf16_small" in c1 and "rpa_decode_splitkv_kernel" in c1 and "waves_per_wg=2" in c1
     assert "prefill" not in c1
     c2 = d(_shape_params(pkg, S=64, decode_end=56, T=8760, Hq=32, Hkv=8, max_q=2048, max_kv=4096, sum_dec=130000))
-    assert "shape=decode_bf16_stream kernel=rpa_decode_balanced_kernel rows=56 waves_per_wg=4 resident_waves=896" in c2
+    assert "shape=decode_bf16_stream kernel=rpa_decode_balanced_kernel rows=56 waves_per_wg=4 resident_waves=1024" in c2
     assert "shape=prefill_pipe kernel=rpa_prefill_pipe_kernel tile=128x1x64 kv_pieces_with_workspace=1" in c2
     c3 = d(_shape_params(pkg, S=16, decode_end=16, T=16, Hq=32, Hkv=8, max_kv=32768, sum_dec=16 * 32768))
     assert "shape=decode_bf16_stream kernel=rpa_decode_splitkv_kernel" in c3 and "merge=rpa_combine_kernel" in c3
     c4 = d(_shape_params(pkg, S=128, decode_end=128, T=128, Hq=64, Hkv=8, fp8=True, max_kv=8192, sum_dec=590000))
-    assert "shape=decode_fp8_stream kernel=rpa_decode_balanced_kernel" in c4 and "resident_waves=2048" in c4
+    assert "shape=decode_fp8_stream kernel=rpa_decode_balanced_kernel" in c4 and "resident_waves=1024" in c4
     # chunks of at most 64 tokens with heads in fours: the short-chunk tile; a long prompt on few heads is cut
     short = d(_shape_params(pkg, S=64, decode_end=0, T=1024, Hq=32, Hkv=8, max_q=16, max_kv=4096))
     assert "shape=prefill_pipe_short" in short and "tile=32x4x64" in short
