@@ -80,7 +80,7 @@ constexpr unsigned kOptPlainOnly = kOptSoftCap | kOptMaskOther | kOptTemperature
 constexpr ShapeRule kShapeRules[] = {
   // ---------------- decode rows (HBM bound: bytes in flight and launch overhead decide)
   {"decode_256", kStageDecode, 0, 256, 0, 0, 0, 0, 0, 0,
-   kKernelRows256, 1, 16, 32, 1, 64, 1, 0, "one wave per (token, kv head, 16 query heads); 5.6-5.75 TB/s on long rows"},
+   kKernelRows256, 1, 16, 32, 1, 64, 1, 0, "one wave per (token, kv head, 16 query heads); 5.9-6.15 TB/s on long rows"},
   {"decode_fp8_stream", kStageDecode, 8, 128, 0, 0, 0, 0, 32ll << 20, 0,
    kKernelDecode, 1, 16, 32, 4, 32, 1, 0, "non-temporal loads: one wave per SIMD; C4 768 waves 226.7 us, 1024 208.7, 1536 245.9, 2048 213.3 (plain loads: 1024 254, 2048 238.5)"},
   {"decode_fp8_small", kStageDecode, 8, 128, 0, 0, 0, 0, 0, 0,
