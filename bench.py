@@ -386,6 +386,8 @@ def measure_ceilings(dev, nbytes=2 << 30, reps=5):
     lib.rpa_ceiling_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64,
                                             ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
     lib.rpa_ceiling_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    lib.rpa_ceiling_lds_dma_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                             ctypes.c_void_p]
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     page_bytes = 256 << 10
@@ -418,6 +420,16 @@ def measure_ceilings(dev, nbytes=2 << 30, reps=5):
                     ms = timed(launch, reps)
                     rows.append({"waves": waves, "order": "contiguous runs" if order == 0 else "interleaved", "paged": paged,
                                  "loads": "non-temporal" if nt else "plain", "ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9})
+    # the same contiguous stream moved into LDS by global_load_lds_dwordx4 (how the prefill and MLA kernels fill their
+    # tile rings), one workgroup of four waves per CU
+    dma_rows = []
+    for nt in (False, True):
+        def launch_dma():
+            rc = lib.rpa_ceiling_lds_dma_read(src.data_ptr(), nbytes, cus * 4, 1 if nt else 0, sink.data_ptr(), stream)
+            if rc != 0:
+                raise RuntimeError(f"rpa_ceiling_lds_dma_read: hip error {rc}")
+        ms = timed(launch_dma, reps)
+        dma_rows.append({"waves": cus * 4, "loads": "non-temporal" if nt else "plain", "ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9})
     iters = 2000
     wgs = 2 * cus
 
@@ -437,10 +449,12 @@ def measure_ceilings(dev, nbytes=2 << 30, reps=5):
                        "hbm_read_gbps_paged_at_decode_plan_waves": best(True, plan_waves),
                        "hbm_read_gbps_plain_loads": max(r["gbps"] for r in rows if r["loads"] == "plain"),
                        "hbm_read_gbps_non_temporal_loads": max(r["gbps"] for r in rows if r["loads"] == "non-temporal"),
+                       "hbm_read_gbps_into_lds_plain": dma_rows[0]["gbps"],
+                       "hbm_read_gbps_into_lds_non_temporal": dma_rows[1]["gbps"],
                        "mfma_bf16_tflops": mfma_tflops},
         "frac_of_published_peak": {"hbm_contiguous": best(False) / HBM_PEAK_GBPS, "hbm_paged": best(True) / HBM_PEAK_GBPS,
                                    "mfma_bf16": mfma_tflops / MFMA_BF16_PEAK_TFLOPS},
-        "mfma_loop_ms": mfma_ms, "stream_read": rows,
+        "mfma_loop_ms": mfma_ms, "stream_read": rows, "stream_read_into_lds": dma_rows,
     }
 
 

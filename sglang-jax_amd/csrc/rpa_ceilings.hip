@@ -7,6 +7,7 @@
 //                             next block requested before the current one is consumed: the decode kernels'
 //                             block and pipeline), contiguous or through a page table, with plain or with
 //                             non-temporal loads (what the decode kernels use), and folds them with xor
+//   rpa_ceiling_lds_dma_read  the same stream moved into LDS by global_load_lds_dwordx4 (the tile rings' way)
 //   rpa_ceiling_mfma          every wave issues v_mfma_f32_32x32x16_bf16 into four independent accumulators,
 //                             two waves per SIMD (two workgroups of four waves per CU, held there by LDS size)
 #include <hip/hip_runtime.h>
@@ -76,6 +77,49 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const char* __restrict
   if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5a17c0deu) sink[0] = (uint32_t)wave;
 }
 
+// The same stream, moved into LDS by global_load_lds_dwordx4 instead of into registers (the way the prefill and MLA
+// kernels fill their tile rings): four waves per workgroup, every wave two 16 KiB buffers, the copies of block i + 1
+// in flight while block i's have landed; one word of every block is read back from LDS and folded.
+template <bool NT>
+__global__ __launch_bounds__(256) void lds_dma_read_kernel(const char* __restrict__ base, int64_t num_blocks,
+                                                          uint32_t* __restrict__ sink) {
+  __shared__ __attribute__((aligned(1024))) char ring[4][2][kBlockBytes];
+  const int lane = threadIdx.x & 63;
+  const int w = threadIdx.x >> 6;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + w;
+  const int64_t waves = (int64_t)gridDim.x * 4;
+  const int64_t per = (num_blocks + waves - 1) / waves;
+  int64_t b = wave * per;
+  const int64_t end = b + per < num_blocks ? b + per : num_blocks;
+  typedef __attribute__((address_space(3))) char* lds_ptr_t;
+  auto copy_block = [&](int slot, int64_t blk) {
+    const char* src = base + blk * kBlockBytes + lane * 16;
+    const uint32_t dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)&ring[w][slot][0]);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if (NT)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(dst + i * 1024), "v"(src + i * 1024) : "memory", "m0");
+      else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst + i * 1024), "v"(src + i * 1024) : "memory", "m0");
+    }
+  };
+  uint32_t acc = 0;
+  if (b < end) {
+    int slot = 0;
+    copy_block(0, b);
+    for (++b; b < end; ++b) {
+      copy_block(slot ^ 1, b);
+      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // all but the newest block's copies have landed
+      acc ^= *reinterpret_cast<const uint32_t*>(&ring[w][slot][lane * 4]);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the slot is read before the block after next overwrites it
+      slot ^= 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    acc ^= *reinterpret_cast<const uint32_t*>(&ring[w][slot][lane * 4]);
+  }
+  if (acc == 0x5a17c0deu) sink[0] = (uint32_t)wave;
+}
+
 __global__ __launch_bounds__(256) void mfma_issue_kernel(int iters, float* __restrict__ sink) {
   extern __shared__ char hold[];  // nothing is kept here: its size limits a CU to two workgroups
   const int lane = threadIdx.x & 63;
@@ -119,6 +163,19 @@ CEIL_API int rpa_ceiling_stream_read(const void* src, int64_t bytes, const int32
   else
     hipLaunchKernelGGL(stream_read_kernel<false>, dim3(waves / 4), dim3(256), 0, (hipStream_t)stream, (const char*)src, table,
                        bytes / kBlockBytes, bpp, page_bytes, order & 3, (uint32_t*)sink);
+  return (int)hipGetLastError();
+}
+
+// The same read through global_load_lds_dwordx4 into LDS: `waves` a multiple of 4, one workgroup of four waves per
+// CU (128 KiB of LDS); nt != 0: with the non-temporal bit.  Returns a hipError_t.
+CEIL_API int rpa_ceiling_lds_dma_read(const void* src, int64_t bytes, int waves, int nt, void* sink, void* stream) {
+  if (bytes <= 0 || bytes % kBlockBytes || waves <= 0 || waves % 4) return (int)hipErrorInvalidValue;
+  if (nt)
+    hipLaunchKernelGGL(lds_dma_read_kernel<true>, dim3(waves / 4), dim3(256), 0, (hipStream_t)stream, (const char*)src,
+                       bytes / kBlockBytes, (uint32_t*)sink);
+  else
+    hipLaunchKernelGGL(lds_dma_read_kernel<false>, dim3(waves / 4), dim3(256), 0, (hipStream_t)stream, (const char*)src,
+                       bytes / kBlockBytes, (uint32_t*)sink);
   return (int)hipGetLastError();
 }
 
