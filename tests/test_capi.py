@@ -64,6 +64,18 @@ def test_library_exports_nothing_but_the_declared_entry_points(pkg):
     assert all(defined[n] == "T" for n in header_functions())
 
 
+def test_measurement_library_exports_its_three_kernels(pkg):
+    """lib/librpa_ceilings.so (bench.py --ceilings) is a library of its own: three launchers, nothing else."""
+    import subprocess
+
+    path = os.path.join(os.path.dirname(pkg._lib.LIB_PATH), "librpa_ceilings.so")
+    assert os.path.exists(path), "build it with __graft_entry__.build()"
+    r = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    names = {ln.split()[2] for ln in r.stdout.splitlines() if len(ln.split()) == 3 and not ln.split()[2].startswith("__hip_")}
+    assert names == {"rpa_ceiling_stream_read", "rpa_ceiling_lds_dma_read", "rpa_ceiling_mfma"}, names
+
+
 def _header_struct_fields(name):
     """Field names of a struct of rpa.h, in declaration order, read from the header's text."""
     text = open(os.path.join(ROOT, "include", "rpa.h")).read()
